@@ -1,0 +1,318 @@
+"""CPU oracle for the fused TTT inner loop -- TEST INFRASTRUCTURE ONLY.
+
+This module restates, in numpy, the arithmetic of the reference's Burn-op inner
+models (the path the reference itself treats as ground truth).  It is the checker
+for the HIP kernels: only the test-suite, the smoke check and the benchmark's
+`cpu_baseline` leg may import it.  Nothing under the product package calls it.
+
+Each function cites the reference lines it follows (paths relative to the
+reference checkout):
+
+  ln_fwd              rust/core/src/util.rs:141-150   (reference/ttt.py:461-475)
+  ln_l2_grad          rust/core/src/util.rs:155-182   (reference/ttt.py:478-505)
+  gelu_tanh           rust/thundercube/src/unary_ops.rs:136-150
+  gelu_tanh_bwd       rust/thundercube/src/unary_ops.rs:152-173 (reference/ttt.py:509-512)
+  linear_mini_batch   rust/core/src/linear.rs:91-149
+  linear_forward      rust/core/src/inner.rs:25-50 + checkpoints as
+                      rust/fused/src/linear_fused_tile/forward/kernel.rs:143-150
+  linear_backward     rust/fused/src/linear_fused_tile/backward/kernel.rs:253-429,
+                      backward/stage.rs:42-1006, layer_norm.rs:428-709
+  mlp_mini_batch      rust/core/src/mlp.rs:127-208
+  mlp_forward         rust/core/src/inner.rs:25-50
+
+How each function is pinned (tests/test_oracle_*.py):
+  ln_fwd            == torch.nn.functional.layer_norm (library routine)
+  ln_l2_grad        == torch autograd of 0.5*||LN(x)-T||^2 w.r.t. x
+  gelu_tanh[_bwd]   == torch gelu(approximate="tanh") and its autograd
+  linear_mini_batch == primal per-token gradient descent written independently
+                       in the test (dual form == primal form invariant), plus the
+                       lr==0 and constant-row closed forms
+  linear_forward    == chaining single mini-batch calls; checkpoint c == state
+                       entering stage c*ci
+  linear_backward   == torch autograd (float64) through the independent primal
+                       formulation, plus central finite differences of
+                       linear_forward
+  mlp_mini_batch    == primal per-token GD on both layers, written in the test
+The reference commits no golden vectors for this path (its fixtures are generated
+at test time), so absolute agreement with Burn-CPU's floating-point results is
+"parity unpinned"; agreement is to tolerance against this float64 restatement.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+GELU_C = 0.7978845608028654  # sqrt(2/pi); reference uses 0.79788456 (unary_ops.rs:136)
+GELU_A = 0.044715
+
+
+# --------------------------------------------------------------------------- LayerNorm
+def ln_fwd(x, gamma, beta, eps=1e-6):
+    """util.rs:141-150. Biased variance, eps inside the sqrt. gamma/beta broadcast on last dim."""
+    mu = x.mean(-1, keepdims=True)
+    var = ((x - mu) ** 2).mean(-1, keepdims=True)
+    std = np.sqrt(var + eps)
+    return gamma * ((x - mu) / std) + beta
+
+
+def ln_l2_grad(x, target, gamma, beta, eps=1e-6):
+    """util.rs:155-182. Returns d/dx 0.5*||LN(x)-target||^2."""
+    d = x.shape[-1]
+    mu = x.mean(-1, keepdims=True)
+    var = ((x - mu) ** 2).mean(-1, keepdims=True)
+    std = np.sqrt(var + eps)
+    xhat = (x - mu) / std
+    out = gamma * xhat + beta
+    dl_dout = out - target
+    dl_dnorm = dl_dout * gamma
+    t1 = dl_dnorm * d
+    t2 = dl_dnorm.sum(-1, keepdims=True)
+    t3 = xhat * (dl_dnorm * xhat).sum(-1, keepdims=True)
+    return (t1 - t2 - t3) / (std * d)
+
+
+# --------------------------------------------------------------------------- GELU
+def gelu_tanh(x):
+    """unary_ops.rs:136-150."""
+    return 0.5 * x * (1.0 + np.tanh(GELU_C * (x + GELU_A * x ** 3)))
+
+
+def gelu_tanh_bwd(x):
+    """unary_ops.rs:152-173; ttt.py:509-512."""
+    t = np.tanh(GELU_C * (x + GELU_A * x ** 3))
+    return 0.5 * (1.0 + t) + 0.5 * x * (1.0 - t * t) * GELU_C * (1.0 + 3.0 * GELU_A * x * x)
+
+
+# --------------------------------------------------------------------------- helpers
+def _hb(p):
+    """[H,d] parameter -> broadcastable [1,H,1,d]."""
+    return p[None, :, None, :]
+
+
+def _eta(token_eta, lr):
+    """linear.rs:111-117: eta[i,j] = token_eta[i]*lr[j], lower triangular. lr [B,H,K]."""
+    k = lr.shape[-1]
+    e = token_eta[None, None, :, None] * lr[:, :, None, :]
+    return e * np.tril(np.ones((k, k), dtype=lr.dtype))
+
+
+def _T(a):
+    return np.swapaxes(a, -1, -2)
+
+
+# --------------------------------------------------------------------------- TTT-Linear
+def linear_mini_batch(W, b, xq, xk, xv, token_eta, lr, gamma, beta, eps=1e-6):
+    """linear.rs:91-149. One mini-batch.
+
+    W [B,H,d,d], b [B,H,d], xq/xk/xv [B,H,K,d], token_eta [K], lr [B,H,K], gamma/beta [H,d].
+    Returns (out [B,H,K,d], W_new, b_new).
+    """
+    k = xq.shape[2]
+    tri = np.tril(np.ones((k, k), dtype=W.dtype))
+    z1 = xk @ W + b[:, :, None, :]                                  # :103
+    target = xv - xk                                                # :105
+    g = ln_l2_grad(z1, target, _hb(gamma), _hb(beta), eps)          # :107-109
+    eta = _eta(token_eta, lr)                                       # :111-117
+    attn = (xq @ _T(xk)) * tri                                      # :119-121
+    b_bar = b[:, :, None, :] - eta @ g                              # :123-124
+    z_bar = xq @ W - (eta * attn) @ g + b_bar                       # :126-128
+    last = eta[:, :, -1, :]                                         # :130-132  [B,H,K]
+    W_new = W - _T(last[..., None] * xk) @ g                        # :134-138
+    b_new = b - (last[..., None] * g).sum(2)                        # :140-144
+    out = xq + ln_fwd(z_bar, _hb(gamma), _hb(beta), eps)            # :146-148
+    return out, W_new, b_new
+
+
+def linear_forward(W0, b0, xq, xk, xv, token_eta, lr, gamma, beta, K=16, eps=1e-6,
+                   checkpoint_interval=0, dtype=np.float64):
+    """inner.rs:25-50: sequential loop over mini-batches; a trailing remainder < K is
+    processed as one short mini-batch (inner.rs:40-47).
+
+    W0 [H,d,d] (or [B,H,d,d]), b0 [H,d] (or [B,H,d]); token_eta is either [seq]
+    (sliced per mini-batch as inner.rs:123-130) or [K] (position inside the mini-batch).
+    If checkpoint_interval > 0 also returns W/b entering every stage c*ci
+    (forward/kernel.rs:143-150), shape [B,H,ceil(N/ci),d,d] / [B,H,ceil(N/ci),d].
+    """
+    xq, xk, xv, lr = (np.asarray(a, dtype=dtype) for a in (xq, xk, xv, lr))
+    gamma, beta = np.asarray(gamma, dtype=dtype), np.asarray(beta, dtype=dtype)
+    token_eta = np.asarray(token_eta, dtype=dtype)
+    B, H, seq, d = xq.shape
+    W = np.asarray(W0, dtype=dtype)
+    b = np.asarray(b0, dtype=dtype)
+    if W.ndim == 3:                                                 # init_state, linear.rs:84-89
+        W = np.broadcast_to(W[None], (B, H, d, d)).copy()
+        b = np.broadcast_to(b[None], (B, H, d)).copy()
+    out = np.zeros_like(xq)
+    Wc, bc = [], []
+    stage = 0
+    for s0 in range(0, seq, K):
+        s1 = min(s0 + K, seq)
+        if checkpoint_interval and stage % checkpoint_interval == 0:
+            Wc.append(W.copy())
+            bc.append(b.copy())
+        te = token_eta[s0:s1] if token_eta.shape[0] == seq and seq != K else token_eta[: s1 - s0]
+        o, W, b = linear_mini_batch(W, b, xq[:, :, s0:s1], xk[:, :, s0:s1], xv[:, :, s0:s1],
+                                    te, lr[:, :, s0:s1], gamma, beta, eps)
+        out[:, :, s0:s1] = o
+        stage += 1
+    if checkpoint_interval:
+        return out, W, b, np.stack(Wc, 2), np.stack(bc, 2)
+    return out, W, b
+
+
+def _ln_l2_parts(z1, target, gamma, beta, eps):
+    d = z1.shape[-1]
+    mu = z1.mean(-1, keepdims=True)
+    std = np.sqrt(((z1 - mu) ** 2).mean(-1, keepdims=True) + eps)
+    xhat = (z1 - mu) / std
+    gO = gamma * xhat + beta - target
+    gx = gO * gamma
+    G = (d * gx - gx.sum(-1, keepdims=True) - xhat * (gx * xhat).sum(-1, keepdims=True)) / (std * d)
+    return xhat, std, gO, gx, G
+
+
+def linear_backward(W0, b0, xq, xk, xv, token_eta, lr, gamma, beta, d_out, K=16, eps=1e-6,
+                    d_W_out=None, d_b_out=None, dtype=np.float64):
+    """Reverse scan over mini-batches (backward/kernel.rs:334-417) applying the one-stage
+    backward (backward/stage.rs:42-1006; second-order LN term layer_norm.rs:428-709).
+
+    seq must be a multiple of K (forward/launch.rs:209-213); token_eta is [K].
+    Returns dict with d_xq,d_xk,d_xv [B,H,seq,d]; d_W0 [B,H,d,d]; d_b0 [B,H,d];
+    d_lr [B,H,seq]; d_token_eta [seq] (per position, summed over batch and heads,
+    backward/kernel.rs:390); d_gamma,d_beta [H,d] (summed over batch; both the output-LN
+    and the through-G contributions, backward/stage.rs:991-994).
+    Upstream grads of the final state default to zero (launch.rs:188-194).
+    """
+    xq, xk, xv, lr, d_out = (np.asarray(a, dtype=dtype) for a in (xq, xk, xv, lr, d_out))
+    gamma, beta = np.asarray(gamma, dtype=dtype), np.asarray(beta, dtype=dtype)
+    te = np.asarray(token_eta, dtype=dtype)
+    B, H, seq, d = xq.shape
+    assert seq % K == 0 and te.shape[0] == K
+    N = seq // K
+    W = np.asarray(W0, dtype=dtype)
+    b = np.asarray(b0, dtype=dtype)
+    if W.ndim == 3:
+        W = np.broadcast_to(W[None], (B, H, d, d)).copy()
+        b = np.broadcast_to(b[None], (B, H, d)).copy()
+    # forward sweep keeping the state entering every stage (checkpoint_interval = 1)
+    Ws, bs = [], []
+    for t in range(N):
+        Ws.append(W)
+        bs.append(b)
+        sl = slice(t * K, (t + 1) * K)
+        _, W, b = linear_mini_batch(W, b, xq[:, :, sl], xk[:, :, sl], xv[:, :, sl], te,
+                                    lr[:, :, sl], gamma, beta, eps)
+    dW = np.zeros((B, H, d, d), dtype) if d_W_out is None else np.asarray(d_W_out, dtype).copy()
+    db = np.zeros((B, H, d), dtype) if d_b_out is None else np.asarray(d_b_out, dtype).copy()
+    g_xq, g_xk, g_xv = np.zeros_like(xq), np.zeros_like(xq), np.zeros_like(xq)
+    g_lr = np.zeros_like(lr)
+    g_te = np.zeros(seq, dtype)
+    g_gamma = np.zeros((H, d), dtype)
+    g_beta = np.zeros((H, d), dtype)
+    gam, bet = _hb(gamma), _hb(beta)
+    tri = np.tril(np.ones((K, K), dtype))
+    for t in range(N - 1, -1, -1):
+        sl = slice(t * K, (t + 1) * K)
+        Q, Kk, V, l = xq[:, :, sl], xk[:, :, sl], xv[:, :, sl], lr[:, :, sl]
+        W, b = Ws[t], bs[t]
+        dO = d_out[:, :, sl]
+        # recompute forward intermediates (stage.rs:123-234)
+        z1 = Kk @ W + b[:, :, None, :]
+        xhat, std, gO, gx, G = _ln_l2_parts(z1, V - Kk, gam, bet, eps)
+        eta = _eta(te, l)
+        A = (Q @ _T(Kk)) * tri
+        zb = Q @ W + b[:, :, None, :] - (eta + eta * A) @ G
+        mu2 = zb.mean(-1, keepdims=True)
+        std2 = np.sqrt(((zb - mu2) ** 2).mean(-1, keepdims=True) + eps)
+        xhat2 = (zb - mu2) / std2
+        last = te[K - 1] * l                                         # [B,H,K]
+        # stage 4: output LayerNorm backward (stage.rs:240-298)
+        g_gamma += (dO * xhat2).sum((0, 2))
+        g_beta += dO.sum((0, 2))
+        gx2 = dO * gam
+        dzb = (d * gx2 - gx2.sum(-1, keepdims=True)
+               - xhat2 * (gx2 * xhat2).sum(-1, keepdims=True)) / (d * std2)
+        # stage 3: dual-form terms (stage.rs:300-648)
+        P = dzb @ _T(G)                                              # [B,H,K,K]
+        dA = -(P * eta) * tri
+        dQ = dO + dzb @ _T(W) + dA @ Kk
+        dK = _T(dA) @ Q - last[..., None] * (G @ _T(dW))
+        S = Kk @ dW + db[:, :, None, :]
+        dG = -_T(eta + eta * A) @ dzb - last[..., None] * S
+        deta = -(P * tri) * (1.0 + A)
+        dlast = -(G * S).sum(-1)                                     # [B,H,K]
+        dl = (deta * te[None, None, :, None]).sum(2) + te[K - 1] * dlast
+        dte = (deta * l[:, :, None, :]).sum(-1)                      # [B,H,K]
+        dte[:, :, K - 1] += (dlast * l).sum(-1)
+        dW_new = dW + _T(Q) @ dzb
+        db_new = db + dzb.sum(2)
+        # stage 2: through G, second-order LayerNorm (layer_norm.rs:428-709)
+        u = -dG / std
+        s1 = u.sum(-1, keepdims=True)
+        s2 = (u * xhat).sum(-1, keepdims=True)
+        dgx = dG / std + s1 / d + xhat * s2 / d
+        dy = gam * dgx
+        dT = -dy
+        g_gamma += (gO * dgx + dy * xhat).sum((0, 2))
+        g_beta += dy.sum((0, 2))
+        dxhat = dy * gam + gx * s2 / d + u * (gx * xhat).sum(-1, keepdims=True) / d
+        dstd = (-(dxhat * xhat + dG * G) / std).sum(-1, keepdims=True)
+        dz1 = dxhat / std - dxhat.sum(-1, keepdims=True) / (d * std) + xhat * dstd / d
+        # stage 1: matmul backward (stage.rs:933-988)
+        g_xq[:, :, sl] = dQ
+        g_xv[:, :, sl] = dT
+        g_xk[:, :, sl] = dK - dT + dz1 @ _T(W)
+        dW = dW_new + _T(Kk) @ dz1
+        db = db_new + dz1.sum(2)
+        g_lr[:, :, sl] = dl
+        g_te[sl] = dte.sum((0, 1))
+    return dict(d_xq=g_xq, d_xk=g_xk, d_xv=g_xv, d_W0=dW, d_b0=db, d_lr=g_lr,
+                d_token_eta=g_te, d_gamma=g_gamma, d_beta=g_beta)
+
+
+# --------------------------------------------------------------------------- TTT-MLP
+def mlp_mini_batch(W1, b1, W2, b2, xq, xk, xv, token_eta, lr, gamma, beta, eps=1e-6):
+    """mlp.rs:127-208. W1 [B,H,d,4d], b1 [B,H,4d], W2 [B,H,4d,d], b2 [B,H,d]."""
+    k = xq.shape[2]
+    tri = np.tril(np.ones((k, k), dtype=W1.dtype))
+    z1 = xk @ W1 + b1[:, :, None, :]                                # :139
+    x2 = gelu_tanh(z1)                                              # :141
+    z2 = x2 @ W2 + b2[:, :, None, :]                                # :143
+    target = xv - xk                                                # :145
+    g2 = ln_l2_grad(z2, target, _hb(gamma), _hb(beta), eps)         # :147-149
+    g1 = (g2 @ _T(W2)) * gelu_tanh_bwd(z1)                          # :151-152
+    eta = _eta(token_eta, lr)                                       # :154-158
+    attn1 = (xq @ _T(xk)) * tri                                     # :160-162
+    b1_bar = b1[:, :, None, :] - eta @ g1                           # :164-165
+    z1_bar = xq @ W1 - (eta * attn1) @ g1 + b1_bar                  # :167-169
+    x2_bar = gelu_tanh(z1_bar)                                      # :171
+    attn2 = (x2_bar @ _T(x2)) * tri                                 # :173
+    b2_bar = b2[:, :, None, :] - eta @ g2                           # :175-176
+    z2_bar = x2_bar @ W2 - (eta * attn2) @ g2 + b2_bar              # :178-180
+    last = eta[:, :, -1, :]                                         # :182-183
+    W1n = W1 - _T(last[..., None] * xk) @ g1                        # :185-188
+    b1n = b1 - (last[..., None] * g1).sum(2)                        # :190-193
+    W2n = W2 - _T(last[..., None] * x2) @ g2                        # :195-198
+    b2n = b2 - (last[..., None] * g2).sum(2)                        # :200-203
+    out = xq + ln_fwd(z2_bar, _hb(gamma), _hb(beta), eps)           # :205-207
+    return out, W1n, b1n, W2n, b2n
+
+
+def mlp_forward(W1_0, b1_0, W2_0, b2_0, xq, xk, xv, token_eta, lr, gamma, beta, K=16,
+                eps=1e-6, dtype=np.float64):
+    """inner.rs:25-50 over mlp_mini_batch. Initial state [H,...] is broadcast over batch
+    (mlp.rs:119-125). Returns (out, W1, b1, W2, b2)."""
+    xq, xk, xv, lr = (np.asarray(a, dtype=dtype) for a in (xq, xk, xv, lr))
+    gamma, beta = np.asarray(gamma, dtype=dtype), np.asarray(beta, dtype=dtype)
+    token_eta = np.asarray(token_eta, dtype=dtype)
+    B, H, seq, d = xq.shape
+    st = [np.asarray(a, dtype=dtype) for a in (W1_0, b1_0, W2_0, b2_0)]
+    if st[0].ndim == 3:
+        st = [np.broadcast_to(a[None], (B,) + a.shape).copy() for a in st]
+    out = np.zeros_like(xq)
+    for s0 in range(0, seq, K):
+        s1 = min(s0 + K, seq)
+        te = token_eta[s0:s1] if token_eta.shape[0] == seq and seq != K else token_eta[: s1 - s0]
+        o, *st = mlp_mini_batch(*st, xq[:, :, s0:s1], xk[:, :, s0:s1], xv[:, :, s0:s1],
+                                te, lr[:, :, s0:s1], gamma, beta, eps)
+        out[:, :, s0:s1] = o
+    return (out, *st)

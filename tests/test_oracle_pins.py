@@ -1,0 +1,285 @@
+"""Pins the numpy oracle against independent statements of the same mathematics.
+
+Nothing here retypes the oracle's dual-form formulas: LayerNorm is torch's library
+routine, G is torch autograd of the reconstruction loss, and the mini-batch result is
+the *primal* per-token gradient-descent form (reference/ttt.py:992-1019 describes it),
+so a dropped term, wrong sign, wrong tril or transposed operand in the oracle fails.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import ttt_oracle as orc
+
+torch.set_default_dtype(torch.float64)
+
+
+def rnd(rng, *shape, scale=1.0):
+    return rng.standard_normal(shape) * scale
+
+
+# ------------------------------------------------------------------ LN / GELU
+def test_ln_fwd_is_torch_layer_norm():
+    rng = np.random.default_rng(0)
+    x, g, b = rnd(rng, 3, 5, 7, 16), rnd(rng, 16), rnd(rng, 16)
+    ref = F.layer_norm(torch.tensor(x), (16,), torch.tensor(g), torch.tensor(b), eps=1e-6)
+    np.testing.assert_allclose(orc.ln_fwd(x, g, b, 1e-6), ref.numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_ln_fwd_constant_rows_give_beta():
+    # validate.py:179-181 style constant inputs: LN of a constant row is beta.
+    x = np.full((2, 3, 8), 0.2)
+    b = np.arange(8.0)
+    np.testing.assert_allclose(orc.ln_fwd(x, np.ones(8), b), np.broadcast_to(b, x.shape), atol=1e-12)
+
+
+@pytest.mark.parametrize("d", [8, 64])
+def test_ln_l2_grad_is_autograd_of_half_sq_loss(d):
+    rng = np.random.default_rng(1)
+    x, t, g, b = rnd(rng, 2, 3, 4, d), rnd(rng, 2, 3, 4, d), rnd(rng, d), rnd(rng, d)
+    xt = torch.tensor(x, requires_grad=True)
+    loss = 0.5 * ((F.layer_norm(xt, (d,), torch.tensor(g), torch.tensor(b), eps=1e-6) - torch.tensor(t)) ** 2).sum()
+    (gx,) = torch.autograd.grad(loss, xt)
+    np.testing.assert_allclose(orc.ln_l2_grad(x, t, g, b, 1e-6), gx.numpy(), rtol=1e-10, atol=1e-12)
+
+
+def test_ln_l2_grad_zero_state_closed_form():
+    # gamma=1,beta=0,x=0 => x_hat=0 and G = -(T - mean T)/sqrt(eps)
+    rng = np.random.default_rng(2)
+    t = rnd(rng, 4, 16)
+    got = orc.ln_l2_grad(np.zeros_like(t), t, np.ones(16), np.zeros(16), 1e-6)
+    np.testing.assert_allclose(got, -(t - t.mean(-1, keepdims=True)) / np.sqrt(1e-6), rtol=1e-12)
+
+
+def test_gelu_matches_torch_tanh_gelu_and_its_derivative():
+    x = np.linspace(-6, 6, 241)
+    xt = torch.tensor(x, requires_grad=True)
+    y = F.gelu(xt, approximate="tanh")
+    (dy,) = torch.autograd.grad(y.sum(), xt)
+    np.testing.assert_allclose(orc.gelu_tanh(x), y.detach().numpy(), rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(orc.gelu_tanh_bwd(x), dy.numpy(), rtol=1e-10, atol=1e-12)
+    # the reference's pre-multiplied constant (ttt.py:511): 3*0.044715*0.79788456
+    assert abs(3 * orc.GELU_A * 0.79788456 - 0.1070322243) < 1e-9
+
+
+# ------------------------------------------------------------------ primal TTT-Linear (torch, independent)
+def primal_linear(W0, b0, xq, xk, xv, te, lr, gamma, beta, K, eps=1e-6, create_graph=False):
+    """Per-token online GD, one token at a time. All tensors torch float64.
+    W0 [B,H,d,d], b0 [B,H,d]; te [K]; returns out, W_final, b_final."""
+    B, H, seq, d = xq.shape
+    W, b = W0, b0
+    outs = []
+    for s0 in range(0, seq, K):
+        k = min(K, seq - s0)
+        xq_, xk_, xv_, lr_ = (a[:, :, s0:s0 + k] for a in (xq, xk, xv, lr))
+        # gradient of the reconstruction loss at the mini-batch's initial state
+        z = torch.einsum("bhki,bhio->bhko", xk_, W) + b[:, :, None, :]
+        if not z.requires_grad:
+            z = z.detach().requires_grad_(True)
+        y = torch.stack([F.layer_norm(z[:, h], (d,), gamma[h], beta[h], eps=eps) for h in range(H)], 1)
+        loss = 0.5 * ((y - (xv_ - xk_)) ** 2).sum()
+        (G,) = torch.autograd.grad(loss, z, create_graph=create_graph)
+        rows = []
+        for i in range(k):
+            Wi, bi = W, b
+            for j in range(i + 1):
+                e = (te[i] * lr_[:, :, j])[..., None, None]
+                Wi = Wi - e * xk_[:, :, j, :, None] * G[:, :, j, None, :]
+                bi = bi - e[..., 0] * G[:, :, j]
+            zi = torch.einsum("bhi,bhio->bho", xq_[:, :, i], Wi) + bi
+            yi = torch.stack([F.layer_norm(zi[:, h], (d,), gamma[h], beta[h], eps=eps) for h in range(H)], 1)
+            rows.append(xq_[:, :, i] + yi)
+        outs.append(torch.stack(rows, 2))
+        W, b = Wi, bi  # state after the last token of the mini-batch
+    return torch.cat(outs, 2), W, b
+
+
+def make_linear_case(seed, B, H, seq, d, K):
+    rng = np.random.default_rng(seed)
+    c = dict(
+        xq=rnd(rng, B, H, seq, d), xk=rnd(rng, B, H, seq, d), xv=rnd(rng, B, H, seq, d),
+        W0=rnd(rng, H, d, d, scale=0.2), b0=rnd(rng, H, d, scale=0.1),
+        gamma=1.0 + rnd(rng, H, d, scale=0.2), beta=rnd(rng, H, d, scale=0.1),
+        lr=rng.uniform(0.01, 0.2, (B, H, seq)), te=1.0 / np.arange(1, K + 1) + rng.uniform(0, 0.1, K),
+    )
+    return c
+
+
+@pytest.mark.parametrize("B,H,seq,d,K", [(2, 2, 12, 8, 4), (1, 3, 16, 16, 16), (2, 1, 11, 8, 4)])
+def test_linear_dual_form_equals_primal_gd(B, H, seq, d, K):
+    c = make_linear_case(10 + seq, B, H, seq, d, K)
+    t = {k: torch.tensor(v) for k, v in c.items()}
+    W0 = t["W0"][None].expand(B, H, d, d)
+    b0 = t["b0"][None].expand(B, H, d)
+    ref_out, ref_W, ref_b = primal_linear(W0, b0, t["xq"], t["xk"], t["xv"], t["te"], t["lr"],
+                                          t["gamma"], t["beta"], K)
+    out, W, b = orc.linear_forward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                                   c["gamma"], c["beta"], K=K)
+    np.testing.assert_allclose(out, ref_out.numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(W, ref_W.numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(b, ref_b.numpy(), rtol=1e-9, atol=1e-10)
+
+
+def test_linear_lr_zero_leaves_state_and_gives_plain_ln():
+    c = make_linear_case(3, 2, 2, 8, 8, 4)
+    c["lr"][:] = 0.0
+    out, W, b = orc.linear_forward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                                   c["gamma"], c["beta"], K=4)
+    z = c["xq"] @ c["W0"][None] + c["b0"][None, :, None, :]
+    exp = c["xq"] + F.layer_norm(torch.tensor(z), (8,), eps=1e-6).numpy() * c["gamma"][None, :, None, :] \
+        + c["beta"][None, :, None, :]
+    np.testing.assert_allclose(out, exp, rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(W, np.broadcast_to(c["W0"][None], W.shape))
+    np.testing.assert_allclose(b, np.broadcast_to(c["b0"][None], b.shape))
+
+
+def test_linear_chained_single_stages_equal_multi_and_checkpoints():
+    # reference tests.rs:49-66: N single-stage calls == one multi-stage call;
+    # checkpoint c holds the state entering stage c*ci (forward/kernel.rs:143-150).
+    B, H, seq, d, K, ci = 2, 2, 32, 8, 4, 3
+    c = make_linear_case(5, B, H, seq, d, K)
+    out, W, b, Wc, bc = orc.linear_forward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                                           c["gamma"], c["beta"], K=K, checkpoint_interval=ci)
+    Ws = np.broadcast_to(c["W0"][None], (B, H, d, d)).copy()
+    bs = np.broadcast_to(c["b0"][None], (B, H, d)).copy()
+    for t in range(seq // K):
+        if t % ci == 0:
+            np.testing.assert_array_equal(Wc[:, :, t // ci], Ws)
+            np.testing.assert_array_equal(bc[:, :, t // ci], bs)
+        sl = slice(t * K, (t + 1) * K)
+        o, Ws, bs = orc.linear_mini_batch(Ws, bs, c["xq"][:, :, sl], c["xk"][:, :, sl], c["xv"][:, :, sl],
+                                          c["te"], c["lr"][:, :, sl], c["gamma"], c["beta"])
+        np.testing.assert_array_equal(out[:, :, sl], o)
+    np.testing.assert_array_equal(W, Ws)
+    assert Wc.shape == (B, H, -(-(seq // K) // ci), d, d)
+
+
+def test_linear_constant_inputs_fixture_shape():
+    # validate.py:179-181: XQ=0.1, XK=0.2, XV=0.3 -> every row of a mini-batch is identical.
+    B, H, seq, d, K = 1, 2, 8, 8, 4
+    c = make_linear_case(6, B, H, seq, d, K)
+    for k, v in (("xq", 0.1), ("xk", 0.2), ("xv", 0.3)):
+        c[k] = np.full((B, H, seq, d), v)
+    c["lr"][:] = 0.0
+    out, _, _ = orc.linear_forward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                                   c["gamma"], c["beta"], K=K)
+    assert np.abs(out - out[:, :, :1]).max() < 1e-12
+
+
+# ------------------------------------------------------------------ backward
+@pytest.mark.parametrize("B,H,N,d,K,state_grads", [(2, 2, 3, 8, 4, False), (1, 2, 2, 8, 4, True)])
+def test_linear_backward_equals_autograd_through_primal(B, H, N, d, K, state_grads):
+    seq = N * K
+    c = make_linear_case(20 + N, B, H, seq, d, K)
+    rng = np.random.default_rng(99)
+    dO = rnd(rng, B, H, seq, d)
+    dWo = rnd(rng, B, H, d, d) if state_grads else None
+    dbo = rnd(rng, B, H, d) if state_grads else None
+    t = {k: torch.tensor(v, requires_grad=True) for k, v in c.items()}
+    W0 = t["W0"][None].expand(B, H, d, d)
+    b0 = t["b0"][None].expand(B, H, d)
+    out, Wf, bf = primal_linear(W0, b0, t["xq"], t["xk"], t["xv"], t["te"], t["lr"],
+                                t["gamma"], t["beta"], K, create_graph=True)
+    loss = (out * torch.tensor(dO)).sum()
+    if state_grads:
+        loss = loss + (Wf * torch.tensor(dWo)).sum() + (bf * torch.tensor(dbo)).sum()
+    names = ["xq", "xk", "xv", "W0", "b0", "lr", "te", "gamma", "beta"]
+    grads = dict(zip(names, torch.autograd.grad(loss, [t[n] for n in names])))
+    got = orc.linear_backward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                              c["gamma"], c["beta"], dO, K=K, d_W_out=dWo, d_b_out=dbo)
+    tol = dict(rtol=1e-7, atol=1e-9)
+    np.testing.assert_allclose(got["d_xq"], grads["xq"].numpy(), **tol)
+    np.testing.assert_allclose(got["d_xk"], grads["xk"].numpy(), **tol)
+    np.testing.assert_allclose(got["d_xv"], grads["xv"].numpy(), **tol)
+    np.testing.assert_allclose(got["d_lr"], grads["lr"].numpy(), **tol)
+    # kernel returns per-batch state grads; the parameter grad is their batch sum
+    np.testing.assert_allclose(got["d_W0"].sum(0), grads["W0"].numpy(), **tol)
+    np.testing.assert_allclose(got["d_b0"].sum(0), grads["b0"].numpy(), **tol)
+    np.testing.assert_allclose(got["d_gamma"], grads["gamma"].numpy(), **tol)
+    np.testing.assert_allclose(got["d_beta"], grads["beta"].numpy(), **tol)
+    # per-position token_eta grads fold mod K onto the K-periodic parameter
+    np.testing.assert_allclose(got["d_token_eta"].reshape(N, K).sum(0), grads["te"].numpy(), **tol)
+
+
+def test_linear_backward_finite_differences_and_linearity():
+    B, H, N, d, K = 1, 1, 2, 4, 4
+    seq = N * K
+    c = make_linear_case(31, B, H, seq, d, K)
+    rng = np.random.default_rng(5)
+    dO = rnd(rng, B, H, seq, d)
+
+    def f(**over):
+        a = {**c, **over}
+        out, _, _ = orc.linear_forward(a["W0"], a["b0"], a["xq"], a["xk"], a["xv"], a["te"], a["lr"],
+                                       a["gamma"], a["beta"], K=K)
+        return (out * dO).sum()
+
+    got = orc.linear_backward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                              c["gamma"], c["beta"], dO, K=K)
+    h = 1e-6
+    for name, key in (("xk", "d_xk"), ("xv", "d_xv"), ("lr", "d_lr"), ("gamma", "d_gamma")):
+        base = c[name]
+        for idx in [tuple(rng.integers(0, s) for s in base.shape) for _ in range(4)]:
+            p, m = base.copy(), base.copy()
+            p[idx] += h
+            m[idx] -= h
+            fd = (f(**{name: p}) - f(**{name: m})) / (2 * h)
+            assert abs(fd - got[key][idx]) <= 1e-5 * max(1.0, abs(fd)), (name, idx, fd, got[key][idx])
+    got2 = orc.linear_backward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                               c["gamma"], c["beta"], 3.0 * dO, K=K)
+    for k in got:
+        np.testing.assert_allclose(got2[k], 3.0 * got[k], rtol=1e-10, atol=1e-12)
+
+
+# ------------------------------------------------------------------ TTT-MLP
+def primal_mlp(W1, b1, W2, b2, xq, xk, xv, te, lr, gamma, beta, K, eps=1e-6):
+    """Per-token GD on both layers (independent of the dual form in mlp.rs)."""
+    B, H, seq, d = xq.shape
+    outs = []
+    for s0 in range(0, seq, K):
+        k = min(K, seq - s0)
+        xq_, xk_, xv_, lr_ = (a[:, :, s0:s0 + k] for a in (xq, xk, xv, lr))
+        W1l = W1.detach().requires_grad_(True)
+        b1l = b1.detach().requires_grad_(True)
+        W2l = W2.detach().requires_grad_(True)
+        b2l = b2.detach().requires_grad_(True)
+        g = [[None] * k for _ in range(4)]
+        for j in range(k):  # per-token parameter gradients at the mini-batch's initial state
+            z1 = torch.einsum("bhi,bhio->bho", xk_[:, :, j], W1l) + b1l
+            z2 = torch.einsum("bhi,bhio->bho", F.gelu(z1, approximate="tanh"), W2l) + b2l
+            y = torch.stack([F.layer_norm(z2[:, h], (d,), gamma[h], beta[h], eps=eps) for h in range(H)], 1)
+            loss = 0.5 * ((y - (xv_[:, :, j] - xk_[:, :, j])) ** 2).sum()
+            gs = torch.autograd.grad(loss, [W1l, b1l, W2l, b2l])
+            for a in range(4):
+                g[a][j] = gs[a]
+        rows = []
+        for i in range(k):
+            cur = [W1, b1, W2, b2]
+            for j in range(i + 1):
+                e = te[i] * lr_[:, :, j]
+                cur = [p - e.reshape(e.shape + (1,) * (p.dim() - 2)) * g[a][j] for a, p in enumerate(cur)]
+            z1 = torch.einsum("bhi,bhio->bho", xq_[:, :, i], cur[0]) + cur[1]
+            z2 = torch.einsum("bhi,bhio->bho", F.gelu(z1, approximate="tanh"), cur[2]) + cur[3]
+            y = torch.stack([F.layer_norm(z2[:, h], (d,), gamma[h], beta[h], eps=eps) for h in range(H)], 1)
+            rows.append(xq_[:, :, i] + y)
+        outs.append(torch.stack(rows, 2))
+        W1, b1, W2, b2 = cur
+    return torch.cat(outs, 2), W1, b1, W2, b2
+
+
+@pytest.mark.parametrize("B,H,seq,d,K", [(2, 2, 8, 4, 4), (1, 2, 7, 8, 4)])
+def test_mlp_dual_form_equals_primal_gd(B, H, seq, d, K):
+    rng = np.random.default_rng(40 + seq)
+    m = 4 * d
+    c = make_linear_case(41 + seq, B, H, seq, d, K)
+    W1, b1 = rnd(rng, H, d, m, scale=0.3), rnd(rng, H, m, scale=0.1)
+    W2, b2 = rnd(rng, H, m, d, scale=0.3), rnd(rng, H, d, scale=0.1)
+    t = {k: torch.tensor(v) for k, v in c.items()}
+    ex = lambda a: torch.tensor(a)[None].expand((B,) + a.shape)
+    ref = primal_mlp(ex(W1), ex(b1), ex(W2), ex(b2), t["xq"], t["xk"], t["xv"], t["te"], t["lr"],
+                     t["gamma"], t["beta"], K)
+    got = orc.mlp_forward(W1, b1, W2, b2, c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                          c["gamma"], c["beta"], K=K)
+    for a, r in zip(got, ref):
+        np.testing.assert_allclose(a, r.numpy(), rtol=1e-8, atol=1e-10)
