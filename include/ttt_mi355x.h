@@ -1,0 +1,129 @@
+/*
+ * ttt_mi355x.h -- C ABI of the MI355X (gfx950) fused TTT inner loop.
+ *
+ * Every entry point is what the reference's FFI for this path would bind.  Paths cited
+ * are relative to the reference (kilyanni/ttt-rs) checkout.
+ *
+ * Conventions
+ *  - All pointers are DEVICE pointers unless stated; the caller owns every buffer; the
+ *    library never allocates or frees device memory and never synchronises: work is
+ *    enqueued on `stream` (a hipStream_t passed as void*; NULL = the default stream).
+ *  - Tensors are contiguous row-major, base pointers 16-byte aligned.
+ *  - Activations xq/xk/xv/out/lr (and their gradients) are stored in `io_dtype`;
+ *    state (W, b), LayerNorm parameters, token_eta and all parameter gradients are f32.
+ *  - Return value: TTT_OK or a negative ttt_status; ttt_last_error() gives the message
+ *    of the calling thread's last failure.  No call aborts the process.
+ */
+#ifndef TTT_MI355X_H
+#define TTT_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  TTT_OK = 0,
+  TTT_ERR_SHAPE = -1,       /* sizes inconsistent (e.g. seq not a multiple of mini_batch) */
+  TTT_ERR_UNSUPPORTED = -2, /* no kernel instantiation for (mini_batch, head_dim, dtype) */
+  TTT_ERR_HIP = -3,         /* a HIP runtime call failed; see ttt_last_error() */
+  TTT_ERR_NULL = -4         /* a required pointer is NULL */
+} ttt_status;
+
+typedef enum { TTT_F32 = 0, TTT_BF16 = 1 } ttt_dtype;
+
+/*
+ * Replaces FusedTttConfig (rust/fused/src/lib.rs:285-328) plus the shapes the reference
+ * reads off its tensors (rust/fused/src/linear_fused_tile/forward/launch.rs:199-226).
+ */
+typedef struct ttt_desc {
+  int32_t batch;               /* B */
+  int32_t heads;               /* H */
+  int32_t seq;                 /* tokens per sequence; must be a multiple of mini_batch */
+  int32_t head_dim;            /* d */
+  int32_t mini_batch;          /* K (1..16) */
+  float eps;                   /* LayerNorm epsilon (reference default 1e-6) */
+  int32_t checkpoint_interval; /* stages between W/b checkpoints, >= 1 */
+  int32_t io_dtype;            /* ttt_dtype of xq, xk, xv, lr, out and their gradients */
+  int32_t state_per_batch;     /* 0: W0/b0 are [H,d,d]/[H,d] shared over the batch
+                                  (TTTLinear::init_state, rust/core/src/linear.rs:84-89);
+                                  1: [B,H,d,d]/[B,H,d] as the reference kernel takes them */
+} ttt_desc;
+
+/* Library / build identification. */
+const char* ttt_version(void);
+/* Message of the calling thread's last error ("" if none). */
+const char* ttt_last_error(void);
+/* TTT_OK if a TTT-Linear kernel exists for this desc, else the status ttt_linear_fwd would
+ * return.  Replaces FusedTttConfig::is_supported (rust/fused/src/lib.rs:313-322). */
+int ttt_linear_supported(const ttt_desc* desc);
+/* Number of checkpoints per (batch, head): ceil((seq/mini_batch)/checkpoint_interval)
+ * (rust/fused/src/linear_fused_tile/forward/launch.rs:221-226). */
+int64_t ttt_linear_num_checkpoints(const ttt_desc* desc);
+
+/*
+ * TTT-Linear multi-stage forward.  Replaces
+ *   FusedKernelBackend<TttTileMultiKernel>::forward
+ *     (rust/kernels/src/kernel.rs:62-69; rust/fused/src/linear_fused_tile/launch.rs:123-161)
+ *   -> forward_multi (rust/fused/src/linear_fused_tile/forward/launch.rs:199-257)
+ * with TttInputs{xq,xk,xv,weight,bias,token_eta,ttt_lr_eta,ln_weight,ln_bias} and
+ * TttOutputs{output,weight,bias} (rust/fused/src/ttt/types.rs:3-13).
+ *
+ *  xq,xk,xv [B,H,seq,d] io   W0 [H,d,d] or [B,H,d,d] f32   b0 [H,d] or [B,H,d] f32
+ *  token_eta [K] f32 (position inside the mini-batch; the reference kernel reads
+ *            token_eta[0..K) of its [seq] tensor, helpers.rs:261-264)
+ *  lr [B,H,seq] io (ttt_lr_eta)        gamma,beta [H,d] f32
+ *  out [B,H,seq,d] io    W_out [B,H,d,d] f32    b_out [B,H,d] f32
+ *  W_ckpt [B,H,C,d,d] f32, b_ckpt [B,H,C,d] f32 with C = ttt_linear_num_checkpoints();
+ *  both may be NULL (no checkpoints written).  Checkpoint c holds the state ENTERING
+ *  stage c*checkpoint_interval (forward/kernel.rs:143-150).
+ */
+int ttt_linear_fwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                   const float* W0, const float* b0, const float* token_eta, const void* lr,
+                   const float* gamma, const float* beta, void* out, float* W_out, float* b_out,
+                   float* W_ckpt, float* b_ckpt, void* stream);
+
+/*
+ * TTT-Linear fused backward.  Replaces
+ *   FusedKernelBackend<TttTileMultiKernel>::backward
+ *     (rust/kernels/src/kernel.rs:71-75; rust/fused/src/linear_fused_tile/launch.rs:163-207)
+ *   -> backward_multi (rust/fused/src/linear_fused_tile/backward/launch.rs:332-438).
+ * Saved state = the nine forward inputs plus the checkpoints written by ttt_linear_fwd
+ * with the same desc (TttSavedStateMulti, launch.rs:30-41).
+ *
+ *  d_out [B,H,seq,d] io.   d_W_out [B,H,d,d], d_b_out [B,H,d] f32: upstream gradients of the
+ *  final state, may be NULL (= zero, which is what the reference assumes, launch.rs:188-194).
+ *  Outputs: d_xq,d_xk,d_xv [B,H,seq,d] io; d_W0 [B,H,d,d] f32 and d_b0 [B,H,d] f32 (per batch
+ *  element; the parameter gradient is their batch sum); d_lr [B,H,seq] io;
+ *  d_token_eta [seq] f32 per position (summed over batch and heads, backward/kernel.rs:390);
+ *  d_gamma,d_beta [H,d] f32 (summed over batch).  The three accumulated outputs
+ *  (d_token_eta, d_gamma, d_beta) are zeroed by the library on `stream` before use.
+ */
+int ttt_linear_bwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                   const float* W0, const float* b0, const float* token_eta, const void* lr,
+                   const float* gamma, const float* beta, const float* W_ckpt,
+                   const float* b_ckpt, const void* d_out, const float* d_W_out,
+                   const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
+                   float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
+                   void* stream);
+
+/*
+ * TTT-MLP multi-stage forward (two-layer inner model d -> 4d -> d, tanh-GELU).  The reference
+ * has no fused kernel for it; this is the fused counterpart of TTTMLP::forward
+ * (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50) behind the same
+ * bundle convention.  W1_0 [H,d,4d] or [B,H,d,4d], b1_0 [H,4d] or [B,H,4d], W2_0 [H,4d,d] or
+ * [B,H,4d,d], b2_0 [H,d] or [B,H,d] (state_per_batch selects); outputs are per batch element.
+ */
+int ttt_mlp_supported(const ttt_desc* desc);
+int ttt_mlp_fwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                void* out, float* W1_out, float* b1_out, float* W2_out, float* b2_out,
+                void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTT_MI355X_H */

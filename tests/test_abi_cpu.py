@@ -1,0 +1,65 @@
+"""CPU-side checks of the C ABI: the library loads, exports every declared symbol, and argument
+validation answers without touching a GPU."""
+import ctypes as C
+import importlib
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ttt_mi355x.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ttt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(P):
+    L = C.CDLL(P.LIB_PATH)
+    syms = declared_symbols()
+    assert set(syms) == set(P.EXPORTS)
+    for s in syms:
+        assert getattr(L, s) is not None
+
+
+def test_version_and_error_strings(P):
+    assert b"gfx950" in P.lib().ttt_version()
+
+
+def desc(P, **kw):
+    base = dict(batch=2, heads=2, seq=32, head_dim=64, mini_batch=16, eps=1e-6,
+                checkpoint_interval=1, io_dtype=P.TTT_F32, state_per_batch=0)
+    base.update(kw)
+    return P.TttDesc(**base)
+
+
+def test_shape_validation(P):
+    L = P.lib()
+    assert L.ttt_linear_supported(C.byref(desc(P))) == P.TTT_OK
+    # seq must be a multiple of mini_batch (forward/launch.rs:209-213 asserts the same)
+    assert L.ttt_linear_supported(C.byref(desc(P, seq=33))) == P.TTT_ERR_SHAPE
+    assert b"multiple" in L.ttt_last_error()
+    assert L.ttt_linear_supported(C.byref(desc(P, head_dim=48))) == P.TTT_ERR_UNSUPPORTED
+    assert L.ttt_linear_supported(C.byref(desc(P, mini_batch=32, seq=64))) == P.TTT_ERR_UNSUPPORTED
+    assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_interval=0))) == P.TTT_ERR_SHAPE
+    assert L.ttt_linear_supported(C.byref(desc(P, io_dtype=7))) == P.TTT_ERR_UNSUPPORTED
+    assert L.ttt_linear_supported(None) == P.TTT_ERR_NULL
+
+
+def test_num_checkpoints(P):
+    L = P.lib()
+    assert L.ttt_linear_num_checkpoints(C.byref(desc(P, seq=16 * 9, checkpoint_interval=4))) == 3
+    assert L.ttt_linear_num_checkpoints(C.byref(desc(P, seq=16 * 8, checkpoint_interval=1))) == 8
+
+
+def test_null_pointers_are_rejected_before_any_launch(P):
+    L = P.lib()
+    rc = L.ttt_linear_fwd(C.byref(desc(P)), *([None] * 15))
+    assert rc == P.TTT_ERR_NULL

@@ -1,0 +1,18 @@
+"""MI355X-native fused TTT inner loop (TTT-Linear / TTT-MLP mini-batch dual form).
+
+Host-side mirror of the reference's inner-model surface (rust/core/src/inner.rs:13-58,
+rust/fused/src/linear_fused_tile/wrapper.rs:81-211) over the C ABI in include/ttt_mi355x.h.
+torch is used only to hold device memory and streams.
+"""
+from ._lib import (TTT_BF16, TTT_ERR_HIP, TTT_ERR_NULL, TTT_ERR_SHAPE, TTT_ERR_UNSUPPORTED,
+                   TTT_F32, TTT_OK, EXPORTS, LIB_PATH, TttDesc, TttError, lib)
+from .inner import (FusedTileMulti, ModelConfig, Qkv, TTTConfig, TTTInputsInner, TTTLinearState,
+                    ttt_linear_forward_raw)
+from . import synthetic
+
+__all__ = [
+    "FusedTileMulti", "ModelConfig", "Qkv", "TTTConfig", "TTTInputsInner", "TTTLinearState",
+    "ttt_linear_forward_raw", "synthetic", "lib", "TttDesc", "TttError", "LIB_PATH", "EXPORTS",
+    "TTT_OK", "TTT_ERR_SHAPE", "TTT_ERR_UNSUPPORTED", "TTT_ERR_HIP", "TTT_ERR_NULL",
+    "TTT_F32", "TTT_BF16",
+]

@@ -1,0 +1,64 @@
+"""ctypes binding of include/ttt_mi355x.h.  Loading fails loudly when the HIP library has not
+been built: there is no CPU fallback anywhere in this package."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libttt_mi355x.so")
+
+TTT_OK, TTT_ERR_SHAPE, TTT_ERR_UNSUPPORTED, TTT_ERR_HIP, TTT_ERR_NULL = 0, -1, -2, -3, -4
+TTT_F32, TTT_BF16 = 0, 1
+
+EXPORTS = (
+    "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_num_checkpoints",
+    "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
+)
+
+
+class TttDesc(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("heads", C.c_int32), ("seq", C.c_int32), ("head_dim", C.c_int32),
+        ("mini_batch", C.c_int32), ("eps", C.c_float), ("checkpoint_interval", C.c_int32),
+        ("io_dtype", C.c_int32), ("state_per_batch", C.c_int32),
+    ]
+
+
+class TttError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"ttt status {code}: {msg}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it first (python ttt-rs_amd/build.py); "
+                "this package has no fallback path")
+        L = C.CDLL(LIB_PATH)
+        vp = C.c_void_p
+        dp = C.POINTER(TttDesc)
+        for name in EXPORTS:
+            getattr(L, name).restype = C.c_int
+        L.ttt_version.restype = C.c_char_p
+        L.ttt_last_error.restype = C.c_char_p
+        L.ttt_linear_supported.argtypes = [dp]
+        L.ttt_linear_num_checkpoints.argtypes = [dp]
+        L.ttt_linear_num_checkpoints.restype = C.c_int64
+        L.ttt_linear_fwd.argtypes = [dp] + [vp] * 15
+        L.ttt_linear_bwd.argtypes = [dp] + [vp] * 24
+        L.ttt_mlp_supported.argtypes = [dp]
+        L.ttt_mlp_fwd.argtypes = [dp] + [vp] * 17
+        _lib = L
+    return _lib
+
+
+def check(rc: int):
+    if rc != TTT_OK:
+        raise TttError(rc, lib().ttt_last_error().decode())

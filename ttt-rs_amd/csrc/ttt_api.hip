@@ -1,0 +1,130 @@
+// C ABI of the MI355X fused TTT inner loop: argument checks and kernel dispatch.
+// Declarations and the reference interfaces they replace: include/ttt_mi355x.h.
+#include "../../include/ttt_mi355x.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "ttt_linear_fwd.hip.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_common(const ttt_desc* d) {
+  if (d == nullptr) return fail(TTT_ERR_NULL, "desc is NULL");
+  if (d->batch <= 0 || d->heads <= 0 || d->seq <= 0 || d->head_dim <= 0 || d->mini_batch <= 0)
+    return fail(TTT_ERR_SHAPE, "batch/heads/seq/head_dim/mini_batch must be positive");
+  if (d->seq % d->mini_batch != 0)
+    return fail(TTT_ERR_SHAPE, "seq (%d) must be a multiple of mini_batch (%d)", d->seq, d->mini_batch);
+  if (d->checkpoint_interval < 1)
+    return fail(TTT_ERR_SHAPE, "checkpoint_interval must be >= 1 (got %d)", d->checkpoint_interval);
+  if (d->io_dtype != TTT_F32 && d->io_dtype != TTT_BF16)
+    return fail(TTT_ERR_UNSUPPORTED, "io_dtype %d is neither TTT_F32 nor TTT_BF16", d->io_dtype);
+  if (!(d->eps > 0.f)) return fail(TTT_ERR_SHAPE, "eps must be positive");
+  if ((int64_t)d->batch * d->heads > 0x7fffffffLL)
+    return fail(TTT_ERR_SHAPE, "batch*heads exceeds the grid limit");
+  return TTT_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int hip_status(hipError_t e, const char* what) {
+  if (e == hipSuccess) return TTT_OK;
+  return fail(TTT_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+template <class T, int D>
+int launch_linear_fwd(const ttt::LinearFwdArgs& a, hipStream_t s) {
+  constexpr int PF = 2;
+  const unsigned grid = (unsigned)(a.B * a.H);
+  hipLaunchKernelGGL((ttt::ttt_linear_fwd_kernel<T, D, PF>), dim3(grid), dim3(64), 0, s, a);
+  return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ttt_version(void) { return "ttt-mi355x 0.1 (gfx950)"; }
+
+const char* ttt_last_error(void) { return g_err; }
+
+int ttt_linear_supported(const ttt_desc* d) {
+  int rc = check_common(d);
+  if (rc != TTT_OK) return rc;
+  if (d->mini_batch > 16)
+    return fail(TTT_ERR_UNSUPPORTED, "mini_batch %d > 16 has no kernel", d->mini_batch);
+  if (d->head_dim != 32 && d->head_dim != 64)
+    return fail(TTT_ERR_UNSUPPORTED, "TTT-Linear head_dim %d has no kernel (32, 64)", d->head_dim);
+  return TTT_OK;
+}
+
+int64_t ttt_linear_num_checkpoints(const ttt_desc* d) {
+  if (check_common(d) != TTT_OK) return -1;
+  const int64_t n = d->seq / d->mini_batch;
+  return (n + d->checkpoint_interval - 1) / d->checkpoint_interval;
+}
+
+int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                   const float* W0, const float* b0, const float* token_eta, const void* lr,
+                   const float* gamma, const float* beta, void* out, float* W_out, float* b_out,
+                   float* W_ckpt, float* b_ckpt, void* stream) {
+  int rc = ttt_linear_supported(d);
+  if (rc != TTT_OK) return rc;
+  if (!xq || !xk || !xv || !W0 || !b0 || !token_eta || !lr || !gamma || !beta || !out || !W_out || !b_out)
+    return fail(TTT_ERR_NULL, "ttt_linear_fwd: a required pointer is NULL");
+  if ((W_ckpt == nullptr) != (b_ckpt == nullptr))
+    return fail(TTT_ERR_NULL, "W_ckpt and b_ckpt must both be given or both be NULL");
+  if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(out))
+    return fail(TTT_ERR_SHAPE, "xq/xk/xv/out must be 16-byte aligned");
+  ttt::LinearFwdArgs a;
+  a.xq = xq; a.xk = xk; a.xv = xv; a.W0 = W0; a.b0 = b0; a.token_eta = token_eta; a.lr = lr;
+  a.gamma = gamma; a.beta = beta; a.out = out; a.W_out = W_out; a.b_out = b_out;
+  a.W_ckpt = W_ckpt; a.b_ckpt = b_ckpt;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.n_stages = d->seq / d->mini_batch;
+  a.ckpt_interval = d->checkpoint_interval;
+  a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
+  a.state_per_batch = d->state_per_batch ? 1 : 0;
+  a.eps = d->eps;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (d->io_dtype == TTT_F32) {
+    if (d->head_dim == 64) return launch_linear_fwd<ttt::F32, 64>(a, s);
+    return launch_linear_fwd<ttt::F32, 32>(a, s);
+  }
+  if (d->head_dim == 64) return launch_linear_fwd<ttt::BF16, 64>(a, s);
+  return launch_linear_fwd<ttt::BF16, 32>(a, s);
+}
+
+int ttt_linear_bwd(const ttt_desc* d, const void*, const void*, const void*, const float*,
+                   const float*, const float*, const void*, const float*, const float*,
+                   const float*, const float*, const void*, const float*, const float*, void*,
+                   void*, void*, float*, float*, void*, float*, float*, float*, void*) {
+  (void)d;
+  return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: not built yet");
+}
+
+int ttt_mlp_supported(const ttt_desc* d) {
+  int rc = check_common(d);
+  if (rc != TTT_OK) return rc;
+  return fail(TTT_ERR_UNSUPPORTED, "ttt_mlp_fwd: not built yet");
+}
+
+int ttt_mlp_fwd(const ttt_desc* d, const void*, const void*, const void*, const float*,
+                const float*, const float*, const float*, const float*, const void*,
+                const float*, const float*, void*, float*, float*, float*, float*, void*) {
+  return ttt_mlp_supported(d);
+}
+
+}  // extern "C"

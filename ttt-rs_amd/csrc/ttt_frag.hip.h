@@ -1,0 +1,160 @@
+// Wave-level building blocks for the gfx950 TTT kernels.
+//
+// One wavefront (64 lanes) is viewed as c = lane & 15 (a column / token index) and
+// g = lane >> 4 (a group of four rows).  All contractions are 16-row MFMAs:
+//
+//   D[m = 4g+r, n = c]  +=  sum_k  A[m = c, k] * B[k, n = c]
+//
+// and a "fragment" is the per-lane slice of one operand for sixteen values of k:
+// lane (c, g) holds slots r = 0..3 standing for k = (g, r).  The pairing of slot and k is
+// the same for A and B, so the k order never has to be the natural one.  This is what lets
+// an accumulator tile D (rows in registers, columns across lanes) be fed back as an operand
+// without moving data:
+//
+//   acc used as B:  B[k = 4g+r, n = c] = D[4g+r, c]      (D itself)
+//   acc used as A:  A[m = c, k = 4g+r] = D[4g+r, c]      (D transposed)
+//
+// Feature axis permutation.  A head_dim index f is split as
+//   f = 32*q + 8*gf + 4*h + r     (q = f/32, gf in 0..3, h in 0..1, r in 0..3)
+// and lives in tile J = 2q+h at in-tile position p = 4*gf + r.  With this choice the eight
+// features a lane needs for tiles 2q and 2q+1 are contiguous in memory
+// (f = 32q + 8g .. 32q + 8g + 7), so a [16 tokens x d] activation tile is fetched with one
+// 16-byte (bf16) or two 16-byte (f32) loads per lane and 32 features.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ttt {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct F32 {};
+struct BF16 {};
+
+// feature index of in-tile position p of tile J
+__device__ __forceinline__ int feat(int J, int p) {
+  return 32 * (J >> 1) + 8 * (p >> 2) + 4 * (J & 1) + (p & 3);
+}
+
+// Sum over the four lane groups g (lanes c, c+16, c+32, c+48); result in every lane.
+__device__ __forceinline__ float xg_sum(float v) {
+#if TTT_XG_SWAP
+  // permlane32_swap(a, b) exchanges a's upper 32 lanes with b's lower 32 lanes; with a == b == v
+  // that leaves {lo,lo} in a and {hi,hi} in b, so a + b is lo + hi in every lane.
+  // permlane16_swap does the same for odd/even rows of 16 lanes.  The two results are copied
+  // into scalars before the float reinterpretation: bit-casting the vector elements in place
+  // makes the front end read element 0 twice.
+  {
+    const uint32_t u = __float_as_uint(v);
+    const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const uint32_t p0 = p[0], p1 = p[1];
+    v = __uint_as_float(p0) + __uint_as_float(p1);
+    const uint32_t w = __float_as_uint(v);
+    const auto q = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    const uint32_t q0 = q[0], q1 = q[1];
+    v = __uint_as_float(q0) + __uint_as_float(q1);
+  }
+#else
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+#endif
+  return v;
+}
+
+template <class T>
+struct Io;
+
+// ---- f32 storage, true-f32 MFMA (v_mfma_f32_16x16x4_f32: one k per lane group and step)
+template <>
+struct Io<F32> {
+  using elem = float;
+  using frag = f32x4;
+  static constexpr int kBytes = 4;
+  __device__ static __forceinline__ frag to_frag(f32x4 v) { return v; }
+  __device__ static __forceinline__ f32x4 to_f32(frag f) { return f; }
+  __device__ static __forceinline__ frag zero() { return frag{0.f, 0.f, 0.f, 0.f}; }
+  __device__ static __forceinline__ void mma(f32x4& acc, frag a, frag b) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], b[r], acc, 0, 0, 0);
+  }
+  __device__ static __forceinline__ void mma2(f32x4& acc, frag a0, frag a1, frag b0, frag b1) {
+    mma(acc, a0, b0);
+    mma(acc, a1, b1);
+  }
+  // eight consecutive elements -> fragments of tiles 2q (lo) and 2q+1 (hi)
+  __device__ static __forceinline__ void load8(const elem* p, bool ok, frag& lo, frag& hi) {
+    if (ok) {
+      lo = *reinterpret_cast<const f32x4*>(p);
+      hi = *reinterpret_cast<const f32x4*>(p + 4);
+    } else {
+      lo = zero();
+      hi = zero();
+    }
+  }
+  __device__ static __forceinline__ void store8(elem* p, f32x4 lo, f32x4 hi) {
+    *reinterpret_cast<f32x4*>(p) = lo;
+    *reinterpret_cast<f32x4*>(p + 4) = hi;
+  }
+  __device__ static __forceinline__ float load1(const elem* p) { return *p; }
+  __device__ static __forceinline__ void store1(elem* p, float v) { *p = v; }
+};
+
+// ---- bf16 storage, bf16 MFMA with f32 accumulation
+template <>
+struct Io<BF16> {
+  using elem = uint16_t;
+  using frag = bf16x4;
+  static constexpr int kBytes = 2;
+  __device__ static __forceinline__ frag to_frag(f32x4 v) { return __builtin_convertvector(v, bf16x4); }
+  __device__ static __forceinline__ f32x4 to_f32(frag f) { return __builtin_convertvector(f, f32x4); }
+  __device__ static __forceinline__ frag zero() {
+    return __builtin_bit_cast(frag, u32x2{0u, 0u});
+  }
+  __device__ static __forceinline__ void mma(f32x4& acc, frag a, frag b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a),
+                                                    __builtin_bit_cast(s16x4, b), acc, 0, 0, 0);
+  }
+  __device__ static __forceinline__ void mma2(f32x4& acc, frag a0, frag a1, frag b0, frag b1) {
+    bf16x8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+    bf16x8 b = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+  }
+  __device__ static __forceinline__ void load8(const elem* p, bool ok, frag& lo, frag& hi) {
+    u32x4 v = ok ? *reinterpret_cast<const u32x4*>(p) : u32x4{0u, 0u, 0u, 0u};
+    lo = __builtin_bit_cast(frag, u32x2{v[0], v[1]});
+    hi = __builtin_bit_cast(frag, u32x2{v[2], v[3]});
+  }
+  __device__ static __forceinline__ void store8(elem* p, f32x4 lo, f32x4 hi) {
+    u32x2 a = __builtin_bit_cast(u32x2, to_frag(lo));
+    u32x2 b = __builtin_bit_cast(u32x2, to_frag(hi));
+    *reinterpret_cast<u32x4*>(p) = u32x4{a[0], a[1], b[0], b[1]};
+  }
+  __device__ static __forceinline__ float load1(const elem* p) {
+    return __builtin_bit_cast(float, static_cast<uint32_t>(*p) << 16);
+  }
+  __device__ static __forceinline__ void store1(elem* p, float v) {
+    *p = __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
+  }
+};
+
+// Identity fragment: as B operand, B[k = 4g+r, n = c] = (c == 4g+r).  acc = mma(0, X, I) turns
+// an A-side fragment X[m = c, k = (g,r)] into the accumulator tile D[4g+r, c] = X^T.
+template <class T>
+__device__ __forceinline__ typename Io<T>::frag identity_frag(int c, int g, float scale = 1.f) {
+  f32x4 v;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) v[r] = (c == 4 * g + r) ? scale : 0.f;
+  return Io<T>::to_frag(v);
+}
+
+template <class T>
+__device__ __forceinline__ typename Io<T>::frag splat_frag(float x) {
+  return Io<T>::to_frag(f32x4{x, x, x, x});
+}
+
+}  // namespace ttt

@@ -1,0 +1,201 @@
+"""Host-side mirror of the reference's inner-model interface for the fused TTT-Linear layer.
+
+Names and argument meaning follow the reference:
+  TTTInnerModel trait            rust/core/src/inner.rs:13-58
+  Qkv / TTTInputsInner           rust/core/src/inner.rs:60-130
+  TTTLinear / TTTLinearState     rust/core/src/linear.rs:17-89
+  Fused<_, TTTLinear, TileMultiKernel> ("fused-tile-multi")
+                                 rust/fused/src/linear_fused_tile/wrapper.rs:81-211
+All arithmetic happens in the HIP library behind include/ttt_mi355x.h.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import TttDesc, check, lib
+
+
+@dataclass
+class TTTConfig:
+    """Subset of rust/config/src/train.rs:11-141 used by the inner loop."""
+    mini_batch_size: int = 16
+    base_lr: float = 1.0
+    epsilon: float = 1e-6
+    checkpoint_interval: int = 1
+    mlp_expansion_factor: int = 4
+
+
+@dataclass
+class ModelConfig:
+    num_heads: int
+    head_dim: int
+    ttt: TTTConfig = field(default_factory=TTTConfig)
+
+
+@dataclass
+class Qkv:
+    """[batch, heads, seq, head_dim] each (inner.rs:60-68)."""
+    xq: torch.Tensor
+    xk: torch.Tensor
+    xv: torch.Tensor
+
+    def slice_seq(self, r: range) -> "Qkv":
+        return Qkv(self.xq[:, :, r.start:r.stop], self.xk[:, :, r.start:r.stop], self.xv[:, :, r.start:r.stop])
+
+
+@dataclass
+class TTTInputsInner:
+    """inner.rs:107-119. token_eta [seq] f32, ttt_lr_eta [batch, heads, seq]."""
+    qkv: Qkv
+    token_eta: torch.Tensor
+    ttt_lr_eta: torch.Tensor
+    start_idx: int = 0
+
+    def slice_seq(self, r: range) -> "TTTInputsInner":
+        return TTTInputsInner(self.qkv.slice_seq(r), self.token_eta[r.start:r.stop],
+                              self.ttt_lr_eta[:, :, r.start:r.stop], r.start)
+
+
+@dataclass
+class TTTLinearState:
+    """linear.rs:27-33: weight [B,H,d,d], bias [B,H,d], always f32."""
+    weight: torch.Tensor
+    bias: torch.Tensor
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _io_dtype(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return _lib.TTT_F32
+    if t.dtype == torch.bfloat16:
+        return _lib.TTT_BF16
+    raise _lib.TttError(_lib.TTT_ERR_UNSUPPORTED, f"activation dtype {t.dtype} (f32 or bf16 only)")
+
+
+def _need(t: torch.Tensor, shape, dtype, name):
+    if tuple(t.shape) != tuple(shape):
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, f"{name}: shape {tuple(t.shape)} != {tuple(shape)}")
+    if t.dtype != dtype:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, f"{name}: dtype {t.dtype} != {dtype}")
+    if not t.is_cuda:
+        raise _lib.TttError(_lib.TTT_ERR_NULL, f"{name} is not a device tensor")
+    return t.contiguous()
+
+
+def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
+                           mini_batch: int, eps: float = 1e-6, checkpoint_interval: int = 1,
+                           want_checkpoints: bool = False):
+    """One call of ttt_linear_fwd on the current stream.
+
+    Counterpart of fused_ttt_tile_forward_multi (rust/fused/src/linear_fused_tile/api.rs:52-83):
+    weight [B,H,d,d] or [H,d,d], bias [B,H,d] or [H,d], token_eta [>=K] (first K entries used).
+    Returns (output, weight_out, bias_out[, weight_ckpt, bias_ckpt]).
+    """
+    B, H, seq, d = xq.shape
+    io = xq.dtype
+    xq = _need(xq, (B, H, seq, d), io, "xq")
+    xk = _need(xk, (B, H, seq, d), io, "xk")
+    xv = _need(xv, (B, H, seq, d), io, "xv")
+    lr = _need(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta")
+    per_batch = weight.dim() == 4
+    weight = _need(weight, (B, H, d, d) if per_batch else (H, d, d), torch.float32, "weight")
+    bias = _need(bias, (B, H, d) if per_batch else (H, d), torch.float32, "bias")
+    ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+    ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+    if token_eta.numel() < mini_batch:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
+    te = token_eta.to(torch.float32).contiguous()
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch))
+    check(lib().ttt_linear_supported(C.byref(desc)))
+    dev = xq.device
+    out = torch.empty_like(xq)
+    w_out = torch.empty((B, H, d, d), dtype=torch.float32, device=dev)
+    b_out = torch.empty((B, H, d), dtype=torch.float32, device=dev)
+    w_ck = b_ck = None
+    if want_checkpoints:
+        n = lib().ttt_linear_num_checkpoints(C.byref(desc))
+        w_ck = torch.empty((B, H, n, d, d), dtype=torch.float32, device=dev)
+        b_ck = torch.empty((B, H, n, d), dtype=torch.float32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_linear_fwd(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(weight), _ptr(bias),
+                                   _ptr(te), _ptr(lr), _ptr(ln_weight), _ptr(ln_bias), _ptr(out),
+                                   _ptr(w_out), _ptr(b_out), _ptr(w_ck), _ptr(b_ck), stream))
+    if want_checkpoints:
+        return out, w_out, b_out, w_ck, b_ck
+    return out, w_out, b_out
+
+
+class FusedTileMulti:
+    """`fused-tile-multi` TTT-Linear layer: Fused<B, TTTLinear<B>, TileMultiKernel>.
+
+    Holds the same parameters as TTTLinear (weight_init [H,d,d], bias_init [H,d], LayerNorm
+    weight/bias [H,d]; linear.rs:17-25) so records are interchangeable with the plain layer
+    (rust/fused/src/lib.rs:183-277).
+    """
+
+    def __init__(self, config: ModelConfig, weight_init, bias_init, ln_weight, ln_bias):
+        H, d = config.num_heads, config.head_dim
+        self.config = config
+        self.weight_init = _need(weight_init, (H, d, d), torch.float32, "weight_init")
+        self.bias_init = _need(bias_init, (H, d), torch.float32, "bias_init")
+        self.ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+        self.ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+
+    @staticmethod
+    def name() -> str:
+        return "FusedTileMultiTTTLinear"  # wrapper.rs:85-87
+
+    @classmethod
+    def new(cls, config: ModelConfig, device, generator: Optional[torch.Generator] = None):
+        """TTTLinear::new (linear.rs:54-78): every parameter ~ Normal(0, 0.02)."""
+        H, d = config.num_heads, config.head_dim
+
+        def init(*shape):
+            return (torch.randn(*shape, generator=generator, dtype=torch.float32) * 0.02).to(device)
+
+        return cls(config, init(H, d, d), init(H, d), init(H, d), init(H, d))
+
+    def get_config(self) -> ModelConfig:
+        return self.config
+
+    def init_state(self, batch_size: int) -> TTTLinearState:
+        """linear.rs:84-89: parameters repeated over the batch."""
+        return TTTLinearState(self.weight_init.unsqueeze(0).repeat(batch_size, 1, 1, 1),
+                              self.bias_init.unsqueeze(0).repeat(batch_size, 1, 1))
+
+    def _launch(self, state: TTTLinearState, inputs: TTTInputsInner, mini_batch: int):
+        t = self.config.ttt
+        out, w, b = ttt_linear_forward_raw(
+            inputs.qkv.xq, inputs.qkv.xk, inputs.qkv.xv, state.weight, state.bias, inputs.token_eta,
+            inputs.ttt_lr_eta, self.ln_weight, self.ln_bias, mini_batch, t.epsilon,
+            t.checkpoint_interval)
+        state.weight, state.bias = w, b
+        return out
+
+    def forward(self, state: TTTLinearState, inputs: TTTInputsInner) -> torch.Tensor:
+        """wrapper.rs:102-164: all full mini-batches in one launch; a trailing remainder is one
+        short mini-batch, as the Burn-op model does it (inner.rs:40-47)."""
+        K = self.config.ttt.mini_batch_size
+        seq = inputs.qkv.xq.shape[2]
+        full = (seq // K) * K
+        outs = []
+        if full > 0:
+            outs.append(self._launch(state, inputs.slice_seq(range(0, full)), K))
+        if full < seq:
+            outs.append(self._launch(state, inputs.slice_seq(range(full, seq)), seq - full))
+        return outs[0] if len(outs) == 1 else torch.cat(outs, 2)
+
+    def forward_mini_batch(self, state: TTTLinearState, inputs: TTTInputsInner, r: range) -> torch.Tensor:
+        """wrapper.rs:166-211: one mini-batch (len(r) <= mini_batch_size)."""
+        if len(r) > self.config.ttt.mini_batch_size or len(r) == 0:
+            raise _lib.TttError(_lib.TTT_ERR_SHAPE, "range longer than mini_batch_size")
+        return self._launch(state, inputs.slice_seq(r), len(r))
