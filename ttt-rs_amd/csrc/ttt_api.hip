@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdio>
 
+#include "ttt_linear_bwd.hip.h"
 #include "ttt_linear_fwd.hip.h"
 
 namespace {
@@ -48,8 +49,24 @@ template <class T, int D>
 int launch_linear_fwd(const ttt::LinearFwdArgs& a, hipStream_t s) {
   constexpr int PF = 2;
   const unsigned grid = (unsigned)(a.B * a.H);
-  hipLaunchKernelGGL((ttt::ttt_linear_fwd_kernel<T, D, PF>), dim3(grid), dim3(64), 0, s, a);
+  if (a.K == 16)
+    hipLaunchKernelGGL((ttt::ttt_linear_fwd_kernel<T, D, PF, true>), dim3(grid), dim3(64), 0, s, a);
+  else
+    hipLaunchKernelGGL((ttt::ttt_linear_fwd_kernel<T, D, PF, false>), dim3(grid), dim3(64), 0, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+}
+
+template <class T, int D>
+int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
+  auto kern = ttt::ttt_linear_bwd_kernel<T, D>;
+  constexpr size_t bytes = ttt::BwdLds<D>::BYTES;
+  // more than the default 64 KiB of LDS per workgroup has to be requested (per device)
+  int rc = hip_status(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
+                      "hipFuncSetAttribute(LDS size)");
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_linear_bwd launch");
 }
 
 }  // namespace
@@ -107,12 +124,51 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   return launch_linear_fwd<ttt::BF16, 32>(a, s);
 }
 
-int ttt_linear_bwd(const ttt_desc* d, const void*, const void*, const void*, const float*,
-                   const float*, const float*, const void*, const float*, const float*,
-                   const float*, const float*, const void*, const float*, const float*, void*,
-                   void*, void*, float*, float*, void*, float*, float*, float*, void*) {
-  (void)d;
-  return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: not built yet");
+int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                   const float* W0, const float* b0, const float* token_eta, const void* lr,
+                   const float* gamma, const float* beta, const float* W_ckpt,
+                   const float* b_ckpt, const void* d_out, const float* d_W_out,
+                   const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
+                   float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
+                   void* stream) {
+  int rc = ttt_linear_supported(d);
+  if (rc != TTT_OK) return rc;
+  // W0/b0 are part of the saved state for interface parity; the state entering every stage is
+  // rebuilt from the checkpoints (checkpoint 0 equals the initial state).
+  (void)W0;
+  (void)b0;
+  if (!xq || !xk || !xv || !token_eta || !lr || !gamma || !beta || !d_out || !d_xq || !d_xk ||
+      !d_xv || !d_W0 || !d_b0 || !d_lr || !d_token_eta || !d_gamma || !d_beta)
+    return fail(TTT_ERR_NULL, "ttt_linear_bwd: a required pointer is NULL");
+  if (!W_ckpt || !b_ckpt)
+    return fail(TTT_ERR_NULL, "ttt_linear_bwd needs the W/b checkpoints written by ttt_linear_fwd");
+  ttt::LinearBwdArgs a;
+  a.xq = xq; a.xk = xk; a.xv = xv; a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta;
+  a.W_ckpt = W_ckpt; a.b_ckpt = b_ckpt; a.d_out = d_out; a.d_W_out = d_W_out; a.d_b_out = d_b_out;
+  a.d_xq = d_xq; a.d_xk = d_xk; a.d_xv = d_xv; a.d_W0 = d_W0; a.d_b0 = d_b0; a.d_lr = d_lr;
+  a.d_token_eta = d_token_eta; a.d_gamma = d_gamma; a.d_beta = d_beta;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.n_stages = d->seq / d->mini_batch;
+  a.ckpt_interval = d->checkpoint_interval;
+  a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
+  a.eps = d->eps;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // accumulated outputs start from zero; a fill kernel (not a memset node) so the sequence
+  // can be captured into a graph
+  const size_t hd = (size_t)d->heads * d->head_dim;
+  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((d->seq + 255) / 256)), dim3(256), 0, s,
+                     d_token_eta, (size_t)d->seq);
+  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((hd + 255) / 256)), dim3(256), 0, s,
+                     d_gamma, hd);
+  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((hd + 255) / 256)), dim3(256), 0, s,
+                     d_beta, hd);
+  const unsigned grid = (unsigned)(a.B * a.H);
+  if (d->io_dtype == TTT_F32) {
+    if (d->head_dim == 64) return launch_linear_bwd<ttt::F32, 64>(a, grid, s);
+    return launch_linear_bwd<ttt::F32, 32>(a, grid, s);
+  }
+  if (d->head_dim == 64) return launch_linear_bwd<ttt::BF16, 64>(a, grid, s);
+  return launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
 }
 
 int ttt_mlp_supported(const ttt_desc* d) {

@@ -1,0 +1,449 @@
+// TTT-Linear fused backward for gfx950: one workgroup (4 wavefronts) per (batch, head).
+//
+// Arithmetic: reverse scan over mini-batches (reference
+// rust/fused/src/linear_fused_tile/backward/kernel.rs:253-429) of the one-stage backward
+// (backward/stage.rs:42-1006; second-order LayerNorm term layer_norm.rs:428-709), with the
+// state entering each stage rebuilt from the forward's checkpoints by re-running the state
+// update (backward/kernel.rs:134-246).  Semantics kept from the reference: upstream gradients
+// of the final state default to zero, d_token_eta is per position and summed over batch and
+// heads with atomics, d_gamma/d_beta carry both the output-LayerNorm and the through-G terms.
+//
+// Design: every operand of a stage ([16 x d] tiles, the [d x d] state W and its gradient dW,
+// the [16 x 16] causal matrices) lives in LDS as f32 with a padded row stride, and all
+// contractions are true-f32 MFMA (v_mfma_f32_16x16x4_f32) whose A/B elements are read from
+// LDS with arbitrary (row, column) strides, so transposed operands cost nothing extra.  dW and
+// db stay in LDS for the whole scan (the reference round-trips them through global memory
+// every stage).  Elementwise work uses thread (t = tid/16, cg = tid%16) for token t and
+// features cg, cg+16, ...; row statistics are 16-lane shuffles.  Arithmetic is f32 for both
+// I/O dtypes; bf16 tensors are converted at the tile loads and stores.
+#pragma once
+#include "ttt_frag.hip.h"
+
+namespace ttt {
+
+struct LinearBwdArgs {
+  const void* xq;
+  const void* xk;
+  const void* xv;
+  const float* token_eta;
+  const void* lr;
+  const float* gamma;
+  const float* beta;
+  const float* W_ckpt;
+  const float* b_ckpt;
+  const void* d_out;
+  const float* d_W_out;
+  const float* d_b_out;
+  void* d_xq;
+  void* d_xk;
+  void* d_xv;
+  float* d_W0;
+  float* d_b0;
+  void* d_lr;
+  float* d_token_eta;
+  float* d_gamma;
+  float* d_beta;
+  int B, H, seq, K, n_stages, ckpt_interval, n_ckpt;
+  float eps;
+};
+
+template <int D>
+struct BwdLds {
+  static constexpr int LD = D + 4;     // padded row stride (floats) of every [*, D] array
+  static constexpr int LK = 17;        // row stride of the [16 x 16] matrices
+  static constexpr int TILE = 16 * LD;
+  static constexpr int WSZ = D * LD;
+  static constexpr int KK = 16 * LK;
+  // offsets in floats
+  static constexpr int W = 0, dW = W + WSZ;
+  static constexpr int XQ = dW + WSZ, XK = XQ + TILE, TG = XK + TILE, DO = TG + TILE, XH = DO + TILE,
+                       G = XH + TILE, XH2 = G + TILE, DZB = XH2 + TILE, S = DZB + TILE,
+                       TMP = S + TILE, DK = TMP + TILE, DZ1 = DK + TILE, DQ = DZ1 + TILE,
+                       DGM = DQ + TILE;
+  static constexpr int A = DGM + TILE, ETA = A + KK, M = ETA + KK, P = M + KK, DA = P + KK,
+                       DETA = DA + KK;
+  static constexpr int b = DETA + KK, db = b + D, gam = db + D, bet = gam + D, lr = bet + D,
+                       te = lr + 16, rstd1 = te + 16, dlast = rstd1 + 16, END = dlast + 16;
+  static constexpr size_t BYTES = sizeof(float) * END;
+};
+
+// C[16*Mt x 16*Nt] (row-major, stride ldc)  = / += / -=  A * B, contraction length Kd (multiple
+// of 4).  A(m,k) = A[m*a_rs + k*a_cs], B(k,n) = B[k*b_rs + n*b_cs].  Output tiles are dealt
+// round-robin to the four waves starting at wave `first`.  MODE 0: set, 1: add, 2: subtract.
+template <int MODE>
+__device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_rs, int a_cs,
+                                       const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
+                                       int wave, int lane, int first = 0) {
+  const int c = lane & 15, g = lane >> 4;
+  const int ntiles = Mt * Nt;
+  for (int tile = (wave - first + 4) & 3; tile < ntiles; tile += 4) {
+    const int tm = tile / Nt, tn = tile - tm * Nt;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float* Ct = C + (16 * tm + 4 * g) * ldc + 16 * tn + c;
+    if (MODE != 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[r] = (MODE == 1) ? Ct[r * ldc] : -Ct[r * ldc];
+    }
+    const float* Ap = A + (16 * tm + c) * a_rs + g * a_cs;
+    const float* Bp = B + g * b_rs + (16 * tn + c) * b_cs;
+#pragma unroll 4
+    for (int k = 0; k < Kd; k += 4)
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ap[k * a_cs], Bp[k * b_rs], acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Ct[r * ldc] = (MODE == 2) ? -acc[r] : acc[r];
+  }
+}
+
+// sum over the 16 lanes that share a token (an aligned group of 16 lanes)
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __shfl_xor(v, 8, 16);
+  v += __shfl_xor(v, 4, 16);
+  v += __shfl_xor(v, 2, 16);
+  v += __shfl_xor(v, 1, 16);
+  return v;
+}
+
+__global__ void ttt_fill_zero_kernel(float* p, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
+template <class T, int D>
+__global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
+  using IO = Io<T>;
+  using elem = typename IO::elem;
+  using L = BwdLds<D>;
+  constexpr int LD = L::LD, LK = L::LK, NJ = D / 16;
+  constexpr float inv_d = 1.0f / D;
+  extern __shared__ float lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int t = tid >> 4, cg = tid & 15;  // elementwise mapping: token t, features cg + 16 j
+  const size_t bh = blockIdx.x;
+  const int h = (int)(bh % a.H);
+  const int K = a.K;
+
+  float* sW = lds + L::W;
+  float* sdW = lds + L::dW;
+  float* sb = lds + L::b;
+  float* sdb = lds + L::db;
+  float* sgam = lds + L::gam;
+  float* sbet = lds + L::bet;
+  float* slr = lds + L::lr;
+  float* ste = lds + L::te;
+
+  // ---- one-time setup
+  for (int i = tid; i < D; i += 256) {
+    sgam[i] = a.gamma[h * D + i];
+    sbet[i] = a.beta[h * D + i];
+    sdb[i] = a.d_b_out ? a.d_b_out[bh * D + i] : 0.f;
+  }
+  for (int i = tid; i < D * D; i += 256) {
+    const int r = i / D, cc = i - r * D;
+    sdW[r * LD + cc] = a.d_W_out ? a.d_W_out[bh * D * D + i] : 0.f;
+  }
+  if (tid < 16) ste[tid] = (tid < K) ? a.token_eta[tid] : 0.f;
+  float dgam_acc[NJ], dbet_acc[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) dgam_acc[j] = dbet_acc[j] = 0.f;
+  __syncthreads();
+  const float te_last = ste[K - 1];
+
+  // load one [K x D] activation tile into LDS as f32 (rows >= K are zero)
+  auto load_tile = [&](float* dst, const void* src, int stage) {
+    const elem* p = static_cast<const elem*>(src) + (bh * a.seq + (size_t)stage * K + t) * D;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) dst[t * LD + cg + 16 * j] = (t < K) ? IO::load1(p + cg + 16 * j) : 0.f;
+  };
+  auto load_lr = [&](int stage) {
+    if (tid < 16)
+      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * a.seq + (size_t)stage * K + tid) : 0.f;
+  };
+
+  // LayerNorm + L2-gradient pieces for this thread's token (row of `z` + bias): returns x_hat,
+  // rstd and G for its NJ features.
+  auto ln1 = [&](const float* z, const float* tg, float (&xh)[NJ], float (&Gv)[NJ], float& rstd) {
+    float zv[NJ], s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      zv[j] = z[t * LD + cg + 16 * j] + sb[cg + 16 * j];
+      s += zv[j];
+    }
+    const float mu = row16_sum(s) * inv_d;
+    float v = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      zv[j] -= mu;
+      v += zv[j] * zv[j];
+    }
+    rstd = __builtin_amdgcn_rsqf(row16_sum(v) * inv_d + a.eps);
+    float gx[NJ], s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const float ga = sgam[cg + 16 * j];
+      xh[j] = zv[j] * rstd;
+      gx[j] = (ga * xh[j] + sbet[cg + 16 * j] - tg[t * LD + cg + 16 * j]) * ga;
+      s1 += gx[j];
+      s2 += gx[j] * xh[j];
+    }
+    s1 = row16_sum(s1) * inv_d;
+    s2 = row16_sum(s2) * inv_d;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) Gv[j] = (gx[j] - s1 - xh[j] * s2) * rstd;
+  };
+
+  for (int st = a.n_stages - 1; st >= 0; --st) {
+    // ================= state entering stage st: checkpoint + re-simulated updates
+    const int ck = st / a.ckpt_interval;
+    {
+      const float* Wg = a.W_ckpt + (bh * a.n_ckpt + ck) * D * D;
+      for (int i = tid; i < D * D; i += 256) {
+        const int r = i / D, cc = i - r * D;
+        sW[r * LD + cc] = Wg[i];
+      }
+      if (tid < D) sb[tid] = a.b_ckpt[(bh * a.n_ckpt + ck) * D + tid];
+    }
+    for (int s2 = ck * a.ckpt_interval; s2 < st; ++s2) {
+      __syncthreads();
+      load_tile(lds + L::XK, a.xk, s2);
+      load_tile(lds + L::TG, a.xv, s2);
+      load_lr(s2);
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) lds[L::TG + t * LD + cg + 16 * j] -= lds[L::XK + t * LD + cg + 16 * j];
+      mm_lds<0>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane);
+      __syncthreads();
+      {
+        float xh[NJ], Gv[NJ], rstd;
+        ln1(lds + L::XH, lds + L::TG, xh, Gv, rstd);
+        const float last = te_last * slr[t];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) lds[L::G + t * LD + cg + 16 * j] = Gv[j] * last;
+      }
+      __syncthreads();
+      // W -= XK^T (last * G) ; b -= colsum(last * G)      (linear.rs:134-144)
+      mm_lds<2>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, 16, wave, lane);
+      if (tid < D) {
+        float s = 0.f;
+        for (int r = 0; r < 16; ++r) s += lds[L::G + r * LD + tid];
+        sb[tid] -= s;
+      }
+    }
+    __syncthreads();
+
+    // ================= load the stage's tiles
+    load_tile(lds + L::XQ, a.xq, st);
+    load_tile(lds + L::XK, a.xk, st);
+    load_tile(lds + L::TG, a.xv, st);
+    load_tile(lds + L::DO, a.d_out, st);
+    load_lr(st);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) lds[L::TG + t * LD + cg + 16 * j] -= lds[L::XK + t * LD + cg + 16 * j];
+    // Z1 = XK W ; Zq = XQ W ; A = XQ XK^T
+    mm_lds<0>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane);
+    mm_lds<0>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, NJ & 3);
+    mm_lds<0>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, (2 * NJ) & 3);
+    __syncthreads();
+
+    // ================= forward intermediates: x_hat, rstd, G; eta, A (tril), M = eta (1 + A)
+    float xh[NJ], Gv[NJ], rstd1;
+    ln1(lds + L::XH, lds + L::TG, xh, Gv, rstd1);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      lds[L::XH + t * LD + cg + 16 * j] = xh[j];
+      lds[L::G + t * LD + cg + 16 * j] = Gv[j];
+    }
+    {
+      const int s = cg;  // (t, s) entry of the [16 x 16] matrices
+      const bool low = s <= t;
+      const float at = low ? lds[L::A + t * LK + s] : 0.f;
+      const float et = low ? ste[t] * slr[s] : 0.f;
+      lds[L::A + t * LK + s] = at;
+      lds[L::ETA + t * LK + s] = et;
+      lds[L::M + t * LK + s] = et * (1.f + at);
+    }
+    __syncthreads();
+    // Zb = XQ W - M G  (+ b added when read)
+    mm_lds<2>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NJ, 16, wave, lane);
+    __syncthreads();
+
+    // ================= output LayerNorm and its backward (stage 4)
+    {
+      float zv[NJ], s = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        zv[j] = lds[L::XH2 + t * LD + cg + 16 * j] + sb[cg + 16 * j];
+        s += zv[j];
+      }
+      const float mu = row16_sum(s) * inv_d;
+      float v = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        zv[j] -= mu;
+        v += zv[j] * zv[j];
+      }
+      const float rstd2 = __builtin_amdgcn_rsqf(row16_sum(v) * inv_d + a.eps);
+      float gx2[NJ], s1 = 0.f, s2 = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const float x2 = zv[j] * rstd2;
+        const float dO = lds[L::DO + t * LD + cg + 16 * j];
+        dgam_acc[j] += dO * x2;
+        dbet_acc[j] += dO;
+        gx2[j] = dO * sgam[cg + 16 * j];
+        s1 += gx2[j];
+        s2 += gx2[j] * x2;
+        zv[j] = x2;
+      }
+      s1 = row16_sum(s1) * inv_d;
+      s2 = row16_sum(s2) * inv_d;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) lds[L::DZB + t * LD + cg + 16 * j] = (gx2[j] - s1 - zv[j] * s2) * rstd2;
+    }
+    __syncthreads();
+
+    // ================= P = dZb G^T ; dQ = dZb W^T ; S = XK dW ; TMP = G dW^T
+    mm_lds<0>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, 1, 1, D, wave, lane, 0);
+    mm_lds<0>(lds + L::DQ, LD, lds + L::DZB, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 1);
+    mm_lds<0>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, LD, 1, 1, NJ, D, wave, lane, (1 + NJ) & 3);
+    mm_lds<0>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, LD, 1, NJ, D, wave, lane, (1 + 2 * NJ) & 3);
+    __syncthreads();
+
+    // ================= dA, d eta ; S += db ; dlast
+    {
+      const int s = cg;
+      const bool low = s <= t;
+      const float p = lds[L::P + t * LK + s];
+      lds[L::DA + t * LK + s] = low ? -p * lds[L::ETA + t * LK + s] : 0.f;
+      lds[L::DETA + t * LK + s] = low ? -p * (1.f + lds[L::A + t * LK + s]) : 0.f;
+      float dl = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const float sv = lds[L::S + t * LD + cg + 16 * j] + sdb[cg + 16 * j];
+        lds[L::S + t * LD + cg + 16 * j] = sv;
+        dl += Gv[j] * sv;
+      }
+      dl = row16_sum(dl);
+      if (cg == 0) lds[L::dlast + t] = -dl;
+    }
+    __syncthreads();
+
+    // ================= dQ += dA XK ; dK = dA^T XQ ; DGM = M^T dZb ; dW += XQ^T dZb ; db += colsum(dZb)
+    mm_lds<1>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NJ, 16, wave, lane, 0);
+    mm_lds<0>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NJ, 16, wave, lane, NJ & 3);
+    mm_lds<0>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, 1, NJ, 16, wave, lane, (2 * NJ) & 3);
+    mm_lds<1>(sdW, LD, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, 16, wave, lane, (3 * NJ) & 3);
+    if (tid < D) {
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += lds[L::DZB + r * LD + tid];
+      sdb[tid] += s;
+    }
+    // d lr and d token_eta (16 threads each)
+    if (tid < 16) {
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += lds[L::DETA + r * LK + tid] * ste[r];
+      s += te_last * lds[L::dlast + tid];
+      if (tid < K) IO::store1(static_cast<elem*>(a.d_lr) + bh * a.seq + (size_t)st * K + tid, s);
+    } else if (tid >= 64 && tid < 80) {
+      const int tt = tid - 64;
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += lds[L::DETA + tt * LK + r] * slr[r];
+      if (tt == K - 1)
+        for (int r = 0; r < 16; ++r) s += lds[L::dlast + r] * slr[r];
+      if (tt < K) atomicAdd(a.d_token_eta + (size_t)st * K + tt, s);
+    }
+    __syncthreads();
+
+    // ================= through G: second-order LayerNorm (stage 2), token-local
+    {
+      const float last = te_last * slr[t];
+      float dG[NJ], u[NJ], gO[NJ], gx[NJ], s1 = 0.f, s2 = 0.f, sgx = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int o = cg + 16 * j;
+        dG[j] = -lds[L::DGM + t * LD + o] - last * lds[L::S + t * LD + o];
+        u[j] = -dG[j] * rstd1;
+        gO[j] = sgam[o] * xh[j] + sbet[o] - lds[L::TG + t * LD + o];
+        gx[j] = gO[j] * sgam[o];
+        s1 += u[j];
+        s2 += u[j] * xh[j];
+        sgx += gx[j] * xh[j];
+      }
+      s1 = row16_sum(s1) * inv_d;
+      s2 = row16_sum(s2) * inv_d;
+      sgx = row16_sum(sgx) * inv_d;
+      float dxh[NJ], dy[NJ], q1 = 0.f, q2 = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int o = cg + 16 * j;
+        const float dgx = -u[j] + s1 + xh[j] * s2;
+        dy[j] = sgam[o] * dgx;
+        dgam_acc[j] += gO[j] * dgx + dy[j] * xh[j];
+        dbet_acc[j] += dy[j];
+        dxh[j] = dy[j] * sgam[o] + gx[j] * s2 + u[j] * sgx;
+        q1 += dxh[j];
+        q2 += dxh[j] * xh[j] + dG[j] * Gv[j];
+      }
+      q1 = row16_sum(q1) * inv_d;
+      const float dsig = -row16_sum(q2) * rstd1;  // d loss / d sigma
+      elem* pv = static_cast<elem*>(a.d_xv) + (bh * a.seq + (size_t)st * K + t) * D;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int o = cg + 16 * j;
+        lds[L::DZ1 + t * LD + o] = (dxh[j] - q1) * rstd1 + xh[j] * dsig * inv_d;
+        // dXV = dT = -dy ; dXK collects dA^T XQ - last (G dW'^T) - dT
+        if (t < K) IO::store1(pv + o, -dy[j]);
+        lds[L::DK + t * LD + o] += dy[j] - last * lds[L::TMP + t * LD + o];
+      }
+    }
+    __syncthreads();
+
+    // ================= dK += dZ1 W^T ; dW += XK^T dZ1 ; db += colsum(dZ1)
+    mm_lds<1>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 0);
+    mm_lds<1>(sdW, LD, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, 16, wave, lane, NJ & 3);
+    if (tid < D) {
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += lds[L::DZ1 + r * LD + tid];
+      sdb[tid] += s;
+    }
+    __syncthreads();
+
+    // ================= store dXQ = dO + dQ, dXK
+    if (t < K) {
+      elem* pq = static_cast<elem*>(a.d_xq) + (bh * a.seq + (size_t)st * K + t) * D;
+      elem* pk = static_cast<elem*>(a.d_xk) + (bh * a.seq + (size_t)st * K + t) * D;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int o = cg + 16 * j;
+        IO::store1(pq + o, lds[L::DQ + t * LD + o] + lds[L::DO + t * LD + o]);
+        IO::store1(pk + o, lds[L::DK + t * LD + o]);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- results carried over the whole scan
+  for (int i = tid; i < D * D; i += 256) {
+    const int r = i / D, cc = i - r * D;
+    a.d_W0[bh * D * D + i] = sdW[r * LD + cc];
+  }
+  if (tid < D) a.d_b0[bh * D + tid] = sdb[tid];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    lds[L::XQ + t * LD + cg + 16 * j] = dgam_acc[j];
+    lds[L::XK + t * LD + cg + 16 * j] = dbet_acc[j];
+  }
+  __syncthreads();
+  if (tid < D) {
+    float sg = 0.f, sbt = 0.f;
+    for (int r = 0; r < 16; ++r) {
+      sg += lds[L::XQ + r * LD + tid];
+      sbt += lds[L::XK + r * LD + tid];
+    }
+    atomicAdd(a.d_gamma + h * D + tid, sg);
+    atomicAdd(a.d_beta + h * D + tid, sbt);
+  }
+}
+
+}  // namespace ttt

@@ -47,13 +47,16 @@ struct StageIn {
   float lr;
 };
 
-template <class T, int D>
+// FULL: mini_batch == 16, so every lane has a token; a prefetch past the last stage re-reads the
+// last stage instead of branching.
+template <class T, int D, bool FULL>
 __device__ __forceinline__ void load_stage(StageIn<T, D / 16>& s, const LinearFwdArgs& a, size_t bh,
                                            int stage, int c, int g) {
   using IO = Io<T>;
   using elem = typename IO::elem;
   constexpr int NT = D / 16;
-  const bool ok = (c < a.K) && (stage < a.n_stages);
+  if (FULL) stage = min(stage, a.n_stages - 1);
+  const bool ok = FULL || ((c < a.K) && (stage < a.n_stages));
   const size_t tok = bh * a.seq + (size_t)stage * a.K + c;
   const elem* pq = static_cast<const elem*>(a.xq) + tok * D + 8 * g;
   const elem* pk = static_cast<const elem*>(a.xk) + tok * D + 8 * g;
@@ -76,7 +79,7 @@ __device__ __forceinline__ float row_sum(const f32x4 (&v)[NT]) {
   return xg_sum(s);
 }
 
-template <class T, int D, int PF>
+template <class T, int D, int PF, bool FULL>
 __global__ void __launch_bounds__(64) ttt_linear_fwd_kernel(LinearFwdArgs a) {
   using IO = Io<T>;
   using frag = typename IO::frag;
@@ -120,7 +123,7 @@ __global__ void __launch_bounds__(64) ttt_linear_fwd_kernel(LinearFwdArgs a) {
 
   StageIn<T, NT> buf[PF];
 #pragma unroll
-  for (int u = 0; u < PF; ++u) load_stage<T, D>(buf[u], a, bh, u, c, g);
+  for (int u = 0; u < PF; ++u) load_stage<T, D, FULL>(buf[u], a, bh, u, c, g);
 
   for (int st0 = 0; st0 < a.n_stages; st0 += PF) {
 #pragma unroll
@@ -128,7 +131,7 @@ __global__ void __launch_bounds__(64) ttt_linear_fwd_kernel(LinearFwdArgs a) {
       const int st = st0 + u;
       if (st >= a.n_stages) break;
       const StageIn<T, NT> cur = buf[u];
-      load_stage<T, D>(buf[u], a, bh, st + PF, c, g);  // prefetch; consumed PF stages later
+      load_stage<T, D, FULL>(buf[u], a, bh, st + PF, c, g);  // prefetch; consumed PF stages later
 
       // ---- checkpoint: state entering stage st
       if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
@@ -184,7 +187,7 @@ __global__ void __launch_bounds__(64) ttt_linear_fwd_kernel(LinearFwdArgs a) {
 #pragma unroll
         for (int J = 0; J < NT; ++J) sq[J] = xh[J] * xh[J];
         const float var = row_sum<NT>(sq) * inv_d;
-        const float rstd = 1.0f / sqrtf(var + a.eps);
+        const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
         f32x4 gx[NT], gxx[NT];
 #pragma unroll
         for (int J = 0; J < NT; ++J) {
@@ -228,8 +231,8 @@ __global__ void __launch_bounds__(64) ttt_linear_fwd_kernel(LinearFwdArgs a) {
           sq[J] = zb[J] * zb[J];
         }
         const float var = row_sum<NT>(sq) * inv_d;
-        const float rstd = 1.0f / sqrtf(var + a.eps);
-        if (c < K) {
+        const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+        if (FULL || c < K) {
           elem* po = static_cast<elem*>(a.out) + (bh * a.seq + (size_t)st * K + c) * D + 8 * g;
 #pragma unroll
           for (int q = 0; q < NT / 2; ++q) {

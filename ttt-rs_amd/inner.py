@@ -134,6 +134,58 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
     return out, w_out, b_out
 
 
+def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
+                            weight_ckpt, bias_ckpt, grad_output, mini_batch: int, eps: float = 1e-6,
+                            checkpoint_interval: int = 1, grad_weight_out=None, grad_bias_out=None):
+    """One call of ttt_linear_bwd on the current stream.
+
+    Counterpart of backward_multi (rust/fused/src/linear_fused_tile/backward/launch.rs:332-438).
+    Returns a dict with the nine input gradients named as TttGradInputs
+    (backward/launch.rs:427-437): grad_xq, grad_xk, grad_xv, grad_weight [B,H,d,d],
+    grad_bias [B,H,d], grad_ttt_lr_eta, grad_token_eta [seq], grad_ln_weight, grad_ln_bias.
+    """
+    B, H, seq, d = xq.shape
+    io = xq.dtype
+    xq = _need(xq, (B, H, seq, d), io, "xq")
+    xk = _need(xk, (B, H, seq, d), io, "xk")
+    xv = _need(xv, (B, H, seq, d), io, "xv")
+    go = _need(grad_output, (B, H, seq, d), io, "grad_output")
+    lr = _need(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta")
+    per_batch = weight.dim() == 4
+    weight = _need(weight, (B, H, d, d) if per_batch else (H, d, d), torch.float32, "weight")
+    bias = _need(bias, (B, H, d) if per_batch else (H, d), torch.float32, "bias")
+    ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+    ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+    te = token_eta.to(torch.float32).contiguous()
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch))
+    check(lib().ttt_linear_supported(C.byref(desc)))
+    n = lib().ttt_linear_num_checkpoints(C.byref(desc))
+    w_ck = _need(weight_ckpt, (B, H, n, d, d), torch.float32, "weight_ckpt")
+    b_ck = _need(bias_ckpt, (B, H, n, d), torch.float32, "bias_ckpt")
+    if grad_weight_out is not None:
+        grad_weight_out = _need(grad_weight_out, (B, H, d, d), torch.float32, "grad_weight_out")
+        grad_bias_out = _need(grad_bias_out, (B, H, d), torch.float32, "grad_bias_out")
+    dev = xq.device
+    g = dict(
+        grad_xq=torch.empty_like(xq), grad_xk=torch.empty_like(xq), grad_xv=torch.empty_like(xq),
+        grad_weight=torch.empty((B, H, d, d), dtype=torch.float32, device=dev),
+        grad_bias=torch.empty((B, H, d), dtype=torch.float32, device=dev),
+        grad_ttt_lr_eta=torch.empty_like(lr),
+        grad_token_eta=torch.empty((seq,), dtype=torch.float32, device=dev),
+        grad_ln_weight=torch.empty((H, d), dtype=torch.float32, device=dev),
+        grad_ln_bias=torch.empty((H, d), dtype=torch.float32, device=dev),
+    )
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_linear_bwd(
+            C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(weight), _ptr(bias), _ptr(te), _ptr(lr),
+            _ptr(ln_weight), _ptr(ln_bias), _ptr(w_ck), _ptr(b_ck), _ptr(go), _ptr(grad_weight_out),
+            _ptr(grad_bias_out), _ptr(g["grad_xq"]), _ptr(g["grad_xk"]), _ptr(g["grad_xv"]),
+            _ptr(g["grad_weight"]), _ptr(g["grad_bias"]), _ptr(g["grad_ttt_lr_eta"]),
+            _ptr(g["grad_token_eta"]), _ptr(g["grad_ln_weight"]), _ptr(g["grad_ln_bias"]), stream))
+    return g
+
+
 class FusedTileMulti:
     """`fused-tile-multi` TTT-Linear layer: Fused<B, TTTLinear<B>, TileMultiKernel>.
 
