@@ -1,0 +1,84 @@
+"""GPU parity: ttt_mlp_fwd and the LDS-resident TTT-Linear forward (head_dim 96/128) through the
+C ABI against the float64 oracle."""
+import importlib
+
+import pytest
+import torch
+
+from helpers import TOL, assert_close, np_inputs, to_dev
+from oracle import ttt_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+def mlp_case(P, seed, B, H, seq, d, K, dtype, style):
+    if style == "baseline":
+        return P.synthetic.baseline_inputs(3, B, H, seq, d, K, io_dtype=dtype, mlp=True)
+    c = P.synthetic.reference_test_inputs(seed, B, H, seq, d, K, io_dtype=dtype)
+    g = torch.Generator().manual_seed(seed + 1)
+    n = lambda *s: torch.randn(*s, generator=g) * 0.02
+    c.pop("W0"), c.pop("b0")
+    c["W1"], c["b1"], c["W2"], c["b2"] = n(H, d, 4 * d), n(H, 4 * d), n(H, 4 * d, d), n(H, d)
+    return c
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("style", ["ref", "baseline"])
+@pytest.mark.parametrize("B,H,d,K,N", [(2, 2, 32, 8, 3), (1, 2, 64, 16, 4), (2, 2, 96, 16, 4),
+                                       (1, 2, 128, 16, 3), (1, 1, 96, 7, 2)])
+def test_mlp_fwd_matches_oracle(P, B, H, d, K, N, style, dtype):
+    print(f"case mlp {style} B{B} H{H} d{d} K{K} N{N} {dtype}", flush=True)
+    c = mlp_case(P, 200 + d + K, B, H, N * K, d, K, dtype, style)
+    dv = to_dev(c)
+    got = P.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
+                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
+                          n["lr"], n["gamma"], n["beta"], K=K)
+    # arithmetic is f32 for both I/O dtypes; only the stored output is rounded for bf16
+    for name, g, r in zip(("out", "W1", "b1", "W2", "b2"), got, ref):
+        assert_close(g, r, TOL[dtype] if name == "out" else 1e-4, name)
+
+
+def test_mlp_inner_model_with_remainder(P):
+    print("case mlp remainder", flush=True)
+    B, H, d, K, seq = 2, 2, 64, 16, 37
+    c = mlp_case(P, 31, B, H, seq, d, K, torch.float32, "ref")
+    te_seq = c["token_eta"].repeat(seq // K + 1)[:seq]
+    dv = to_dev(c)
+    model = P.FusedMlp(P.ModelConfig(H, d, P.TTTConfig(mini_batch_size=K)), dv["W1"], dv["b1"], dv["W2"],
+                       dv["b2"], dv["gamma"], dv["beta"])
+    state = model.init_state(B)
+    out = model.forward(state, P.TTTInputsInner(P.Qkv(dv["xq"], dv["xk"], dv["xv"]), te_seq.to("cuda:0"),
+                                                dv["lr"]))
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"],
+                          te_seq.double().numpy(), n["lr"], n["gamma"], n["beta"], K=K)
+    for name, g, r in zip(("out", "W1", "b1", "W2", "b2"), (out, state.w1, state.b1, state.w2, state.b2), ref):
+        assert_close(g, r, 1e-4, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("B,H,d,K,N,ci", [(2, 2, 96, 16, 4, 1), (1, 3, 128, 16, 5, 2), (1, 2, 128, 6, 3, 1)])
+def test_linear_fwd_wide_heads(P, B, H, d, K, N, ci, dtype):
+    """head_dim 96 / 128 run the LDS-resident kernel (f32 arithmetic for both I/O dtypes)."""
+    print(f"case linear wide B{B} H{H} d{d} K{K} N{N} ci{ci} {dtype}", flush=True)
+    c = P.synthetic.reference_test_inputs(300 + d, B, H, N * K, d, K, io_dtype=dtype)
+    dv = to_dev(c)
+    out, W, b, Wc, bc = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
+                                                 dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K,
+                                                 1e-6, ci, want_checkpoints=True)
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ro, rW, rb, rWc, rbc = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"],
+                                              n["lr"], n["gamma"], n["beta"], K=K, checkpoint_interval=ci)
+    assert_close(out, ro, TOL[dtype], "out")
+    for name, g, r in (("W", W, rW), ("b", b, rb), ("W_ckpt", Wc, rWc), ("b_ckpt", bc, rbc)):
+        assert_close(g, r, 1e-4, name)

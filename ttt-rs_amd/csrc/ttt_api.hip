@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdio>
 
+#include "ttt_engine_fwd.hip.h"
 #include "ttt_linear_bwd.hip.h"
 #include "ttt_linear_fwd.hip.h"
 
@@ -56,14 +57,39 @@ int launch_linear_fwd(const ttt::LinearFwdArgs& a, hipStream_t s) {
   return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
 }
 
+template <class K>
+int opt_in_lds(K kern, size_t bytes) {
+  // more than the default 64 KiB of LDS per workgroup has to be requested (per device)
+  return hip_status(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
+                    "hipFuncSetAttribute(LDS size)");
+}
+
+template <class T, int D>
+int launch_linear_fwd_lds(const ttt::LinearFwdArgs& a, hipStream_t s) {
+  auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D>;
+  constexpr size_t bytes = ttt::LinFwdLds<D>::BYTES;
+  int rc = opt_in_lds(kern, bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(256), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_linear_fwd (LDS kernel) launch");
+}
+
+template <class T, int D>
+int launch_mlp_fwd(const ttt::MlpFwdArgs& a, hipStream_t s) {
+  auto kern = ttt::ttt_mlp_fwd_kernel<T, D>;
+  constexpr size_t bytes = ttt::MlpLds<D>::BYTES;
+  int rc = opt_in_lds(kern, bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_mlp_fwd launch");
+}
+
 template <class T, int D>
 int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
   auto kern = ttt::ttt_linear_bwd_kernel<T, D>;
   constexpr size_t bytes = ttt::BwdLds<D>::BYTES;
-  // more than the default 64 KiB of LDS per workgroup has to be requested (per device)
-  int rc = hip_status(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
-                      "hipFuncSetAttribute(LDS size)");
+  int rc = opt_in_lds(kern, bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_bwd launch");
@@ -82,8 +108,8 @@ int ttt_linear_supported(const ttt_desc* d) {
   if (rc != TTT_OK) return rc;
   if (d->mini_batch > 16)
     return fail(TTT_ERR_UNSUPPORTED, "mini_batch %d > 16 has no kernel", d->mini_batch);
-  if (d->head_dim != 32 && d->head_dim != 64)
-    return fail(TTT_ERR_UNSUPPORTED, "TTT-Linear head_dim %d has no kernel (32, 64)", d->head_dim);
+  if (d->head_dim != 32 && d->head_dim != 64 && d->head_dim != 96 && d->head_dim != 128)
+    return fail(TTT_ERR_UNSUPPORTED, "TTT-Linear head_dim %d has no kernel (32, 64, 96, 128)", d->head_dim);
   return TTT_OK;
 }
 
@@ -116,12 +142,14 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.state_per_batch = d->state_per_batch ? 1 : 0;
   a.eps = d->eps;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (d->io_dtype == TTT_F32) {
-    if (d->head_dim == 64) return launch_linear_fwd<ttt::F32, 64>(a, s);
-    return launch_linear_fwd<ttt::F32, 32>(a, s);
+  // head_dim 32/64: register-resident single-wave kernel; 96/128: LDS-resident kernel
+  const bool f32 = d->io_dtype == TTT_F32;
+  switch (d->head_dim) {
+    case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, s) : launch_linear_fwd<ttt::BF16, 32>(a, s);
+    case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, s) : launch_linear_fwd<ttt::BF16, 64>(a, s);
+    case 96: return f32 ? launch_linear_fwd_lds<ttt::F32, 96>(a, s) : launch_linear_fwd_lds<ttt::BF16, 96>(a, s);
+    default: return f32 ? launch_linear_fwd_lds<ttt::F32, 128>(a, s) : launch_linear_fwd_lds<ttt::BF16, 128>(a, s);
   }
-  if (d->head_dim == 64) return launch_linear_fwd<ttt::BF16, 64>(a, s);
-  return launch_linear_fwd<ttt::BF16, 32>(a, s);
 }
 
 int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
@@ -133,6 +161,8 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
                    void* stream) {
   int rc = ttt_linear_supported(d);
   if (rc != TTT_OK) return rc;
+  if (d->head_dim > 64)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim %d has no kernel (32, 64)", d->head_dim);
   // W0/b0 are part of the saved state for interface parity; the state entering every stage is
   // rebuilt from the checkpoints (checkpoint 0 equals the initial state).
   (void)W0;
@@ -174,13 +204,41 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
 int ttt_mlp_supported(const ttt_desc* d) {
   int rc = check_common(d);
   if (rc != TTT_OK) return rc;
-  return fail(TTT_ERR_UNSUPPORTED, "ttt_mlp_fwd: not built yet");
+  if (d->mini_batch > 16)
+    return fail(TTT_ERR_UNSUPPORTED, "mini_batch %d > 16 has no kernel", d->mini_batch);
+  if (d->head_dim != 32 && d->head_dim != 64 && d->head_dim != 96 && d->head_dim != 128)
+    return fail(TTT_ERR_UNSUPPORTED, "TTT-MLP head_dim %d has no kernel (32, 64, 96, 128)", d->head_dim);
+  return TTT_OK;
 }
 
-int ttt_mlp_fwd(const ttt_desc* d, const void*, const void*, const void*, const float*,
-                const float*, const float*, const float*, const float*, const void*,
-                const float*, const float*, void*, float*, float*, float*, float*, void*) {
-  return ttt_mlp_supported(d);
+int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                void* out, float* W1_out, float* b1_out, float* W2_out, float* b2_out,
+                void* stream) {
+  int rc = ttt_mlp_supported(d);
+  if (rc != TTT_OK) return rc;
+  if (!xq || !xk || !xv || !W1_0 || !b1_0 || !W2_0 || !b2_0 || !token_eta || !lr || !gamma || !beta ||
+      !out || !W1_out || !b1_out || !W2_out || !b2_out)
+    return fail(TTT_ERR_NULL, "ttt_mlp_fwd: a required pointer is NULL");
+  if (W1_out == W1_0 || W2_out == W2_0)
+    return fail(TTT_ERR_SHAPE, "ttt_mlp_fwd: W1_out/W2_out are the live state and must not alias W1_0/W2_0");
+  ttt::MlpFwdArgs a;
+  a.xq = xq; a.xk = xk; a.xv = xv; a.W1_0 = W1_0; a.b1_0 = b1_0; a.W2_0 = W2_0; a.b2_0 = b2_0;
+  a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
+  a.W1 = W1_out; a.b1 = b1_out; a.W2 = W2_out; a.b2 = b2_out;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.n_stages = d->seq / d->mini_batch;
+  a.state_per_batch = d->state_per_batch ? 1 : 0;
+  a.eps = d->eps;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool f32 = d->io_dtype == TTT_F32;
+  switch (d->head_dim) {
+    case 32: return f32 ? launch_mlp_fwd<ttt::F32, 32>(a, s) : launch_mlp_fwd<ttt::BF16, 32>(a, s);
+    case 64: return f32 ? launch_mlp_fwd<ttt::F32, 64>(a, s) : launch_mlp_fwd<ttt::BF16, 64>(a, s);
+    case 96: return f32 ? launch_mlp_fwd<ttt::F32, 96>(a, s) : launch_mlp_fwd<ttt::BF16, 96>(a, s);
+    default: return f32 ? launch_mlp_fwd<ttt::F32, 128>(a, s) : launch_mlp_fwd<ttt::BF16, 128>(a, s);
+  }
 }
 
 }  // extern "C"

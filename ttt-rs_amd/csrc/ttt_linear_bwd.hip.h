@@ -17,7 +17,7 @@
 // features cg, cg+16, ...; row statistics are 16-lane shuffles.  Arithmetic is f32 for both
 // I/O dtypes; bf16 tensors are converted at the tile loads and stores.
 #pragma once
-#include "ttt_frag.hip.h"
+#include "ttt_engine.hip.h"
 
 namespace ttt {
 
@@ -66,47 +66,6 @@ struct BwdLds {
                        te = lr + 16, rstd1 = te + 16, dlast = rstd1 + 16, END = dlast + 16;
   static constexpr size_t BYTES = sizeof(float) * END;
 };
-
-// C[16*Mt x 16*Nt] (row-major, stride ldc)  = / += / -=  A * B, contraction length Kd (multiple
-// of 4).  A(m,k) = A[m*a_rs + k*a_cs], B(k,n) = B[k*b_rs + n*b_cs].  Output tiles are dealt
-// round-robin to the four waves starting at wave `first`.  MODE 0: set, 1: add, 2: subtract.
-template <int MODE>
-__device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_rs, int a_cs,
-                                       const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
-                                       int wave, int lane, int first = 0) {
-  const int c = lane & 15, g = lane >> 4;
-  const int ntiles = Mt * Nt;
-  for (int tile = (wave - first + 4) & 3; tile < ntiles; tile += 4) {
-    const int tm = tile / Nt, tn = tile - tm * Nt;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    float* Ct = C + (16 * tm + 4 * g) * ldc + 16 * tn + c;
-    if (MODE != 0) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc[r] = (MODE == 1) ? Ct[r * ldc] : -Ct[r * ldc];
-    }
-    const float* Ap = A + (16 * tm + c) * a_rs + g * a_cs;
-    const float* Bp = B + g * b_rs + (16 * tn + c) * b_cs;
-#pragma unroll 4
-    for (int k = 0; k < Kd; k += 4)
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ap[k * a_cs], Bp[k * b_rs], acc, 0, 0, 0);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) Ct[r * ldc] = (MODE == 2) ? -acc[r] : acc[r];
-  }
-}
-
-// sum over the 16 lanes that share a token (an aligned group of 16 lanes)
-__device__ __forceinline__ float row16_sum(float v) {
-  v += __shfl_xor(v, 8, 16);
-  v += __shfl_xor(v, 4, 16);
-  v += __shfl_xor(v, 2, 16);
-  v += __shfl_xor(v, 1, 16);
-  return v;
-}
-
-__global__ void ttt_fill_zero_kernel(float* p, size_t n) {
-  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0.f;
-}
 
 template <class T, int D>
 __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {

@@ -186,6 +186,119 @@ def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_
     return g
 
 
+def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias,
+                        mini_batch: int, eps: float = 1e-6):
+    """One call of ttt_mlp_fwd on the current stream: the fused counterpart of
+    TTTMLP::forward (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50).
+    w1 [B,H,d,4d] or [H,d,4d], b1 [..,4d], w2 [..,4d,d], b2 [..,d].
+    Returns (output, w1_out, b1_out, w2_out, b2_out), state per batch element."""
+    B, H, seq, d = xq.shape
+    m = w1.shape[-1]
+    io = xq.dtype
+    xq = _need(xq, (B, H, seq, d), io, "xq")
+    xk = _need(xk, (B, H, seq, d), io, "xk")
+    xv = _need(xv, (B, H, seq, d), io, "xv")
+    lr = _need(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta")
+    per_batch = w1.dim() == 4
+    lead = (B, H) if per_batch else (H,)
+    if m != 4 * d:
+        raise _lib.TttError(_lib.TTT_ERR_UNSUPPORTED, f"mlp_dim {m} != 4*head_dim (only expansion 4)")
+    w1 = _need(w1, lead + (d, m), torch.float32, "w1")
+    b1 = _need(b1, lead + (m,), torch.float32, "b1")
+    w2 = _need(w2, lead + (m, d), torch.float32, "w2")
+    b2 = _need(b2, lead + (d,), torch.float32, "b2")
+    ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+    ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+    if token_eta.numel() < mini_batch:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
+    te = token_eta.to(torch.float32).contiguous()
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), int(per_batch))
+    check(lib().ttt_mlp_supported(C.byref(desc)))
+    dev = xq.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    out = torch.empty_like(xq)
+    o = [torch.empty((B, H, d, m), **f32), torch.empty((B, H, m), **f32),
+         torch.empty((B, H, m, d), **f32), torch.empty((B, H, d), **f32)]
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_mlp_fwd(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(w1), _ptr(b1), _ptr(w2),
+                                _ptr(b2), _ptr(te), _ptr(lr), _ptr(ln_weight), _ptr(ln_bias), _ptr(out),
+                                *[_ptr(x) for x in o], stream))
+    return (out, *o)
+
+
+@dataclass
+class TTTMLPState:
+    """mlp.rs:43-53: w1 [B,H,d,4d], b1 [B,H,4d], w2 [B,H,4d,d], b2 [B,H,d], always f32."""
+    w1: torch.Tensor
+    b1: torch.Tensor
+    w2: torch.Tensor
+    b2: torch.Tensor
+
+
+class FusedMlp:
+    """Fused TTT-MLP layer with the TTTMLP parameter set (mlp.rs:29-41) and the TTTInnerModel
+    surface (inner.rs:13-58)."""
+
+    def __init__(self, config: ModelConfig, w1_init, b1_init, w2_init, b2_init, ln_weight, ln_bias):
+        H, d = config.num_heads, config.head_dim
+        m = config.ttt.mlp_expansion_factor * d
+        self.config = config
+        self.w1_init = _need(w1_init, (H, d, m), torch.float32, "w1_init")
+        self.b1_init = _need(b1_init, (H, m), torch.float32, "b1_init")
+        self.w2_init = _need(w2_init, (H, m, d), torch.float32, "w2_init")
+        self.b2_init = _need(b2_init, (H, d), torch.float32, "b2_init")
+        self.ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+        self.ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+
+    @staticmethod
+    def name() -> str:
+        return "FusedTTTMLP"
+
+    @classmethod
+    def new(cls, config: ModelConfig, device, generator: Optional[torch.Generator] = None):
+        """TTTMLP::new (mlp.rs:76-113): every parameter ~ Normal(0, 0.02)."""
+        H, d = config.num_heads, config.head_dim
+        m = config.ttt.mlp_expansion_factor * d
+
+        def init(*shape):
+            return (torch.randn(*shape, generator=generator, dtype=torch.float32) * 0.02).to(device)
+
+        return cls(config, init(H, d, m), init(H, m), init(H, m, d), init(H, d), init(H, d), init(H, d))
+
+    def get_config(self) -> ModelConfig:
+        return self.config
+
+    def init_state(self, batch_size: int) -> TTTMLPState:
+        """mlp.rs:119-125."""
+        rep = lambda p: p.unsqueeze(0).repeat(batch_size, *([1] * p.dim()))
+        return TTTMLPState(rep(self.w1_init), rep(self.b1_init), rep(self.w2_init), rep(self.b2_init))
+
+    def _launch(self, state: TTTMLPState, inputs: TTTInputsInner, mini_batch: int):
+        out, state.w1, state.b1, state.w2, state.b2 = ttt_mlp_forward_raw(
+            inputs.qkv.xq, inputs.qkv.xk, inputs.qkv.xv, state.w1, state.b1, state.w2, state.b2,
+            inputs.token_eta, inputs.ttt_lr_eta, self.ln_weight, self.ln_bias, mini_batch,
+            self.config.ttt.epsilon)
+        return out
+
+    def forward(self, state: TTTMLPState, inputs: TTTInputsInner) -> torch.Tensor:
+        """inner.rs:25-50 in at most two launches: all full mini-batches, then the remainder."""
+        K = self.config.ttt.mini_batch_size
+        seq = inputs.qkv.xq.shape[2]
+        full = (seq // K) * K
+        outs = []
+        if full > 0:
+            outs.append(self._launch(state, inputs.slice_seq(range(0, full)), K))
+        if full < seq:
+            outs.append(self._launch(state, inputs.slice_seq(range(full, seq)), seq - full))
+        return outs[0] if len(outs) == 1 else torch.cat(outs, 2)
+
+    def forward_mini_batch(self, state: TTTMLPState, inputs: TTTInputsInner, r: range) -> torch.Tensor:
+        if len(r) > self.config.ttt.mini_batch_size or len(r) == 0:
+            raise _lib.TttError(_lib.TTT_ERR_SHAPE, "range longer than mini_batch_size")
+        return self._launch(state, inputs.slice_seq(r), len(r))
+
+
 class FusedTileMulti:
     """`fused-tile-multi` TTT-Linear layer: Fused<B, TTTLinear<B>, TileMultiKernel>.
 
