@@ -6,6 +6,7 @@ resident in HBM.  Default workload = the TTT-Linear forward at the 125M shape
 
 Throughput follows the reference's definition: tokens/s = batch*seq / seconds of the inner
 loop only, with Q/K/V, lr and token_eta precomputed (reference rust/cli/src/bench.rs:153-191,329).
+Other workloads (--workload) cover the remaining benchmark configurations.
 """
 from __future__ import annotations
 
@@ -20,46 +21,60 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+F32_MFMA_PEAK_TF = 157.3   # MI355X dense fp32 matrix
+BF16_MFMA_PEAK_TF = 2500.0
 
 WORKLOADS = {
-    # name: (config_idx, B, H, d, seq, K, io dtype, kind)
-    "linear_fwd_125m_bf16": (1, 32, 12, 64, 2048, 16, "bf16", "linear_fwd"),
-    "linear_fwd_125m_f32_b8": (2, 8, 12, 64, 2048, 16, "f32", "linear_fwd"),
-    "linear_fwd_cfg0_f32": (0, 1, 4, 64, 256, 16, "f32", "linear_fwd"),
+    # name: dict(cfg=config index, B, H, d, seq, K, io, kind)
+    "linear_fwd_125m_bf16": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="linear_fwd"),
+    "linear_fwd_cfg0_f32": dict(cfg=0, B=1, H=4, d=64, seq=256, K=16, io="f32", kind="linear_fwd"),
+    "linear_fwd_125m_f32_b8": dict(cfg=2, B=8, H=12, d=64, seq=2048, K=16, io="f32", kind="linear_fwd"),
+    "linear_fwd_bwd_125m_f32_b8": dict(cfg=2, B=8, H=12, d=64, seq=2048, K=16, io="f32", kind="linear_fwd_bwd"),
+    "mlp_fwd_d96_bf16": dict(cfg=3, B=8, H=16, d=96, seq=2048, K=16, io="bf16", kind="mlp_fwd"),
+    "stack8_d128_seq8192_bf16": dict(cfg=4, B=4, H=16, d=128, seq=8192, K=16, io="bf16", kind="stack"),
 }
 
 
-def algorithmic_bytes(B, H, seq, d, s):
-    """Compulsory traffic of the forward: xq, xk, xv in, out written once, lr in."""
+def linear_fwd_bytes(B, H, seq, d, s):
+    """Compulsory traffic of a forward: xq, xk, xv in, out written once, lr in."""
     return B * H * seq * (4 * d * s + s)
 
 
-def cpu_baseline(c, K, budget_s=20.0):
-    """Times the C port of the reference CPU path (oracle/ttt_oracle.c) on the host cores, on
-    the same inputs (f32 arithmetic on the stored values)."""
+def linear_bwd_bytes(B, H, seq, d, s):
+    """Backward: xq, xk, xv, d_out in; d_xq, d_xk, d_xv out; lr in, d_lr out."""
+    return B * H * seq * (7 * d * s + 2 * s)
+
+
+def cpu_baseline(c, K, kind, budget_s=20.0):
+    """Times the C/OpenMP port of the reference CPU path (oracle/ttt_oracle.c) on the host cores
+    on the same inputs (f32 arithmetic on the stored values), on a bounded batch slice."""
     import numpy as np
     from oracle import c_oracle
     cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "9999")))
     n = {k: v.float().numpy() for k, v in c.items()}
     B, H, seq, d = n["xq"].shape
-    args = (n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"], n["gamma"], n["beta"])
-    # bounded sample: whole workload when it fits the time budget, else a batch slice
+    if kind == "mlp_fwd":
+        fn = c_oracle.mlp_fwd
+        keys = ("W1", "b1", "W2", "b2", "xq", "xk", "xv", "token_eta", "lr", "gamma", "beta")
+    else:
+        fn = c_oracle.linear_fwd
+        keys = ("W0", "b0", "xq", "xk", "xv", "token_eta", "lr", "gamma", "beta")
+    bsl = lambda nb: [n[k][:nb] if k in ("xq", "xk", "xv", "lr") else n[k] for k in keys]
     t0 = time.perf_counter()
-    c_oracle.linear_fwd(*[a[:1] if a.ndim >= 3 and a.shape[0] == B else a for a in args], K=K,
-                        dtype=np.float32, nthreads=cores)
+    fn(*bsl(1), K=K, dtype=np.float32, nthreads=cores)
     t_one = time.perf_counter() - t0
     Bs = max(1, min(B, int(budget_s / 4 / max(t_one, 1e-4))))
-    sl = [a[:Bs] if a.ndim >= 3 and a.shape[0] == B else a for a in args]
     times = []
     for _ in range(3):
         t0 = time.perf_counter()
-        c_oracle.linear_fwd(*sl, K=K, dtype=np.float32, nthreads=cores)
+        fn(*bsl(Bs), K=K, dtype=np.float32, nthreads=cores)
         times.append(time.perf_counter() - t0)
     t = sum(times) / len(times)
+    what = "forward" if kind != "linear_fwd_bwd" else "forward only (the C port has no backward)"
     return {"value": Bs * seq / t, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"C/OpenMP f32 port of the reference CPU path, same inputs, batch {Bs} of {B} "
-                      f"(tokens/s is batch-normalised), mean of 3 runs, {t:.3f} s per run"}
+            "sample": f"C/OpenMP f32 port of the reference CPU path, {what}, same inputs, batch {Bs} of "
+                      f"{B} (tokens/s is batch-normalised), mean of 3 runs, {t:.3f} s per run"}
 
 
 def main():
@@ -68,6 +83,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="linear_fwd_125m_bf16", choices=sorted(WORKLOADS))
+    ap.add_argument("--checkpoint-interval", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -76,16 +92,54 @@ def main():
 
     import torch
     pkg = importlib.import_module("ttt-rs_amd")
-    cfg, B, H, d, seq, K, io, kind = WORKLOADS[a.workload]
+    w = WORKLOADS[a.workload]
+    B, H, d, seq, K, io, kind = w["B"], w["H"], w["d"], w["seq"], w["K"], w["io"], w["kind"]
     dtype = {"bf16": torch.bfloat16, "f32": torch.float32}[io]
     s = 2 if io == "bf16" else 4
-    c = pkg.synthetic.baseline_inputs(cfg, B, H, seq, d, K, io_dtype=dtype)
+    ci = a.checkpoint_interval
     dev = torch.device("cuda:0")
-    dv = {k: v.to(dev) for k, v in c.items()}
+    th = B * H * seq  # token-heads
 
-    def step():
-        return pkg.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
-                                          dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+    if kind == "stack":
+        # 8 layers (6 TTT-Linear then 2 TTT-MLP); layer input = previous output + fresh projections
+        layers = []
+        for li in range(8):
+            c = pkg.synthetic.baseline_inputs(40 + li, B, H, seq, d, K, io_dtype=dtype, mlp=li >= 6)
+            layers.append({k: v.to(dev) for k, v in c.items()})
+        c = None
+
+        def step():
+            x = None
+            for li, L in enumerate(layers):
+                q, k, v = (L["xq"], L["xk"], L["xv"]) if x is None else (x + L["xq"], x + L["xk"], x + L["xv"])
+                if li < 6:
+                    x = pkg.ttt_linear_forward_raw(q, k, v, L["W0"], L["b0"], L["token_eta"], L["lr"],
+                                                   L["gamma"], L["beta"], K)[0]
+                else:
+                    x = pkg.ttt_mlp_forward_raw(q, k, v, L["W1"], L["b1"], L["W2"], L["b2"], L["token_eta"],
+                                                L["lr"], L["gamma"], L["beta"], K)[0]
+            return (x,)
+    else:
+        c = pkg.synthetic.baseline_inputs(w["cfg"], B, H, seq, d, K, io_dtype=dtype,
+                                          with_dout=kind == "linear_fwd_bwd", mlp=kind == "mlp_fwd")
+        dv = {k: v.to(dev) for k, v in c.items()}
+        if kind == "linear_fwd":
+            def step():
+                return pkg.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
+                                                  dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+        elif kind == "mlp_fwd":
+            def step():
+                return pkg.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
+                                               dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+        else:
+            def step():
+                out, W, b, Wc, bc = pkg.ttt_linear_forward_raw(
+                    dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                    dv["gamma"], dv["beta"], K, 1e-6, ci, want_checkpoints=True)
+                g = pkg.ttt_linear_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
+                                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], Wc, bc,
+                                                dv["d_out"], K, 1e-6, ci)
+                return (out, g["grad_xq"])
 
     for _ in range(a.warmup):
         step()
@@ -94,41 +148,68 @@ def main():
           for _ in range(a.steps)]
     t0 = time.perf_counter()
     for e0, e1 in ev:
-        e0.record()          # events sit on the stream the kernel is launched on
-        out = step()
+        e0.record()          # events sit on the stream the kernels are launched on
+        res = step()
         e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    kern_ms = [e0.elapsed_time(e1) for e0, e1 in ev]
-    avg_kernel_s = sum(kern_ms) / len(kern_ms) / 1e3
-    assert torch.isfinite(out[0].float()).all()
+    dev_s = sum(e0.elapsed_time(e1) for e0, e1 in ev) / len(ev) / 1e3  # device time of one step
+    assert all(torch.isfinite(r.float()).all() for r in res)
 
-    ms_per_step = wall / a.steps * 1e3
-    alg = algorithmic_bytes(B, H, seq, d, s)
-    achieved = alg / avg_kernel_s / 1e9
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(a.workload)
-    res = {
-        "metric": "inner-loop tokens/sec (fwd) at 125M shape",
+    pass_name = {"linear_fwd": "fwd", "linear_fwd_bwd": "fwd+bwd", "mlp_fwd": "fwd", "stack": "fwd"}[kind]
+    out = {
+        "metric": f"inner-loop tokens/sec ({pass_name}) at 125M shape" if d == 64 else
+                  f"inner-loop tokens/sec ({pass_name})",
         "value": B * seq / (wall / a.steps),
         "unit": "tokens/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": wall / a.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 I/O, f32 state and accumulation" if io == "bf16" else "f32",
         "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "heads": H, "head_dim": d, "seq_len": seq,
-                   "mini_batch": K, "io_dtype": io, "inner_model": "TTT-Linear", "pass": "forward"},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "ttt_linear_fwd_kernel", "kernel_avg_us": avg_kernel_s * 1e6,
-                     "algorithmic_bytes": alg},
+                   "mini_batch": K, "io_dtype": io, "pass": pass_name},
     }
-    if not a.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(c, K)
-    print(json.dumps(res))
+    if kind == "linear_fwd":
+        alg = linear_fwd_bytes(B, H, seq, d, s)
+        out["dtype"] = "bf16" if io == "bf16" and d <= 64 else "f32"
+        out["config"]["inner_model"] = "TTT-Linear"
+        out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                           "kernel": "ttt_linear_fwd_kernel", "kernel_avg_us": dev_s * 1e6,
+                           "algorithmic_bytes": alg}
+    elif kind == "linear_fwd_bwd":
+        # the backward kernel dominates; it computes in f32 MFMA: 18 d^2 + 22 K d flop per token-head
+        flops = th * (24 * d * d + 26 * K * d)
+        out["dtype"] = "f32"
+        out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci)
+        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
+                           "kernel": "ttt_linear_fwd_kernel + ttt_linear_bwd_kernel (whole step)",
+                           "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops,
+                           "algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)}
+    elif kind == "mlp_fwd":
+        flops = th * (56 * d * d + 20 * K * d)
+        out["dtype"] = "f32"   # bf16 I/O, f32 MFMA arithmetic
+        out["config"]["inner_model"] = "TTT-MLP"
+        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
+                           "frac_of_bf16_peak": flops / dev_s / 1e12 / BF16_MFMA_PEAK_TF,
+                           "kernel": "ttt_mlp_fwd_kernel", "kernel_avg_us": dev_s * 1e6,
+                           "algorithmic_flops": flops}
+    else:
+        flops = th * (6 * (6 * d * d + 4 * K * d) + 2 * (56 * d * d + 20 * K * d))
+        out["dtype"] = "f32"
+        out["config"]["inner_model"] = "6 x TTT-Linear + 2 x TTT-MLP"
+        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
+                           "kernel": "8 layer launches + input adds (whole step)",
+                           "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        out["roofline"]["traffic"] = json.load(open(tpath)).get(a.workload)
+    if not a.no_cpu_baseline and c is not None:
+        out["cpu_baseline"] = cpu_baseline(c, K, kind)
+    print(json.dumps(out))
 
 
 if __name__ == "__main__":
