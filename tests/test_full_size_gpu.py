@@ -1,0 +1,151 @@
+"""GPU parity at the benchmark's full sizes.
+
+The float64 oracle is too slow for whole configurations, so each case checks
+  * oracle agreement on a slice of (batch, head) units over the FULL sequence length (all
+    mini-batches chained), and
+  * size-independent properties on the whole tensor: a sequence processed in two calls with the
+    state carried over equals one call bit for bit, and (batch, head) units are independent.
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import TOL, assert_close, to_np
+from oracle import ttt_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+def dev(c):
+    return {k: v.to("cuda:0") for k, v in c.items()}
+
+
+def sub(c, bs, hs, keys_bh=("xq", "xk", "xv", "lr", "d_out")):
+    """Slice of the inputs: batch entries bs, heads hs (numpy float64)."""
+    o = {}
+    for k, v in c.items():
+        if k in keys_bh:
+            o[k] = to_np(v[bs][:, hs])
+        elif k == "token_eta":
+            o[k] = to_np(v)
+        else:
+            o[k] = to_np(v[hs])
+    return o
+
+
+def test_config1_linear_fwd_bf16_full(P):
+    B, H, d, seq, K = 32, 12, 64, 2048, 16
+    print("case config1 full", flush=True)
+    c = P.synthetic.baseline_inputs(1, B, H, seq, d, K, io_dtype=torch.bfloat16)
+    dv = dev(c)
+    args = lambda s: (dv["xq"][:, :, s].contiguous(), dv["xk"][:, :, s].contiguous(), dv["xv"][:, :, s].contiguous())
+    out, W, b = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"],
+                                         dv["lr"], dv["gamma"], dv["beta"], K)
+    # two halves with carried state == one call, bit for bit
+    h1 = slice(0, seq // 2)
+    h2 = slice(seq // 2, seq)
+    o1, W1, b1 = P.ttt_linear_forward_raw(*args(h1), dv["W0"], dv["b0"], dv["token_eta"],
+                                          dv["lr"][:, :, h1].contiguous(), dv["gamma"], dv["beta"], K)
+    o2, W2, b2 = P.ttt_linear_forward_raw(*args(h2), W1, b1, dv["token_eta"],
+                                          dv["lr"][:, :, h2].contiguous(), dv["gamma"], dv["beta"], K)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([o1, o2], 2), out)
+    assert torch.equal(W2, W) and torch.equal(b2, b)
+    # oracle on four (b, h) units over all 128 mini-batches
+    bs, hs = [0, 31], [0, 11]
+    n = sub(c, bs, hs)
+    ro, rW, rb = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                                    n["gamma"], n["beta"], K=K)
+    assert_close(out[bs][:, hs], ro, TOL[torch.bfloat16], "out")
+    assert_close(W[bs][:, hs], rW, TOL[torch.bfloat16], "W_out")
+    assert_close(b[bs][:, hs], rb, TOL[torch.bfloat16], "b_out")
+
+
+def test_config2_linear_fwd_bwd_f32_full(P):
+    B, H, d, seq, K = 8, 12, 64, 2048, 16
+    print("case config2 full", flush=True)
+    c = P.synthetic.baseline_inputs(2, B, H, seq, d, K, with_dout=True)
+    dv = dev(c)
+
+    def fwd_bwd(x, ci):
+        out, W, b, Wc, bc = P.ttt_linear_forward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"],
+                                                     x["lr"], x["gamma"], x["beta"], K, 1e-6, ci,
+                                                     want_checkpoints=True)
+        g = P.ttt_linear_backward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"],
+                                      x["gamma"], x["beta"], Wc, bc, x["d_out"], K, 1e-6, ci)
+        return out, g
+
+    out, g = fwd_bwd(dv, 1)
+    # a coarser checkpoint interval (re-simulated states) must give the same gradients
+    _, g16 = fwd_bwd(dv, 16)
+    torch.cuda.synchronize()
+    for k in g:
+        assert_close(g16[k], g[k].double(), 1e-5, "ci16 " + k)
+    # one batch entry alone: per-unit gradients are identical, reduced ones are that entry's share
+    one = {k: (v[3:4].contiguous() if k in ("xq", "xk", "xv", "lr", "d_out") else v) for k, v in dv.items()}
+    o1, g1 = fwd_bwd(one, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, out[3:4])
+    for k in ("grad_xq", "grad_xk", "grad_xv", "grad_weight", "grad_bias", "grad_ttt_lr_eta"):
+        assert torch.equal(g1[k], g[k][3:4]), k
+    # oracle (all 128 stages, all heads of that batch entry, all nine gradients)
+    n = sub(c, [3], list(range(H)))
+    r = orc.linear_backward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                            n["gamma"], n["beta"], n["d_out"], K=K)
+    names = [("grad_xq", "d_xq"), ("grad_xk", "d_xk"), ("grad_xv", "d_xv"), ("grad_weight", "d_W0"),
+             ("grad_bias", "d_b0"), ("grad_ttt_lr_eta", "d_lr"), ("grad_token_eta", "d_token_eta"),
+             ("grad_ln_weight", "d_gamma"), ("grad_ln_bias", "d_beta")]
+    for gn, rn in names:
+        assert_close(g1[gn], r[rn], 1e-4, gn)
+
+
+def test_config3_mlp_fwd_bf16_full(P):
+    B, H, d, seq, K = 8, 16, 96, 2048, 16
+    print("case config3 full", flush=True)
+    c = P.synthetic.baseline_inputs(3, B, H, seq, d, K, io_dtype=torch.bfloat16, mlp=True)
+    dv = dev(c)
+    got = P.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
+                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+    torch.cuda.synchronize()
+    bs, hs = [0, 7], [0, 15]
+    n = sub(c, bs, hs)
+    ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
+                          n["lr"], n["gamma"], n["beta"], K=K)
+    for name, gv, rv in zip(("out", "W1", "b1", "W2", "b2"), got, ref):
+        assert_close(gv[bs][:, hs], rv, TOL[torch.bfloat16] if name == "out" else 1e-4, name)
+
+
+def test_config4_layers_d128_seq8192(P):
+    """One TTT-Linear and one TTT-MLP layer of the long-context stack at its real shape
+    (512 chained mini-batches), checked on a slice of units."""
+    B, H, d, seq, K = 4, 16, 128, 8192, 16
+    print("case config4 layers", flush=True)
+    bs, hs = [1], [0, 15]
+    c = P.synthetic.baseline_inputs(40, B, H, seq, d, K, io_dtype=torch.bfloat16)
+    dv = dev(c)
+    out, W, b = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"],
+                                         dv["lr"], dv["gamma"], dv["beta"], K)
+    torch.cuda.synchronize()
+    n = sub(c, bs, hs)
+    ro, rW, rb = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                                    n["gamma"], n["beta"], K=K)
+    assert_close(out[bs][:, hs], ro, TOL[torch.bfloat16], "linear out")
+    assert_close(W[bs][:, hs], rW, 1e-4, "linear W")
+    del dv, out, W, b
+    c = P.synthetic.baseline_inputs(46, B, H, seq, d, K, io_dtype=torch.bfloat16, mlp=True)
+    dv = dev(c)
+    got = P.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
+                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+    torch.cuda.synchronize()
+    n = sub(c, bs, hs)
+    ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
+                          n["lr"], n["gamma"], n["beta"], K=K)
+    for name, gv, rv in zip(("out", "W1", "b1", "W2", "b2"), got, ref):
+        assert_close(gv[bs][:, hs], rv, TOL[torch.bfloat16] if name == "out" else 1e-4, "mlp " + name)
