@@ -82,7 +82,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="linear_fwd_125m_bf16", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="linear_fwd_125m_bf16", choices=sorted(WORKLOADS) + ["hbm_copy_calibration"])
     ap.add_argument("--checkpoint-interval", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     a = ap.parse_args()
@@ -91,6 +91,18 @@ def main():
                  "batch*heads with no communication, see DESIGN.md)")
 
     import torch
+    if a.workload == "hbm_copy_calibration":
+        # plain device-to-device copy of known size: reference point for the FETCH_SIZE / WRITE_SIZE
+        # counters (rocprofv3 --pmc) that the `traffic` figures are scaled by
+        nbytes = 512 << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(a.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": a.workload, "copy_bytes": nbytes, "steps": a.steps}))
+        return
     pkg = importlib.import_module("ttt-rs_amd")
     w = WORKLOADS[a.workload]
     B, H, d, seq, K, io, kind = w["B"], w["H"], w["d"], w["seq"], w["K"], w["io"], w["kind"]
