@@ -12,7 +12,7 @@ import torch.nn.functional as F
 
 from oracle import ttt_oracle as orc
 
-torch.set_default_dtype(torch.float64)
+
 
 
 def rnd(rng, *shape, scale=1.0):

@@ -19,6 +19,9 @@ HIPCC_FLAGS = [
     "-DTTT_XG_SWAP=1",
     # keep the compiler from forming packed-f32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # let MFMA results live in ordinary VGPRs: the kernels consume them with VALU code right away,
+    # and the default AGPR placement costs a v_accvgpr move per register and use
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 

@@ -6,10 +6,14 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 
 #include "ttt_engine_fwd.hip.h"
 #include "ttt_linear_bwd.hip.h"
 #include "ttt_linear_fwd.hip.h"
+#include "ttt_linear_fwd_mw.hip.h"
+#include "ttt_linear_fwd_sk.hip.h"
 
 namespace {
 
@@ -46,15 +50,53 @@ int hip_status(hipError_t e, const char* what) {
   return fail(TTT_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// ---- TTT-Linear forward, head_dim 32/64: kernel choice --------------------------------------
+// A (batch, head) unit is a strictly sequential chain of mini-batches, so the launch is latency
+// bound until there are more units than SIMDs.  Few units: split each unit over several waves
+// (skewed workgroup kernel).  Many units: one wave per unit (no exchange at all).
+// TTT_LINEAR_FWD_WAVES = 1 | 2 | 4 overrides the number of waves per unit (tuning / tests).
+int fwd_waves_override() {
+  const char* e = std::getenv("TTT_LINEAR_FWD_WAVES");
+  return e ? std::atoi(e) : 0;
+}
+
+template <class T, int D, int NW>
+int launch_linear_fwd_nw(const ttt::LinearFwdArgs& a, hipStream_t s) {
+  constexpr int PF = 2;  // mini-batches prefetched ahead, in registers
+  const dim3 grid((unsigned)(a.B * a.H)), block(64 * NW);
+  if (NW == 1) {
+    if (a.K == 16)
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, true>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, false>), grid, block, 0, s, a);
+  } else {
+    constexpr int NWS = NW > 1 ? NW : 2;  // the skewed kernel needs at least two waves
+    if (a.K == 16)
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, false>), grid, block, 0, s, a);
+  }
+  return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+}
+
 template <class T, int D>
 int launch_linear_fwd(const ttt::LinearFwdArgs& a, hipStream_t s) {
-  constexpr int PF = 2;
-  const unsigned grid = (unsigned)(a.B * a.H);
-  if (a.K == 16)
-    hipLaunchKernelGGL((ttt::ttt_linear_fwd_kernel<T, D, PF, true>), dim3(grid), dim3(64), 0, s, a);
-  else
-    hipLaunchKernelGGL((ttt::ttt_linear_fwd_kernel<T, D, PF, false>), dim3(grid), dim3(64), 0, s, a);
-  return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+  constexpr int max_nw = D / 16;
+  constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
+  const long units = (long)a.B * a.H;
+  int nw = fwd_waves_override();
+  if (nw <= 0) {
+    // measured on MI355X (256 CUs x 4 SIMDs): bf16 is VALU-latency bound and likes 2 waves per unit
+    // up to ~2 units per CU; f32 is MFMA bound (16x16x4 f32) and likes 4 until the CUs are shared
+    if (f32)
+      nw = units <= 256 ? 4 : (units <= 512 ? 2 : 1);
+    else
+      nw = units <= 512 ? 2 : 1;
+  }
+  if (nw > max_nw) nw = max_nw;
+  if (nw >= 4) return launch_linear_fwd_nw<T, D, (max_nw >= 4 ? 4 : 2)>(a, s);
+  if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(a, s);
+  return launch_linear_fwd_nw<T, D, 1>(a, s);
 }
 
 template <class K>

@@ -27,6 +27,8 @@
 namespace ttt {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -64,6 +66,21 @@ __device__ __forceinline__ float xg_sum(float v) {
   v += __shfl_xor(v, 32);
 #endif
   return v;
+}
+
+// Reduce four values over the four lane groups at once: returns, in lane group g, the sum over
+// all groups of the g-th argument.  One 32-lane swap per pair sends each half the partner's copy of
+// the value it keeps; one 16-lane swap finishes both pairs: 3 swaps + 3 adds for four sums.
+__device__ __forceinline__ float xg_sum4_scatter(float a, float b, float c, float d) {
+  const auto p = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(c), false, false);
+  const uint32_t p0 = p[0], p1 = p[1];
+  const float ac = __uint_as_float(p0) + __uint_as_float(p1);  // lower half: a, upper half: c (2 rows each)
+  const auto q = __builtin_amdgcn_permlane32_swap(__float_as_uint(b), __float_as_uint(d), false, false);
+  const uint32_t q0 = q[0], q1 = q[1];
+  const float bd = __uint_as_float(q0) + __uint_as_float(q1);  // lower half: b, upper half: d
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(ac), __float_as_uint(bd), false, false);
+  const uint32_t r0 = r[0], r1 = r[1];
+  return __uint_as_float(r0) + __uint_as_float(r1);            // rows: a, b, c, d
 }
 
 template <class T>
@@ -110,7 +127,13 @@ struct Io<BF16> {
   using elem = uint16_t;
   using frag = bf16x4;
   static constexpr int kBytes = 2;
-  __device__ static __forceinline__ frag to_frag(f32x4 v) { return __builtin_convertvector(v, bf16x4); }
+  // two packed conversions (v_cvt_pk_bf16_f32); converting the 4-vector in one go makes the
+  // compiler convert element by element and re-pack with v_perm
+  __device__ static __forceinline__ frag to_frag(f32x4 v) {
+    const bf16x2 lo = __builtin_convertvector(f32x2{v[0], v[1]}, bf16x2);
+    const bf16x2 hi = __builtin_convertvector(f32x2{v[2], v[3]}, bf16x2);
+    return __builtin_bit_cast(frag, u32x2{__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)});
+  }
   __device__ static __forceinline__ f32x4 to_f32(frag f) { return __builtin_convertvector(f, f32x4); }
   __device__ static __forceinline__ frag zero() {
     return __builtin_bit_cast(frag, u32x2{0u, 0u});

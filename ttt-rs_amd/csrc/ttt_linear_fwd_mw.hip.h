@@ -1,0 +1,375 @@
+// TTT-Linear multi-stage forward for gfx950, one workgroup of NW wavefronts per (batch, head):
+// wave w owns TPW = (d/16)/NW output-feature tiles (16*TPW features).  NW = 1 needs no LDS and no
+// barrier; NW = d/16 gives every wave one tile.
+//
+// Arithmetic as ttt_linear_fwd.hip.h (reference rust/core/src/linear.rs:91-149 looped as
+// rust/core/src/inner.rs:25-50; checkpoints as
+// rust/fused/src/linear_fused_tile/forward/kernel.rs:143-150).
+//
+// What is split and what is not:
+//  * Wave w keeps the column slice W[:, own tiles] (NT*TPW accumulator tiles), its slice of
+//    b, gamma, beta, and computes its 16 features of Z1, G, Zbar and of the output.  The state
+//    update of that slice needs only the wave's own G tile, so W never crosses waves.
+//  * Every wave loads the full XK and XQ rows (they are the k-side operands of its products)
+//    and recomputes the [16 x 16] attention block; HBM sees each byte once, the repeats hit L1.
+//  * LayerNorm statistics need all d features of a token.  Each wave reduces raw moments of its
+//    own 16 features and the waves exchange them through LDS: ONE exchange (six sums) for the
+//    LN-L2 gradient, one (two sums) for the output LayerNorm, so two barriers per mini-batch.
+//    With z the pre-norm row, a = gamma^2 and q = gamma*(beta - target), the six sums
+//    sum z, sum z^2, sum a z, sum a z^2, sum q, sum q z  give mean, variance and both reductions of
+//    the gradient formula (reference rust/core/src/util.rs:171-179).
+#pragma once
+#include "ttt_linear_fwd.hip.h"
+
+namespace ttt {
+
+// Workgroup barrier for LDS exchanges only: waits for this wave's LDS traffic, not for the
+// global prefetches in flight (a full __syncthreads() would drain those every mini-batch).
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <class T, int NT, int TPW>
+struct StageInMw {
+  typename Io<T>::frag q[NT], k[NT];               // full rows: k-side operands
+  typename Io<T>::frag qo[TPW], ko[TPW], vo[TPW];  // this wave's features of xq, xk, xv
+  float lr;
+};
+
+template <class T>
+__device__ __forceinline__ typename Io<T>::frag load4(const typename Io<T>::elem* p);
+template <>
+__device__ __forceinline__ Io<F32>::frag load4<F32>(const float* p) {
+  return *reinterpret_cast<const f32x4*>(p);
+}
+template <>
+__device__ __forceinline__ Io<BF16>::frag load4<BF16>(const uint16_t* p) {
+  return __builtin_bit_cast(bf16x4, *reinterpret_cast<const u32x2*>(p));
+}
+template <class T>
+__device__ __forceinline__ void store4(typename Io<T>::elem* p, f32x4 v);
+template <>
+__device__ __forceinline__ void store4<F32>(float* p, f32x4 v) {
+  *reinterpret_cast<f32x4*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void store4<BF16>(uint16_t* p, f32x4 v) {
+  *reinterpret_cast<u32x2*>(p) = __builtin_bit_cast(u32x2, Io<BF16>::to_frag(v));
+}
+
+// Offset (in elements) of the features of own tile jj held by lane group g: four contiguous
+// features feat(J, 4g .. 4g+3), J = w*TPW + jj.
+template <int TPW>
+__device__ __forceinline__ int own_offset(int w, int jj, int g) {
+  const int J = w * TPW + jj;
+  return 32 * (J >> 1) + 8 * g + 4 * (J & 1);
+}
+
+template <class T, int D, int NW, bool FULL>
+__device__ __forceinline__ void load_stage_mw(StageInMw<T, D / 16, D / 16 / NW>& s, const LinearFwdArgs& a,
+                                              size_t bh, int stage, int c, int g, int w) {
+  using IO = Io<T>;
+  using elem = typename IO::elem;
+  constexpr int NT = D / 16, TPW = NT / NW;
+  if (FULL) stage = min(stage, a.n_stages - 1);
+  const bool ok = FULL || ((c < a.K) && (stage < a.n_stages));
+  const size_t tok = bh * a.seq + (size_t)stage * a.K + c;
+  const elem* pq = static_cast<const elem*>(a.xq) + tok * D;
+  const elem* pk = static_cast<const elem*>(a.xk) + tok * D;
+  const elem* pv = static_cast<const elem*>(a.xv) + tok * D;
+#pragma unroll
+  for (int q = 0; q < NT / 2; ++q) {
+    IO::load8(pq + 32 * q + 8 * g, ok, s.q[2 * q], s.q[2 * q + 1]);
+    IO::load8(pk + 32 * q + 8 * g, ok, s.k[2 * q], s.k[2 * q + 1]);
+  }
+  if (NW == 1) {
+    // the wave owns every feature: xq/xk are already there, only xv is extra
+#pragma unroll
+    for (int q = 0; q < NT / 2; ++q) IO::load8(pv + 32 * q + 8 * g, ok, s.vo[2 * q], s.vo[2 * q + 1]);
+  } else if (TPW == 1) {
+    const int off = own_offset<TPW>(w, 0, g);
+    if (ok) {
+      s.qo[0] = load4<T>(pq + off);
+      s.ko[0] = load4<T>(pk + off);
+      s.vo[0] = load4<T>(pv + off);
+    } else {
+      s.qo[0] = s.ko[0] = s.vo[0] = IO::zero();
+    }
+  } else {
+#pragma unroll
+    for (int qq = 0; qq < TPW / 2; ++qq) {
+      const int off = own_offset<TPW>(w, 2 * qq, g);  // eight contiguous features: tiles 2qq, 2qq+1
+      IO::load8(pq + off, ok, s.qo[2 * qq], s.qo[2 * qq + 1]);
+      IO::load8(pk + off, ok, s.ko[2 * qq], s.ko[2 * qq + 1]);
+      IO::load8(pv + off, ok, s.vo[2 * qq], s.vo[2 * qq + 1]);
+    }
+  }
+  s.lr = ok ? IO::load1(static_cast<const elem*>(a.lr) + tok) : 0.f;
+}
+
+// Sum over the four lane groups.  MF: one f32 MFMA against a ones operand (keeps the VALU free);
+// otherwise the lane-swap reduction.
+template <bool MF>
+__device__ __forceinline__ float xg_reduce(float v) {
+  if (MF) {
+    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    z = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, v, z, 0, 0, 0);
+    return z[0];
+  }
+  return xg_sum(v);
+}
+
+template <class T, int D, int NW, int PF, bool FULL>
+__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArgs a) {
+  using IO = Io<T>;
+  using frag = typename IO::frag;
+  using elem = typename IO::elem;
+  constexpr int NT = D / 16, TPW = NT / NW;
+  constexpr bool BF = sizeof(elem) == 2;  // bf16 storage: MFMA pipe has room for helper products
+  constexpr float inv_d = 1.0f / D;
+  __shared__ float ex1[6 * 16 * NW];
+  __shared__ float ex2[2 * 16 * NW];
+
+  const int lane = threadIdx.x & 63, w = (threadIdx.x >> 6) % NW;
+  const int c = lane & 15, g = lane >> 4;
+  const size_t bh = blockIdx.x;
+  const int h = (int)(bh % a.H);
+  const int K = a.K;
+
+  // eta_last = token_eta[K-1] * lr is folded into G itself: G'' = -sc * lr * G with
+  // sc = token_eta[K-1], so the state update is W += XK^T G'' with no further scaling and the
+  // causal matrix becomes (token_eta[t] / sc) (1 + A[t][s]).  sc == 0 (no state update at all)
+  // falls back to sc = 1 and skips the update.
+  const float te_last = a.token_eta[K - 1];
+  const bool upd = te_last != 0.f;
+  const float sc = upd ? te_last : 1.f;
+  const float rho_c = (c < K) ? a.token_eta[c] / sc : 0.f;
+  const frag ident = identity_frag<T>(c, g);
+  const frag nident = identity_frag<T>(c, g, -1.f);
+  const frag ones = splat_frag<T>(1.f);
+  const size_t sb = a.state_per_batch ? bh : (size_t)h;
+  f32x4 gam[TPW], bet[TPW], bT[TPW], a2[TPW];
+  float sum_a = 0.f;
+#pragma unroll
+  for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int f = own_offset<TPW>(w, jj, g) + r;
+      gam[jj][r] = a.gamma[h * D + f];
+      bet[jj][r] = a.beta[h * D + f];
+      bT[jj][r] = a.b0[sb * D + f];
+      a2[jj][r] = gam[jj][r] * gam[jj][r];
+    }
+  for (int f = 0; f < D; ++f) sum_a += a.gamma[h * D + f] * a.gamma[h * D + f];
+  // Wc[I][jj][r] = W[feat(I,4g+r)][feat(w*TPW+jj, c)]
+  f32x4 Wc[NT][TPW];
+  {
+    const float* W0 = a.W0 + sb * D * D;
+#pragma unroll
+    for (int I = 0; I < NT; ++I)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Wc[I][jj][r] = W0[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)];
+  }
+
+  // Ring of R = PF+1 register sets, loop unrolled by R: step u consumes set u and refills the set
+  // that step u-1 consumed, so every set has fixed registers and a load is never copied (a copy
+  // at the loop back-edge would have to wait for the load, i.e. undo the prefetch).
+  constexpr int R = PF + 1;
+  StageInMw<T, NT, TPW> buf[R];
+#pragma unroll
+  for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], a, bh, u, c, g, w);
+
+  for (int st0 = 0; st0 < a.n_stages; st0 += R) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int st = st0 + u;
+      load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], a, bh, st + PF, c, g, w);
+      if (st >= a.n_stages) continue;
+      const StageInMw<T, NT, TPW>& cur = buf[u];
+
+      if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
+        const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
+        float* Wd = a.W_ckpt + ci * D * D;
+#pragma unroll
+        for (int I = 0; I < NT; ++I)
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+        if (c == 0)
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
+      }
+
+      // ---- Z1^T, Zbar^T (this wave's feature rows) and the attention block
+      f32x4 z1[TPW], zb[TPW], At = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        z1[jj] = bT[jj];
+        zb[jj] = bT[jj];
+      }
+#pragma unroll
+      for (int q = 0; q < NT / 2; ++q) {
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          const frag w0 = IO::to_frag(Wc[2 * q][jj]), w1 = IO::to_frag(Wc[2 * q + 1][jj]);
+          IO::mma2(z1[jj], w0, w1, cur.k[2 * q], cur.k[2 * q + 1]);
+          IO::mma2(zb[jj], w0, w1, cur.q[2 * q], cur.q[2 * q + 1]);
+        }
+        IO::mma2(At, cur.k[2 * q], cur.k[2 * q + 1], cur.q[2 * q], cur.q[2 * q + 1]);
+      }
+      // ---- raw moments of this wave's features
+      f32x4 bq[TPW];
+      float S[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const frag ko = (NW == 1) ? cur.k[jj] : cur.ko[jj];
+        f32x4 uu;  // beta - (xv - xk)
+        if (BF) {
+          uu = bet[jj];
+          IO::mma2(uu, nident, ident, cur.vo[jj], ko);
+        } else {
+          uu = bet[jj] - (IO::to_f32(cur.vo[jj]) - IO::to_f32(ko));
+        }
+        bq[jj] = gam[jj] * uu;
+        const f32x4 az = a2[jj] * z1[jj];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          S[0] += z1[jj][r];
+          S[1] += z1[jj][r] * z1[jj][r];
+          S[2] += az[r];
+          S[3] += az[r] * z1[jj][r];
+          S[4] += bq[jj][r];
+          S[5] += bq[jj][r] * z1[jj][r];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 6; ++i) S[i] = xg_reduce<BF>(S[i]);
+      if (NW > 1) {
+        // lane group g publishes sums g and g+4; every lane then adds up the waves
+        float v0 = S[0], v1 = S[4];
+        if (g == 1) { v0 = S[1]; v1 = S[5]; }
+        if (g == 2) v0 = S[2];
+        if (g == 3) v0 = S[3];
+        ex1[(g * 16 + c) * NW + w] = v0;
+        if (g < 2) ex1[((g + 4) * 16 + c) * NW + w] = v1;
+        lds_barrier();
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+          float s = 0.f;
+#pragma unroll
+          for (int ww = 0; ww < NW; ++ww) s += ex1[(i * 16 + c) * NW + ww];
+          S[i] = s;
+        }
+      }
+      f32x4 G[TPW];
+      {
+        const float mu = S[0] * inv_d;
+        const float var = S[1] * inv_d - mu * mu;
+        const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+        const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
+        const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
+        // G'' = p (gx - s1/d - xh s2/d), gx = a2 xh + bq, xh = (z - mu) rstd, p = -sc lr rstd
+        //     = (z - mu) (c1 a2 + c2) + (p bq + c3)
+        const float p = -sc * cur.lr * rstd;
+        const float c1 = p * rstd, c2 = -c1 * s2 * inv_d, c3 = -p * s1 * inv_d;
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) G[jj] = (z1[jj] - mu) * (a2[jj] * c1 + c2) + (bq[jj] * p + c3);
+      }
+      // ---- G'' with tokens along k; causal correction Zbar^T += G''^T M''^T
+      frag Gd[TPW];
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+        IO::mma(t, IO::to_frag(G[jj]), ident);
+        Gd[jj] = IO::to_frag(t);
+      }
+      {
+        f32x4 m;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + At[r]) : 0.f;
+        const frag Mf = IO::to_frag(m);
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) IO::mma(zb[jj], Gd[jj], Mf);
+      }
+      // ---- output LayerNorm
+      {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            s0 += zb[jj][r];
+            s1 += zb[jj][r] * zb[jj][r];
+          }
+        s0 = xg_reduce<BF>(s0);
+        s1 = xg_reduce<BF>(s1);
+        if (NW > 1) {
+          if (g < 2) ex2[(g * 16 + c) * NW + w] = (g == 0) ? s0 : s1;
+          lds_barrier();
+          s0 = s1 = 0.f;
+#pragma unroll
+          for (int ww = 0; ww < NW; ++ww) {
+            s0 += ex2[c * NW + ww];
+            s1 += ex2[(16 + c) * NW + ww];
+          }
+        }
+        const float mu = s0 * inv_d;
+        const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
+        if (FULL || c < K) {
+          elem* po = static_cast<elem*>(a.out) + (bh * a.seq + (size_t)st * K + c) * D;
+          f32x4 o[TPW];
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) {
+            const frag qo = (NW == 1) ? cur.q[jj] : cur.qo[jj];
+            f32x4 qb;  // xq + beta
+            if (BF) {
+              qb = bet[jj];
+              IO::mma(qb, ident, qo);
+            } else {
+              qb = IO::to_f32(qo) + bet[jj];
+            }
+            o[jj] = qb + gam[jj] * ((zb[jj] - mu) * rstd);
+          }
+          if (TPW == 1) {
+            store4<T>(po + own_offset<TPW>(w, 0, g), o[0]);
+          } else {
+#pragma unroll
+            for (int qq = 0; qq < TPW / 2; ++qq)
+              IO::store8(po + own_offset<TPW>(w, 2 * qq, g), o[2 * qq], o[2 * qq + 1]);
+          }
+        }
+      }
+      // ---- state update of this wave's column slice (linear.rs:134-144): W += XK^T G'', b += colsum G''
+      if (upd) {
+#pragma unroll
+        for (int I = 0; I < NT; ++I) {
+          f32x4 t = {0.f, 0.f, 0.f, 0.f};
+          IO::mma(t, cur.k[I], ident);  // t[r] = XK[s = 4g+r][feat(I,c)]
+          const frag kd = IO::to_frag(t);
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd, Gd[jj]);
+        }
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones);
+      }
+    }
+  }
+
+  {
+    float* Wd = a.W_out + bh * D * D;
+#pragma unroll
+    for (int I = 0; I < NT; ++I)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+    if (c == 0)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_out + bh * D + own_offset<TPW>(w, jj, g), bT[jj]);
+  }
+}
+
+}  // namespace ttt

@@ -1,0 +1,278 @@
+// TTT-Linear multi-stage forward for gfx950: the workgroup kernel of ttt_linear_fwd_mw.hip.h with
+// the output path skewed by one mini-batch.
+//
+// Per mini-batch t a wave has two dependency chains:
+//   recurrence  W_t -> Z1 -> LayerNorm statistics -> G -> W_{t+1}     (must finish before t+1 starts)
+//   output      Zbar_t -> LayerNorm statistics -> out_t               (nothing waits for it)
+// Each needs its own cross-wave exchange of row sums.  Here the output chain of mini-batch t-1 runs
+// inside iteration t: its two sums travel in the same LDS exchange as the six sums of the
+// recurrence (lane group g publishes sums g and g+4: eight in all), so there is ONE barrier per
+// mini-batch, and between two barriers the instruction stream always holds two independent chains
+// for the in-order issue to interleave.  The exchange buffer is double-buffered by parity because
+// one barrier per iteration does not separate a fast wave's next write from a slow wave's read.
+#pragma once
+#include "ttt_linear_fwd_mw.hip.h"
+
+namespace ttt {
+
+template <class T, int D, int NW, int PF, bool FULL>
+__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArgs a) {
+  using IO = Io<T>;
+  using frag = typename IO::frag;
+  using elem = typename IO::elem;
+  constexpr int NT = D / 16, TPW = NT / NW;
+  constexpr bool BF = sizeof(elem) == 2;
+  constexpr float inv_d = 1.0f / D;
+  static_assert(NW > 1, "the skewed kernel is for two or more waves per unit");
+  __shared__ float ex[2][8 * 16 * NW];
+
+  const int lane = threadIdx.x & 63, w = (threadIdx.x >> 6) % NW;
+  const int c = lane & 15, g = lane >> 4;
+  const size_t bh = blockIdx.x;
+  const int h = (int)(bh % a.H);
+  const int K = a.K;
+
+  // same scale folding as the unskewed kernel: G'' = -sc lr G, M'' = (token_eta[t]/sc)(1 + A)
+  const float te_last = a.token_eta[K - 1];
+  const bool upd = te_last != 0.f;
+  const float sc = upd ? te_last : 1.f;
+  const float rho_c = (c < K) ? a.token_eta[c] / sc : 0.f;
+  const frag ident = identity_frag<T>(c, g);
+  const frag nident = identity_frag<T>(c, g, -1.f);
+  const frag ones = splat_frag<T>(1.f);
+  const size_t sb = a.state_per_batch ? bh : (size_t)h;
+  f32x4 gam[TPW], bet[TPW], bT[TPW], a2[TPW];
+  float sum_a = 0.f;
+#pragma unroll
+  for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int f = own_offset<TPW>(w, jj, g) + r;
+      gam[jj][r] = a.gamma[h * D + f];
+      bet[jj][r] = a.beta[h * D + f];
+      bT[jj][r] = a.b0[sb * D + f];
+      a2[jj][r] = gam[jj][r] * gam[jj][r];
+    }
+  for (int f = 0; f < D; ++f) sum_a += a.gamma[h * D + f] * a.gamma[h * D + f];
+  f32x4 Wc[NT][TPW];
+  {
+    const float* W0 = a.W0 + sb * D * D;
+#pragma unroll
+    for (int I = 0; I < NT; ++I)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Wc[I][jj][r] = W0[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)];
+  }
+
+  // pending output of the previous mini-batch
+  f32x4 zbp[TPW];
+  frag qop[TPW];
+#pragma unroll
+  for (int jj = 0; jj < TPW; ++jj) {
+    zbp[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+    qop[jj] = IO::zero();
+  }
+
+  // publish this lane group's two sums, wait for the other waves, add up
+  auto exchange8 = [&](float (&S)[8], int parity) {
+    // lane group g ends up with sums g and g+4 reduced over the wave, and publishes them
+    const float v0 = xg_sum4_scatter(S[0], S[1], S[2], S[3]);
+    const float v1 = xg_sum4_scatter(S[4], S[5], S[6], S[7]);
+    float* e = ex[parity];
+    e[(g * 16 + c) * NW + w] = v0;
+    e[((g + 4) * 16 + c) * NW + w] = v1;
+    lds_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float s = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < NW; ++ww) s += e[(i * 16 + c) * NW + ww];
+      S[i] = s;
+    }
+  };
+  // out = xq + gamma (zbar - mu) rstd + beta for the pending mini-batch
+  auto emit_output = [&](float s0, float s1, int stage) {
+    const float mu = s0 * inv_d;
+    const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
+    if (FULL || c < K) {
+      elem* po = static_cast<elem*>(a.out) + (bh * a.seq + (size_t)stage * K + c) * D;
+      f32x4 o[TPW];
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        f32x4 qb;
+        if (BF) {
+          qb = bet[jj];
+          IO::mma(qb, ident, qop[jj]);
+        } else {
+          qb = IO::to_f32(qop[jj]) + bet[jj];
+        }
+        o[jj] = qb + gam[jj] * ((zbp[jj] - mu) * rstd);
+      }
+      if (TPW == 1) {
+        store4<T>(po + own_offset<TPW>(w, 0, g), o[0]);
+      } else {
+#pragma unroll
+        for (int qq = 0; qq < TPW / 2; ++qq)
+          IO::store8(po + own_offset<TPW>(w, 2 * qq, g), o[2 * qq], o[2 * qq + 1]);
+      }
+    }
+  };
+
+  constexpr int R = PF + 1;
+  StageInMw<T, NT, TPW> buf[R];
+#pragma unroll
+  for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], a, bh, u, c, g, w);
+
+  for (int st0 = 0; st0 < a.n_stages; st0 += R) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int st = st0 + u;
+      load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], a, bh, st + PF, c, g, w);
+      if (st >= a.n_stages) continue;
+      const StageInMw<T, NT, TPW>& cur = buf[u];
+
+      if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
+        const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
+        float* Wd = a.W_ckpt + ci * D * D;
+#pragma unroll
+        for (int I = 0; I < NT; ++I)
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+        if (c == 0)
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
+      }
+
+      // ---- XK with tokens along k for the state update: depends on nothing computed here, so it
+      // is issued first and fills the gaps of the dependent chain below
+      frag kd[NT];
+#pragma unroll
+      for (int I = 0; I < NT; ++I) {
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+        IO::mma(t, cur.k[I], ident);  // t[r] = XK[s = 4g+r][feat(I,c)]
+        kd[I] = IO::to_frag(t);
+      }
+      // ---- Z1^T, Zbar^T (this wave's feature rows) and the attention block
+      f32x4 z1[TPW], zb[TPW], At = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        z1[jj] = bT[jj];
+        zb[jj] = bT[jj];
+      }
+#pragma unroll
+      for (int q = 0; q < NT / 2; ++q) {
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          const frag w0 = IO::to_frag(Wc[2 * q][jj]), w1 = IO::to_frag(Wc[2 * q + 1][jj]);
+          IO::mma2(z1[jj], w0, w1, cur.k[2 * q], cur.k[2 * q + 1]);
+          IO::mma2(zb[jj], w0, w1, cur.q[2 * q], cur.q[2 * q + 1]);
+        }
+        IO::mma2(At, cur.k[2 * q], cur.k[2 * q + 1], cur.q[2 * q], cur.q[2 * q + 1]);
+      }
+      // ---- row sums: six raw moments of Z1 (this mini-batch), two of the pending Zbar
+      f32x4 bq[TPW];
+      float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        f32x4 uu;  // beta - (xv - xk)
+        if (BF) {
+          uu = bet[jj];
+          IO::mma2(uu, nident, ident, cur.vo[jj], cur.ko[jj]);
+        } else {
+          uu = bet[jj] - (IO::to_f32(cur.vo[jj]) - IO::to_f32(cur.ko[jj]));
+        }
+        bq[jj] = gam[jj] * uu;
+        const f32x4 az = a2[jj] * z1[jj];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          S[0] += z1[jj][r];
+          S[1] += z1[jj][r] * z1[jj][r];
+          S[2] += az[r];
+          S[3] += az[r] * z1[jj][r];
+          S[4] += bq[jj][r];
+          S[5] += bq[jj][r] * z1[jj][r];
+          S[6] += zbp[jj][r];
+          S[7] += zbp[jj][r] * zbp[jj][r];
+        }
+      }
+      exchange8(S, st & 1);
+
+      // ---- pending output (previous mini-batch): independent of everything below
+      if (st > 0) emit_output(S[6], S[7], st - 1);
+
+      // ---- recurrence: G'' , causal correction, state update
+      f32x4 G[TPW];
+      {
+        const float mu = S[0] * inv_d;
+        const float var = S[1] * inv_d - mu * mu;
+        const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+        const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
+        const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
+        const float p = -sc * cur.lr * rstd;
+        const float c1 = p * rstd, c2 = -c1 * s2 * inv_d, c3 = -p * s1 * inv_d;
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) G[jj] = (z1[jj] - mu) * (a2[jj] * c1 + c2) + (bq[jj] * p + c3);
+      }
+      frag Gd[TPW];
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+        IO::mma(t, IO::to_frag(G[jj]), ident);
+        Gd[jj] = IO::to_frag(t);
+      }
+      {
+        f32x4 m;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + At[r]) : 0.f;
+        const frag Mf = IO::to_frag(m);
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) IO::mma(zb[jj], Gd[jj], Mf);
+      }
+      if (upd) {
+#pragma unroll
+        for (int I = 0; I < NT; ++I)
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones);
+      }
+      // this mini-batch's Zbar and xq become the pending output
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        zbp[jj] = zb[jj];
+        qop[jj] = cur.qo[jj];
+      }
+    }
+  }
+
+  // ---- flush the last mini-batch's output
+  {
+    float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        S[6] += zbp[jj][r];
+        S[7] += zbp[jj][r] * zbp[jj][r];
+      }
+    exchange8(S, a.n_stages & 1);
+    emit_output(S[6], S[7], a.n_stages - 1);
+  }
+  {
+    float* Wd = a.W_out + bh * D * D;
+#pragma unroll
+    for (int I = 0; I < NT; ++I)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+    if (c == 0)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_out + bh * D + own_offset<TPW>(w, jj, g), bT[jj]);
+  }
+}
+
+}  // namespace ttt

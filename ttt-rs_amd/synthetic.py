@@ -27,11 +27,11 @@ def baseline_inputs(config_idx: int, B: int, H: int, seq: int, d: int, K: int = 
     c["xq"], c["xk"], c["xv"] = n(B, H, seq, d), n(B, H, seq, d), n(B, H, seq, d)
     if mlp:
         c["W1"], c["W2"] = n(H, d, 4 * d) * 0.02, n(H, 4 * d, d) * 0.02
-        c["b1"], c["b2"] = torch.zeros(H, 4 * d), torch.zeros(H, d)
+        c["b1"], c["b2"] = torch.zeros(H, 4 * d, dtype=torch.float32), torch.zeros(H, d, dtype=torch.float32)
     else:
         c["W0"] = n(H, d, d) * 0.02
-        c["b0"] = torch.zeros(H, d)
-    c["gamma"], c["beta"] = torch.ones(H, d), torch.zeros(H, d)
+        c["b0"] = torch.zeros(H, d, dtype=torch.float32)
+    c["gamma"], c["beta"] = torch.ones(H, d, dtype=torch.float32), torch.zeros(H, d, dtype=torch.float32)
     c["lr"] = (base_lr / d) * torch.sigmoid(n(B, H, seq))
     c["token_eta"] = 1.0 / torch.arange(1, K + 1, dtype=torch.float32)
     if with_dout:
@@ -55,7 +55,7 @@ def reference_test_inputs(seed: int, B: int, H: int, seq: int, d: int, K: int,
     if trained_params:
         c["gamma"], c["beta"] = n(H, d) * 0.02, n(H, d) * 0.02
     else:
-        c["gamma"], c["beta"] = torch.ones(H, d), torch.zeros(H, d)
+        c["gamma"], c["beta"] = torch.ones(H, d, dtype=torch.float32), torch.zeros(H, d, dtype=torch.float32)
     c["lr"] = 0.01 + 0.04 * torch.rand(B, H, seq, generator=g, dtype=torch.float32)
     c["token_eta"] = 1.0 / torch.arange(1, K + 1, dtype=torch.float32)
     for k in ("xq", "xk", "xv", "lr"):
