@@ -11,34 +11,77 @@
 namespace ttt {
 
 // C[16*Mt x 16*Nt] (row-major, stride ldc)  op=  A * B over k in [k0, k0+Kd), Kd a multiple of 4.
-// A(m,k) = A[m*a_rs + k*a_cs], B(k,n) = B[k*b_rs + n*b_cs].  Output tiles are dealt round-robin
-// to the NW waves of the workgroup, starting at wave `first`.
+// A(m,k) = A[m*a_rs + k*a_cs], B(k,n) = B[k*b_rs + n*b_cs].
 // MODE 0: C = AB   1: C += AB   2: C -= AB   3: C *= AB (elementwise)
-template <int MODE, int NW = 4>
+//
+// Work split: the tile row tm and a block of NB consecutive tile columns form one job; jobs are
+// dealt round-robin to the NW waves of the workgroup, starting at wave `first`.  Inside a job the
+// A element of a k-step is loaded once and feeds NB MFMAs, and KU k-steps of operands are fetched
+// before the first MFMA of the group issues, so the loads of a group overlap its MFMAs.
+template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8)>
 __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_rs, int a_cs,
                                        const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
                                        int wave, int lane, int first = 0, int k0 = 0) {
   const int c = lane & 15, g = lane >> 4;
-  const int ntiles = Mt * Nt;
-  for (int tile = (wave - first + NW) % NW; tile < ntiles; tile += NW) {
-    const int tm = tile / Nt, tn = tile - tm * Nt;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    float* Ct = C + (size_t)(16 * tm + 4 * g) * ldc + 16 * tn + c;
-    if (MODE == 1 || MODE == 2) {
+  const int nblk = (Nt + NB - 1) / NB;
+  const int njobs = Mt * nblk;
+#pragma nounroll
+  for (int job = (wave - first + NW) % NW; job < njobs; job += NW) {
+    const int tm = job / nblk, tn0 = (job - tm * nblk) * NB;
+    // 32-bit element offsets from the (wave-uniform) base pointers keep the address math in
+    // single registers: base in SGPRs, one VGPR offset per access
+    f32x4 acc[NB];
+    const int coff = (16 * tm + 4 * g) * ldc + 16 * tn0 + c;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[r] = (MODE == 1) ? Ct[(size_t)r * ldc] : -Ct[(size_t)r * ldc];
+    for (int j = 0; j < NB; ++j) {
+      const bool live = tn0 + j < Nt;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = 0.f;
+        if ((MODE == 1 || MODE == 2) && live) v = C[coff + r * ldc + 16 * j];
+        acc[j][r] = (MODE == 2) ? -v : v;
+      }
     }
-    const float* Ap = A + (size_t)(16 * tm + c) * a_rs + (size_t)(k0 + g) * a_cs;
-    const float* Bp = B + (size_t)(k0 + g) * b_rs + (size_t)(16 * tn + c) * b_cs;
-#pragma unroll 4
-    for (int k = 0; k < Kd; k += 4)
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ap[(size_t)k * a_cs], Bp[(size_t)k * b_rs], acc, 0, 0, 0);
+    const int aoff = (16 * tm + c) * a_rs + (k0 + g) * a_cs;
+    const int boff = (k0 + g) * b_rs + (16 * tn0 + c) * b_cs;
+    const int astep = 4 * a_cs, bstep = 4 * b_rs, bcol = 16 * b_cs;
+    int k = 0;
+#pragma nounroll
+    for (; k + 4 * KU <= Kd; k += 4 * KU) {
+      float av[KU], bv[KU][NB];
+      const int ak = aoff + k * a_cs, bk = boff + k * b_rs;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      if (MODE == 3)
-        Ct[(size_t)r * ldc] *= acc[r];
-      else
-        Ct[(size_t)r * ldc] = (MODE == 2) ? -acc[r] : acc[r];
+      for (int u = 0; u < KU; ++u) {
+        av[u] = A[ak + u * astep];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) bv[u][j] = (tn0 + j < Nt) ? B[bk + u * bstep + j * bcol] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < KU; ++u)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u][j], acc[j], 0, 0, 0);
+    }
+#pragma nounroll
+    for (; k < Kd; k += 4) {
+      const float av = A[aoff + k * a_cs];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const float bv = (tn0 + j < Nt) ? B[boff + k * b_rs + j * bcol] : 0.f;
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[j], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      if (tn0 + j >= Nt) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float* p = C + coff + r * ldc + 16 * j;
+        if (MODE == 3)
+          *p *= acc[j][r];
+        else
+          *p = (MODE == 2) ? -acc[j][r] : acc[j][r];
+      }
     }
   }
 }

@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a
       lds[L::M + t * LK + s] = (s <= t) ? ste[t] * slr[s] * (1.f + at) : 0.f;
     }
     __syncthreads();
-    mm_lds<2>(lds + L::ZB, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NT, 16, wave, lane);
+    mm_lds<2, 4, 1, 4>(lds + L::ZB, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NT, 16, wave, lane);
     __syncthreads();
     {
       float xh[NJ], rstd;
@@ -151,7 +151,7 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a
       }
     }
     __syncthreads();
-    mm_lds<2>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NT, NT, 16, wave, lane);
+    mm_lds<2, 4, (NT % 4 == 0 ? 4 : 2), 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NT, NT, 16, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < 16; ++r) s += lds[L::G + r * LD + tid];
@@ -210,6 +210,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
   using L = MlpLds<D>;
   constexpr int M = L::M, LD = L::LD, LM = L::LM, LK = L::LK;
   constexpr int NW = 8, GW = 32, NJD = D / GW, NJM = M / GW, NTD = D / 16, NTM = M / 16;
+  constexpr int NBM = NTM / NW;  // hidden-side tile columns per job: one job per wave
+  constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
   extern __shared__ float lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int t = tid >> 5, cg = tid & 31;
@@ -252,10 +254,9 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
       slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * a.seq + (size_t)st * K + tid) : 0.f;
     __syncthreads();
     // ---- Z1 = XK W1 ; Zbar1 = XQ W1 ; A1 = XQ XK^T            (mlp.rs:139,160,167)
-    mm_lds<0, NW>(lds + L::BA, LM, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
-    mm_lds<0, NW>(lds + L::BC, LM, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane, NTM % NW);
-    mm_lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane,
-                  (2 * NTM) % NW);
+    mm_lds<0, NW, NBM>(lds + L::BA, LM, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
+    mm_lds<0, NW, NBM>(lds + L::BC, LM, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
+    mm_lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane);
     __syncthreads();
     // ---- X2 = gelu(Z1 + b1), keep gelu'(Z1 + b1) ; eta, M1 = eta (1 + A1)   (mlp.rs:141,154-162)
 #pragma unroll
@@ -285,10 +286,10 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
     }
     __syncthreads();
     // ---- G1 = (G2 W2^T) * gelu'(Z1)                           (mlp.rs:151-152)
-    mm_lds<3, NW>(lds + L::BA, LM, lds + L::Z2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<3, NW, NBM>(lds + L::BA, LM, lds + L::Z2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- Zbar1 -= M1 G1                                       (mlp.rs:164-169)
-    mm_lds<2, NW>(lds + L::BC, LM, lds + L::M1, LK, 1, lds + L::BA, LM, 1, 1, NTM, 16, wave, lane);
+    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(lds + L::BC, LM, lds + L::M1, LK, 1, lds + L::BA, LM, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
     // ---- Xbar2 = gelu(Zbar1 + b1)                             (mlp.rs:171)
 #pragma unroll
@@ -322,7 +323,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
     }
     __syncthreads();
     // ---- Zbar2 -= M2 G2                                       (mlp.rs:175-180)
-    mm_lds<2, NW>(lds + L::ZB2, LD, lds + L::M2, LK, 1, lds + L::Z2, LD, 1, 1, NTD, 16, wave, lane);
+    mm_lds<2, NW, 1, 4>(lds + L::ZB2, LD, lds + L::M2, LK, 1, lds + L::Z2, LD, 1, 1, NTD, 16, wave, lane);
     __syncthreads();
     // ---- out = XQ + LN(Zbar2 + b2) ; scale G1, G2 by eta_last  (mlp.rs:182-207)
     {
@@ -342,9 +343,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
     }
     __syncthreads();
     // ---- W1 -= XK^T G1l ; W2 -= X2^T G2l ; b1 -= colsum(G1l) ; b2 -= colsum(G2l)
-    mm_lds<2, NW>(W1, M, lds + L::XK, 1, LD, lds + L::BA, LM, 1, NTD, NTM, 16, wave, lane);
-    mm_lds<2, NW>(W2, D, lds + L::BB, 1, LM, lds + L::Z2, LD, 1, NTM, NTD, 16, wave, lane,
-                  (NTD * NTM) % NW);
+    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(W1, M, lds + L::XK, 1, LD, lds + L::BA, LM, 1, NTD, NTM, 16, wave, lane);
+    mm_lds<2, NW, NBD, (NBD >= 3 ? 1 : 2)>(W2, D, lds + L::BB, 1, LM, lds + L::Z2, LD, 1, NTM, NTD, 16, wave, lane);
     if (tid < M) {
       float s = 0.f;
       for (int r = 0; r < 16; ++r) s += lds[L::BA + r * LM + tid];

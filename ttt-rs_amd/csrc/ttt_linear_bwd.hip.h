@@ -181,7 +181,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       }
       __syncthreads();
       // W -= XK^T (last * G) ; b -= colsum(last * G)      (linear.rs:134-144)
-      mm_lds<2>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, 16, wave, lane);
+      mm_lds<2, 4, NJ, 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, 16, wave, lane);
       if (tid < D) {
         float s = 0.f;
         for (int r = 0; r < 16; ++r) s += lds[L::G + r * LD + tid];
@@ -224,7 +224,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     }
     __syncthreads();
     // Zb = XQ W - M G  (+ b added when read)
-    mm_lds<2>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NJ, 16, wave, lane);
+    mm_lds<2, 4, 1, 4>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NJ, 16, wave, lane);
     __syncthreads();
 
     // ================= output LayerNorm and its backward (stage 4)
@@ -289,10 +289,10 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     __syncthreads();
 
     // ================= dQ += dA XK ; dK = dA^T XQ ; DGM = M^T dZb ; dW += XQ^T dZb ; db += colsum(dZb)
-    mm_lds<1>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NJ, 16, wave, lane, 0);
-    mm_lds<0>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NJ, 16, wave, lane, NJ & 3);
-    mm_lds<0>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, 1, NJ, 16, wave, lane, (2 * NJ) & 3);
-    mm_lds<1>(sdW, LD, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, 16, wave, lane, (3 * NJ) & 3);
+    mm_lds<1, 4, 1, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NJ, 16, wave, lane, 0);
+    mm_lds<0, 4, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NJ, 16, wave, lane, NJ & 3);
+    mm_lds<0, 4, 1, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, 1, NJ, 16, wave, lane, (2 * NJ) & 3);
+    mm_lds<1, 4, NJ, 4>(sdW, LD, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, 16, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < 16; ++r) s += lds[L::DZB + r * LD + tid];
@@ -360,7 +360,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
 
     // ================= dK += dZ1 W^T ; dW += XK^T dZ1 ; db += colsum(dZ1)
     mm_lds<1>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 0);
-    mm_lds<1>(sdW, LD, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, 16, wave, lane, NJ & 3);
+    mm_lds<1, 4, NJ, 4>(sdW, LD, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, 16, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < 16; ++r) s += lds[L::DZ1 + r * LD + tid];
