@@ -45,22 +45,40 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
     const int aoff = (16 * tm + c) * a_rs + (k0 + g) * a_cs;
     const int boff = (k0 + g) * b_rs + (16 * tn0 + c) * b_cs;
     const int astep = 4 * a_cs, bstep = 4 * b_rs, bcol = 16 * b_cs;
-    int k = 0;
-#pragma nounroll
-    for (; k + 4 * KU <= Kd; k += 4 * KU) {
-      float av[KU], bv[KU][NB];
-      const int ak = aoff + k * a_cs, bk = boff + k * b_rs;
+    // two operand buffers in ping-pong: the loads of the next group of KU k-steps are in flight
+    // while the MFMAs of the current group issue (fixed buffers, so no load is ever copied)
+    float avA[KU], bvA[KU][NB], avB[KU], bvB[KU][NB];
+    auto fetch = [&](float (&av)[KU], float (&bv)[KU][NB], int kk) {
+      const int ak = aoff + kk * a_cs, bk = boff + kk * b_rs;
 #pragma unroll
       for (int u = 0; u < KU; ++u) {
         av[u] = A[ak + u * astep];
 #pragma unroll
         for (int j = 0; j < NB; ++j) bv[u][j] = (tn0 + j < Nt) ? B[bk + u * bstep + j * bcol] : 0.f;
       }
+    };
+    auto fma_group = [&](const float (&av)[KU], const float (&bv)[KU][NB]) {
 #pragma unroll
       for (int u = 0; u < KU; ++u)
 #pragma unroll
         for (int j = 0; j < NB; ++j)
           acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u][j], acc[j], 0, 0, 0);
+    };
+    constexpr int KG = 4 * KU;
+    const int ngroups = Kd / KG;
+    int k = 0;
+    if (ngroups > 0) {
+      fetch(avA, bvA, 0);
+      int gi = 0;
+#pragma nounroll
+      for (; gi + 2 <= ngroups; gi += 2) {
+        fetch(avB, bvB, (gi + 1) * KG);
+        fma_group(avA, bvA);
+        if (gi + 2 < ngroups) fetch(avA, bvA, (gi + 2) * KG);
+        fma_group(avB, bvB);
+      }
+      if (gi < ngroups) fma_group(avA, bvA);
+      k = ngroups * KG;
     }
 #pragma nounroll
     for (; k < Kd; k += 4) {
