@@ -50,6 +50,11 @@ typedef struct ttt_desc {
   int32_t state_per_batch;     /* 0: W0/b0 are [H,d,d]/[H,d] shared over the batch
                                   (TTTLinear::init_state, rust/core/src/linear.rs:84-89);
                                   1: [B,H,d,d]/[B,H,d] as the reference kernel takes them */
+  int32_t seq_stride;          /* tokens between consecutive (batch, head) units in xq, xk, xv, lr,
+                                  out and their gradients; 0 = seq (dense).  A window of a longer
+                                  sequence (the reference's slice_seq, rust/core/src/inner.rs:70-77)
+                                  is processed in place by pointing at its first token and passing
+                                  the full length here. */
 } ttt_desc;
 
 /* Library / build identification. */

@@ -140,3 +140,25 @@ def test_inner_model_forward_with_remainder(P):
     assert_close(out, ro, 1e-4, "out")
     assert_close(state.weight, rW, 1e-4, "W")
     assert_close(state.bias, rb, 1e-4, "b")
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_sequence_windows_in_place(P, d):
+    """desc.seq_stride: a window of a longer sequence is processed where it lies (inputs, lr and
+    the output share the pitch); the result equals the packed call bit for bit."""
+    print(f"case windows d={d}", flush=True)
+    B, H, K, seq = 2, 2, 16, 16 * 6
+    c = to_dev(P.synthetic.reference_test_inputs(21, B, H, seq, d, K))
+    lo, hi = 32, 80
+    win = lambda t: t[:, :, lo:hi]
+    out_full = torch.full_like(c["xq"], float("nan"))
+    o1, W1, b1 = P.ttt_linear_forward_raw(win(c["xq"]), win(c["xk"]), win(c["xv"]), c["W0"], c["b0"],
+                                          c["token_eta"], win(c["lr"]), c["gamma"], c["beta"], K,
+                                          out=win(out_full))
+    o2, W2, b2 = P.ttt_linear_forward_raw(win(c["xq"]).contiguous(), win(c["xk"]).contiguous(),
+                                          win(c["xv"]).contiguous(), c["W0"], c["b0"], c["token_eta"],
+                                          win(c["lr"]).contiguous(), c["gamma"], c["beta"], K)
+    torch.cuda.synchronize()
+    assert o1.data_ptr() == win(out_full).data_ptr()
+    assert torch.equal(o1, o2) and torch.equal(W1, W2) and torch.equal(b1, b2)
+    assert torch.isnan(out_full[:, :, :lo]).all() and torch.isnan(out_full[:, :, hi:]).all()

@@ -21,7 +21,7 @@ class TttDesc(C.Structure):
     _fields_ = [
         ("batch", C.c_int32), ("heads", C.c_int32), ("seq", C.c_int32), ("head_dim", C.c_int32),
         ("mini_batch", C.c_int32), ("eps", C.c_float), ("checkpoint_interval", C.c_int32),
-        ("io_dtype", C.c_int32), ("state_per_batch", C.c_int32),
+        ("io_dtype", C.c_int32), ("state_per_batch", C.c_int32), ("seq_stride", C.c_int32),
     ]
 
 

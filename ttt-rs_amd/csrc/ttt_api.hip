@@ -38,6 +38,8 @@ int check_common(const ttt_desc* d) {
   if (d->io_dtype != TTT_F32 && d->io_dtype != TTT_BF16)
     return fail(TTT_ERR_UNSUPPORTED, "io_dtype %d is neither TTT_F32 nor TTT_BF16", d->io_dtype);
   if (!(d->eps > 0.f)) return fail(TTT_ERR_SHAPE, "eps must be positive");
+  if (d->seq_stride != 0 && d->seq_stride < d->seq)
+    return fail(TTT_ERR_SHAPE, "seq_stride (%d) must be 0 or >= seq (%d)", d->seq_stride, d->seq);
   if ((int64_t)d->batch * d->heads > 0x7fffffffLL)
     return fail(TTT_ERR_SHAPE, "batch*heads exceeds the grid limit");
   return TTT_OK;
@@ -178,6 +180,7 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.gamma = gamma; a.beta = beta; a.out = out; a.W_out = W_out; a.b_out = b_out;
   a.W_ckpt = W_ckpt; a.b_ckpt = b_ckpt;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.n_stages = d->seq / d->mini_batch;
   a.ckpt_interval = d->checkpoint_interval;
   a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
@@ -220,6 +223,7 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.d_xq = d_xq; a.d_xk = d_xk; a.d_xv = d_xv; a.d_W0 = d_W0; a.d_b0 = d_b0; a.d_lr = d_lr;
   a.d_token_eta = d_token_eta; a.d_gamma = d_gamma; a.d_beta = d_beta;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.n_stages = d->seq / d->mini_batch;
   a.ckpt_interval = d->checkpoint_interval;
   a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
@@ -270,6 +274,7 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
   a.W1 = W1_out; a.b1 = b1_out; a.W2 = W2_out; a.b2 = b2_out;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.n_stages = d->seq / d->mini_batch;
   a.state_per_batch = d->state_per_batch ? 1 : 0;
   a.eps = d->eps;

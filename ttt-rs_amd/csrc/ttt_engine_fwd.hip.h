@@ -103,7 +103,7 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a
   const float te_last = ste[K - 1];
 
   for (int st = 0; st < a.n_stages; ++st) {
-    const size_t row = bh * a.seq + (size_t)st * K + t;
+    const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
     if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
       const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
       for (int i = tid; i < D * D; i += 256) a.W_ckpt[ci * D * D + i] = sW[(i / D) * LD + (i % D)];
@@ -119,7 +119,7 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a
       lds[L::TG + t * LD + o] = (ok ? IO::load1(static_cast<const elem*>(a.xv) + row * D + o) : 0.f) - k;
     }
     if (tid < 16)
-      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * a.seq + (size_t)st * K + tid) : 0.f;
+      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid) : 0.f;
     __syncthreads();
     mm_lds<0>(lds + L::G, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NT, D, wave, lane);
     mm_lds<0>(lds + L::ZB, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NT, D, wave, lane, NT & 3);
@@ -183,7 +183,7 @@ struct MlpFwdArgs {
   float* b1;
   float* W2;  // [B,H,M,D]
   float* b2;
-  int B, H, seq, K, n_stages, state_per_batch;
+  int B, H, seq, seq_stride, K, n_stages, state_per_batch;
   float eps;
 };
 
@@ -239,7 +239,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
   const float te_last = ste[K - 1];
 
   for (int st = 0; st < a.n_stages; ++st) {
-    const size_t row = bh * a.seq + (size_t)st * K + t;
+    const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
     // ---- load XQ, XK, target = XV - XK
 #pragma unroll
     for (int j = 0; j < NJD; ++j) {
@@ -251,7 +251,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
       lds[L::TG + t * LD + o] = (ok ? IO::load1(static_cast<const elem*>(a.xv) + row * D + o) : 0.f) - k;
     }
     if (tid < 16)
-      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * a.seq + (size_t)st * K + tid) : 0.f;
+      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid) : 0.f;
     __syncthreads();
     // ---- Z1 = XK W1 ; Zbar1 = XQ W1 ; A1 = XQ XK^T            (mlp.rs:139,160,167)
     mm_lds<0, NW, NBM>(lds + L::BA, LM, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);

@@ -43,7 +43,7 @@ struct LinearBwdArgs {
   float* d_token_eta;
   float* d_gamma;
   float* d_beta;
-  int B, H, seq, K, n_stages, ckpt_interval, n_ckpt;
+  int B, H, seq, seq_stride, K, n_stages, ckpt_interval, n_ckpt;
   float eps;
 };
 
@@ -110,13 +110,13 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
 
   // load one [K x D] activation tile into LDS as f32 (rows >= K are zero)
   auto load_tile = [&](float* dst, const void* src, int stage) {
-    const elem* p = static_cast<const elem*>(src) + (bh * a.seq + (size_t)stage * K + t) * D;
+    const elem* p = static_cast<const elem*>(src) + (bh * (size_t)a.seq_stride + (size_t)stage * K + t) * D;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) dst[t * LD + cg + 16 * j] = (t < K) ? IO::load1(p + cg + 16 * j) : 0.f;
   };
   auto load_lr = [&](int stage) {
     if (tid < 16)
-      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * a.seq + (size_t)stage * K + tid) : 0.f;
+      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
   };
 
   // LayerNorm + L2-gradient pieces for this thread's token (row of `z` + bias): returns x_hat,
@@ -303,7 +303,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       float s = 0.f;
       for (int r = 0; r < 16; ++r) s += lds[L::DETA + r * LK + tid] * ste[r];
       s += te_last * lds[L::dlast + tid];
-      if (tid < K) IO::store1(static_cast<elem*>(a.d_lr) + bh * a.seq + (size_t)st * K + tid, s);
+      if (tid < K) IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid, s);
     } else if (tid >= 64 && tid < 80) {
       const int tt = tid - 64;
       float s = 0.f;
@@ -346,7 +346,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       }
       q1 = row16_sum(q1) * inv_d;
       const float dsig = -row16_sum(q2) * rstd1;  // d loss / d sigma
-      elem* pv = static_cast<elem*>(a.d_xv) + (bh * a.seq + (size_t)st * K + t) * D;
+      elem* pv = static_cast<elem*>(a.d_xv) + (bh * (size_t)a.seq_stride + (size_t)st * K + t) * D;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const int o = cg + 16 * j;
@@ -370,8 +370,8 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
 
     // ================= store dXQ = dO + dQ, dXK
     if (t < K) {
-      elem* pq = static_cast<elem*>(a.d_xq) + (bh * a.seq + (size_t)st * K + t) * D;
-      elem* pk = static_cast<elem*>(a.d_xk) + (bh * a.seq + (size_t)st * K + t) * D;
+      elem* pq = static_cast<elem*>(a.d_xq) + (bh * (size_t)a.seq_stride + (size_t)st * K + t) * D;
+      elem* pk = static_cast<elem*>(a.d_xk) + (bh * (size_t)a.seq_stride + (size_t)st * K + t) * D;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const int o = cg + 16 * j;

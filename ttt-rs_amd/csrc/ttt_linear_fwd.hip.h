@@ -21,7 +21,7 @@ struct LinearFwdArgs {
   float* b_out;
   float* W_ckpt;
   float* b_ckpt;
-  int B, H, seq, K, n_stages, ckpt_interval, n_ckpt, state_per_batch;
+  int B, H, seq, seq_stride, K, n_stages, ckpt_interval, n_ckpt, state_per_batch;
   float eps;
 };
 

@@ -73,7 +73,7 @@ __device__ __forceinline__ void load_stage_mw(StageInMw<T, D / 16, D / 16 / NW>&
   constexpr int NT = D / 16, TPW = NT / NW;
   if (FULL) stage = min(stage, a.n_stages - 1);
   const bool ok = FULL || ((c < a.K) && (stage < a.n_stages));
-  const size_t tok = bh * a.seq + (size_t)stage * a.K + c;
+  const size_t tok = bh * (size_t)a.seq_stride + (size_t)stage * a.K + c;
   const elem* pq = static_cast<const elem*>(a.xq) + tok * D;
   const elem* pk = static_cast<const elem*>(a.xk) + tok * D;
   const elem* pv = static_cast<const elem*>(a.xv) + tok * D;
@@ -319,7 +319,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
         const float mu = s0 * inv_d;
         const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
         if (FULL || c < K) {
-          elem* po = static_cast<elem*>(a.out) + (bh * a.seq + (size_t)st * K + c) * D;
+          elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
           f32x4 o[TPW];
 #pragma unroll
           for (int jj = 0; jj < TPW; ++jj) {

@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
     const float mu = s0 * inv_d;
     const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
     if (FULL || c < K) {
-      elem* po = static_cast<elem*>(a.out) + (bh * a.seq + (size_t)stage * K + c) * D;
+      elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D;
       f32x4 o[TPW];
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) {

@@ -90,9 +90,42 @@ def _need(t: torch.Tensor, shape, dtype, name):
     return t.contiguous()
 
 
+def _seq_pitch(t: torch.Tensor) -> Optional[int]:
+    """Tokens between consecutive (batch, head) units if `t` ([B,H,seq,d] or [B,H,seq]) is a
+    window along seq of a dense tensor (what slicing dim 2 of a contiguous tensor gives), else None."""
+    trail = t.shape[3] if t.dim() == 4 else 1
+    st = t.stride()
+    if t.dim() == 4 and (st[3] != 1 or st[2] != trail):
+        return None
+    if t.dim() == 3 and st[2] != 1:
+        return None
+    if st[1] % trail or st[0] != t.shape[1] * st[1]:
+        return None
+    pitch = st[1] // trail
+    return pitch if pitch >= t.shape[2] else None
+
+
+def _common_pitch(seq: int, *tensors) -> int:
+    """The shared sequence pitch of the given windows, or 0 when they have to be packed."""
+    pitches = {_seq_pitch(t) for t in tensors}
+    if len(pitches) == 1 and None not in pitches:
+        p = pitches.pop()
+        return 0 if p == seq else p
+    return 0
+
+
+def _need_win(t: torch.Tensor, shape, dtype, name, pitch: int):
+    """Like _need, but keeps a sequence window in place when a pitch is in use."""
+    if pitch == 0:
+        return _need(t, shape, dtype, name)
+    if tuple(t.shape) != tuple(shape) or t.dtype != dtype or not t.is_cuda:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, f"{name}: expected {tuple(shape)} {dtype} on the device")
+    return t
+
+
 def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
                            mini_batch: int, eps: float = 1e-6, checkpoint_interval: int = 1,
-                           want_checkpoints: bool = False):
+                           want_checkpoints: bool = False, out: Optional[torch.Tensor] = None):
     """One call of ttt_linear_fwd on the current stream.
 
     Counterpart of fused_ttt_tile_forward_multi (rust/fused/src/linear_fused_tile/api.rs:52-83):
@@ -101,10 +134,13 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
     """
     B, H, seq, d = xq.shape
     io = xq.dtype
-    xq = _need(xq, (B, H, seq, d), io, "xq")
-    xk = _need(xk, (B, H, seq, d), io, "xk")
-    xv = _need(xv, (B, H, seq, d), io, "xv")
-    lr = _need(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta")
+    # sequence windows of dense tensors are processed in place (desc.seq_stride) when inputs and
+    # the caller's output window share one pitch; anything else is packed first
+    pitch = _common_pitch(seq, xq, xk, xv, ttt_lr_eta, out) if out is not None else 0
+    xq = _need_win(xq, (B, H, seq, d), io, "xq", pitch)
+    xk = _need_win(xk, (B, H, seq, d), io, "xk", pitch)
+    xv = _need_win(xv, (B, H, seq, d), io, "xv", pitch)
+    lr = _need_win(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta", pitch)
     per_batch = weight.dim() == 4
     weight = _need(weight, (B, H, d, d) if per_batch else (H, d, d), torch.float32, "weight")
     bias = _need(bias, (B, H, d) if per_batch else (H, d), torch.float32, "bias")
@@ -113,10 +149,14 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
     if token_eta.numel() < mini_batch:
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
     te = token_eta.to(torch.float32).contiguous()
-    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch))
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), pitch)
     check(lib().ttt_linear_supported(C.byref(desc)))
     dev = xq.device
-    out = torch.empty_like(xq)
+    if out is None or (pitch == 0 and not out.is_contiguous()):
+        dst, out = out, torch.empty((B, H, seq, d), dtype=io, device=dev)
+    else:
+        dst = None
+        out = _need_win(out, (B, H, seq, d), io, "out", pitch)
     w_out = torch.empty((B, H, d, d), dtype=torch.float32, device=dev)
     b_out = torch.empty((B, H, d), dtype=torch.float32, device=dev)
     w_ck = b_ck = None
@@ -129,6 +169,9 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
         check(lib().ttt_linear_fwd(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(weight), _ptr(bias),
                                    _ptr(te), _ptr(lr), _ptr(ln_weight), _ptr(ln_bias), _ptr(out),
                                    _ptr(w_out), _ptr(b_out), _ptr(w_ck), _ptr(b_ck), stream))
+    if dst is not None:
+        dst.copy_(out)
+        out = dst
     if want_checkpoints:
         return out, w_out, b_out, w_ck, b_ck
     return out, w_out, b_out
@@ -157,7 +200,7 @@ def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_
     ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
     ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
     te = token_eta.to(torch.float32).contiguous()
-    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch))
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), 0)
     check(lib().ttt_linear_supported(C.byref(desc)))
     n = lib().ttt_linear_num_checkpoints(C.byref(desc))
     w_ck = _need(weight_ckpt, (B, H, n, d, d), torch.float32, "weight_ckpt")
@@ -212,7 +255,7 @@ def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_we
     if token_eta.numel() < mini_batch:
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
     te = token_eta.to(torch.float32).contiguous()
-    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), int(per_batch))
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), int(per_batch), 0)
     check(lib().ttt_mlp_supported(C.byref(desc)))
     dev = xq.device
     f32 = dict(dtype=torch.float32, device=dev)
@@ -337,12 +380,12 @@ class FusedTileMulti:
         return TTTLinearState(self.weight_init.unsqueeze(0).repeat(batch_size, 1, 1, 1),
                               self.bias_init.unsqueeze(0).repeat(batch_size, 1, 1))
 
-    def _launch(self, state: TTTLinearState, inputs: TTTInputsInner, mini_batch: int):
+    def _launch(self, state: TTTLinearState, inputs: TTTInputsInner, mini_batch: int, out=None):
         t = self.config.ttt
         out, w, b = ttt_linear_forward_raw(
             inputs.qkv.xq, inputs.qkv.xk, inputs.qkv.xv, state.weight, state.bias, inputs.token_eta,
             inputs.ttt_lr_eta, self.ln_weight, self.ln_bias, mini_batch, t.epsilon,
-            t.checkpoint_interval)
+            t.checkpoint_interval, out=out)
         state.weight, state.bias = w, b
         return out
 
@@ -352,12 +395,13 @@ class FusedTileMulti:
         K = self.config.ttt.mini_batch_size
         seq = inputs.qkv.xq.shape[2]
         full = (seq // K) * K
-        outs = []
+        # one output tensor; both launches read and write sequence windows in place
+        output = torch.empty(inputs.qkv.xq.shape, dtype=inputs.qkv.xq.dtype, device=inputs.qkv.xq.device)
         if full > 0:
-            outs.append(self._launch(state, inputs.slice_seq(range(0, full)), K))
+            self._launch(state, inputs.slice_seq(range(0, full)), K, out=output[:, :, :full])
         if full < seq:
-            outs.append(self._launch(state, inputs.slice_seq(range(full, seq)), seq - full))
-        return outs[0] if len(outs) == 1 else torch.cat(outs, 2)
+            self._launch(state, inputs.slice_seq(range(full, seq)), seq - full, out=output[:, :, full:])
+        return output
 
     def forward_mini_batch(self, state: TTTLinearState, inputs: TTTInputsInner, r: range) -> torch.Tensor:
         """wrapper.rs:166-211: one mini-batch (len(r) <= mini_batch_size)."""
