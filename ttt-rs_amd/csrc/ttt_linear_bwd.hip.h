@@ -151,17 +151,59 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     for (int j = 0; j < NJ; ++j) Gv[j] = (gx[j] - s1 - xh[j] * s2) * rstd;
   };
 
+  // ---- register prefetch of everything a stage reads from HBM: the checkpoint (W, b) and the four
+  // activation tiles of the NEXT stage to be processed are fetched while the current one computes,
+  // and only copied into LDS at the top of that stage.  Thread tid owns EP contiguous elements of
+  // each [16 x D] tile and WP float4 pieces of the checkpoint.
+  constexpr int EP = D / 16;          // 16*D elements / 256 threads
+  constexpr int WP = D * D / 1024;    // D*D floats / (256 threads * 4)
+  const int pt = (tid * EP) / D, pc = (tid * EP) % D;  // token row / first feature of this thread's piece
+  struct Prefetch {
+    f32x4 w[WP];
+    float b, lr;
+    float q[EP], k[EP], v[EP], o[EP];
+  } pre;
+  auto fetch_tile = [&](float (&dst)[EP], const void* src, int stage) {
+    const elem* p = static_cast<const elem*>(src) + (bh * (size_t)a.seq_stride + (size_t)stage * K + pt) * D + pc;
+#pragma unroll
+    for (int e = 0; e < EP; ++e) dst[e] = (pt < K) ? IO::load1(p + e) : 0.f;
+  };
+  auto fetch_stage = [&](int stage) {
+    const int ckp = stage / a.ckpt_interval;
+    const f32x4* Wg = reinterpret_cast<const f32x4*>(a.W_ckpt + (bh * a.n_ckpt + ckp) * D * D);
+#pragma unroll
+    for (int i = 0; i < WP; ++i) pre.w[i] = Wg[tid + 256 * i];
+    pre.b = (tid < D) ? a.b_ckpt[(bh * a.n_ckpt + ckp) * D + tid] : 0.f;
+    pre.lr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
+    fetch_tile(pre.q, a.xq, stage);
+    fetch_tile(pre.k, a.xk, stage);
+    fetch_tile(pre.v, a.xv, stage);
+    fetch_tile(pre.o, a.d_out, stage);
+  };
+  auto commit_state = [&]() {
+#pragma unroll
+    for (int i = 0; i < WP; ++i) {
+      const int idx = (tid + 256 * i) * 4;
+      *reinterpret_cast<f32x4*>(sW + (idx / D) * LD + (idx % D)) = pre.w[i];
+    }
+    if (tid < D) sb[tid] = pre.b;
+  };
+  auto commit_tiles = [&]() {
+#pragma unroll
+    for (int e = 0; e < EP; ++e) {
+      lds[L::XQ + pt * LD + pc + e] = pre.q[e];
+      lds[L::XK + pt * LD + pc + e] = pre.k[e];
+      lds[L::TG + pt * LD + pc + e] = pre.v[e] - pre.k[e];
+      lds[L::DO + pt * LD + pc + e] = pre.o[e];
+    }
+    if (tid < 16) slr[tid] = pre.lr;
+  };
+  fetch_stage(a.n_stages - 1);
+
   for (int st = a.n_stages - 1; st >= 0; --st) {
     // ================= state entering stage st: checkpoint + re-simulated updates
     const int ck = st / a.ckpt_interval;
-    {
-      const float* Wg = a.W_ckpt + (bh * a.n_ckpt + ck) * D * D;
-      for (int i = tid; i < D * D; i += 256) {
-        const int r = i / D, cc = i - r * D;
-        sW[r * LD + cc] = Wg[i];
-      }
-      if (tid < D) sb[tid] = a.b_ckpt[(bh * a.n_ckpt + ck) * D + tid];
-    }
+    commit_state();
     for (int s2 = ck * a.ckpt_interval; s2 < st; ++s2) {
       __syncthreads();
       load_tile(lds + L::XK, a.xk, s2);
@@ -188,17 +230,12 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
         sb[tid] -= s;
       }
     }
-    __syncthreads();
+    if (ck * a.ckpt_interval < st) __syncthreads();  // the re-simulation used the XK / target tiles
 
-    // ================= load the stage's tiles
-    load_tile(lds + L::XQ, a.xq, st);
-    load_tile(lds + L::XK, a.xk, st);
-    load_tile(lds + L::TG, a.xv, st);
-    load_tile(lds + L::DO, a.d_out, st);
-    load_lr(st);
+    // ================= this stage's tiles (target = XV - XK formed on the way), then prefetch the next
+    commit_tiles();
     __syncthreads();
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) lds[L::TG + t * LD + cg + 16 * j] -= lds[L::XK + t * LD + cg + 16 * j];
+    if (st > 0) fetch_stage(st - 1);
     // Z1 = XK W ; Zq = XQ W ; A = XQ XK^T
     mm_lds<0>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane);
     mm_lds<0>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, NJ & 3);
