@@ -102,6 +102,23 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a
   __syncthreads();
   const float te_last = ste[K - 1];
 
+  // the next mini-batch's xq/xk/xv/lr are fetched into registers while this one computes
+  float pq[NJ], pk[NJ], pv[NJ], plr = 0.f;
+  auto fetch = [&](int stage) {
+    const size_t r = (bh * (size_t)a.seq_stride + (size_t)stage * K + t) * D;
+    const bool ok = t < K;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int o = cg + 16 * j;
+      pq[j] = ok ? IO::load1(static_cast<const elem*>(a.xq) + r + o) : 0.f;
+      pk[j] = ok ? IO::load1(static_cast<const elem*>(a.xk) + r + o) : 0.f;
+      pv[j] = ok ? IO::load1(static_cast<const elem*>(a.xv) + r + o) : 0.f;
+    }
+    if (tid < 16)
+      plr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
+  };
+  fetch(0);
+
   for (int st = 0; st < a.n_stages; ++st) {
     const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
     if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
@@ -112,15 +129,13 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int o = cg + 16 * j;
-      const bool ok = t < K;
-      const float k = ok ? IO::load1(static_cast<const elem*>(a.xk) + row * D + o) : 0.f;
-      lds[L::XQ + t * LD + o] = ok ? IO::load1(static_cast<const elem*>(a.xq) + row * D + o) : 0.f;
-      lds[L::XK + t * LD + o] = k;
-      lds[L::TG + t * LD + o] = (ok ? IO::load1(static_cast<const elem*>(a.xv) + row * D + o) : 0.f) - k;
+      lds[L::XQ + t * LD + o] = pq[j];
+      lds[L::XK + t * LD + o] = pk[j];
+      lds[L::TG + t * LD + o] = pv[j] - pk[j];
     }
-    if (tid < 16)
-      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid) : 0.f;
+    if (tid < 16) slr[tid] = plr;
     __syncthreads();
+    if (st + 1 < a.n_stages) fetch(st + 1);
     mm_lds<0>(lds + L::G, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NT, D, wave, lane);
     mm_lds<0>(lds + L::ZB, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NT, D, wave, lane, NT & 3);
     mm_lds<0>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, (2 * NT) & 3);
@@ -238,21 +253,36 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
   __syncthreads();
   const float te_last = ste[K - 1];
 
-  for (int st = 0; st < a.n_stages; ++st) {
-    const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
-    // ---- load XQ, XK, target = XV - XK
+  // the next mini-batch's xq/xk/xv/lr are fetched into registers while this one computes
+  float pq[NJD], pk[NJD], pv[NJD], plr = 0.f;
+  auto fetch = [&](int stage) {
+    const size_t r = (bh * (size_t)a.seq_stride + (size_t)stage * K + t) * D;
+    const bool ok = t < K;
 #pragma unroll
     for (int j = 0; j < NJD; ++j) {
       const int o = cg + GW * j;
-      const bool ok = t < K;
-      const float k = ok ? IO::load1(static_cast<const elem*>(a.xk) + row * D + o) : 0.f;
-      lds[L::XQ + t * LD + o] = ok ? IO::load1(static_cast<const elem*>(a.xq) + row * D + o) : 0.f;
-      lds[L::XK + t * LD + o] = k;
-      lds[L::TG + t * LD + o] = (ok ? IO::load1(static_cast<const elem*>(a.xv) + row * D + o) : 0.f) - k;
+      pq[j] = ok ? IO::load1(static_cast<const elem*>(a.xq) + r + o) : 0.f;
+      pk[j] = ok ? IO::load1(static_cast<const elem*>(a.xk) + r + o) : 0.f;
+      pv[j] = ok ? IO::load1(static_cast<const elem*>(a.xv) + r + o) : 0.f;
     }
     if (tid < 16)
-      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid) : 0.f;
+      plr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
+  };
+  fetch(0);
+
+  for (int st = 0; st < a.n_stages; ++st) {
+    const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
+    // ---- XQ, XK, target = XV - XK from the prefetch registers
+#pragma unroll
+    for (int j = 0; j < NJD; ++j) {
+      const int o = cg + GW * j;
+      lds[L::XQ + t * LD + o] = pq[j];
+      lds[L::XK + t * LD + o] = pk[j];
+      lds[L::TG + t * LD + o] = pv[j] - pk[j];
+    }
+    if (tid < 16) slr[tid] = plr;
     __syncthreads();
+    if (st + 1 < a.n_stages) fetch(st + 1);
     // ---- Z1 = XK W1 ; Zbar1 = XQ W1 ; A1 = XQ XK^T            (mlp.rs:139,160,167)
     mm_lds<0, NW, NBM>(lds + L::BA, LM, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
     mm_lds<0, NW, NBM>(lds + L::BC, LM, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
