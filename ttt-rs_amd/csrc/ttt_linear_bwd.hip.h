@@ -73,6 +73,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   using elem = typename IO::elem;
   using L = BwdLds<D>;
   constexpr int LD = L::LD, LK = L::LK, NJ = D / 16;
+  constexpr int NB2 = NJ >= 2 ? 2 : 1;  // tile columns per job of a [16 x D] product
   constexpr float inv_d = 1.0f / D;
   extern __shared__ float lds[];
 
@@ -237,9 +238,11 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     __syncthreads();
     if (st > 0) fetch_stage(st - 1);
     // Z1 = XK W ; Zq = XQ W ; A = XQ XK^T
-    mm_lds<0>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane);
-    mm_lds<0>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, NJ & 3);
-    mm_lds<0>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, (2 * NJ) & 3);
+    // every product is cut into jobs of NB2 tile columns: two or more accumulator chains per wave keep the
+    // matrix pipe busy (a single chain waits out the full MFMA latency between dependent steps)
+    mm_lds<0, 4, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, 0);
+    mm_lds<0, 4, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, 2);
+    mm_lds<0>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, 1);
     __syncthreads();
 
     // ================= forward intermediates: x_hat, rstd, G; eta, A (tril), M = eta (1 + A)
@@ -300,10 +303,10 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     __syncthreads();
 
     // ================= P = dZb G^T ; dQ = dZb W^T ; S = XK dW ; TMP = G dW^T
-    mm_lds<0>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, 1, 1, D, wave, lane, 0);
-    mm_lds<0>(lds + L::DQ, LD, lds + L::DZB, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 1);
-    mm_lds<0>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, LD, 1, 1, NJ, D, wave, lane, (1 + NJ) & 3);
-    mm_lds<0>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, LD, 1, NJ, D, wave, lane, (1 + 2 * NJ) & 3);
+    mm_lds<0, 4, NB2>(lds + L::DQ, LD, lds + L::DZB, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 0);
+    mm_lds<0, 4, NB2>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, LD, 1, NJ, D, wave, lane, 0);
+    mm_lds<0, 4, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, LD, 1, 1, NJ, D, wave, lane, 2);
+    mm_lds<0>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, 1, 1, D, wave, lane, 3);
     __syncthreads();
 
     // ================= dA, d eta ; S += db ; dlast
@@ -326,9 +329,9 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     __syncthreads();
 
     // ================= dQ += dA XK ; dK = dA^T XQ ; DGM = M^T dZb ; dW += XQ^T dZb ; db += colsum(dZb)
-    mm_lds<1, 4, 1, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NJ, 16, wave, lane, 0);
-    mm_lds<0, 4, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NJ, 16, wave, lane, NJ & 3);
-    mm_lds<0, 4, 1, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, 1, NJ, 16, wave, lane, (2 * NJ) & 3);
+    mm_lds<1, 4, NJ, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NJ, 16, wave, lane, 0);
+    mm_lds<0, 4, NJ, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NJ, 16, wave, lane, 1);
+    mm_lds<0, 4, NJ, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, 1, NJ, 16, wave, lane, 2);
     mm_lds<1, 4, NJ, 4>(sdW, LD, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, 16, wave, lane);
     if (tid < D) {
       float s = 0.f;
@@ -396,7 +399,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     __syncthreads();
 
     // ================= dK += dZ1 W^T ; dW += XK^T dZ1 ; db += colsum(dZ1)
-    mm_lds<1>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 0);
+    mm_lds<1, 4, NB2>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 2);
     mm_lds<1, 4, NJ, 4>(sdW, LD, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, 16, wave, lane);
     if (tid < D) {
       float s = 0.f;
