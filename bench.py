@@ -201,13 +201,16 @@ def main():
                            "algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)}
     elif kind == "mlp_fwd":
         flops = th * (56 * d * d + 20 * K * d)
-        out["dtype"] = "f32"   # bf16 I/O, f32 MFMA arithmetic
+        # bf16 I/O with d <= 96: register-resident kernel, bf16 MFMA operands with f32 accumulation and
+        # state; otherwise the LDS-tile kernel with f32 MFMA
+        rr = io == "bf16" and d <= 96 and os.environ.get("TTT_MLP_FWD_KERNEL") != "lds"
+        peak = BF16_MFMA_PEAK_TF if rr else F32_MFMA_PEAK_TF
+        out["dtype"] = "bf16" if rr else "f32"
         out["config"]["inner_model"] = "TTT-MLP"
-        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
-                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
-                           "frac_of_bf16_peak": flops / dev_s / 1e12 / BF16_MFMA_PEAK_TF,
-                           "kernel": "ttt_mlp_fwd_kernel", "kernel_avg_us": dev_s * 1e6,
-                           "algorithmic_flops": flops}
+        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": peak,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / peak, "traffic": None,
+                           "kernel": "ttt_mlp_fwd_rr_kernel" if rr else "ttt_mlp_fwd_kernel",
+                           "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     else:
         flops = th * (6 * (6 * d * d + 4 * K * d) + 2 * (56 * d * d + 20 * K * d))
         out["dtype"] = "f32"

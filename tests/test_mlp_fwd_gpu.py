@@ -41,9 +41,12 @@ def test_mlp_fwd_matches_oracle(P, B, H, d, K, N, style, dtype):
     n = np_inputs(c)
     ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
                           n["lr"], n["gamma"], n["beta"], K=K)
-    # arithmetic is f32 for both I/O dtypes; only the stored output is rounded for bf16
+    # bf16 I/O with d <= 96 runs the register-resident kernel, whose products take bf16 operands
+    # (f32 accumulation and state): everything is held to the bf16 bar.  The other cases compute in
+    # f32 throughout and only round the stored output.
+    f32_products = dtype == torch.float32 or d > 96
     for name, g, r in zip(("out", "W1", "b1", "W2", "b2"), got, ref):
-        assert_close(g, r, TOL[dtype] if name == "out" else 1e-4, name)
+        assert_close(g, r, 1e-4 if (f32_products and name != "out") else TOL[dtype], name)
 
 
 def test_mlp_inner_model_with_remainder(P):

@@ -14,6 +14,7 @@
 #include "ttt_linear_fwd.hip.h"
 #include "ttt_linear_fwd_mw.hip.h"
 #include "ttt_linear_fwd_sk.hip.h"
+#include "ttt_mlp_fwd_rr.hip.h"
 
 namespace {
 
@@ -127,6 +128,17 @@ int launch_mlp_fwd(const ttt::MlpFwdArgs& a, hipStream_t s) {
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_mlp_fwd launch");
+}
+
+// register-resident kernel (d <= 96, bf16 operands on the matrix cores)
+template <class T, int D>
+int launch_mlp_fwd_rr(const ttt::MlpFwdArgs& a, hipStream_t s) {
+  auto kern = ttt::ttt_mlp_fwd_rr_kernel<T, D>;
+  constexpr size_t bytes = ttt::MlpRrLds<D, sizeof(typename ttt::Io<T>::elem)>::BYTES;
+  int rc = opt_in_lds(kern, bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_mlp_fwd (register-resident kernel) launch");
 }
 
 template <class T, int D>
@@ -280,6 +292,16 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   a.eps = d->eps;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool f32 = d->io_dtype == TTT_F32;
+  // bf16 I/O, d <= 96: the state fits the register file of one CU.  TTT_MLP_FWD_KERNEL=lds forces
+  // the LDS-tile kernel (f32 products, state in global memory) that the other cases use.
+  const char* force = getenv("TTT_MLP_FWD_KERNEL");
+  if (!f32 && d->head_dim <= 96 && !(force && strcmp(force, "lds") == 0)) {
+    switch (d->head_dim) {
+      case 32: return launch_mlp_fwd_rr<ttt::BF16, 32>(a, s);
+      case 64: return launch_mlp_fwd_rr<ttt::BF16, 64>(a, s);
+      default: return launch_mlp_fwd_rr<ttt::BF16, 96>(a, s);
+    }
+  }
   switch (d->head_dim) {
     case 32: return f32 ? launch_mlp_fwd<ttt::F32, 32>(a, s) : launch_mlp_fwd<ttt::BF16, 32>(a, s);
     case 64: return f32 ? launch_mlp_fwd<ttt::F32, 64>(a, s) : launch_mlp_fwd<ttt::BF16, 64>(a, s);

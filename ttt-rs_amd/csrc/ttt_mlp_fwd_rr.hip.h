@@ -1,0 +1,503 @@
+// TTT-MLP multi-stage forward for gfx950 with the whole state resident in registers.
+//
+// Arithmetic: reference rust/core/src/mlp.rs:127-208 (one mini-batch) looped over the sequence as
+// rust/core/src/inner.rs:25-50; GELU constants rust/thundercube/src/unary_ops.rs:136-173.
+//
+// One workgroup of eight waves per (batch, head).  The hidden axis (4 d units) is cut into eight
+// slices; wave w keeps, as MFMA accumulator tiles in VGPRs for the whole sequence,
+//     W1[:, slice]  (d x 4d/8)   rows (d features) in registers, hidden units across lanes
+//     W2[slice, :]  (4d/8 x d)   hidden units in registers, d features across lanes
+//     b1[slice]
+// which is 2 * (d/16) * (d/32) tiles = 144 VGPRs at d = 96.  Everything that is elementwise in the
+// hidden axis (Z1, GELU, G1, Zbar1, Xbar2, both state updates) stays inside the wave.  The three
+// contractions OVER the hidden axis (Z2 = X2 W2, Zbar2 = Xbar2 W2, A2 = Xbar2 X2^T) are split-k:
+// every wave writes its partial tiles to LDS and wave I < d/16 (a "reducer") adds up d-feature
+// tile I, owns b2 / gamma / beta of those sixteen features and does the LayerNorm work on them.
+//
+// Per mini-batch there are three barriers on the recurrence W -> Z1 -> X2 -> Z2 -> G2 -> G1 -> W':
+//   B1  partial Z2 tiles (and last mini-batch's partial Zbar2 / A2) are in LDS
+//   B2  the reducers' row moments (six for the LN-L2 gradient of this mini-batch, two for the output
+//       LayerNorm of the previous one) are in LDS
+//   B3  G2 (as both operand orientations, already scaled by -eta_last) is in LDS
+// The output of mini-batch t needs nothing the recurrence waits for, so it is finished one
+// mini-batch late, inside the reducers' part of mini-batch t+1, and shares its barriers.
+//
+// An odd hidden tile at the end of a split-k chain is issued as a k = 32 MFMA with a zero second
+// half, not as a k = 16 one: a 16x16x16 bf16 MFMA accumulating straight onto the result of a
+// 16x16x32 one was measured to give wrong sums on gfx950 with this toolchain.
+//
+// Contractions over the d axis against W2 (G1 = G2 W2^T) need W2 tiles with d in the k position;
+// the accumulator layout has it across lanes, so those operand tiles are transposed on the matrix
+// pipe (one 16x16x16 MFMA against an identity fragment each).
+#pragma once
+#include "ttt_engine_fwd.hip.h"
+#include "ttt_linear_fwd_mw.hip.h"
+
+namespace ttt {
+
+template <int D, int ES>
+struct MlpRrLds {
+  static constexpr int NW = 8, NT = D / 16;
+  static constexpr int TILE = 16 * D * ES;    // one [16 x d] input tile, rows unpadded
+  static constexpr int IN1 = 3 * TILE;        // xq, xk, xv tiles of one mini-batch
+  static constexpr int IN = 0;                // [3 buffers][3][16][d]
+  static constexpr int LR = IN + 3 * IN1;     // [3][16] floats
+  static constexpr int P1 = LR + 3 * 64 + 64;  // [NW][NT][64] f32x4: partial Z2^T tiles
+  static constexpr int P2 = P1 + NW * NT * 1024;  // partial Zbar2^T tiles
+  static constexpr int PA = P2 + NW * NT * 1024;  // [NW][64] f32x4: partial A2^T
+  static constexpr int EX = PA + NW * 1024;       // [8 sums][2][16 tokens] f32x4 (reducer index % 4)
+  static constexpr int GT = EX + 8 * 2 * 16 * 16;  // [NT][64] frag: G2^T tiles (d along k)
+  static constexpr int GD = GT + NT * 64 * 4 * ES;  // [NT][64] frag: G2 tiles (tokens along k)
+  static constexpr int KD = GD + NT * 64 * 4 * ES;  // [2][NT][64] frag: XK tiles (tokens along k)
+  static constexpr int PRM = KD + 2 * NT * 64 * 4 * ES;  // gamma[d], beta[d], b1[4d] floats
+  static constexpr int BYTES = PRM + (2 * D + 4 * D) * 4;
+  static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
+  static_assert(NT <= NW && D % 32 == 0, "one reducer wave per d-feature tile");
+  static_assert(TILE % 1024 == 0 && P1 % 16 == 0, "input tiles are staged in 1 KiB wave blocks");
+};
+
+// y = gelu_tanh(x), dy = its derivative.  With r = 1 / (1 + exp(2u)), u = c (x + a x^3):
+// (1 + tanh u) / 2 = 1 - r and 1 - tanh^2 u = 4 r (1 - r).
+__device__ __forceinline__ void gelu_fast_pair(float x, float& y, float& dy) {
+  const float c2 = 2.f * 0.7978845608f;
+  const float x2 = x * x;
+  const float u = x * __builtin_fmaf(0.044715f, x2, 1.f);
+  const float e = __builtin_amdgcn_exp2f(u * (c2 * 1.4426950409f));
+  const float r = __builtin_amdgcn_rcpf(1.f + e);
+  const float hp = 1.f - r;
+  y = x * hp;
+  dy = hp * __builtin_fmaf(c2 * __builtin_fmaf(3.f * 0.044715f, x2, 1.f), x * r, 1.f);
+}
+__device__ __forceinline__ float gelu_fast(float x) {
+  const float u = x * __builtin_fmaf(0.044715f, x * x, 1.f);
+  const float e = __builtin_amdgcn_exp2f(u * (2.f * 0.7978845608f * 1.4426950409f));
+  return x - x * __builtin_amdgcn_rcpf(1.f + e);
+}
+
+// Makes the compiler forget what it knows about v.  The bf16 operand copies of the W2 tiles are
+// needed at three places of a mini-batch; without this the compiler keeps the converted copies
+// (36 VGPRs at d = 96) alive across the barriers and spills state tiles to scratch instead.
+__device__ __forceinline__ void forget(f32x4& v) { asm volatile("" : "+v"(v)); }
+// Orders memory accesses around the point where v is complete: keeps a reduction loop from issuing
+// all its LDS loads (four VGPRs each) before the first add.
+__device__ __forceinline__ void pin(f32x4& v) { asm volatile("" : "+v"(v)::"memory"); }
+__device__ __forceinline__ void pin(float& v) { asm volatile("" : "+v"(v)::"memory"); }
+
+template <class T, int D>
+__global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
+  using IO = Io<T>;
+  using frag = typename IO::frag;
+  using elem = typename IO::elem;
+  constexpr int ES = sizeof(elem);
+  using L = MlpRrLds<D, ES>;
+  constexpr int NW = 8, NT = D / 16, F = 4 * D, HT = F / 16 / NW;
+  constexpr float inv_d = 1.0f / D;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  // the wave index is read through an SGPR so that everything keyed on it is scalar control flow
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15, g = lane >> 4;
+  const size_t bh = blockIdx.x;
+  const int h = (int)(bh % a.H), K = a.K;
+  const bool red = w < NT;  // this wave reduces d-feature tile w
+
+  f32x4* const P1 = reinterpret_cast<f32x4*>(smem + L::P1);
+  f32x4* const P2 = reinterpret_cast<f32x4*>(smem + L::P2);
+  f32x4* const PA = reinterpret_cast<f32x4*>(smem + L::PA);
+  float* const EX = reinterpret_cast<float*>(smem + L::EX);
+  frag* const GT = reinterpret_cast<frag*>(smem + L::GT);
+  frag* const GD = reinterpret_cast<frag*>(smem + L::GD);
+  frag* const KD = reinterpret_cast<frag*>(smem + L::KD);
+  float* const LRs = reinterpret_cast<float*>(smem + L::LR);
+  float* const GAM = reinterpret_cast<float*>(smem + L::PRM);
+  float* const BET = GAM + D;
+  float* const B1s = BET + D;  // b1: each wave reads and updates only its own slice
+
+  // scale folding as in the TTT-Linear kernels: G'' = -sc lr G, M'' = (token_eta[t] / sc)(1 + A)
+  const float te_last = a.token_eta[K - 1];
+  const bool upd = te_last != 0.f;
+  const float sc = upd ? te_last : 1.f;
+  const float rho_c = (c < K) ? a.token_eta[c] / sc : 0.f;
+  const frag ident = identity_frag<T>(c, g);
+  const frag ones = splat_frag<T>(1.f);
+  const size_t sb = a.state_per_batch ? bh : (size_t)h;
+  const int own = own_offset<1>(red ? w : 0, 0, g);  // first of this lane's four features of tile w
+
+  // ---- state and parameters
+  f32x4 W1c[NT][HT], W2c[HT][NT];
+  {
+    const float* W1 = a.W1_0 + sb * (size_t)D * F;
+    const float* W2 = a.W2_0 + sb * (size_t)D * F;
+#pragma unroll
+    for (int j = 0; j < HT; ++j) {
+      const int hb = 16 * (w * HT + j);
+#pragma unroll
+      for (int I = 0; I < NT; ++I)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          W1c[I][j][r] = W1[(size_t)feat(I, 4 * g + r) * F + hb + c];
+          W2c[j][I][r] = W2[(size_t)(hb + 4 * g + r) * D + feat(I, c)];
+        }
+    }
+  }
+  f32x4 b2T;
+  float sum_a = 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) b2T[r] = a.b2_0[sb * D + own + r];
+  for (int f = 0; f < D; ++f) sum_a += a.gamma[h * D + f] * a.gamma[h * D + f];
+  for (int i = tid; i < D; i += 512) {
+    GAM[i] = a.gamma[h * D + i];
+    BET[i] = a.beta[h * D + i];
+  }
+  for (int i = tid; i < F; i += 512) B1s[i] = a.b1_0[sb * F + i];
+
+  // ---- staging of the xq / xk / xv rows of a mini-batch: global -> LDS without passing through
+  // registers, in wave blocks of 64 lanes x 16 bytes.  A block never straddles two tensors; lanes
+  // whose token is past a short mini-batch are masked off and their LDS rows keep the zeros
+  // written below.  Three buffers: mini-batch st+1 is fetched while st is computed, and rows of
+  // st are still read (for the W1 update) after the slowest wave has started st+1's fetch.
+  constexpr int NBLK = L::IN1 / 1024, NBI = (NBLK + NW - 1) / NW;
+  int goff[NBI];
+#pragma unroll
+  for (int it = 0; it < NBI; ++it) {
+    const int rem = (1024 * (w + NW * it) + 16 * lane) % L::TILE, tok = rem / (D * ES);
+    goff[it] = (tok < K) ? rem : -1;
+  }
+  auto fetch = [&](int stage) {
+    if (stage >= a.n_stages) return;
+    unsigned char* dst = smem + L::IN + (stage % 3) * L::IN1;
+    const size_t tok0 = (bh * (size_t)a.seq_stride + (size_t)stage * K) * D * ES;
+#pragma unroll
+    for (int it = 0; it < NBI; ++it) {
+      const int b = w + NW * it;  // wave-uniform
+      if (b < NBLK) {
+        const int ten = (1024 * b) / L::TILE;
+        const unsigned char* src =
+            static_cast<const unsigned char*>(ten == 0 ? a.xq : ten == 1 ? a.xk : a.xv) + tok0;
+        if (goff[it] >= 0)
+          __builtin_amdgcn_global_load_lds(
+              (const __attribute__((address_space(1))) void*)(src + goff[it]),
+              (__attribute__((address_space(3))) void*)(dst + 1024 * b), 16, 0, 0);
+      }
+    }
+    if (tid < 16 && tid < K)
+      LRs[(stage % 3) * 16 + tid] =
+          IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid);
+  };
+  // staged row of token c of tensor ten (0 xq, 1 xk, 2 xv)
+  auto row = [&](int buf, int ten) -> const elem* {
+    return reinterpret_cast<const elem*>(smem + L::IN + buf * L::IN1 + ten * L::TILE) + c * D;
+  };
+
+  for (int i = tid; i < (L::P1 - L::IN) / 4; i += 512) reinterpret_cast<float*>(smem)[i] = 0.f;
+  for (int i = tid; i < 8 * 2 * 16 * 4; i += 512) EX[i] = 0.f;
+  __syncthreads();
+  fetch(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  // pending output of the previous mini-batch (reducers)
+
+  // Zbar2^T tile of the previous mini-batch from the split-k partials
+  auto reduce_pending = [&]() -> f32x4 {
+    // few loads in flight at a time: the registers are needed for the state
+    f32x4 zq = {0.f, 0.f, 0.f, 0.f}, at = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) {
+      zq += P2[(ww * NT + w) * 64 + lane];
+      at += PA[ww * 64 + lane];
+      if (ww & 1) {
+        pin(zq);
+        pin(at);
+      }
+    }
+    f32x4 m;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + at[r]) : 0.f;
+    IO::mma(zq, GD[w * 64 + lane], IO::to_frag(m));  // still the previous mini-batch's G2 tile
+    return zq;
+  };
+  // lane group g publishes sums g and g + 4 of reducer w
+  auto publish = [&](const float (&S)[8]) {
+    const float v0 = xg_sum4_scatter(S[0], S[1], S[2], S[3]);
+    const float v1 = xg_sum4_scatter(S[4], S[5], S[6], S[7]);
+    EX[(((g)*2 + (w >> 2)) * 16 + c) * 4 + (w & 3)] = v0;
+    EX[(((g + 4) * 2 + (w >> 2)) * 16 + c) * 4 + (w & 3)] = v1;
+  };
+  auto collect = [&](int i) -> float {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(EX + ((i * 2 + 0) * 16 + c) * 4);
+    float s = (lo[0] + lo[1]) + (lo[2] + lo[3]);
+    if (NT > 4) {
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(EX + ((i * 2 + 1) * 16 + c) * 4);
+      s += (hi[0] + hi[1]) + (hi[2] + hi[3]);
+    }
+    return s;
+  };
+  auto emit_output = [&](f32x4 zbp, float s0, float s1, int stage) {
+    const float mu = s0 * inv_d;
+    const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
+    if (c < K) {
+      const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + own), bet = *reinterpret_cast<const f32x4*>(BET + own);
+      const frag qo = load4<T>(row(stage % 3, 0) + own);
+      elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D + own;
+      store4<T>(po, IO::to_f32(qo) + bet + gam * ((zbp - mu) * rstd));
+    }
+  };
+
+  for (int st = 0; st < a.n_stages; ++st) {
+    const int buf = st % 3, par = st & 1;
+    fetch(st + 1);
+
+    // ================= phase A: everything that needs only W1, W2 and the inputs
+    f32x4 z1[HT];
+    // XK tile w with tokens along k, for everybody's W1 update
+    if (red) {
+      f32x4 t = {0.f, 0.f, 0.f, 0.f};
+      IO::mma(t, load4<T>(row(buf, 1) + own), ident);
+      KD[(par * NT + w) * 64 + lane] = IO::to_frag(t);
+    }
+    // Z1^T for this wave's hidden units
+#pragma unroll
+    for (int j = 0; j < HT; ++j) z1[j] = *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g);
+#pragma unroll
+    for (int q = 0; q < NT / 2; ++q) {
+      frag k0, k1;
+      IO::load8(row(buf, 1) + 32 * q + 8 * g, true, k0, k1);
+#pragma unroll
+      for (int j = 0; j < HT; ++j)
+        IO::mma2(z1[j], IO::to_frag(W1c[2 * q][j]), IO::to_frag(W1c[2 * q + 1][j]), k0, k1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const float lrc = LRs[buf * 16 + c];
+    // X2 = gelu(Z1), gelu'(Z1)
+    frag x2f[HT];
+    f32x4 dg[HT];
+#pragma unroll
+    for (int j = 0; j < HT; ++j) {
+      f32x4 y, dy;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float yy, dd;
+        gelu_fast_pair(z1[j][r], yy, dd);
+        y[r] = yy;
+        dy[r] = dd;
+      }
+      x2f[j] = IO::to_frag(y);
+      dg[j] = dy;
+      // materialise both now: left to itself the compiler postpones gelu' to its use after the
+      // barriers and keeps (or spills) twice as many intermediates until then
+      asm volatile("" : "+v"(x2f[j]), "+v"(dg[j]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // partial Z2^T over this wave's hidden units
+#pragma unroll
+    for (int I = 0; I < NT; ++I) {
+      f32x4 p = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j + 1 < HT; j += 2)
+        IO::mma2(p, IO::to_frag(W2c[j][I]), IO::to_frag(W2c[j + 1][I]), x2f[j], x2f[j + 1]);
+      if (HT & 1) IO::mma2(p, IO::to_frag(W2c[HT - 1][I]), IO::zero(), x2f[HT - 1], IO::zero());
+      P1[(w * NT + I) * 64 + lane] = p;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    lds_barrier();  // ---- B1
+
+    // ================= phase B (reducers): full Z2 tile, pending Zbar2 tile, row moments
+    f32x4 z = {0.f, 0.f, 0.f, 0.f}, bq = z, zbp = z;
+    if (red) {
+      z = b2T;
+#pragma unroll
+      for (int ww = 0; ww < NW; ++ww) {
+        z += P1[(ww * NT + w) * 64 + lane];
+        if ((ww & 3) == 3) pin(z);
+      }
+      const frag ko = load4<T>(row(buf, 1) + own), vo = load4<T>(row(buf, 2) + own);
+      const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + own), bet = *reinterpret_cast<const f32x4*>(BET + own);
+      bq = gam * (bet - (IO::to_f32(vo) - IO::to_f32(ko)));
+      if (st > 0) zbp = reduce_pending();
+      float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      const f32x4 az = gam * gam * z;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        S[0] += z[r];
+        S[1] += z[r] * z[r];
+        S[2] += az[r];
+        S[3] += az[r] * z[r];
+        S[4] += bq[r];
+        S[5] += bq[r] * z[r];
+        S[6] += zbp[r];
+        S[7] += zbp[r] * zbp[r];
+      }
+      publish(S);
+    }
+    lds_barrier();  // ---- B2
+
+    // ================= phase C (reducers): previous output, G2'' in both orientations
+    if (red) {
+      float S[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        S[i] = collect(i);
+        if (i & 1) pin(S[i]);
+      }
+      if (st > 0) emit_output(zbp, S[6], S[7], st - 1);
+      const float mu = S[0] * inv_d;
+      const float var = S[1] * inv_d - mu * mu;
+      const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+      const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
+      const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
+      const float p = -sc * lrc * rstd;
+      const float c1 = p * rstd, c2 = -c1 * s2 * inv_d, c3 = -p * s1 * inv_d;
+      const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + own);
+      const f32x4 G = (z - mu) * (gam * gam * c1 + c2) + (bq * p + c3);
+      const frag gt = IO::to_frag(G);
+      f32x4 t = {0.f, 0.f, 0.f, 0.f};
+      IO::mma(t, gt, ident);
+      GT[w * 64 + lane] = gt;
+      GD[w * 64 + lane] = IO::to_frag(t);
+    }
+    // the next mini-batch's rows must have landed before anybody passes B3
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();  // ---- B3
+
+    // ================= phase D: G1, Zbar1, Xbar2, split-k partials of the output path, updates
+#pragma unroll
+    for (int j = 0; j < HT; ++j)
+#pragma unroll
+      for (int I = 0; I < NT; ++I) forget(W2c[j][I]);
+    frag G1d[HT];
+#pragma unroll
+    for (int j = 0; j < HT; ++j) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int q = 0; q < NT / 2; ++q) {
+        f32x4 t0 = {0.f, 0.f, 0.f, 0.f}, t1 = {0.f, 0.f, 0.f, 0.f};
+        IO::mma(t0, IO::to_frag(W2c[j][2 * q]), ident);
+        IO::mma(t1, IO::to_frag(W2c[j][2 * q + 1]), ident);
+        IO::mma2(acc, IO::to_frag(t0), IO::to_frag(t1), GT[(2 * q) * 64 + lane], GT[(2 * q + 1) * 64 + lane]);
+      }
+      f32x4 t = {0.f, 0.f, 0.f, 0.f};
+      IO::mma(t, IO::to_frag(acc * dg[j]), ident);
+      G1d[j] = IO::to_frag(t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // Zbar1^T = (XQ W1 + b1)^T + G1''^T M1, with M1[s][t] = (token_eta[t] / sc)(1 + A1[t][s]) for s <= t.
+    // Computed here rather than next to Z1 so that it does not occupy registers across the barriers.
+#pragma unroll
+    for (int j = 0; j < HT; ++j)
+#pragma unroll
+      for (int I = 0; I < NT; ++I) forget(W1c[I][j]);
+    f32x4 zq[HT], At = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < HT; ++j) zq[j] = *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g);
+#pragma unroll
+    for (int q = 0; q < NT / 2; ++q) {
+      frag k0, k1, q0, q1;
+      IO::load8(row(buf, 1) + 32 * q + 8 * g, true, k0, k1);
+      IO::load8(row(buf, 0) + 32 * q + 8 * g, true, q0, q1);
+#pragma unroll
+      for (int j = 0; j < HT; ++j)
+        IO::mma2(zq[j], IO::to_frag(W1c[2 * q][j]), IO::to_frag(W1c[2 * q + 1][j]), q0, q1);
+      IO::mma2(At, k0, k1, q0, q1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    {
+      f32x4 m;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + At[r]) : 0.f;
+      const frag Mf = IO::to_frag(m);
+#pragma unroll
+      for (int j = 0; j < HT; ++j) IO::mma(zq[j], G1d[j], Mf);
+    }
+    frag xbf[HT];
+#pragma unroll
+    for (int j = 0; j < HT; ++j) {
+      f32x4 y;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) y[r] = gelu_fast(zq[j][r]);
+      xbf[j] = IO::to_frag(y);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int j = 0; j < HT; ++j)
+#pragma unroll
+      for (int I = 0; I < NT; ++I) forget(W2c[j][I]);
+    {
+      f32x4 p = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j + 1 < HT; j += 2) IO::mma2(p, x2f[j], x2f[j + 1], xbf[j], xbf[j + 1]);
+      if (HT & 1) IO::mma2(p, x2f[HT - 1], IO::zero(), xbf[HT - 1], IO::zero());
+      PA[w * 64 + lane] = p;
+    }
+#pragma unroll
+    for (int I = 0; I < NT; ++I) {
+      f32x4 p = (I == w) ? b2T : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j + 1 < HT; j += 2)
+        IO::mma2(p, IO::to_frag(W2c[j][I]), IO::to_frag(W2c[j + 1][I]), xbf[j], xbf[j + 1]);
+      if (HT & 1) IO::mma2(p, IO::to_frag(W2c[HT - 1][I]), IO::zero(), xbf[HT - 1], IO::zero());
+      P2[(w * NT + I) * 64 + lane] = p;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (upd) {
+      frag x2d[HT];
+#pragma unroll
+      for (int j = 0; j < HT; ++j) {
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+        IO::mma(t, x2f[j], ident);
+        x2d[j] = IO::to_frag(t);
+        f32x4 b = *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g);
+        IO::mma(b, G1d[j], ones);
+        if (c == 0) *reinterpret_cast<f32x4*>(B1s + 16 * (w * HT + j) + 4 * g) = b;
+      }
+#pragma unroll
+      for (int I = 0; I < NT; ++I) {
+        const frag kd = KD[(par * NT + I) * 64 + lane], g2d = GD[I * 64 + lane];
+#pragma unroll
+        for (int j = 0; j < HT; ++j) {
+          IO::mma(W1c[I][j], kd, G1d[j]);
+          IO::mma(W2c[j][I], x2d[j], g2d);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (red) IO::mma(b2T, GD[w * 64 + lane], ones);
+    }
+  }
+
+  // ---- the last mini-batch's output
+  lds_barrier();
+  f32x4 zbp = {0.f, 0.f, 0.f, 0.f};
+  if (red) {
+    zbp = reduce_pending();
+    float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      S[6] += zbp[r];
+      S[7] += zbp[r] * zbp[r];
+    }
+    publish(S);
+  }
+  lds_barrier();
+  if (red) emit_output(zbp, collect(6), collect(7), a.n_stages - 1);
+
+  // ---- final state
+  {
+    float* W1 = a.W1 + bh * (size_t)D * F;
+    float* W2 = a.W2 + bh * (size_t)D * F;
+#pragma unroll
+    for (int j = 0; j < HT; ++j) {
+      const int hb = 16 * (w * HT + j);
+#pragma unroll
+      for (int I = 0; I < NT; ++I)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          W1[(size_t)feat(I, 4 * g + r) * F + hb + c] = W1c[I][j][r];
+          W2[(size_t)(hb + 4 * g + r) * D + feat(I, c)] = W2c[j][I][r];
+        }
+      if (c == 0) store4<F32>(a.b1 + bh * F + hb + 4 * g, *reinterpret_cast<const f32x4*>(B1s + hb + 4 * g));
+    }
+    if (red && c == 0) store4<F32>(a.b2 + bh * D + own, b2T);
+  }
+}
+
+}  // namespace ttt
