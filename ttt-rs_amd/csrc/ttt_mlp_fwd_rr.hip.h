@@ -50,7 +50,8 @@ struct MlpRrLds {
   static constexpr int GD = GT + NT * 64 * 4 * ES;  // [NT][64] frag: G2 tiles (tokens along k)
   static constexpr int KD = GD + NT * 64 * 4 * ES;  // [2][NT][64] frag: XK tiles (tokens along k)
   static constexpr int PRM = KD + 2 * NT * 64 * 4 * ES;  // gamma[d], beta[d], b1[4d] floats
-  static constexpr int BYTES = PRM + (2 * D + 4 * D) * 4;
+  static constexpr int EXO = PRM + (2 * D + 4 * D) * 4;    // [2 sums][2][16 tokens] f32x4 (output tile % 4)
+  static constexpr int BYTES = EXO + 2 * 2 * 16 * 16;
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
   static_assert(NT <= NW && D % 32 == 0, "one reducer wave per d-feature tile");
   static_assert(TILE % 1024 == 0 && P1 % 16 == 0, "input tiles are staged in 1 KiB wave blocks");
@@ -83,6 +84,12 @@ __device__ __forceinline__ void forget(f32x4& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void pin(f32x4& v) { asm volatile("" : "+v"(v)::"memory"); }
 __device__ __forceinline__ void pin(float& v) { asm volatile("" : "+v"(v)::"memory"); }
 
+// The LDS addresses derived from the lane index are many (the regions span 150 KiB, beyond the
+// 64 KiB reach of an instruction offset) and all loop-invariant: hoisted out of the loop they are
+// spilled and reloaded from scratch.  Hiding the lane index from the optimiser at the start of each
+// phase makes them cheap phase-local recomputations instead.
+#define RELANE() asm volatile("" : "+v"(lane))
+
 template <class T, int D>
 __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
   using IO = Io<T>;
@@ -95,7 +102,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   // the wave index is read through an SGPR so that everything keyed on it is scalar control flow
-  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int lane = tid & 63;  // refreshed (see RELANE) at every phase of the main loop
   const int c = lane & 15, g = lane >> 4;
   const size_t bh = blockIdx.x;
   const int h = (int)(bh % a.H), K = a.K;
@@ -105,6 +113,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
   f32x4* const P2 = reinterpret_cast<f32x4*>(smem + L::P2);
   f32x4* const PA = reinterpret_cast<f32x4*>(smem + L::PA);
   float* const EX = reinterpret_cast<float*>(smem + L::EX);
+  float* const EXO = reinterpret_cast<float*>(smem + L::EXO);
   frag* const GT = reinterpret_cast<frag*>(smem + L::GT);
   frag* const GD = reinterpret_cast<frag*>(smem + L::GD);
   frag* const KD = reinterpret_cast<frag*>(smem + L::KD);
@@ -191,6 +200,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
 
   for (int i = tid; i < (L::P1 - L::IN) / 4; i += 512) reinterpret_cast<float*>(smem)[i] = 0.f;
   for (int i = tid; i < 8 * 2 * 16 * 4; i += 512) EX[i] = 0.f;
+  if (tid < 2 * 2 * 16 * 4) EXO[tid] = 0.f;
   __syncthreads();
   fetch(0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -198,31 +208,12 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
 
   // pending output of the previous mini-batch (reducers)
 
-  // Zbar2^T tile of the previous mini-batch from the split-k partials
-  auto reduce_pending = [&]() -> f32x4 {
-    // few loads in flight at a time: the registers are needed for the state
-    f32x4 zq = {0.f, 0.f, 0.f, 0.f}, at = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ww = 0; ww < NW; ++ww) {
-      zq += P2[(ww * NT + w) * 64 + lane];
-      at += PA[ww * 64 + lane];
-      if (ww & 1) {
-        pin(zq);
-        pin(at);
-      }
-    }
-    f32x4 m;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + at[r]) : 0.f;
-    IO::mma(zq, GD[w * 64 + lane], IO::to_frag(m));  // still the previous mini-batch's G2 tile
-    return zq;
-  };
-  // lane group g publishes sums g and g + 4 of reducer w
-  auto publish = [&](const float (&S)[8]) {
+  // ---- reducers: lane group g publishes sums g and g + 4 (six in all) of reducer w
+  auto publish = [&](const float (&S)[6]) {
     const float v0 = xg_sum4_scatter(S[0], S[1], S[2], S[3]);
-    const float v1 = xg_sum4_scatter(S[4], S[5], S[6], S[7]);
+    const float v1 = xg_sum4_scatter(S[4], S[5], 0.f, 0.f);
     EX[(((g)*2 + (w >> 2)) * 16 + c) * 4 + (w & 3)] = v0;
-    EX[(((g + 4) * 2 + (w >> 2)) * 16 + c) * 4 + (w & 3)] = v1;
+    if (g < 2) EX[(((g + 4) * 2 + (w >> 2)) * 16 + c) * 4 + (w & 3)] = v1;
   };
   auto collect = [&](int i) -> float {
     const f32x4 lo = *reinterpret_cast<const f32x4*>(EX + ((i * 2 + 0) * 16 + c) * 4);
@@ -233,19 +224,65 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
     }
     return s;
   };
-  auto emit_output = [&](f32x4 zbp, float s0, float s1, int stage) {
-    const float mu = s0 * inv_d;
-    const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
+
+  // ---- output path: finishing the OUTPUT of the previous mini-batch is spread over the waves with
+  // the most slack: d-feature tile I goes to wave (NT + I) % NW, i.e. first to the waves that reduce
+  // no Z2 tile, then to reducers 0, 1, ...  Each wave has at most one output tile.
+  const int otile = (w - NT + NW) % NW;  // this wave's output tile
+  const bool outw = otile < NT;
+  const int ooff = own_offset<1>(outw ? otile : 0, 0, g);
+  f32x4 zb = {0.f, 0.f, 0.f, 0.f};
+  // part 1 (before B2): Zbar2^T tile from the split-k partials, causal correction, row moments
+  auto output_reduce = [&]() {
+    f32x4 at = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) at += PA[ww * 64 + lane];
+    pin(at);
+    f32x4 m;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + at[r]) : 0.f;
+    zb = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) zb += P2[(ww * NT + otile) * 64 + lane];
+    pin(zb);
+    IO::mma(zb, GD[otile * 64 + lane], IO::to_frag(m));  // GD still holds the previous mini-batch's G2
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      s0 += zb[r];
+      s1 += zb[r] * zb[r];
+    }
+    s0 = xg_sum(s0);
+    s1 = xg_sum(s1);
+    if (g == 0) {
+      EXO[((0 * 2 + (otile >> 2)) * 16 + c) * 4 + (otile & 3)] = s0;
+      EXO[((1 * 2 + (otile >> 2)) * 16 + c) * 4 + (otile & 3)] = s1;
+    }
+  };
+  auto collect_o = [&](int i) -> float {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(EXO + ((i * 2 + 0) * 16 + c) * 4);
+    float s = (lo[0] + lo[1]) + (lo[2] + lo[3]);
+    if (NT > 4) {
+      const f32x4 hi = *reinterpret_cast<const f32x4*>(EXO + ((i * 2 + 1) * 16 + c) * 4);
+      s += (hi[0] + hi[1]) + (hi[2] + hi[3]);
+    }
+    return s;
+  };
+  // part 2 (after B2): out = xq + gamma (zbar - mu) rstd + beta
+  auto output_emit = [&](int stage) {
+    const float mu = collect_o(0) * inv_d;
+    const float rstd = __builtin_amdgcn_rsqf(collect_o(1) * inv_d - mu * mu + a.eps);
     if (c < K) {
-      const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + own), bet = *reinterpret_cast<const f32x4*>(BET + own);
-      const frag qo = load4<T>(row(stage % 3, 0) + own);
-      elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D + own;
-      store4<T>(po, IO::to_f32(qo) + bet + gam * ((zbp - mu) * rstd));
+      const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + ooff), bet = *reinterpret_cast<const f32x4*>(BET + ooff);
+      const frag qo = load4<T>(row(stage % 3, 0) + ooff);
+      elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D + ooff;
+      store4<T>(po, IO::to_f32(qo) + bet + gam * ((zb - mu) * rstd));
     }
   };
 
   for (int st = 0; st < a.n_stages; ++st) {
     const int buf = st % 3, par = st & 1;
+    RELANE();
     fetch(st + 1);
 
     // ================= phase A: everything that needs only W1, W2 and the inputs
@@ -301,9 +338,11 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
     lds_barrier();  // ---- B1
+    RELANE();
 
-    // ================= phase B (reducers): full Z2 tile, pending Zbar2 tile, row moments
-    f32x4 z = {0.f, 0.f, 0.f, 0.f}, bq = z, zbp = z;
+    // ================= phase B: reducers: full Z2 tile and its row moments;
+    //                          output waves: Zbar2 tiles of the previous mini-batch and their moments
+    f32x4 z = {0.f, 0.f, 0.f, 0.f}, bq = z;
     if (red) {
       z = b2T;
 #pragma unroll
@@ -314,8 +353,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
       const frag ko = load4<T>(row(buf, 1) + own), vo = load4<T>(row(buf, 2) + own);
       const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + own), bet = *reinterpret_cast<const f32x4*>(BET + own);
       bq = gam * (bet - (IO::to_f32(vo) - IO::to_f32(ko)));
-      if (st > 0) zbp = reduce_pending();
-      float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      float S[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       const f32x4 az = gam * gam * z;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -325,22 +363,20 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
         S[3] += az[r] * z[r];
         S[4] += bq[r];
         S[5] += bq[r] * z[r];
-        S[6] += zbp[r];
-        S[7] += zbp[r] * zbp[r];
       }
       publish(S);
     }
+    if (outw && st > 0) output_reduce();
     lds_barrier();  // ---- B2
+    RELANE();
 
-    // ================= phase C (reducers): previous output, G2'' in both orientations
+    // ================= phase C: reducers: G2'' in both orientations; output waves: store the output
     if (red) {
-      float S[8];
+      float S[6];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < 6; ++i) {
         S[i] = collect(i);
-        if (i & 1) pin(S[i]);
       }
-      if (st > 0) emit_output(zbp, S[6], S[7], st - 1);
       const float mu = S[0] * inv_d;
       const float var = S[1] * inv_d - mu * mu;
       const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
@@ -356,9 +392,11 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
       GT[w * 64 + lane] = gt;
       GD[w * 64 + lane] = IO::to_frag(t);
     }
+    if (outw && st > 0) output_emit(st - 1);
     // the next mini-batch's rows must have landed before anybody passes B3
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();  // ---- B3
+    RELANE();
 
     // ================= phase D: G1, Zbar1, Xbar2, split-k partials of the output path, updates
 #pragma unroll
@@ -466,19 +504,9 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
 
   // ---- the last mini-batch's output
   lds_barrier();
-  f32x4 zbp = {0.f, 0.f, 0.f, 0.f};
-  if (red) {
-    zbp = reduce_pending();
-    float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      S[6] += zbp[r];
-      S[7] += zbp[r] * zbp[r];
-    }
-    publish(S);
-  }
+  if (outw) output_reduce();
   lds_barrier();
-  if (red) emit_output(zbp, collect(6), collect(7), a.n_stages - 1);
+  if (outw) output_emit(a.n_stages - 1);
 
   // ---- final state
   {
@@ -499,5 +527,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
     if (red && c == 0) store4<F32>(a.b2 + bh * D + own, b2T);
   }
 }
+
+#undef RELANE
 
 }  // namespace ttt
