@@ -82,6 +82,17 @@ def gelu_tanh_bwd(x):
     return 0.5 * (1.0 + t) + 0.5 * x * (1.0 - t * t) * GELU_C * (1.0 + 3.0 * GELU_A * x * x)
 
 
+def gelu_tanh_bwd2(x):
+    """Second derivative of the tanh-GELU (unary_ops.rs:175-195), needed by the TTT-MLP backward.
+    With u = c (x + a x^3), t = tanh u, u' = c (1 + 3 a x^2), u'' = 6 a c x:
+    gelu'' = (1 - t^2) u' + 0.5 x (1 - t^2) (u'' - 2 t u'^2)."""
+    t = np.tanh(GELU_C * (x + GELU_A * x ** 3))
+    du = GELU_C * (1.0 + 3.0 * GELU_A * x * x)
+    ddu = 6.0 * GELU_A * GELU_C * x
+    s = 1.0 - t * t
+    return s * du + 0.5 * x * s * (ddu - 2.0 * t * du * du)
+
+
 # --------------------------------------------------------------------------- helpers
 def _hb(p):
     """[H,d] parameter -> broadcastable [1,H,1,d]."""
@@ -316,3 +327,128 @@ def mlp_forward(W1_0, b1_0, W2_0, b2_0, xq, xk, xv, token_eta, lr, gamma, beta, 
                                 te, lr[:, :, s0:s1], gamma, beta, eps)
         out[:, :, s0:s1] = o
     return (out, *st)
+
+
+def _ln_l2_second_order(dG, xhat, std, gO, gx, G, gam, d):
+    """Backward of G = ln_l2_grad(z, T) given dG (layer_norm.rs:428-709): returns dz, dT and the
+    [B,H,K,d] summands of d_gamma, d_beta."""
+    u = -dG / std
+    s1 = u.sum(-1, keepdims=True)
+    s2 = (u * xhat).sum(-1, keepdims=True)
+    dgx = dG / std + s1 / d + xhat * s2 / d
+    dy = gam * dgx
+    dxhat = dy * gam + gx * s2 / d + u * (gx * xhat).sum(-1, keepdims=True) / d
+    dstd = (-(dxhat * xhat + dG * G) / std).sum(-1, keepdims=True)
+    dz = dxhat / std - dxhat.sum(-1, keepdims=True) / (d * std) + xhat * dstd / d
+    return dz, -dy, gO * dgx + dy * xhat, dy
+
+
+def mlp_backward(W1_0, b1_0, W2_0, b2_0, xq, xk, xv, token_eta, lr, gamma, beta, d_out, K=16,
+                 eps=1e-6, d_state_out=None, dtype=np.float64):
+    """Reverse scan of the TTT-MLP inner loop: the gradient of sum(out * d_out) (plus the inner
+    product of the final state with d_state_out = (dW1, db1, dW2, db2), if given) through
+    mlp_mini_batch (mlp.rs:127-208) looped as inner.rs:25-50.  The reference has no fused MLP
+    backward; it differentiates these ops with Burn autodiff, which this restates in closed form.
+
+    seq must be a multiple of K; token_eta is [K].  Returns a dict: d_xq,d_xk,d_xv [B,H,seq,d];
+    d_W1 [B,H,d,4d], d_b1 [B,H,4d], d_W2 [B,H,4d,d], d_b2 [B,H,d] (per batch: the parameter grads are
+    their batch sums); d_lr [B,H,seq]; d_token_eta [seq] (per position, summed over batch and
+    heads); d_gamma, d_beta [H,d] (summed over batch).
+    """
+    xq, xk, xv, lr, d_out = (np.asarray(a, dtype=dtype) for a in (xq, xk, xv, lr, d_out))
+    gamma, beta = np.asarray(gamma, dtype=dtype), np.asarray(beta, dtype=dtype)
+    te = np.asarray(token_eta, dtype=dtype)
+    B, H, seq, d = xq.shape
+    assert seq % K == 0 and te.shape[0] == K
+    N = seq // K
+    st = [np.asarray(a, dtype=dtype) for a in (W1_0, b1_0, W2_0, b2_0)]
+    if st[0].ndim == 3:
+        st = [np.broadcast_to(a[None], (B,) + a.shape).copy() for a in st]
+    states = []
+    for t in range(N):
+        states.append(st)
+        sl = slice(t * K, (t + 1) * K)
+        _, *st = mlp_mini_batch(*st, xq[:, :, sl], xk[:, :, sl], xv[:, :, sl], te, lr[:, :, sl],
+                                gamma, beta, eps)
+    if d_state_out is None:
+        dW1, db1, dW2, db2 = (np.zeros_like(a) for a in st)
+    else:
+        dW1, db1, dW2, db2 = (np.asarray(a, dtype).copy() for a in d_state_out)
+    g_xq, g_xk, g_xv = np.zeros_like(xq), np.zeros_like(xq), np.zeros_like(xq)
+    g_lr = np.zeros_like(lr)
+    g_te = np.zeros(seq, dtype)
+    g_gamma = np.zeros((H, d), dtype)
+    g_beta = np.zeros((H, d), dtype)
+    gam, bet = _hb(gamma), _hb(beta)
+    tri = np.tril(np.ones((K, K), dtype))
+    for t in range(N - 1, -1, -1):
+        sl = slice(t * K, (t + 1) * K)
+        Q, Kk, V, l = xq[:, :, sl], xk[:, :, sl], xv[:, :, sl], lr[:, :, sl]
+        W1, b1, W2, b2 = states[t]
+        dO = d_out[:, :, sl]
+        # ---- forward intermediates of this mini-batch (mlp.rs:139-183)
+        z1 = Kk @ W1 + b1[:, :, None, :]
+        x2, ph1 = gelu_tanh(z1), gelu_tanh_bwd(z1)
+        z2 = x2 @ W2 + b2[:, :, None, :]
+        xhat, std, gO, gx, G2 = _ln_l2_parts(z2, V - Kk, gam, bet, eps)
+        U = G2 @ _T(W2)
+        G1 = U * ph1
+        eta = _eta(te, l)
+        A1 = (Q @ _T(Kk)) * tri
+        z1b = Q @ W1 + b1[:, :, None, :] - (eta + eta * A1) @ G1
+        x2b, ph1b = gelu_tanh(z1b), gelu_tanh_bwd(z1b)
+        A2 = (x2b @ _T(x2)) * tri
+        z2b = x2b @ W2 + b2[:, :, None, :] - (eta + eta * A2) @ G2
+        mu2 = z2b.mean(-1, keepdims=True)
+        std2 = np.sqrt(((z2b - mu2) ** 2).mean(-1, keepdims=True) + eps)
+        xhat2 = (z2b - mu2) / std2
+        last = te[K - 1] * l
+        # ---- output LayerNorm
+        g_gamma += (dO * xhat2).sum((0, 2))
+        g_beta += dO.sum((0, 2))
+        gx2 = dO * gam
+        dz2b = (d * gx2 - gx2.sum(-1, keepdims=True)
+                - xhat2 * (gx2 * xhat2).sum(-1, keepdims=True)) / (d * std2)
+        # ---- second layer, dual-form terms
+        P2 = dz2b @ _T(G2)
+        dA2 = -(P2 * eta) * tri
+        deta = -(P2 * tri) * (1.0 + A2)
+        dx2b = dz2b @ _T(W2) + dA2 @ x2
+        dx2 = _T(dA2) @ x2b - last[..., None] * (G2 @ _T(dW2))
+        S2 = x2 @ dW2 + db2[:, :, None, :]
+        dG2 = -_T(eta + eta * A2) @ dz2b - last[..., None] * S2
+        dlast = -(G2 * S2).sum(-1)
+        # ---- first layer, dual-form terms
+        dz1b = dx2b * ph1b
+        P1 = dz1b @ _T(G1)
+        dA1 = -(P1 * eta) * tri
+        deta += -(P1 * tri) * (1.0 + A1)
+        dQ = dO + dz1b @ _T(W1) + dA1 @ Kk
+        dK = _T(dA1) @ Q - last[..., None] * (G1 @ _T(dW1))
+        S1 = Kk @ dW1 + db1[:, :, None, :]
+        dG1 = -_T(eta + eta * A1) @ dz1b - last[..., None] * S1
+        dlast += -(G1 * S1).sum(-1)
+        # ---- G1 = (G2 W2^T) * gelu'(z1)
+        dU = dG1 * ph1
+        dG2 = dG2 + dU @ W2
+        # ---- G2 = LN-L2 gradient of z2: second-order LayerNorm
+        dz2, dT, sg, sb = _ln_l2_second_order(dG2, xhat, std, gO, gx, G2, gam, d)
+        g_gamma += sg.sum((0, 2))
+        g_beta += sb.sum((0, 2))
+        dx2 = dx2 + dz2 @ _T(W2)
+        dz1 = dG1 * U * gelu_tanh_bwd2(z1) + dx2 * ph1
+        # ---- parameter and input gradients
+        dW2 = dW2 + _T(x2b) @ dz2b + _T(dU) @ G2 + _T(x2) @ dz2
+        db2 = db2 + dz2b.sum(2) + dz2.sum(2)
+        dW1 = dW1 + _T(Q) @ dz1b + _T(Kk) @ dz1
+        db1 = db1 + dz1b.sum(2) + dz1.sum(2)
+        g_xq[:, :, sl] = dQ
+        g_xv[:, :, sl] = dT
+        g_xk[:, :, sl] = dK - dT + dz1 @ _T(W1)
+        dl = (deta * te[None, None, :, None]).sum(2) + te[K - 1] * dlast
+        dte = (deta * l[:, :, None, :]).sum(-1)
+        dte[:, :, K - 1] += (dlast * l).sum(-1)
+        g_lr[:, :, sl] = dl
+        g_te[sl] = dte.sum((0, 1))
+    return dict(d_xq=g_xq, d_xk=g_xk, d_xv=g_xv, d_W1=dW1, d_b1=db1, d_W2=dW2, d_b2=db2,
+                d_lr=g_lr, d_token_eta=g_te, d_gamma=g_gamma, d_beta=g_beta)

@@ -283,3 +283,84 @@ def test_mlp_dual_form_equals_primal_gd(B, H, seq, d, K):
                           c["gamma"], c["beta"], K=K)
     for a, r in zip(got, ref):
         np.testing.assert_allclose(a, r.numpy(), rtol=1e-8, atol=1e-10)
+
+
+# ------------------------------------------------------------------ TTT-MLP backward
+def test_gelu_second_derivative_is_autograd():
+    x = torch.linspace(-4, 4, 101, dtype=torch.float64, requires_grad=True)
+    (dy,) = torch.autograd.grad(F.gelu(x, approximate="tanh").sum(), x, create_graph=True)
+    (ddy,) = torch.autograd.grad(dy.sum(), x)
+    np.testing.assert_allclose(orc.gelu_tanh_bwd2(x.detach().numpy()), ddy.numpy(), rtol=1e-9, atol=1e-12)
+
+
+def torch_mlp_dual(W1, b1, W2, b2, xq, xk, xv, te, lr, gamma, beta, K, eps=1e-6):
+    """The dual form of mlp.rs:127-208 in differentiable torch ops; the LN-L2 gradient is taken by
+    autograd (create_graph) rather than from the closed form, so this shares no formula with the
+    oracle's backward."""
+    B, H, seq, d = xq.shape
+    ln = lambda z: torch.stack([F.layer_norm(z[:, h], (d,), gamma[h], beta[h], eps=eps) for h in range(H)], 1)
+    outs = []
+    for s0 in range(0, seq, K):
+        q, k, v, l = (a[:, :, s0:s0 + K] for a in (xq, xk, xv, lr))
+        tri = torch.tril(torch.ones(K, K, dtype=xq.dtype))
+        z1 = k @ W1 + b1[:, :, None, :]
+        x2 = F.gelu(z1, approximate="tanh")
+        z2 = x2 @ W2 + b2[:, :, None, :]
+        # gradient of the reconstruction loss w.r.t. z2 and (through it) z1, as functions of the state
+        z2d = z2
+        loss = 0.5 * ((ln(z2d) - (v - k)) ** 2).sum()
+        (g2,) = torch.autograd.grad(loss, z2d, create_graph=True)
+        (dphi,) = torch.autograd.grad(x2.sum(), z1, create_graph=True)
+        g1 = (g2 @ W2.transpose(-1, -2)) * dphi
+        eta = (te[None, None, :, None] * l[:, :, None, :]) * tri
+        a1 = (q @ k.transpose(-1, -2)) * tri
+        z1b = q @ W1 + b1[:, :, None, :] - (eta + eta * a1) @ g1
+        x2b = F.gelu(z1b, approximate="tanh")
+        a2 = (x2b @ x2.transpose(-1, -2)) * tri
+        z2b = x2b @ W2 + b2[:, :, None, :] - (eta + eta * a2) @ g2
+        outs.append(q + ln(z2b))
+        last = eta[:, :, -1, :]
+        W1 = W1 - (last[..., None] * k).transpose(-1, -2) @ g1
+        b1 = b1 - (last[..., None] * g1).sum(2)
+        W2 = W2 - (last[..., None] * x2).transpose(-1, -2) @ g2
+        b2 = b2 - (last[..., None] * g2).sum(2)
+    return torch.cat(outs, 2), W1, b1, W2, b2
+
+
+@pytest.mark.parametrize("B,H,N,d,K,state_grads", [(2, 2, 3, 4, 4, False), (1, 2, 2, 8, 4, True)])
+def test_mlp_backward_equals_autograd_through_dual(B, H, N, d, K, state_grads):
+    seq, m = N * K, 4 * d
+    c = make_linear_case(60 + N, B, H, seq, d, K)
+    rng = np.random.default_rng(61 + N)
+    c.update(W1=rnd(rng, H, d, m, scale=0.3), b1=rnd(rng, H, m, scale=0.1),
+             W2=rnd(rng, H, m, d, scale=0.3), b2=rnd(rng, H, d, scale=0.1))
+    dO = rnd(rng, B, H, seq, d)
+    dst = [rnd(rng, B, H, d, m), rnd(rng, B, H, m), rnd(rng, B, H, m, d), rnd(rng, B, H, d)] if state_grads else None
+    t = {k: torch.tensor(v, requires_grad=True) for k, v in c.items()}
+    ex = lambda a: a[None].expand((B,) + tuple(a.shape))
+    # forward of the torch restatement agrees with the oracle's forward (itself pinned to primal GD)
+    out, *fin = torch_mlp_dual(ex(t["W1"]), ex(t["b1"]), ex(t["W2"]), ex(t["b2"]), t["xq"], t["xk"], t["xv"],
+                               t["te"], t["lr"], t["gamma"], t["beta"], K)
+    ref = orc.mlp_forward(c["W1"], c["b1"], c["W2"], c["b2"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                          c["gamma"], c["beta"], K=K)
+    for a, r in zip((out, *fin), ref):
+        np.testing.assert_allclose(a.detach().numpy(), r, rtol=1e-9, atol=1e-11)
+    loss = (out * torch.tensor(dO)).sum()
+    if state_grads:
+        loss = loss + sum((f * torch.tensor(g)).sum() for f, g in zip(fin, dst))
+    names = ["xq", "xk", "xv", "W1", "b1", "W2", "b2", "lr", "te", "gamma", "beta"]
+    grads = dict(zip(names, torch.autograd.grad(loss, [t[n] for n in names])))
+    got = orc.mlp_backward(c["W1"], c["b1"], c["W2"], c["b2"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                           c["gamma"], c["beta"], dO, K=K, d_state_out=dst)
+    tol = dict(rtol=1e-7, atol=1e-9)
+    for k in ("xq", "xk", "xv", "lr", "gamma", "beta"):
+        np.testing.assert_allclose(got["d_" + k], grads[k].numpy(), err_msg=k, **tol)
+    for k in ("W1", "b1", "W2", "b2"):  # per-batch state grads: the parameter grad is their batch sum
+        np.testing.assert_allclose(got["d_" + k].sum(0), grads[k].numpy(), err_msg=k, **tol)
+    np.testing.assert_allclose(got["d_token_eta"].reshape(N, K).sum(0), grads["te"].numpy(), **tol)
+    # linearity in the upstream gradient
+    got3 = orc.mlp_backward(c["W1"], c["b1"], c["W2"], c["b2"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"],
+                            c["gamma"], c["beta"], 3.0 * dO, K=K,
+                            d_state_out=None if dst is None else [3.0 * g for g in dst])
+    for k in got:
+        np.testing.assert_allclose(got3[k], 3.0 * got[k], rtol=1e-10, atol=1e-12)
