@@ -128,6 +128,38 @@ int ttt_mlp_fwd(const ttt_desc* desc, const void* xq, const void* xk, const void
                 void* out, float* W1_out, float* b1_out, float* W2_out, float* b2_out,
                 void* stream);
 
+/*
+ * TTT-MLP fused backward: gradients of sum(out * d_out) (plus the inner product of the final state
+ * with d_W1_out .. d_b2_out, if given) through the inner loop that ttt_mlp_fwd runs.  The
+ * reference has no fused MLP kernel: it differentiates TTTMLP::forward_mini_batch
+ * (rust/core/src/mlp.rs:127-208) with Burn autodiff, and this call replaces that autodiff path
+ * the way ttt_linear_bwd replaces fused_ttt_backward_kernel_multi (GELU second derivative:
+ * rust/thundercube/src/unary_ops.rs:175-195; second-order LayerNorm:
+ * rust/fused/src/linear_fused_tile/layer_norm.rs:428-709).
+ *
+ * Inputs are those of ttt_mlp_fwd (the call re-runs the forward sweep itself, so nothing has to be
+ * saved by the caller) plus d_out [B,H,seq,d] io and the optional upstream gradients of the final
+ * state (all four or none; NULL = zero): d_W1_out [B,H,d,4d], d_b1_out [B,H,4d],
+ * d_W2_out [B,H,4d,d], d_b2_out [B,H,d], f32.
+ * Outputs: d_xq,d_xk,d_xv [B,H,seq,d] io; d_W1 [B,H,d,4d], d_b1 [B,H,4d], d_W2 [B,H,4d,d],
+ * d_b2 [B,H,d] f32 per batch element (the parameter gradients are their batch sums);
+ * d_lr [B,H,seq] io; d_token_eta [seq] f32 per position (summed over batch and heads);
+ * d_gamma, d_beta [H,d] f32 (summed over batch).  The accumulated outputs are zeroed by the
+ * library on `stream`.
+ * workspace: ttt_mlp_bwd_workspace_bytes(desc) bytes of device memory, 16-byte aligned, owned by
+ * the caller and free to reuse after the call's work on `stream` has finished.  It holds the
+ * rolling state, the per-mini-batch update factors of the forward sweep and scratch tiles.
+ * seq must be a multiple of mini_batch.
+ */
+int64_t ttt_mlp_bwd_workspace_bytes(const ttt_desc* desc);
+int ttt_mlp_bwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                const void* d_out, const float* d_W1_out, const float* d_b1_out,
+                const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
+                float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
+                float* d_gamma, float* d_beta, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,69 @@
+"""GPU parity: ttt_mlp_bwd through the C ABI against the float64 oracle (itself pinned to torch
+autograd in test_oracle_pins.py)."""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import TOL, assert_close, np_inputs, to_dev
+from oracle import ttt_oracle as orc
+from test_mlp_fwd_gpu import mlp_case
+
+pytestmark = pytest.mark.gpu
+
+GRADS = ("d_xq", "d_xk", "d_xv", "d_W1", "d_b1", "d_W2", "d_b2", "d_lr", "d_token_eta", "d_gamma", "d_beta")
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+def run_case(P, B, H, d, K, N, dtype, style, state_grads=False, seed=0):
+    seq = N * K
+    c = mlp_case(P, 300 + d + K + seed, B, H, seq, d, K, dtype, style)
+    g = torch.Generator().manual_seed(77 + seed)
+    d_out = torch.randn(B, H, seq, d, generator=g).to(dtype)
+    dst = None
+    if state_grads:
+        m = 4 * d
+        dst = [torch.randn(*s, generator=g) * 0.1 for s in ((B, H, d, m), (B, H, m), (B, H, m, d), (B, H, d))]
+    dv = to_dev(c)
+    got = P.ttt_mlp_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
+                                 dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], d_out.to("cuda:0"), K,
+                                 d_state_out=None if dst is None else [x.to("cuda:0") for x in dst])
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ref = orc.mlp_backward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                           n["gamma"], n["beta"], d_out.double().numpy(), K=K,
+                           d_state_out=None if dst is None else [x.double().numpy() for x in dst])
+    return got, ref
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("B,H,d,K,N,style,state_grads", [
+    (2, 2, 32, 8, 3, "ref", False), (1, 2, 64, 16, 4, "ref", True), (1, 2, 96, 16, 3, "baseline", False),
+    (1, 1, 128, 16, 2, "ref", False), (1, 2, 32, 16, 1, "ref", True)])
+def test_mlp_bwd_matches_oracle(P, B, H, d, K, N, style, state_grads, dtype):
+    print(f"case mlp bwd {style} B{B} H{H} d{d} K{K} N{N} {dtype} state_grads={state_grads}", flush=True)
+    got, ref = run_case(P, B, H, d, K, N, dtype, style, state_grads)
+    # arithmetic is f32 for both I/O dtypes; bf16 rounds the stored activation gradients
+    for k in GRADS:
+        io_out = k in ("d_xq", "d_xk", "d_xv", "d_lr")
+        assert_close(got[k], ref[k], TOL[dtype] if io_out else 1e-4, k)
+
+
+def test_mlp_bwd_is_linear_in_upstream_gradient(P):
+    print("case mlp bwd linearity", flush=True)
+    B, H, d, K, N = 1, 2, 64, 16, 3
+    c = mlp_case(P, 411, B, H, N * K, d, K, torch.float32, "ref")
+    dv = to_dev(c)
+    g = torch.Generator().manual_seed(5)
+    dO = torch.randn(B, H, N * K, d, generator=g).to("cuda:0")
+    f = lambda x: P.ttt_mlp_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
+                                         dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], x, K)
+    g1, g2 = f(dO), f(2.0 * dO)
+    torch.cuda.synchronize()
+    for k in GRADS:
+        assert_close(g2[k], 2.0 * g1[k].double().cpu().numpy(), 1e-5, k)

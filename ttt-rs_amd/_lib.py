@@ -14,6 +14,7 @@ TTT_F32, TTT_BF16 = 0, 1
 EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
+    "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd",
 )
 
 
@@ -55,6 +56,9 @@ def lib() -> C.CDLL:
         L.ttt_linear_bwd.argtypes = [dp] + [vp] * 24
         L.ttt_mlp_supported.argtypes = [dp]
         L.ttt_mlp_fwd.argtypes = [dp] + [vp] * 17
+        L.ttt_mlp_bwd_workspace_bytes.argtypes = [dp]
+        L.ttt_mlp_bwd_workspace_bytes.restype = C.c_int64
+        L.ttt_mlp_bwd.argtypes = [dp] + [vp] * 29
         _lib = L
     return _lib
 

@@ -14,6 +14,7 @@
 #include "ttt_linear_fwd.hip.h"
 #include "ttt_linear_fwd_mw.hip.h"
 #include "ttt_linear_fwd_sk.hip.h"
+#include "ttt_mlp_bwd.hip.h"
 #include "ttt_mlp_fwd_rr.hip.h"
 
 namespace {
@@ -151,6 +152,41 @@ int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s)
   return hip_status(hipGetLastError(), "ttt_linear_bwd launch");
 }
 
+template <class T, int D>
+int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
+  auto kern = ttt::ttt_mlp_bwd_kernel<T, D>;
+  constexpr size_t bytes = ttt::MlpBwdLds<D>::BYTES;
+  int rc = opt_in_lds(kern, bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_mlp_bwd launch");
+}
+
+// dst = src, or zeros when src is null (a kernel, not a memcpy/memset node: capturable)
+__global__ void ttt_copy_or_zero_kernel(float* dst, const float* src, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src ? src[i] : 0.f;
+}
+void copy_or_zero(float* dst, const float* src, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(ttt_copy_or_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, dst, src, n);
+}
+
+// float offsets of the pieces of the ttt_mlp_bwd workspace
+struct MlpBwdWs {
+  size_t W1, W2, b1, b2, G1s, G2s, mt, total;
+  explicit MlpBwdWs(const ttt_desc* d) {
+    const size_t U = (size_t)d->batch * d->heads, D = d->head_dim, M = 4 * D, N = d->seq / d->mini_batch;
+    W1 = 0;
+    W2 = W1 + U * D * M;
+    b1 = W2 + U * M * D;
+    b2 = b1 + U * M;
+    G1s = b2 + U * D;
+    G2s = G1s + U * N * 16 * M;
+    mt = G2s + U * N * 16 * D;
+    total = mt + U * ttt::kMlpBwdMTiles * 16 * M;
+  }
+};
+
 }  // namespace
 
 extern "C" {
@@ -285,6 +321,7 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   a.xq = xq; a.xk = xk; a.xv = xv; a.W1_0 = W1_0; a.b1_0 = b1_0; a.W2_0 = W2_0; a.b2_0 = b2_0;
   a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
   a.W1 = W1_out; a.b1 = b1_out; a.W2 = W2_out; a.b2 = b2_out;
+  a.G1_save = nullptr; a.G2_save = nullptr;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
   a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.n_stages = d->seq / d->mini_batch;
@@ -307,6 +344,82 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
     case 64: return f32 ? launch_mlp_fwd<ttt::F32, 64>(a, s) : launch_mlp_fwd<ttt::BF16, 64>(a, s);
     case 96: return f32 ? launch_mlp_fwd<ttt::F32, 96>(a, s) : launch_mlp_fwd<ttt::BF16, 96>(a, s);
     default: return f32 ? launch_mlp_fwd<ttt::F32, 128>(a, s) : launch_mlp_fwd<ttt::BF16, 128>(a, s);
+  }
+}
+
+int64_t ttt_mlp_bwd_workspace_bytes(const ttt_desc* d) {
+  if (ttt_mlp_supported(d) != TTT_OK) return -1;
+  return (int64_t)(MlpBwdWs(d).total * sizeof(float));
+}
+
+int ttt_mlp_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                const void* d_out, const float* d_W1_out, const float* d_b1_out,
+                const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
+                float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
+                float* d_gamma, float* d_beta, void* workspace, void* stream) {
+  int rc = ttt_mlp_supported(d);
+  if (rc != TTT_OK) return rc;
+  if (!xq || !xk || !xv || !W1_0 || !b1_0 || !W2_0 || !b2_0 || !token_eta || !lr || !gamma || !beta ||
+      !d_out || !d_xq || !d_xk || !d_xv || !d_W1 || !d_b1 || !d_W2 || !d_b2 || !d_lr || !d_token_eta ||
+      !d_gamma || !d_beta || !workspace)
+    return fail(TTT_ERR_NULL, "ttt_mlp_bwd: a required pointer is NULL");
+  const bool up = d_W1_out || d_b1_out || d_W2_out || d_b2_out;
+  if (up && !(d_W1_out && d_b1_out && d_W2_out && d_b2_out))
+    return fail(TTT_ERR_NULL, "ttt_mlp_bwd: the four upstream state gradients must all be given or all be NULL");
+  if (!aligned16(workspace)) return fail(TTT_ERR_SHAPE, "ttt_mlp_bwd: workspace must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const MlpBwdWs w(d);
+  float* ws = static_cast<float*>(workspace);
+  const bool f32 = d->io_dtype == TTT_F32;
+  const size_t U = (size_t)d->batch * d->heads, D = d->head_dim, M = 4 * D;
+
+  // forward sweep with the LDS-tile kernel (f32 products): final state and, per mini-batch, the
+  // rank-16 factors of the state update
+  ttt::MlpFwdArgs fa;
+  fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
+  fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
+  fa.W1 = ws + w.W1; fa.b1 = ws + w.b1; fa.W2 = ws + w.W2; fa.b2 = ws + w.b2;
+  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s;
+  fa.B = d->batch; fa.H = d->heads; fa.seq = d->seq; fa.K = d->mini_batch;
+  fa.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
+  fa.n_stages = d->seq / d->mini_batch;
+  fa.state_per_batch = d->state_per_batch ? 1 : 0;
+  fa.eps = d->eps;
+  switch (d->head_dim) {
+    case 32: rc = f32 ? launch_mlp_fwd<ttt::F32, 32>(fa, s) : launch_mlp_fwd<ttt::BF16, 32>(fa, s); break;
+    case 64: rc = f32 ? launch_mlp_fwd<ttt::F32, 64>(fa, s) : launch_mlp_fwd<ttt::BF16, 64>(fa, s); break;
+    case 96: rc = f32 ? launch_mlp_fwd<ttt::F32, 96>(fa, s) : launch_mlp_fwd<ttt::BF16, 96>(fa, s); break;
+    default: rc = f32 ? launch_mlp_fwd<ttt::F32, 128>(fa, s) : launch_mlp_fwd<ttt::BF16, 128>(fa, s); break;
+  }
+  if (rc != TTT_OK) return rc;
+
+  // gradient accumulators start from the upstream state gradients (or zero); the reductions over
+  // batch / heads start from zero
+  copy_or_zero(d_W1, d_W1_out, U * D * M, s);
+  copy_or_zero(d_b1, d_b1_out, U * M, s);
+  copy_or_zero(d_W2, d_W2_out, U * M * D, s);
+  copy_or_zero(d_b2, d_b2_out, U * D, s);
+  copy_or_zero(d_token_eta, nullptr, (size_t)d->seq, s);
+  copy_or_zero(d_gamma, nullptr, (size_t)d->heads * D, s);
+  copy_or_zero(d_beta, nullptr, (size_t)d->heads * D, s);
+  rc = hip_status(hipGetLastError(), "ttt_mlp_bwd fills");
+  if (rc != TTT_OK) return rc;
+
+  ttt::MlpBwdArgs a;
+  a.xq = xq; a.xk = xk; a.xv = xv; a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta;
+  a.d_out = d_out; a.G1s = ws + w.G1s; a.G2s = ws + w.G2s; a.W1 = ws + w.W1; a.W2 = ws + w.W2;
+  a.b1f = ws + w.b1; a.b2f = ws + w.b2; a.mt = ws + w.mt;
+  a.d_xq = d_xq; a.d_xk = d_xk; a.d_xv = d_xv; a.d_W1 = d_W1; a.d_b1 = d_b1; a.d_W2 = d_W2; a.d_b2 = d_b2;
+  a.d_lr = d_lr; a.d_token_eta = d_token_eta; a.d_gamma = d_gamma; a.d_beta = d_beta;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.seq_stride = fa.seq_stride; a.n_stages = fa.n_stages; a.eps = d->eps;
+  switch (d->head_dim) {
+    case 32: return f32 ? launch_mlp_bwd<ttt::F32, 32>(a, s) : launch_mlp_bwd<ttt::BF16, 32>(a, s);
+    case 64: return f32 ? launch_mlp_bwd<ttt::F32, 64>(a, s) : launch_mlp_bwd<ttt::BF16, 64>(a, s);
+    case 96: return f32 ? launch_mlp_bwd<ttt::F32, 96>(a, s) : launch_mlp_bwd<ttt::BF16, 96>(a, s);
+    default: return f32 ? launch_mlp_bwd<ttt::F32, 128>(a, s) : launch_mlp_bwd<ttt::BF16, 128>(a, s);
   }
 }
 

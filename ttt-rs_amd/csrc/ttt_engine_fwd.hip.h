@@ -198,6 +198,10 @@ struct MlpFwdArgs {
   float* b1;
   float* W2;  // [B,H,M,D]
   float* b2;
+  // optional (LDS-tile kernel only): per mini-batch, the rank-16 factors of the state update,
+  // eta_last * G1 [B*H][N][16][M] and eta_last * G2 [B*H][N][16][D], for ttt_mlp_bwd; out may then be null
+  float* G1_save;
+  float* G2_save;
   int B, H, seq, seq_stride, K, n_stages, state_per_batch;
   float eps;
 };
@@ -363,13 +367,20 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
 #pragma unroll
       for (int j = 0; j < NJD; ++j) {
         const int o = cg + GW * j;
-        if (t < K)
+        if (t < K && a.out != nullptr)
           IO::store1(static_cast<elem*>(a.out) + row * D + o,
                      lds[L::XQ + t * LD + o] + (sgam[o] * xh[j] + sbet[o]));
         lds[L::Z2 + t * LD + o] *= last;
       }
 #pragma unroll
       for (int j = 0; j < NJM; ++j) lds[L::BA + t * LM + cg + GW * j] *= last;
+      if (a.G1_save != nullptr) {
+        const size_t srow = (bh * (size_t)a.n_stages + st) * 16 + t;
+#pragma unroll
+        for (int j = 0; j < NJD; ++j) a.G2_save[srow * D + cg + GW * j] = lds[L::Z2 + t * LD + cg + GW * j];
+#pragma unroll
+        for (int j = 0; j < NJM; ++j) a.G1_save[srow * M + cg + GW * j] = lds[L::BA + t * LM + cg + GW * j];
+      }
     }
     __syncthreads();
     // ---- W1 -= XK^T G1l ; W2 -= X2^T G2l ; b1 -= colsum(G1l) ; b2 -= colsum(G2l)

@@ -1,0 +1,495 @@
+// TTT-MLP fused backward for gfx950: one workgroup (8 wavefronts) per (batch, head).
+//
+// Arithmetic: the gradient of the TTT-MLP inner loop (reference rust/core/src/mlp.rs:127-208
+// looped as rust/core/src/inner.rs:25-50).  The reference has no fused MLP kernel and
+// differentiates these ops with Burn autodiff; this kernel applies the closed-form one-mini-batch
+// backward in a reverse scan, the way the reference's TTT-Linear backward does
+// (rust/fused/src/linear_fused_tile/backward/kernel.rs:253-429), including the second-order
+// LayerNorm term (layer_norm.rs:428-709) and the second derivative of the tanh-GELU
+// (rust/thundercube/src/unary_ops.rs:175-195).
+//
+// State without checkpoints.  The state (W1 [d,4d], W2 [4d,d], b1, b2) entering mini-batch t is
+// not stored by the forward.  The forward sweep saves, per mini-batch, the two rank-16 factors of
+// its state update, G1l = eta_last * G1 [16,4d] and G2l = eta_last * G2 [16,d] (30 KiB at d = 96
+// against 590 KiB for the state), and hands over the FINAL state; the reverse scan un-applies the
+// update of mini-batch t (W1 += XK^T G1l, W2 += X2^T G2l, ...) before it differentiates it.  The
+// roll-back is exact up to one f32 rounding per element and mini-batch.
+//
+// Data placement: [16 x d] tiles, the [16 x 16] causal matrices, biases and their gradients live
+// in LDS; the [16 x 4d] tiles, the rolling state and the gradient accumulators dW1, dW2 live in
+// global memory (caller's workspace / output buffers, an L2-resident working set) and are read
+// in place as MFMA operands.  All contractions are true-f32 MFMA for both I/O dtypes.
+#pragma once
+#include "ttt_engine_fwd.hip.h"
+
+namespace ttt {
+
+struct MlpBwdArgs {
+  const void* xq;
+  const void* xk;
+  const void* xv;
+  const float* token_eta;
+  const void* lr;
+  const float* gamma;
+  const float* beta;
+  const void* d_out;
+  const float* G1s;  // [B*H][N][16][4d]  eta_last * G1 per mini-batch (forward sweep)
+  const float* G2s;  // [B*H][N][16][d]
+  float* W1;         // [B*H][d][4d] final state on entry, initial state on exit
+  float* W2;         // [B*H][4d][d]
+  const float* b1f;  // [B*H][4d] final biases
+  const float* b2f;  // [B*H][d]
+  float* mt;         // [B*H][NMT][16][4d] scratch tiles
+  void* d_xq;
+  void* d_xk;
+  void* d_xv;
+  float* d_W1;  // [B*H][d][4d]; holds the upstream gradient (or zeros) on entry
+  float* d_b1;
+  float* d_W2;
+  float* d_b2;
+  void* d_lr;
+  float* d_token_eta;
+  float* d_gamma;
+  float* d_beta;
+  int B, H, seq, seq_stride, K, n_stages;
+  float eps;
+};
+
+constexpr int kMlpBwdMTiles = 9;  // [16 x 4d] scratch tiles per (batch, head)
+
+template <int D>
+struct MlpBwdLds {
+  static constexpr int M = 4 * D, LD = D + 4, LK = 17, KK = 16 * LK, TD = 16 * LD;
+  static constexpr int XQ = 0, XK = XQ + TD, TG = XK + TD, DO = TG + TD, XH = DO + TD, G2 = XH + TD,
+                       XH2 = G2 + TD, DZB2 = XH2 + TD, DG2 = DZB2 + TD, DZ2 = DG2 + TD, DT = DZ2 + TD,
+                       DQ = DT + TD, DK = DQ + TD;
+  static constexpr int ETA = DK + TD, A1 = ETA + KK, M1 = A1 + KK, M2 = M1 + KK, P = M2 + KK,
+                       DA = P + KK, DETA = DA + KK, PART = DETA + KK;
+  static constexpr int b1 = PART + 8 * 256, b2 = b1 + M, db1 = b2 + D, db2 = db1 + M, gam = db2 + D,
+                       bet = gam + D, lr = bet + D, te = lr + 16, rstd1 = te + 16, dlast = rstd1 + 16,
+                       END = dlast + 16;
+  static constexpr size_t BYTES = sizeof(float) * END;
+  static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
+};
+
+// tanh-GELU with first and second derivative
+__device__ __forceinline__ void gelu_tanh_all(float x, float& y, float& dy, float& ddy) {
+  const float c = 0.7978845608f, a = 0.044715f;
+  const float t = tanhf(c * (x + a * x * x * x));
+  const float du = c * (1.f + 3.f * a * x * x), ddu = 6.f * a * c * x, s = 1.f - t * t;
+  y = 0.5f * x * (1.f + t);
+  dy = 0.5f * (1.f + t) + 0.5f * x * s * du;
+  ddy = s * du + 0.5f * x * s * (ddu - 2.f * t * du * du);
+}
+
+template <class T, int D>
+__global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
+  using IO = Io<T>;
+  using elem = typename IO::elem;
+  using L = MlpBwdLds<D>;
+  constexpr int M = L::M, LD = L::LD, LK = L::LK;
+  constexpr int NW = 8, GW = 32, NJD = D / GW, NJM = M / GW, NTD = D / 16, NTM = M / 16;
+  constexpr int NBM = NTM / NW;  // [16 x 4d] products: one job of NBM tile columns per wave
+  constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
+  constexpr float inv_d = 1.0f / D;
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int t = tid >> 5, cg = tid & 31;  // elementwise mapping: token t, columns cg + 32 j
+  const size_t bh = blockIdx.x;
+  const int h = (int)(bh % a.H), K = a.K, N = a.n_stages;
+  float *sb1 = lds + L::b1, *sb2 = lds + L::b2, *sdb1 = lds + L::db1, *sdb2 = lds + L::db2,
+        *sgam = lds + L::gam, *sbet = lds + L::bet, *slr = lds + L::lr, *ste = lds + L::te;
+  float* W1 = a.W1 + bh * (size_t)D * M;
+  float* W2 = a.W2 + bh * (size_t)M * D;
+  float* dW1 = a.d_W1 + bh * (size_t)D * M;
+  float* dW2 = a.d_W2 + bh * (size_t)M * D;
+  // [16 x 4d] scratch tiles
+  float* mt = a.mt + bh * (size_t)kMlpBwdMTiles * 16 * M;
+  float *mZ1 = mt, *mX2 = mt + 16 * M, *mU = mt + 2 * 16 * M, *mG1 = mt + 3 * 16 * M, *mZB1 = mt + 4 * 16 * M,
+        *mXB2 = mt + 5 * 16 * M, *mDXB = mt + 6 * 16 * M, *mDX2 = mt + 7 * 16 * M, *mS1 = mt + 8 * 16 * M;
+
+  for (int i = tid; i < M; i += 512) {
+    sb1[i] = a.b1f[bh * M + i];
+    sdb1[i] = a.d_b1[bh * M + i];
+  }
+  for (int i = tid; i < D; i += 512) {
+    sb2[i] = a.b2f[bh * D + i];
+    sdb2[i] = a.d_b2[bh * D + i];
+    sgam[i] = a.gamma[h * D + i];
+    sbet[i] = a.beta[h * D + i];
+  }
+  if (tid < 16) ste[tid] = (tid < K) ? a.token_eta[tid] : 0.f;
+  float dgam_acc[NJD], dbet_acc[NJD];
+#pragma unroll
+  for (int j = 0; j < NJD; ++j) dgam_acc[j] = dbet_acc[j] = 0.f;
+  __syncthreads();
+  const float te_last = ste[K - 1];
+
+  auto load_tile = [&](float* dst, const void* src, int stage) {
+    const elem* p = static_cast<const elem*>(src) + (bh * (size_t)a.seq_stride + (size_t)stage * K + t) * D;
+#pragma unroll
+    for (int j = 0; j < NJD; ++j) dst[t * LD + cg + GW * j] = (t < K) ? IO::load1(p + cg + GW * j) : 0.f;
+  };
+  // C[16 x 16] (PART slices) = X Y^T over the 4d columns of two [16 x 4d] tiles, one k-slice per wave
+  auto splitk_xyT = [&](const float* X, const float* Y) {
+    const int c = lane & 15, g = lane >> 4;
+    constexpr int KS = M / NW;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const float* Ap = X + c * M + wave * KS + g;
+    const float* Bp = Y + c * M + wave * KS + g;
+#pragma unroll 4
+    for (int k = 0; k < KS; k += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ap[k], Bp[k], acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) lds[L::PART + wave * 256 + (4 * g + r) * 16 + c] = acc[r];
+  };
+  auto part_sum = [&](int tt, int s) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) v += lds[L::PART + w * 256 + tt * 16 + s];
+    return v;
+  };
+
+  for (int st = N - 1; st >= 0; --st) {
+    const float* G1l = a.G1s + ((bh * N + st) * (size_t)16) * M;
+    const float* G2l = a.G2s + ((bh * N + st) * (size_t)16) * D;
+    const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
+
+    // ---- 1. inputs of this mini-batch
+    load_tile(lds + L::XQ, a.xq, st);
+    load_tile(lds + L::XK, a.xk, st);
+    load_tile(lds + L::TG, a.xv, st);
+    load_tile(lds + L::DO, a.d_out, st);
+    if (tid < 16)
+      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid) : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NJD; ++j) lds[L::TG + t * LD + cg + GW * j] -= lds[L::XK + t * LD + cg + GW * j];
+    const float last = te_last * slr[t];
+    // ---- 2. roll W1, b1 back to the state entering this mini-batch
+    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, 16, wave, lane);
+    if (tid < M) {
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += G1l[r * M + tid];
+      sb1[tid] += s;
+    }
+    __syncthreads();
+    // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
+    mm_lds<0, NW, NBM>(mZ1, M, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) {
+      const int o = cg + GW * j;
+      float y, dy;
+      const float z = mZ1[t * M + o] + sb1[o];
+      gelu_tanh_pair(z, y, dy);
+      mZ1[t * M + o] = z;
+      mX2[t * M + o] = y;
+    }
+    __syncthreads();
+    // ---- 4. roll W2, b2 back
+    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, 16, wave, lane);
+    if (tid < D) {
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += G2l[r * D + tid];
+      sb2[tid] += s;
+    }
+    __syncthreads();
+    // ---- 5. Z2 = X2 W2 ; A1 = XQ XK^T ; eta
+    mm_lds<0, NW>(lds + L::XH, LD, mX2, M, 1, W2, D, 1, 1, NTD, M, wave, lane);
+    mm_lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, NTD % NW);
+    if (tid < 256) {
+      const int tt = tid >> 4, s = tid & 15;
+      lds[L::ETA + tt * LK + s] = (s <= tt) ? ste[tt] * slr[s] : 0.f;
+    }
+    __syncthreads();
+    // ---- 6. LayerNorm of Z2 + b2: x_hat, rstd, G2 ; M1 = eta (1 + A1)
+    float rstd1;
+    {
+      float xh[NJD], gx[NJD], s1 = 0.f, s2 = 0.f;
+      ln_stats<D, GW>(lds + L::XH + t * LD, sb2, cg, a.eps, xh, rstd1);
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        gx[j] = (sgam[o] * xh[j] + sbet[o] - lds[L::TG + t * LD + o]) * sgam[o];
+        s1 += gx[j];
+        s2 += gx[j] * xh[j];
+      }
+      s1 = rowgroup_sum<GW>(s1) * inv_d;
+      s2 = rowgroup_sum<GW>(s2) * inv_d;
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        lds[L::XH + t * LD + o] = xh[j];
+        lds[L::G2 + t * LD + o] = (gx[j] - s1 - xh[j] * s2) * rstd1;
+      }
+    }
+    if (tid < 256) {
+      const int tt = tid >> 4, s = tid & 15;
+      lds[L::M1 + tt * LK + s] = lds[L::ETA + tt * LK + s] * (1.f + lds[L::A1 + tt * LK + s]);
+    }
+    __syncthreads();
+    // ---- 7. U = G2 W2^T ; Zbar1 = XQ W1
+    mm_lds<0, NW, NBM>(mU, M, lds + L::G2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
+    __syncthreads();
+    // ---- 8. G1 = U gelu'(Z1)
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) {
+      const int o = cg + GW * j;
+      float y, dy;
+      gelu_tanh_pair(mZ1[t * M + o], y, dy);
+      mG1[t * M + o] = mU[t * M + o] * dy;
+    }
+    __syncthreads();
+    // ---- 9. Zbar1 -= M1 G1 ; then + b1, Xbar2 = gelu
+    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(mZB1, M, lds + L::M1, LK, 1, mG1, M, 1, 1, NTM, 16, wave, lane);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) {
+      const int o = cg + GW * j;
+      float y, dy;
+      const float z = mZB1[t * M + o] + sb1[o];
+      gelu_tanh_pair(z, y, dy);
+      mZB1[t * M + o] = z;
+      mXB2[t * M + o] = y;
+    }
+    __syncthreads();
+    // ---- 10. A2 = Xbar2 X2^T (split-k) ; Zbar2 = Xbar2 W2
+    splitk_xyT(mXB2, mX2);
+    mm_lds<0, NW>(lds + L::XH2, LD, mXB2, M, 1, W2, D, 1, 1, NTD, M, wave, lane);
+    __syncthreads();
+    if (tid < 256) {
+      const int tt = tid >> 4, s = tid & 15;
+      lds[L::M2 + tt * LK + s] = lds[L::ETA + tt * LK + s] * (1.f + part_sum(tt, s));
+    }
+    __syncthreads();
+    mm_lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M2, LK, 1, lds + L::G2, LD, 1, 1, NTD, 16, wave, lane);
+    __syncthreads();
+    // ---- 11. output LayerNorm backward: dZbar2
+    {
+      float xh[NJD], rstd2, gx2[NJD], s1 = 0.f, s2 = 0.f;
+      ln_stats<D, GW>(lds + L::XH2 + t * LD, sb2, cg, a.eps, xh, rstd2);
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        const float dO = lds[L::DO + t * LD + o];
+        dgam_acc[j] += dO * xh[j];
+        dbet_acc[j] += dO;
+        gx2[j] = dO * sgam[o];
+        s1 += gx2[j];
+        s2 += gx2[j] * xh[j];
+      }
+      s1 = rowgroup_sum<GW>(s1) * inv_d;
+      s2 = rowgroup_sum<GW>(s2) * inv_d;
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) lds[L::DZB2 + t * LD + cg + GW * j] = (gx2[j] - s1 - xh[j] * s2) * rstd2;
+    }
+    __syncthreads();
+    // ---- 12. P2 = dZbar2 G2^T ; dXbar2 = dZbar2 W2^T ; S2 = X2 dW2
+    mm_lds<0, NW>(lds + L::P, LK, lds + L::DZB2, LD, 1, lds + L::G2, 1, LD, 1, 1, D, wave, lane, NW - 1);
+    mm_lds<0, NW, NBM>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<0, NW>(lds + L::DG2, LD, mX2, M, 1, dW2, D, 1, 1, NTD, M, wave, lane);
+    __syncthreads();
+    // ---- 13. dA2, d eta ; dG2 = -last (S2 + db2) ; d last
+    if (tid < 256) {
+      const int tt = tid >> 4, s = tid & 15;
+      const float p = (s <= tt) ? lds[L::P + tt * LK + s] : 0.f;
+      const float et = lds[L::ETA + tt * LK + s];
+      lds[L::DA + tt * LK + s] = -p * et;
+      // 1 + A2 = M2 / eta is not safe for eta = 0: recompute from the split-k sums still in PART
+      lds[L::DETA + tt * LK + s] = -p * (1.f + part_sum(tt, s));
+    }
+    {
+      float q = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        const float s2v = lds[L::DG2 + t * LD + o] + sdb2[o];
+        q += lds[L::G2 + t * LD + o] * s2v;
+        lds[L::DG2 + t * LD + o] = -last * s2v;
+      }
+      q = rowgroup_sum<GW>(q);
+      if (cg == 0) lds[L::dlast + t] = -q;
+    }
+    __syncthreads();
+    // ---- 14. dXbar2 += dA2 X2 ; dG2 -= M2^T dZbar2 ; dX2 = dA2^T Xbar2
+    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(mDXB, M, lds + L::DA, LK, 1, mX2, M, 1, 1, NTM, 16, wave, lane);
+    mm_lds<2, NW, 1, 4>(lds + L::DG2, LD, lds + L::M2, 1, LK, lds + L::DZB2, LD, 1, 1, NTD, 16, wave, lane);
+    mm_lds<0, NW, NBM, (NBM >= 3 ? 1 : 2)>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
+    __syncthreads();
+    // ---- 15. dX2 -= (last G2) dW2^T ; dZbar1 = dXbar2 gelu'(Zbar1)
+    mm_lds<2, NW, NBM>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) {
+      const int o = cg + GW * j;
+      float y, dy;
+      gelu_tanh_pair(mZB1[t * M + o], y, dy);
+      mDXB[t * M + o] *= dy;
+    }
+    __syncthreads();
+    // ---- 16. P1 = dZbar1 G1^T (split-k) ; dQ = dZbar1 W1^T ; S1 = XK dW1
+    splitk_xyT(mDXB, mG1);
+    mm_lds<0, NW>(lds + L::DQ, LD, mDXB, M, 1, W1, 1, M, 1, NTD, M, wave, lane);
+    mm_lds<0, NW, NBM>(mS1, M, lds + L::XK, LD, 1, dW1, M, 1, 1, NTM, D, wave, lane);
+    __syncthreads();
+    // ---- 17. dA1, d eta ; dG1 = -last (S1 + db1) ; d last
+    if (tid < 256) {
+      const int tt = tid >> 4, s = tid & 15;
+      const float p = (s <= tt) ? part_sum(tt, s) : 0.f;
+      lds[L::DA + tt * LK + s] = -p * lds[L::ETA + tt * LK + s];
+      lds[L::DETA + tt * LK + s] += -p * (1.f + lds[L::A1 + tt * LK + s]);
+    }
+    {
+      float q = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJM; ++j) {
+        const int o = cg + GW * j;
+        const float s1v = mS1[t * M + o] + sdb1[o];
+        q += mG1[t * M + o] * s1v;
+        mS1[t * M + o] = -last * s1v;
+      }
+      q = rowgroup_sum<GW>(q);
+      if (cg == 0) lds[L::dlast + t] -= q;
+    }
+    __syncthreads();
+    // ---- 18. dG1 -= M1^T dZbar1 ; dQ += dA1 XK ; dK = dA1^T XQ
+    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(mS1, M, lds + L::M1, 1, LK, mDXB, M, 1, 1, NTM, 16, wave, lane);
+    mm_lds<1, NW, 1, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NTD, 16, wave, lane);
+    mm_lds<0, NW, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NTD, 16, wave, lane, NTD % NW);
+    __syncthreads();
+    // ---- 19. dK -= (last G1) dW1^T ; dU = dG1 gelu'(Z1) (kept in mU's place after saving U * gelu'')
+    mm_lds<2, NW>(lds + L::DK, LD, G1l, M, 1, dW1, 1, M, 1, NTD, M, wave, lane);
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) {
+      const int o = cg + GW * j;
+      float y, dy, ddy;
+      gelu_tanh_all(mZ1[t * M + o], y, dy, ddy);
+      const float dg1 = mS1[t * M + o];
+      mS1[t * M + o] = dg1 * mU[t * M + o] * ddy;  // first term of dZ1
+      mU[t * M + o] = dg1 * dy;                    // dU
+    }
+    __syncthreads();
+    // ---- 20. dG2 += dU W2
+    mm_lds<1, NW>(lds + L::DG2, LD, mU, M, 1, W2, D, 1, 1, NTD, M, wave, lane);
+    __syncthreads();
+    // ---- 21. second-order LayerNorm: dZ2, dT, d gamma, d beta
+    {
+      float xh[NJD], dG[NJD], u[NJD], gO[NJD], gx[NJD], s1 = 0.f, s2 = 0.f, sgx = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        xh[j] = lds[L::XH + t * LD + o];
+        dG[j] = lds[L::DG2 + t * LD + o];
+        u[j] = -dG[j] * rstd1;
+        gO[j] = sgam[o] * xh[j] + sbet[o] - lds[L::TG + t * LD + o];
+        gx[j] = gO[j] * sgam[o];
+        s1 += u[j];
+        s2 += u[j] * xh[j];
+        sgx += gx[j] * xh[j];
+      }
+      s1 = rowgroup_sum<GW>(s1) * inv_d;
+      s2 = rowgroup_sum<GW>(s2) * inv_d;
+      sgx = rowgroup_sum<GW>(sgx) * inv_d;
+      float dxh[NJD], dy[NJD], q1 = 0.f, q2 = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        const float dgx = -u[j] + s1 + xh[j] * s2;
+        dy[j] = sgam[o] * dgx;
+        dgam_acc[j] += gO[j] * dgx + dy[j] * xh[j];
+        dbet_acc[j] += dy[j];
+        dxh[j] = dy[j] * sgam[o] + gx[j] * s2 + u[j] * sgx;
+        q1 += dxh[j];
+        q2 += dxh[j] * xh[j] + dG[j] * lds[L::G2 + t * LD + o];
+      }
+      q1 = rowgroup_sum<GW>(q1) * inv_d;
+      const float dsig = -rowgroup_sum<GW>(q2) * rstd1;
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        lds[L::DZ2 + t * LD + o] = (dxh[j] - q1) * rstd1 + xh[j] * dsig * inv_d;
+        lds[L::DT + t * LD + o] = -dy[j];
+      }
+    }
+    __syncthreads();
+    // ---- 22. dX2 += dZ2 W2^T ; then dZ1 = dG1 U gelu''(Z1) + dX2 gelu'(Z1)
+    mm_lds<1, NW, NBM>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) {
+      const int o = cg + GW * j;
+      float y, dy;
+      gelu_tanh_pair(mZ1[t * M + o], y, dy);
+      mDX2[t * M + o] = mS1[t * M + o] + mDX2[t * M + o] * dy;  // dZ1
+    }
+    __syncthreads();
+    // ---- 23. gradient accumulation; dK += dZ1 W1^T
+    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mXB2, 1, M, lds + L::DZB2, LD, 1, NTM, NTD, 16, wave, lane);
+    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mU, 1, M, lds + L::G2, LD, 1, NTM, NTD, 16, wave, lane);
+    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, 16, wave, lane);
+    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, 16, wave, lane);
+    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(dW1, M, lds + L::XK, 1, LD, mDX2, M, 1, NTD, NTM, 16, wave, lane);
+    mm_lds<1, NW>(lds + L::DK, LD, mDX2, M, 1, W1, 1, M, 1, NTD, M, wave, lane);
+    if (tid < M) {
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += mDXB[r * M + tid] + mDX2[r * M + tid];
+      sdb1[tid] += s;
+    }
+    if (tid < D) {
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += lds[L::DZB2 + r * LD + tid] + lds[L::DZ2 + r * LD + tid];
+      sdb2[tid] += s;
+    }
+    __syncthreads();
+    // ---- 24. stores
+    if (t < K) {
+      elem* pq = static_cast<elem*>(a.d_xq) + row * D;
+      elem* pk = static_cast<elem*>(a.d_xk) + row * D;
+      elem* pv = static_cast<elem*>(a.d_xv) + row * D;
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = cg + GW * j;
+        const float dT = lds[L::DT + t * LD + o];
+        IO::store1(pq + o, lds[L::DQ + t * LD + o] + lds[L::DO + t * LD + o]);
+        IO::store1(pk + o, lds[L::DK + t * LD + o] - dT);
+        IO::store1(pv + o, dT);
+      }
+    }
+    if (tid < 16) {
+      const int s = tid;
+      float dl = te_last * lds[L::dlast + s];
+      for (int r = 0; r < 16; ++r) dl += lds[L::DETA + r * LK + s] * ste[r];
+      if (s < K)
+        IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + s, dl);
+    } else if (tid >= 64 && tid < 80) {
+      const int tt = tid - 64;
+      float s = 0.f;
+      for (int r = 0; r < 16; ++r) s += lds[L::DETA + tt * LK + r] * slr[r];
+      if (tt == K - 1)
+        for (int r = 0; r < 16; ++r) s += lds[L::dlast + r] * slr[r];
+      if (tt < K) atomicAdd(a.d_token_eta + (size_t)st * K + tt, s);
+    }
+    __syncthreads();
+  }
+
+  // ---- results carried over the whole scan
+  for (int i = tid; i < M; i += 512) a.d_b1[bh * M + i] = sdb1[i];
+  for (int i = tid; i < D; i += 512) a.d_b2[bh * D + i] = sdb2[i];
+#pragma unroll
+  for (int j = 0; j < NJD; ++j) {
+    lds[L::XQ + t * LD + cg + GW * j] = dgam_acc[j];
+    lds[L::XK + t * LD + cg + GW * j] = dbet_acc[j];
+  }
+  __syncthreads();
+  if (tid < D) {
+    float sg = 0.f, sbt = 0.f;
+    for (int r = 0; r < 16; ++r) {
+      sg += lds[L::XQ + r * LD + tid];
+      sbt += lds[L::XK + r * LD + tid];
+    }
+    atomicAdd(a.d_gamma + h * D + tid, sg);
+    atomicAdd(a.d_beta + h * D + tid, sbt);
+  }
+}
+
+}  // namespace ttt

@@ -270,6 +270,64 @@ def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_we
     return (out, *o)
 
 
+def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias, d_out,
+                         mini_batch: int, eps: float = 1e-6, d_state_out=None):
+    """One call of ttt_mlp_bwd on the current stream: gradients of the TTT-MLP inner loop
+    (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50; the reference gets them
+    from Burn autodiff).  Arguments as ttt_mlp_forward_raw plus d_out [B,H,seq,d] and the optional
+    upstream gradients of the final state d_state_out = (dW1, db1, dW2, db2), per batch element.
+    Returns a dict: d_xq, d_xk, d_xv, d_W1 [B,H,d,4d], d_b1, d_W2, d_b2 (per batch element), d_lr,
+    d_token_eta [seq], d_gamma, d_beta [H,d]."""
+    B, H, seq, d = xq.shape
+    m = w1.shape[-1]
+    io = xq.dtype
+    xq = _need(xq, (B, H, seq, d), io, "xq")
+    xk = _need(xk, (B, H, seq, d), io, "xk")
+    xv = _need(xv, (B, H, seq, d), io, "xv")
+    d_out = _need(d_out, (B, H, seq, d), io, "d_out")
+    lr = _need(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta")
+    per_batch = w1.dim() == 4
+    lead = (B, H) if per_batch else (H,)
+    if m != 4 * d:
+        raise _lib.TttError(_lib.TTT_ERR_UNSUPPORTED, f"mlp_dim {m} != 4*head_dim (only expansion 4)")
+    w1 = _need(w1, lead + (d, m), torch.float32, "w1")
+    b1 = _need(b1, lead + (m,), torch.float32, "b1")
+    w2 = _need(w2, lead + (m, d), torch.float32, "w2")
+    b2 = _need(b2, lead + (d,), torch.float32, "b2")
+    ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+    ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+    if token_eta.numel() < mini_batch:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
+    te = token_eta.to(torch.float32).contiguous()
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), int(per_batch), 0)
+    check(lib().ttt_mlp_supported(C.byref(desc)))
+    dev = xq.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    shapes = [(B, H, d, m), (B, H, m), (B, H, m, d), (B, H, d)]
+    up = [None] * 4
+    if d_state_out is not None:
+        up = [_need(g, sh, torch.float32, "d_state_out") for g, sh in zip(d_state_out, shapes)]
+    g_act = [torch.empty_like(xq) for _ in range(3)]
+    g_st = [torch.empty(sh, **f32) for sh in shapes]
+    g_lr = torch.empty_like(lr)
+    g_te = torch.empty(seq, **f32)
+    g_gam, g_bet = torch.empty((H, d), **f32), torch.empty((H, d), **f32)
+    nbytes = lib().ttt_mlp_bwd_workspace_bytes(C.byref(desc))
+    if nbytes < 0:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, "ttt_mlp_bwd_workspace_bytes failed")
+    ws = torch.empty((nbytes + 3) // 4, **f32)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    null = C.c_void_p(None)
+    with torch.cuda.device(dev):
+        check(lib().ttt_mlp_bwd(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(w1), _ptr(b1), _ptr(w2),
+                                _ptr(b2), _ptr(te), _ptr(lr), _ptr(ln_weight), _ptr(ln_bias), _ptr(d_out),
+                                *[null if g is None else _ptr(g) for g in up],
+                                *[_ptr(g) for g in g_act], *[_ptr(g) for g in g_st], _ptr(g_lr), _ptr(g_te),
+                                _ptr(g_gam), _ptr(g_bet), _ptr(ws), stream))
+    return dict(d_xq=g_act[0], d_xk=g_act[1], d_xv=g_act[2], d_W1=g_st[0], d_b1=g_st[1], d_W2=g_st[2],
+                d_b2=g_st[3], d_lr=g_lr, d_token_eta=g_te, d_gamma=g_gam, d_beta=g_bet)
+
+
 @dataclass
 class TTTMLPState:
     """mlp.rs:43-53: w1 [B,H,d,4d], b1 [B,H,4d], w2 [B,H,4d,d], b2 [B,H,d], always f32."""
