@@ -32,6 +32,8 @@ WORKLOADS = {
     "linear_fwd_125m_f32_b8": dict(cfg=2, B=8, H=12, d=64, seq=2048, K=16, io="f32", kind="linear_fwd"),
     "linear_fwd_bwd_125m_f32_b8": dict(cfg=2, B=8, H=12, d=64, seq=2048, K=16, io="f32", kind="linear_fwd_bwd"),
     "mlp_fwd_d96_bf16": dict(cfg=3, B=8, H=16, d=96, seq=2048, K=16, io="bf16", kind="mlp_fwd"),
+    "mlp_fwd_bwd_d96_bf16": dict(cfg=3, B=8, H=16, d=96, seq=2048, K=16, io="bf16", kind="mlp_fwd_bwd"),
+    "linear_fwd_bwd_125m_bf16_b32": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="linear_fwd_bwd"),
     "stack8_d128_seq8192_bf16": dict(cfg=4, B=4, H=16, d=128, seq=8192, K=16, io="bf16", kind="stack"),
 }
 
@@ -54,7 +56,7 @@ def cpu_baseline(c, K, kind, budget_s=20.0):
     cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "9999")))
     n = {k: v.float().numpy() for k, v in c.items()}
     B, H, seq, d = n["xq"].shape
-    if kind == "mlp_fwd":
+    if kind in ("mlp_fwd", "mlp_fwd_bwd"):
         fn = c_oracle.mlp_fwd
         keys = ("W1", "b1", "W2", "b2", "xq", "xk", "xv", "token_eta", "lr", "gamma", "beta")
     else:
@@ -71,7 +73,7 @@ def cpu_baseline(c, K, kind, budget_s=20.0):
         fn(*bsl(Bs), K=K, dtype=np.float32, nthreads=cores)
         times.append(time.perf_counter() - t0)
     t = sum(times) / len(times)
-    what = "forward" if kind != "linear_fwd_bwd" else "forward only (the C port has no backward)"
+    what = "forward" if kind not in ("linear_fwd_bwd", "mlp_fwd_bwd") else "forward only (the C port has no backward)"
     return {"value": Bs * seq / t, "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"C/OpenMP f32 port of the reference CPU path, {what}, same inputs, batch {Bs} of "
                       f"{B} (tokens/s is batch-normalised), mean of 3 runs, {t:.3f} s per run"}
@@ -133,7 +135,8 @@ def main():
             return (x,)
     else:
         c = pkg.synthetic.baseline_inputs(w["cfg"], B, H, seq, d, K, io_dtype=dtype,
-                                          with_dout=kind == "linear_fwd_bwd", mlp=kind == "mlp_fwd")
+                                          with_dout=kind in ("linear_fwd_bwd", "mlp_fwd_bwd"),
+                                          mlp=kind in ("mlp_fwd", "mlp_fwd_bwd"))
         dv = {k: v.to(dev) for k, v in c.items()}
         if kind == "linear_fwd":
             def step():
@@ -143,6 +146,14 @@ def main():
             def step():
                 return pkg.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
                                                dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+        elif kind == "mlp_fwd_bwd":
+            def step():
+                fw = pkg.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
+                                             dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+                g = pkg.ttt_mlp_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
+                                             dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"],
+                                             dv["d_out"], K)
+                return (fw[0], g["d_xq"])
         else:
             def step():
                 out, W, b, Wc, bc = pkg.ttt_linear_forward_raw(
@@ -168,7 +179,8 @@ def main():
     dev_s = sum(e0.elapsed_time(e1) for e0, e1 in ev) / len(ev) / 1e3  # device time of one step
     assert all(torch.isfinite(r.float()).all() for r in res)
 
-    pass_name = {"linear_fwd": "fwd", "linear_fwd_bwd": "fwd+bwd", "mlp_fwd": "fwd", "stack": "fwd"}[kind]
+    pass_name = {"linear_fwd": "fwd", "linear_fwd_bwd": "fwd+bwd", "mlp_fwd": "fwd", "mlp_fwd_bwd": "fwd+bwd",
+                 "stack": "fwd"}[kind]
     out = {
         "metric": f"inner-loop tokens/sec ({pass_name}) at 125M shape" if d == 64 else
                   f"inner-loop tokens/sec ({pass_name})",
@@ -210,6 +222,16 @@ def main():
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": peak,
                            "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / peak, "traffic": None,
                            "kernel": "ttt_mlp_fwd_rr_kernel" if rr else "ttt_mlp_fwd_kernel",
+                           "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
+    elif kind == "mlp_fwd_bwd":
+        # forward (56 d^2 + 20 K d) plus the backward's own forward sweep and its 14 state-sized and
+        # 7 rank-16 products: (56 + 56 + 14*8 + 7*8) d^2 flop per token-head, K-sized terms aside
+        flops = th * (280 * d * d)
+        out["dtype"] = "f32"
+        out["config"]["inner_model"] = "TTT-MLP"
+        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
+                           "kernel": "ttt_mlp_fwd_rr_kernel + ttt_mlp_fwd_kernel + ttt_mlp_bwd_kernel (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     else:
         flops = th * (6 * (6 * d * d + 4 * K * d) + 2 * (56 * d * d + 20 * K * d))

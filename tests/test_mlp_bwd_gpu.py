@@ -67,3 +67,12 @@ def test_mlp_bwd_is_linear_in_upstream_gradient(P):
     torch.cuda.synchronize()
     for k in GRADS:
         assert_close(g2[k], 2.0 * g1[k].double().cpu().numpy(), 1e-5, k)
+
+
+def test_mlp_bwd_long_sequence_rollback(P):
+    """128 mini-batches at the TTT-MLP benchmark head size: the state is rolled back 128 times from
+    the final state, so this bounds the accumulated rounding of the roll-back."""
+    print("case mlp bwd long", flush=True)
+    got, ref = run_case(P, 1, 2, 96, 16, 128, torch.float32, "baseline", seed=3)
+    for k in GRADS:
+        assert_close(got[k], ref[k], 1e-4, k)

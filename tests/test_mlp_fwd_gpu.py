@@ -49,6 +49,24 @@ def test_mlp_fwd_matches_oracle(P, B, H, d, K, N, style, dtype):
         assert_close(g, r, 1e-4 if (f32_products and name != "out") else TOL[dtype], name)
 
 
+def test_mlp_fwd_bf16_lds_kernel_keeps_f32_products(P, monkeypatch):
+    """TTT_MLP_FWD_KERNEL=lds selects the LDS-tile kernel for bf16 I/O too: f32 products, so the
+    state meets the f32 bar."""
+    print("case mlp bf16 lds kernel", flush=True)
+    monkeypatch.setenv("TTT_MLP_FWD_KERNEL", "lds")
+    B, H, d, K, N = 2, 2, 96, 16, 4
+    c = mlp_case(P, 77, B, H, N * K, d, K, torch.bfloat16, "ref")
+    dv = to_dev(c)
+    got = P.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
+                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
+                          n["lr"], n["gamma"], n["beta"], K=K)
+    for name, g, r in zip(("out", "W1", "b1", "W2", "b2"), got, ref):
+        assert_close(g, r, TOL[torch.bfloat16] if name == "out" else 1e-4, name)
+
+
 def test_mlp_inner_model_with_remainder(P):
     print("case mlp remainder", flush=True)
     B, H, d, K, seq = 2, 2, 64, 16, 37
