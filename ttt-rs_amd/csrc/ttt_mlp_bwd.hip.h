@@ -60,8 +60,9 @@ constexpr int kMlpBwdMTiles = 9;  // [16 x 4d] scratch tiles per (batch, head)
 template <int D>
 struct MlpBwdLds {
   static constexpr int M = 4 * D, LD = D + 4, LK = 17, KK = 16 * LK, TD = 16 * LD;
-  static constexpr int XQ = 0, XK = XQ + TD, TG = XK + TD, DO = TG + TD, XH = DO + TD, G2 = XH + TD,
-                       XH2 = G2 + TD, DZB2 = XH2 + TD, DG2 = DZB2 + TD, DZ2 = DG2 + TD, DT = DZ2 + TD,
+  // (XQ, XK) and (DZ2, G2, DZB2) are consecutive on purpose: see the fused accumulations of step 23
+  static constexpr int XQ = 0, XK = XQ + TD, TG = XK + TD, DO = TG + TD, XH = DO + TD, DZ2 = XH + TD,
+                       G2 = DZ2 + TD, DZB2 = G2 + TD, XH2 = DZB2 + TD, DG2 = XH2 + TD, DT = DG2 + TD,
                        DQ = DT + TD, DK = DQ + TD;
   static constexpr int ETA = DK + TD, A1 = ETA + KK, M1 = A1 + KK, M2 = M1 + KK, P = M2 + KK,
                        DA = P + KK, DETA = DA + KK, PART = DETA + KK;
@@ -105,8 +106,10 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
   float* dW2 = a.d_W2 + bh * (size_t)M * D;
   // [16 x 4d] scratch tiles
   float* mt = a.mt + bh * (size_t)kMlpBwdMTiles * 16 * M;
-  float *mZ1 = mt, *mX2 = mt + 16 * M, *mU = mt + 2 * 16 * M, *mG1 = mt + 3 * 16 * M, *mZB1 = mt + 4 * 16 * M,
-        *mXB2 = mt + 5 * 16 * M, *mDXB = mt + 6 * 16 * M, *mDX2 = mt + 7 * 16 * M, *mS1 = mt + 8 * 16 * M;
+  // (X2, U, Xbar2) and (dZbar1, dZ1) are consecutive: each group is the k-side operand of one fused
+  // rank-48 / rank-32 accumulation into dW2 / dW1
+  float *mZ1 = mt, *mX2 = mt + 16 * M, *mU = mt + 2 * 16 * M, *mXB2 = mt + 3 * 16 * M, *mG1 = mt + 4 * 16 * M,
+        *mZB1 = mt + 5 * 16 * M, *mDXB = mt + 6 * 16 * M, *mDX2 = mt + 7 * 16 * M, *mS1 = mt + 8 * 16 * M;
 
   for (int i = tid; i < M; i += 512) {
     sb1[i] = a.b1f[bh * M + i];
@@ -142,6 +145,17 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) lds[L::PART + wave * 256 + (4 * g + r) * 16 + c] = acc[r];
   };
+  // this thread's NJM elements of a [16 x 4d] tile, all loads issued before any use (the tiles are
+  // in global memory and may alias as far as the compiler knows, so a load-compute-store loop would
+  // pay the full memory latency per element)
+  auto ldm = [&](const float* tile, float (&v)[NJM]) {
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) v[j] = tile[t * M + cg + GW * j];
+  };
+  auto stm = [&](float* tile, const float (&v)[NJM]) {
+#pragma unroll
+    for (int j = 0; j < NJM; ++j) tile[t * M + cg + GW * j] = v[j];
+  };
   auto part_sum = [&](int tt, int s) {
     float v = 0.f;
 #pragma unroll
@@ -176,14 +190,17 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
     mm_lds<0, NW, NBM>(mZ1, M, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
+    {
+      float z[NJM], y[NJM];
+      ldm(mZ1, z);
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) {
-      const int o = cg + GW * j;
-      float y, dy;
-      const float z = mZ1[t * M + o] + sb1[o];
-      gelu_tanh_pair(z, y, dy);
-      mZ1[t * M + o] = z;
-      mX2[t * M + o] = y;
+      for (int j = 0; j < NJM; ++j) {
+        float dy;
+        z[j] += sb1[cg + GW * j];
+        gelu_tanh_pair(z[j], y[j], dy);
+      }
+      stm(mZ1, z);
+      stm(mX2, y);
     }
     __syncthreads();
     // ---- 4. roll W2, b2 back
@@ -233,25 +250,33 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     mm_lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 8. G1 = U gelu'(Z1)
+    {
+      float z[NJM], u[NJM];
+      ldm(mZ1, z);
+      ldm(mU, u);
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) {
-      const int o = cg + GW * j;
-      float y, dy;
-      gelu_tanh_pair(mZ1[t * M + o], y, dy);
-      mG1[t * M + o] = mU[t * M + o] * dy;
+      for (int j = 0; j < NJM; ++j) {
+        float y, dy;
+        gelu_tanh_pair(z[j], y, dy);
+        u[j] *= dy;
+      }
+      stm(mG1, u);
     }
     __syncthreads();
     // ---- 9. Zbar1 -= M1 G1 ; then + b1, Xbar2 = gelu
     mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(mZB1, M, lds + L::M1, LK, 1, mG1, M, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
+    {
+      float z[NJM], y[NJM];
+      ldm(mZB1, z);
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) {
-      const int o = cg + GW * j;
-      float y, dy;
-      const float z = mZB1[t * M + o] + sb1[o];
-      gelu_tanh_pair(z, y, dy);
-      mZB1[t * M + o] = z;
-      mXB2[t * M + o] = y;
+      for (int j = 0; j < NJM; ++j) {
+        float dy;
+        z[j] += sb1[cg + GW * j];
+        gelu_tanh_pair(z[j], y[j], dy);
+      }
+      stm(mZB1, z);
+      stm(mXB2, y);
     }
     __syncthreads();
     // ---- 10. A2 = Xbar2 X2^T (split-k) ; Zbar2 = Xbar2 W2
@@ -319,12 +344,17 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     __syncthreads();
     // ---- 15. dX2 -= (last G2) dW2^T ; dZbar1 = dXbar2 gelu'(Zbar1)
     mm_lds<2, NW, NBM>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
+    {
+      float z[NJM], v[NJM];
+      ldm(mZB1, z);
+      ldm(mDXB, v);
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) {
-      const int o = cg + GW * j;
-      float y, dy;
-      gelu_tanh_pair(mZB1[t * M + o], y, dy);
-      mDXB[t * M + o] *= dy;
+      for (int j = 0; j < NJM; ++j) {
+        float y, dy;
+        gelu_tanh_pair(z[j], y, dy);
+        v[j] *= dy;
+      }
+      stm(mDXB, v);
     }
     __syncthreads();
     // ---- 16. P1 = dZbar1 G1^T (split-k) ; dQ = dZbar1 W1^T ; S1 = XK dW1
@@ -340,14 +370,16 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
       lds[L::DETA + tt * LK + s] += -p * (1.f + lds[L::A1 + tt * LK + s]);
     }
     {
-      float q = 0.f;
+      float q = 0.f, sv[NJM], gv[NJM];
+      ldm(mS1, sv);
+      ldm(mG1, gv);
 #pragma unroll
       for (int j = 0; j < NJM; ++j) {
-        const int o = cg + GW * j;
-        const float s1v = mS1[t * M + o] + sdb1[o];
-        q += mG1[t * M + o] * s1v;
-        mS1[t * M + o] = -last * s1v;
+        const float s1v = sv[j] + sdb1[cg + GW * j];
+        q += gv[j] * s1v;
+        sv[j] = -last * s1v;
       }
+      stm(mS1, sv);
       q = rowgroup_sum<GW>(q);
       if (cg == 0) lds[L::dlast + t] -= q;
     }
@@ -359,14 +391,20 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     __syncthreads();
     // ---- 19. dK -= (last G1) dW1^T ; dU = dG1 gelu'(Z1) (kept in mU's place after saving U * gelu'')
     mm_lds<2, NW>(lds + L::DK, LD, G1l, M, 1, dW1, 1, M, 1, NTD, M, wave, lane);
+    {
+      float z[NJM], dg1[NJM], u[NJM];
+      ldm(mZ1, z);
+      ldm(mS1, dg1);
+      ldm(mU, u);
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) {
-      const int o = cg + GW * j;
-      float y, dy, ddy;
-      gelu_tanh_all(mZ1[t * M + o], y, dy, ddy);
-      const float dg1 = mS1[t * M + o];
-      mS1[t * M + o] = dg1 * mU[t * M + o] * ddy;  // first term of dZ1
-      mU[t * M + o] = dg1 * dy;                    // dU
+      for (int j = 0; j < NJM; ++j) {
+        float y, dy, ddy;
+        gelu_tanh_all(z[j], y, dy, ddy);
+        z[j] = dg1[j] * u[j] * ddy;  // first term of dZ1
+        u[j] = dg1[j] * dy;          // dU
+      }
+      stm(mS1, z);
+      stm(mU, u);
     }
     __syncthreads();
     // ---- 20. dG2 += dU W2
@@ -415,20 +453,25 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     // ---- 22. dX2 += dZ2 W2^T ; then dZ1 = dG1 U gelu''(Z1) + dX2 gelu'(Z1)
     mm_lds<1, NW, NBM>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
+    {
+      float z[NJM], f1[NJM], dx[NJM];
+      ldm(mZ1, z);
+      ldm(mS1, f1);
+      ldm(mDX2, dx);
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) {
-      const int o = cg + GW * j;
-      float y, dy;
-      gelu_tanh_pair(mZ1[t * M + o], y, dy);
-      mDX2[t * M + o] = mS1[t * M + o] + mDX2[t * M + o] * dy;  // dZ1
+      for (int j = 0; j < NJM; ++j) {
+        float y, dy;
+        gelu_tanh_pair(z[j], y, dy);
+        dx[j] = f1[j] + dx[j] * dy;  // dZ1
+      }
+      stm(mDX2, dx);
     }
     __syncthreads();
     // ---- 23. gradient accumulation; dK += dZ1 W1^T
-    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mXB2, 1, M, lds + L::DZB2, LD, 1, NTM, NTD, 16, wave, lane);
-    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mU, 1, M, lds + L::G2, LD, 1, NTM, NTD, 16, wave, lane);
-    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, 16, wave, lane);
-    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, 16, wave, lane);
-    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(dW1, M, lds + L::XK, 1, LD, mDX2, M, 1, NTD, NTM, 16, wave, lane);
+    // dW2 += X2^T dZ2 + dU^T G2 + Xbar2^T dZbar2 as ONE rank-48 pass over dW2 (operands consecutive)
+    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, 48, wave, lane);
+    // dW1 += XQ^T dZbar1 + XK^T dZ1 as one rank-32 pass
+    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, 32, wave, lane);
     mm_lds<1, NW>(lds + L::DK, LD, mDX2, M, 1, W1, 1, M, 1, NTD, M, wave, lane);
     if (tid < M) {
       float s = 0.f;
