@@ -17,6 +17,7 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
         #include <cstdio>
         #include <cstring>
         #include "ttt-rs_amd/host/fused_tile_multi.hpp"
+        #include "ttt-rs_amd/host/fused_mlp.hpp"
         int main() {
           ttt::ModelConfig cfg; cfg.num_heads = 2; cfg.head_dim = 64;
           float dummy[4] = {0.f, 0.f, 0.f, 0.f};
@@ -30,6 +31,18 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
           in.seq_len = 32;                                          // valid shape, null tensors
           try { m.forward(st, in, out, ttt::Checkpoints{}, nullptr); return 5; }
           catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 6; std::printf("%s\n", e.what()); }
+          // TTT-MLP host class: workspace query, shape and null-pointer rejection
+          cfg.head_dim = 96;
+          ttt::FusedMlp mlp(cfg, dummy, dummy, dummy, dummy, dummy, dummy);
+          if (std::strcmp(mlp.name(), "FusedTTTMLP")) return 7;
+          // per (batch, head): 2 d M + M + d + N 16 (M + d) + 9 * 16 M floats, M = 4 d
+          const long long per_unit = 2LL * 96 * 384 + 384 + 96 + 2LL * 16 * (384 + 96) + 9LL * 16 * 384;
+          if (mlp.backward_workspace_bytes(2, 32, TTT_BF16) != 4 * 2 * 2 * per_unit) return 8;
+          ttt::TTTMLPState ms;
+          try { mlp.forward_mini_batch(ms, in, 0, 17, out, nullptr); return 9; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_SHAPE) return 10; }
+          try { mlp.backward(in, ms, out, nullptr, nullptr, nullptr, nullptr, ttt::TTTMLPGrads{}, out, nullptr); return 11; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 12; }
           return 0;
         }
     '''))

@@ -76,3 +76,25 @@ def test_mlp_bwd_long_sequence_rollback(P):
     got, ref = run_case(P, 1, 2, 96, 16, 128, torch.float32, "baseline", seed=3)
     for k in GRADS:
         assert_close(got[k], ref[k], 1e-4, k)
+
+
+def test_mlp_inner_model_backward_from_parameters(P):
+    """FusedMlp.backward with state0 = None: [H,..] parameters broadcast over batch; the parameter
+    gradient is the batch sum of the per-batch state gradients."""
+    print("case mlp model backward", flush=True)
+    B, H, d, K, N = 2, 2, 32, 16, 2
+    c = mlp_case(P, 512, B, H, N * K, d, K, torch.float32, "ref")
+    dv = to_dev(c)
+    model = P.FusedMlp(P.ModelConfig(H, d, P.TTTConfig(mini_batch_size=K)), dv["W1"], dv["b1"], dv["W2"],
+                       dv["b2"], dv["gamma"], dv["beta"])
+    g = torch.Generator().manual_seed(9)
+    dO = torch.randn(B, H, N * K, d, generator=g)
+    got = model.backward(None, P.TTTInputsInner(P.Qkv(dv["xq"], dv["xk"], dv["xv"]), dv["token_eta"], dv["lr"]),
+                         dO.to("cuda:0"))
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ref = orc.mlp_backward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                           n["gamma"], n["beta"], dO.double().numpy(), K=K)
+    for k in GRADS:
+        assert_close(got[k], ref[k], 1e-4, k)
+    assert_close(got["d_W1"].sum(0), ref["d_W1"].sum(0), 1e-4, "parameter grad W1")

@@ -399,6 +399,17 @@ class FusedMlp:
             raise _lib.TttError(_lib.TTT_ERR_SHAPE, "range longer than mini_batch_size")
         return self._launch(state, inputs.slice_seq(r), len(r))
 
+    def backward(self, state0: Optional[TTTMLPState], inputs: TTTInputsInner, grad_output, grad_state_out=None):
+        """Gradients of forward() over a sequence that is a multiple of mini_batch_size, starting from
+        state0 (None: the [H,..] parameters broadcast over batch, init_state).  The reference gets these
+        from Burn autodiff over mlp.rs:127-208.  Returns the dict of ttt_mlp_backward_raw."""
+        st = (self.w1_init, self.b1_init, self.w2_init, self.b2_init) if state0 is None else \
+            (state0.w1, state0.b1, state0.w2, state0.b2)
+        return ttt_mlp_backward_raw(inputs.qkv.xq, inputs.qkv.xk, inputs.qkv.xv, *st, inputs.token_eta,
+                                    inputs.ttt_lr_eta, self.ln_weight, self.ln_bias, grad_output,
+                                    self.config.ttt.mini_batch_size, self.config.ttt.epsilon,
+                                    d_state_out=grad_state_out)
+
 
 class FusedTileMulti:
     """`fused-tile-multi` TTT-Linear layer: Fused<B, TTTLinear<B>, TileMultiKernel>.
