@@ -34,6 +34,9 @@ WORKLOADS = {
     "mlp_fwd_d96_bf16": dict(cfg=3, B=8, H=16, d=96, seq=2048, K=16, io="bf16", kind="mlp_fwd"),
     "mlp_fwd_bwd_d96_bf16": dict(cfg=3, B=8, H=16, d=96, seq=2048, K=16, io="bf16", kind="mlp_fwd_bwd"),
     "linear_fwd_bwd_125m_bf16_b32": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="linear_fwd_bwd"),
+    # the elementwise passes either side of the inner loop at the 125M shape (hidden 768)
+    "inner_inputs_125m_bf16": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="inner_inputs"),
+    "layer_epilogue_125m_bf16": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="layer_epilogue"),
     "stack8_d128_seq8192_bf16": dict(cfg=4, B=4, H=16, d=128, seq=8192, K=16, io="bf16", kind="stack"),
 }
 
@@ -133,6 +136,26 @@ def main():
                     x = pkg.ttt_mlp_forward_raw(q, k, v, L["W1"], L["b1"], L["W2"], L["b2"], L["token_eta"],
                                                 L["lr"], L["gamma"], L["beta"], K)[0]
             return (x,)
+    elif kind in ("inner_inputs", "layer_epilogue"):
+        c = None
+        g = torch.Generator().manual_seed(1234 + w["cfg"])
+        rn = lambda *sh: torch.randn(*sh, generator=g).to(dtype).to(dev)
+        if kind == "inner_inputs":
+            xq, xk, xv, lg = rn(B, seq, H, d), rn(B, seq, H, d), rn(B, seq, H, d), rn(B, seq, H)
+            bias = torch.zeros(H, device=dev)
+            tidx = (1.0 / torch.arange(1, K + 1, dtype=torch.float32)).to(dev)
+            ltidx = torch.zeros(K, device=dev)
+            rope = pkg.rope_cos_sin(K, 0, None, d, dev)
+
+            def step():
+                r = pkg.inner_loop_inputs_raw(xq, xk, xv, lg, bias, 1.0, tidx, ltidx, K, rope=rope, pos_wrap=K)
+                return (r.qkv.xq, r.ttt_lr_eta)
+        else:
+            x, gate = rn(B, H, seq, d), rn(B, seq, H * d)
+            gam, bet = torch.ones(H * d, device=dev), torch.zeros(H * d, device=dev)
+
+            def step():
+                return (pkg.layer_epilogue_raw(x, gam, bet, gate),)
     else:
         c = pkg.synthetic.baseline_inputs(w["cfg"], B, H, seq, d, K, io_dtype=dtype,
                                           with_dout=kind in ("linear_fwd_bwd", "mlp_fwd_bwd"),
@@ -180,7 +203,7 @@ def main():
     assert all(torch.isfinite(r.float()).all() for r in res)
 
     pass_name = {"linear_fwd": "fwd", "linear_fwd_bwd": "fwd+bwd", "mlp_fwd": "fwd", "mlp_fwd_bwd": "fwd+bwd",
-                 "stack": "fwd"}[kind]
+                 "stack": "fwd", "inner_inputs": "inner-loop inputs", "layer_epilogue": "layer epilogue"}[kind]
     out = {
         "metric": f"inner-loop tokens/sec ({pass_name}) at 125M shape" if d == 64 else
                   f"inner-loop tokens/sec ({pass_name})",
@@ -201,6 +224,14 @@ def main():
                            "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
                            "kernel": "ttt_linear_fwd_kernel", "kernel_avg_us": dev_s * 1e6,
                            "algorithmic_bytes": alg}
+    elif kind in ("inner_inputs", "layer_epilogue"):
+        # inner_inputs: xq, xk, xv read and written once, logits in, lr out; epilogue: inner_out and gate in, out written
+        alg = th * (6 * d * s + 2 * s) if kind == "inner_inputs" else th * 3 * d * s
+        out["dtype"] = "f32"
+        out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                           "kernel": "ttt_inner_inputs_kernel" if kind == "inner_inputs" else "ttt_layer_epilogue_kernel",
+                           "kernel_avg_us": dev_s * 1e6, "algorithmic_bytes": alg}
     elif kind == "linear_fwd_bwd":
         # the backward kernel dominates; it computes in f32 MFMA: 18 d^2 + 22 K d flop per token-head
         flops = th * (24 * d * d + 26 * K * d)

@@ -160,6 +160,38 @@ int ttt_mlp_bwd(const ttt_desc* desc, const void* xq, const void* xk, const void
                 float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
                 float* d_gamma, float* d_beta, void* workspace, void* stream);
 
+/*
+ * The elementwise work either side of the inner loop, one HBM-bound pass each (the GEMMs of the
+ * projections stay with the BLAS the caller uses).  desc supplies batch, heads, seq, head_dim,
+ * mini_batch and io_dtype; the other fields are ignored.
+ *
+ * ttt_inner_inputs: TTT::get_inner_loop_inputs after the projections
+ * (rust/layer/src/ttt.rs:147-194 get_qkv, :205-227 get_lr, :247-268).
+ *   xq,xk,xv [B,seq,H,d] io as the q/k/v projections (and q/k convolutions) leave them;
+ *   lr_logits [B,seq,H] io = x . learnable_ttt_lr_weight^T; lr_bias [H] f32; token_idx,
+ *   learnable_token_idx [mini_batch] f32; rope_cos, rope_sin [npos, d/2] f32 as
+ *   RotaryEmbedding::get_cos_sin builds them (rust/core/src/util.rs:289-322; its two halves are
+ *   equal, pass one), or both NULL for no position encoding.  Token t uses table row
+ *   (pos_offset + t), modulo pos_wrap when pos_wrap > 0 (ttt.rs:183-189: RopeGlobal passes
+ *   (start_idx, none), the default passes (start_idx % mini_batch, mini_batch)).
+ *   Outputs: xq_out,xk_out,xv_out [B,H,seq,d] io (head split; xq,xk rotated: permute_qk ->
+ *   rotate-half RoPE -> undo_permute_qk, ttt.rs:26-41, util.rs:349-392); lr_out [B,H,seq] io =
+ *   base_lr * sigmoid(lr_logits + lr_bias) / d; token_eta_out [seq] f32 =
+ *   max(token_idx + learnable_token_idx, 0) tiled.  Outputs must not alias inputs.
+ *
+ * ttt_layer_epilogue: TTT::forward after the inner model (ttt.rs:285-297) up to the output
+ * projection: inner_out [B,H,seq,d] io -> head merge -> post_norm LayerNorm over H*d (weight, bias
+ * [H*d] f32, eps) -> times gelu_tanh(gate [B,seq,H*d] io) when gate is not NULL -> out [B,seq,H*d] io.
+ * H*d <= 2048.
+ */
+int ttt_inner_inputs(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                     const void* lr_logits, const float* lr_bias, float base_lr, const float* token_idx,
+                     const float* learnable_token_idx, const float* rope_cos, const float* rope_sin,
+                     int pos_offset, int pos_wrap, void* xq_out, void* xk_out, void* xv_out, void* lr_out,
+                     float* token_eta_out, void* stream);
+int ttt_layer_epilogue(const ttt_desc* desc, const void* inner_out, const float* post_norm_weight,
+                       const float* post_norm_bias, float eps, const void* gate, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -452,3 +452,74 @@ def mlp_backward(W1_0, b1_0, W2_0, b2_0, xq, xk, xv, token_eta, lr, gamma, beta,
         g_te[sl] = dte.sum((0, 1))
     return dict(d_xq=g_xq, d_xk=g_xk, d_xv=g_xv, d_W1=dW1, d_b1=db1, d_W2=dW2, d_b2=db2,
                 d_lr=g_lr, d_token_eta=g_te, d_gamma=g_gamma, d_beta=g_beta)
+
+
+# --------------------------------------------------------------------------- either side of the inner loop
+def rope_cos_sin(seq, offset, wrap, head_dim, base=10000.0):
+    """RotaryEmbeddingConfig::init + get_cos_sin (util.rs:266-322): inv_freq[i] = 1/base^(2i/d) rounded
+    to f32, positions (offset + t), taken modulo `wrap` when given, freqs = pos * inv_freq formed in
+    f32 as the reference's backend does; returns (cos, sin) [seq, d/2] (the reference concatenates
+    the half twice to [seq, d])."""
+    half = head_dim // 2
+    inv_freq = np.array([np.float32(1.0 / base ** ((2 * i) / head_dim)) for i in range(half)], np.float32)
+    pos = np.arange(seq, dtype=np.float32) + np.float32(offset)
+    if wrap is not None:
+        pos = np.fmod(pos, np.float32(wrap))
+    freqs = (pos[:, None] * inv_freq[None, :]).astype(np.float32).astype(np.float64)
+    return np.cos(freqs), np.sin(freqs)
+
+
+def _permute_qk(x):
+    """ttt.rs:26-32: [..., d] -> [..., d/2, 2] -> swap -> [..., 2, d/2] -> [..., d]."""
+    s = x.shape
+    return np.swapaxes(x.reshape(s[:-1] + (s[-1] // 2, 2)), -1, -2).reshape(s)
+
+
+def _undo_permute_qk(x):
+    """ttt.rs:35-41."""
+    s = x.shape
+    return np.swapaxes(x.reshape(s[:-1] + (2, s[-1] // 2)), -1, -2).reshape(s)
+
+
+def _rotate_half(x):
+    """util.rs:349-364: [x1, x2] -> [-x2, x1]."""
+    h = x.shape[-1] // 2
+    return np.concatenate([-x[..., h:], x[..., :h]], -1)
+
+
+def rope_apply(x, cos, sin):
+    """permute_qk -> x*cos + rotate_half(x)*sin -> undo_permute_qk (ttt.rs:179-194,
+    util.rs:385-392).  x [B,H,seq,d]; cos/sin [seq, d/2]."""
+    c = np.concatenate([cos, cos], -1)[None, None]
+    s = np.concatenate([sin, sin], -1)[None, None]
+    y = _permute_qk(x)
+    return _undo_permute_qk(y * c + _rotate_half(y) * s)
+
+
+def inner_loop_inputs(xq, xk, xv, lr_logits, lr_bias, base_lr, token_idx, learnable_token_idx, K,
+                      cos=None, sin=None, dtype=np.float64):
+    """TTT::get_inner_loop_inputs after the projections (ttt.rs:147-194, 205-227, 247-268).
+    xq,xk,xv [B,seq,H,d] as the projections (and convolutions) leave them; lr_logits [B,seq,H] =
+    x @ learnable_ttt_lr_weight^T.  Returns xq,xk,xv [B,H,seq,d] (RoPE on xq,xk when cos/sin
+    [seq,d/2] are given), ttt_lr_eta [B,H,seq], token_eta [seq]."""
+    xq, xk, xv, lg = (np.asarray(a, dtype) for a in (xq, xk, xv, lr_logits))
+    B, seq, H, d = xq.shape
+    q, k, v = (np.transpose(a, (0, 2, 1, 3)) for a in (xq, xk, xv))
+    if cos is not None:
+        q, k = rope_apply(q, cos, sin), rope_apply(k, cos, sin)
+    z = lg + np.asarray(lr_bias, dtype)[None, None, :]
+    lr = base_lr * (1.0 / (1.0 + np.exp(-np.transpose(z, (0, 2, 1))))) / d
+    te = np.asarray(token_idx, dtype) + np.asarray(learnable_token_idx, dtype)
+    te = np.maximum(np.tile(te, -(-seq // K))[:seq], 0.0)
+    return q, k, v, lr, te
+
+
+def layer_epilogue(inner_out, post_gamma, post_beta, gate=None, eps=1e-6):
+    """TTT::forward after the inner model (ttt.rs:285-297): [B,H,seq,d] -> [B,seq,H*d], post_norm
+    LayerNorm over the hidden axis (eps 1e-6), times gelu_tanh(gate) when the gate projection exists.
+    The output projection that follows is a plain GEMM and not part of this."""
+    x = np.asarray(inner_out, np.float64)
+    B, H, seq, d = x.shape
+    y = ln_fwd(np.transpose(x, (0, 2, 1, 3)).reshape(B, seq, H * d), np.asarray(post_gamma, np.float64),
+               np.asarray(post_beta, np.float64), eps)
+    return y if gate is None else gelu_tanh(np.asarray(gate, np.float64)) * y

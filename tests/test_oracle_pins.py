@@ -364,3 +364,53 @@ def test_mlp_backward_equals_autograd_through_dual(B, H, N, d, K, state_grads):
                             d_state_out=None if dst is None else [3.0 * g for g in dst])
     for k in got:
         np.testing.assert_allclose(got3[k], 3.0 * got[k], rtol=1e-10, atol=1e-12)
+
+
+# ------------------------------------------------------------------ either side of the inner loop
+def test_rope_is_complex_rotation_of_adjacent_pairs():
+    """permute_qk -> rotate_half RoPE -> undo_permute_qk (ttt.rs:26-41, util.rs:349-392) is a rotation
+    of the adjacent pairs (x[2i], x[2i+1]) by the angle pos * inv_freq[i]."""
+    rng = np.random.default_rng(3)
+    B, H, seq, d = 2, 3, 40, 16
+    x = rnd(rng, B, H, seq, d)
+    for offset, wrap in ((0, None), (5, 16), (37, None)):
+        cos, sin = orc.rope_cos_sin(seq, offset, wrap, d)
+        got = orc.rope_apply(x, cos, sin)
+        z = (x[..., 0::2] + 1j * x[..., 1::2]) * (cos + 1j * sin)[None, None]
+        np.testing.assert_allclose(got[..., 0::2], z.real, rtol=1e-12, atol=1e-14)
+        np.testing.assert_allclose(got[..., 1::2], z.imag, rtol=1e-12, atol=1e-14)
+        # positions: first frequency is 1 (inv_freq[0] = 1), so cos[:, 0] = cos(pos)
+        pos = np.arange(seq) + offset
+        if wrap is not None:
+            pos = pos % wrap
+        np.testing.assert_allclose(cos[:, 0], np.cos(pos.astype(np.float64)), atol=1e-12)
+    # torch restatement of apply_rotary_pos_emb_single on the permuted layout
+    t = torch.tensor(orc._permute_qk(x))
+    c = torch.tensor(np.concatenate([cos, cos], -1))
+    s = torch.tensor(np.concatenate([sin, sin], -1))
+    rot = torch.cat([-t[..., d // 2:], t[..., : d // 2]], -1)
+    np.testing.assert_allclose(orc._permute_qk(got), (t * c + rot * s).numpy(), rtol=1e-12, atol=1e-14)
+
+
+def test_inner_loop_inputs_and_epilogue_pieces():
+    rng = np.random.default_rng(8)
+    B, seq, H, d, K = 2, 19, 3, 8, 8
+    xq, xk, xv = (rnd(rng, B, seq, H, d) for _ in range(3))
+    lg, bias = rnd(rng, B, seq, H), rnd(rng, H)
+    tidx, ltidx = 1.0 / np.arange(1, K + 1), rnd(rng, K, scale=0.3) - 0.2
+    q, k, v, lr, te = orc.inner_loop_inputs(xq, xk, xv, lg, bias, 0.7, tidx, ltidx, K)
+    np.testing.assert_array_equal(v, np.transpose(xv, (0, 2, 1, 3)))
+    np.testing.assert_array_equal(q, np.transpose(xq, (0, 2, 1, 3)))
+    ref_lr = 0.7 * torch.sigmoid(torch.tensor(lg + bias).permute(0, 2, 1)) / d
+    np.testing.assert_allclose(lr, ref_lr.numpy(), rtol=1e-12)
+    ref_te = (torch.tensor(tidx) + torch.tensor(ltidx)).repeat(3)[:seq].clamp_min(0.0)
+    np.testing.assert_allclose(te, ref_te.numpy(), rtol=1e-14)
+    assert (te >= 0).all() and (te == 0).any()
+    # epilogue = torch layer_norm over the merged heads times torch tanh-GELU of the gate
+    inner = rnd(rng, B, H, seq, d)
+    g, b, gate = 1.0 + rnd(rng, H * d, scale=0.2), rnd(rng, H * d, scale=0.1), rnd(rng, B, seq, H * d)
+    merged = torch.tensor(inner).permute(0, 2, 1, 3).reshape(B, seq, H * d)
+    ref = F.layer_norm(merged, (H * d,), torch.tensor(g), torch.tensor(b), eps=1e-6)
+    np.testing.assert_allclose(orc.layer_epilogue(inner, g, b), ref.numpy(), rtol=1e-10, atol=1e-12)
+    ref = F.gelu(torch.tensor(gate), approximate="tanh") * ref
+    np.testing.assert_allclose(orc.layer_epilogue(inner, g, b, gate), ref.numpy(), rtol=1e-10, atol=1e-12)

@@ -10,6 +10,7 @@
 #include <cstring>
 
 #include "ttt_engine_fwd.hip.h"
+#include "ttt_layer_io.hip.h"
 #include "ttt_linear_bwd.hip.h"
 #include "ttt_linear_fwd.hip.h"
 #include "ttt_linear_fwd_mw.hip.h"
@@ -186,6 +187,15 @@ struct MlpBwdWs {
     total = mt + U * ttt::kMlpBwdMTiles * 16 * M;
   }
 };
+
+template <class T>
+void launch_epilogue(const ttt::LayerEpilogueArgs& a, int nc, dim3 grid, hipStream_t s) {
+  switch (nc) {
+    case 1: hipLaunchKernelGGL((ttt::ttt_layer_epilogue_kernel<T, 1>), grid, dim3(256), 0, s, a); break;
+    case 2: hipLaunchKernelGGL((ttt::ttt_layer_epilogue_kernel<T, 2>), grid, dim3(256), 0, s, a); break;
+    default: hipLaunchKernelGGL((ttt::ttt_layer_epilogue_kernel<T, 4>), grid, dim3(256), 0, s, a); break;
+  }
+}
 
 }  // namespace
 
@@ -421,6 +431,73 @@ int ttt_mlp_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
     case 96: return f32 ? launch_mlp_bwd<ttt::F32, 96>(a, s) : launch_mlp_bwd<ttt::BF16, 96>(a, s);
     default: return f32 ? launch_mlp_bwd<ttt::F32, 128>(a, s) : launch_mlp_bwd<ttt::BF16, 128>(a, s);
   }
+}
+
+int ttt_inner_inputs(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                     const void* lr_logits, const float* lr_bias, float base_lr, const float* token_idx,
+                     const float* learnable_token_idx, const float* rope_cos, const float* rope_sin,
+                     int pos_offset, int pos_wrap, void* xq_out, void* xk_out, void* xv_out, void* lr_out,
+                     float* token_eta_out, void* stream) {
+  if (!d) return fail(TTT_ERR_NULL, "ttt_inner_inputs: desc is NULL");
+  if (d->batch <= 0 || d->heads <= 0 || d->seq <= 0 || d->head_dim <= 0 || d->mini_batch <= 0)
+    return fail(TTT_ERR_SHAPE, "ttt_inner_inputs: batch, heads, seq, head_dim, mini_batch must be positive");
+  if (d->head_dim % 8 != 0)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_inner_inputs: head_dim %d is not a multiple of 8", d->head_dim);
+  if (d->io_dtype != TTT_F32 && d->io_dtype != TTT_BF16)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_inner_inputs: io_dtype %d", d->io_dtype);
+  if (!xq || !xk || !xv || !lr_logits || !lr_bias || !token_idx || !learnable_token_idx || !xq_out ||
+      !xk_out || !xv_out || !lr_out || !token_eta_out)
+    return fail(TTT_ERR_NULL, "ttt_inner_inputs: a required pointer is NULL");
+  if ((rope_cos == nullptr) != (rope_sin == nullptr))
+    return fail(TTT_ERR_NULL, "ttt_inner_inputs: rope_cos and rope_sin must both be given or both be NULL");
+  if (pos_offset < 0 || pos_wrap < 0) return fail(TTT_ERR_SHAPE, "ttt_inner_inputs: negative position");
+  if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(xq_out) || !aligned16(xk_out) ||
+      !aligned16(xv_out) || !aligned16(rope_cos) || !aligned16(rope_sin))
+    return fail(TTT_ERR_SHAPE, "ttt_inner_inputs: activation and table pointers must be 16-byte aligned");
+  ttt::InnerInputsArgs a;
+  a.xq = xq; a.xk = xk; a.xv = xv; a.lr_logits = lr_logits; a.lr_bias = lr_bias; a.token_idx = token_idx;
+  a.learnable_token_idx = learnable_token_idx; a.cos = rope_cos; a.sin = rope_sin;
+  a.xq_out = xq_out; a.xk_out = xk_out; a.xv_out = xv_out; a.lr_out = lr_out; a.token_eta_out = token_eta_out;
+  a.lr_scale = base_lr / (float)d->head_dim;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.D = d->head_dim; a.K = d->mini_batch;
+  a.pos_offset = pos_offset; a.pos_wrap = pos_wrap;
+  const size_t total = (size_t)a.B * a.seq * a.H * (a.D / 8);
+  const dim3 grid((unsigned)((total + 255) / 256));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (d->io_dtype == TTT_F32)
+    hipLaunchKernelGGL(ttt::ttt_inner_inputs_kernel<ttt::F32>, grid, dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL(ttt::ttt_inner_inputs_kernel<ttt::BF16>, grid, dim3(256), 0, s, a);
+  return hip_status(hipGetLastError(), "ttt_inner_inputs launch");
+}
+
+int ttt_layer_epilogue(const ttt_desc* d, const void* inner_out, const float* post_norm_weight,
+                       const float* post_norm_bias, float eps, const void* gate, void* out, void* stream) {
+  if (!d) return fail(TTT_ERR_NULL, "ttt_layer_epilogue: desc is NULL");
+  if (d->batch <= 0 || d->heads <= 0 || d->seq <= 0 || d->head_dim <= 0)
+    return fail(TTT_ERR_SHAPE, "ttt_layer_epilogue: batch, heads, seq, head_dim must be positive");
+  const int hidden = d->heads * d->head_dim;
+  if (d->head_dim % 8 != 0 || hidden > 2048)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_layer_epilogue: head_dim %d (multiple of 8) / hidden %d (<= 2048)",
+                d->head_dim, hidden);
+  if (d->io_dtype != TTT_F32 && d->io_dtype != TTT_BF16)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_layer_epilogue: io_dtype %d", d->io_dtype);
+  if (!inner_out || !post_norm_weight || !post_norm_bias || !out)
+    return fail(TTT_ERR_NULL, "ttt_layer_epilogue: a required pointer is NULL");
+  if (!aligned16(inner_out) || !aligned16(out) || !aligned16(gate) || !aligned16(post_norm_weight) ||
+      !aligned16(post_norm_bias))
+    return fail(TTT_ERR_SHAPE, "ttt_layer_epilogue: pointers must be 16-byte aligned");
+  ttt::LayerEpilogueArgs a;
+  a.inner_out = inner_out; a.gamma = post_norm_weight; a.beta = post_norm_bias; a.gate = gate; a.out = out;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.D = d->head_dim; a.eps = eps;
+  const int nch = hidden / 8, nc = nch <= 64 ? 1 : nch <= 128 ? 2 : 4;
+  const dim3 grid((unsigned)(((size_t)a.B * a.seq + 3) / 4));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (d->io_dtype == TTT_F32)
+    launch_epilogue<ttt::F32>(a, nc, grid, s);
+  else
+    launch_epilogue<ttt::BF16>(a, nc, grid, s);
+  return hip_status(hipGetLastError(), "ttt_layer_epilogue launch");
 }
 
 }  // extern "C"

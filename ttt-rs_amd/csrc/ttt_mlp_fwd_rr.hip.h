@@ -57,24 +57,6 @@ struct MlpRrLds {
   static_assert(TILE % 1024 == 0 && P1 % 16 == 0, "input tiles are staged in 1 KiB wave blocks");
 };
 
-// y = gelu_tanh(x), dy = its derivative.  With r = 1 / (1 + exp(2u)), u = c (x + a x^3):
-// (1 + tanh u) / 2 = 1 - r and 1 - tanh^2 u = 4 r (1 - r).
-__device__ __forceinline__ void gelu_fast_pair(float x, float& y, float& dy) {
-  const float c2 = 2.f * 0.7978845608f;
-  const float x2 = x * x;
-  const float u = x * __builtin_fmaf(0.044715f, x2, 1.f);
-  const float e = __builtin_amdgcn_exp2f(u * (c2 * 1.4426950409f));
-  const float r = __builtin_amdgcn_rcpf(1.f + e);
-  const float hp = 1.f - r;
-  y = x * hp;
-  dy = hp * __builtin_fmaf(c2 * __builtin_fmaf(3.f * 0.044715f, x2, 1.f), x * r, 1.f);
-}
-__device__ __forceinline__ float gelu_fast(float x) {
-  const float u = x * __builtin_fmaf(0.044715f, x * x, 1.f);
-  const float e = __builtin_amdgcn_exp2f(u * (2.f * 0.7978845608f * 1.4426950409f));
-  return x - x * __builtin_amdgcn_rcpf(1.f + e);
-}
-
 // Makes the compiler forget what it knows about v.  The bf16 operand copies of the W2 tiles are
 // needed at three places of a mini-batch; without this the compiler keeps the converted copies
 // (36 VGPRs at d = 96) alive across the barriers and spills state tiles to scratch instead.

@@ -477,3 +477,70 @@ class FusedTileMulti:
         if len(r) > self.config.ttt.mini_batch_size or len(r) == 0:
             raise _lib.TttError(_lib.TTT_ERR_SHAPE, "range longer than mini_batch_size")
         return self._launch(state, inputs.slice_seq(r), len(r))
+
+
+# --------------------------------------------------------------------------- either side of the inner loop
+def rope_cos_sin(seq_len: int, offset: int, wrap: Optional[int], head_dim: int, device, base: float = 10000.0):
+    """RotaryEmbeddingConfig::init + RotaryEmbedding::get_cos_sin (rust/core/src/util.rs:266-322) in f32:
+    returns (cos, sin) [seq_len, head_dim/2] (the reference repeats this half twice)."""
+    half = head_dim // 2
+    inv_freq = torch.tensor([1.0 / base ** ((2 * i) / head_dim) for i in range(half)], dtype=torch.float32)
+    pos = torch.arange(seq_len, dtype=torch.float32) + float(offset)
+    if wrap is not None:
+        pos = torch.remainder(pos, float(wrap))
+    freqs = pos[:, None] * inv_freq[None, :]
+    return freqs.cos().to(device), freqs.sin().to(device)
+
+
+def inner_loop_inputs_raw(xq, xk, xv, lr_logits, lr_bias, base_lr: float, token_idx, learnable_token_idx,
+                          mini_batch: int, rope=None, pos_offset: int = 0, pos_wrap: int = 0) -> TTTInputsInner:
+    """One call of ttt_inner_inputs: TTT::get_inner_loop_inputs after the projections
+    (rust/layer/src/ttt.rs:147-194, 205-227, 247-268).  xq,xk,xv [B,seq,H,d]; lr_logits [B,seq,H];
+    rope = (cos, sin) tables [npos, d/2] f32 or None."""
+    B, seq, H, d = xq.shape
+    io = xq.dtype
+    xq = _need(xq, (B, seq, H, d), io, "xq")
+    xk = _need(xk, (B, seq, H, d), io, "xk")
+    xv = _need(xv, (B, seq, H, d), io, "xv")
+    lg = _need(lr_logits, (B, seq, H), io, "lr_logits")
+    lb = _need(lr_bias.reshape(-1), (H,), torch.float32, "lr_bias")
+    ti = _need(token_idx, (mini_batch,), torch.float32, "token_idx")
+    lti = _need(learnable_token_idx, (mini_batch,), torch.float32, "learnable_token_idx")
+    null = C.c_void_p(None)
+    cos = sin = None
+    if rope is not None:
+        cos = _need(rope[0], (rope[0].shape[0], d // 2), torch.float32, "rope cos")
+        sin = _need(rope[1], (rope[0].shape[0], d // 2), torch.float32, "rope sin")
+        last = (pos_offset + seq - 1) if pos_wrap == 0 else min(pos_wrap - 1, pos_offset + seq - 1)
+        if last >= cos.shape[0]:
+            raise _lib.TttError(_lib.TTT_ERR_SHAPE, "rope table shorter than the positions used")
+    dev = xq.device
+    q, k, v = (torch.empty((B, H, seq, d), dtype=io, device=dev) for _ in range(3))
+    lr = torch.empty((B, H, seq), dtype=io, device=dev)
+    te = torch.empty(seq, dtype=torch.float32, device=dev)
+    desc = TttDesc(B, H, seq, d, mini_batch, 0.0, 1, _io_dtype(xq), 0, 0)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_inner_inputs(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(lg), _ptr(lb),
+                                     C.c_float(base_lr), _ptr(ti), _ptr(lti),
+                                     null if cos is None else _ptr(cos), null if sin is None else _ptr(sin),
+                                     pos_offset, pos_wrap, _ptr(q), _ptr(k), _ptr(v), _ptr(lr), _ptr(te), stream))
+    return TTTInputsInner(Qkv(q, k, v), te, lr)
+
+
+def layer_epilogue_raw(inner_out, post_norm_weight, post_norm_bias, gate=None, eps: float = 1e-6):
+    """One call of ttt_layer_epilogue: head merge + post_norm LayerNorm (+ tanh-GELU gate) of
+    TTT::forward (rust/layer/src/ttt.rs:285-297).  inner_out [B,H,seq,d] -> [B,seq,H*d]."""
+    B, H, seq, d = inner_out.shape
+    io = inner_out.dtype
+    x = _need(inner_out, (B, H, seq, d), io, "inner_out")
+    g = _need(post_norm_weight, (H * d,), torch.float32, "post_norm_weight")
+    b = _need(post_norm_bias, (H * d,), torch.float32, "post_norm_bias")
+    gt = None if gate is None else _need(gate, (B, seq, H * d), io, "gate")
+    out = torch.empty((B, seq, H * d), dtype=io, device=x.device)
+    desc = TttDesc(B, H, seq, d, 1, eps, 1, _io_dtype(x), 0, 0)
+    stream = C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+    with torch.cuda.device(x.device):
+        check(lib().ttt_layer_epilogue(C.byref(desc), _ptr(x), _ptr(g), _ptr(b), C.c_float(eps),
+                                       C.c_void_p(None) if gt is None else _ptr(gt), _ptr(out), stream))
+    return out
