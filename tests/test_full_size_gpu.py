@@ -147,7 +147,7 @@ def test_config4_layers_d128_seq8192(P):
     ro, rW, rb = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
                                     n["gamma"], n["beta"], K=K)
     assert_close(out[bs][:, hs], ro, TOL[torch.bfloat16], "linear out")
-    assert_close(W[bs][:, hs], rW, 1e-4, "linear W")
+    assert_close(W[bs][:, hs], rW, TOL[torch.bfloat16], "linear W")  # bf16 operands, f32 state
     del dv, out, W, b
     c = P.synthetic.baseline_inputs(46, B, H, seq, d, K, io_dtype=torch.bfloat16, mlp=True)
     dv = dev(c)

@@ -104,6 +104,23 @@ int launch_linear_fwd(const ttt::LinearFwdArgs& a, hipStream_t s) {
   return launch_linear_fwd_nw<T, D, 1>(a, s);
 }
 
+// ---- TTT-Linear forward, head_dim 96/128: the same register-resident skewed kernel with two
+// feature tiles per wave (3 waves at d = 96, 4 at d = 128; one tile per wave was measured slower for
+// every shape tried: twice the waves exchange twice the row sums).  The LDS-tile kernel stays
+// available through TTT_LINEAR_FWD_KERNEL=lds.
+template <class T, int D>
+int launch_linear_fwd_wide(const ttt::LinearFwdArgs& a, hipStream_t s) {
+  constexpr int NW = D / 32;
+  constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
+  constexpr int PF = f32 ? 1 : 2;  // f32 fragments are twice as large: prefetch one mini-batch ahead
+  const dim3 grid((unsigned)(a.B * a.H)), block(64 * NW);
+  if (a.K == 16)
+    hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, true>), grid, block, 0, s, a);
+  else
+    hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, false>), grid, block, 0, s, a);
+  return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+}
+
 template <class K>
 int opt_in_lds(K kern, size_t bytes) {
   // more than the default 64 KiB of LDS per workgroup has to be requested (per device)
@@ -245,14 +262,22 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.state_per_batch = d->state_per_batch ? 1 : 0;
   a.eps = d->eps;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // head_dim 32/64: register-resident single-wave kernel; 96/128: LDS-resident kernel
+  // register-resident kernels for every head_dim; the LDS-tile kernel (96/128) only on request
   const bool f32 = d->io_dtype == TTT_F32;
   switch (d->head_dim) {
     case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, s) : launch_linear_fwd<ttt::BF16, 32>(a, s);
     case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, s) : launch_linear_fwd<ttt::BF16, 64>(a, s);
-    case 96: return f32 ? launch_linear_fwd_lds<ttt::F32, 96>(a, s) : launch_linear_fwd_lds<ttt::BF16, 96>(a, s);
-    default: return f32 ? launch_linear_fwd_lds<ttt::F32, 128>(a, s) : launch_linear_fwd_lds<ttt::BF16, 128>(a, s);
+    default: break;
   }
+  const char* force = getenv("TTT_LINEAR_FWD_KERNEL");
+  if (force && strcmp(force, "lds") == 0) {
+    if (d->head_dim == 96)
+      return f32 ? launch_linear_fwd_lds<ttt::F32, 96>(a, s) : launch_linear_fwd_lds<ttt::BF16, 96>(a, s);
+    return f32 ? launch_linear_fwd_lds<ttt::F32, 128>(a, s) : launch_linear_fwd_lds<ttt::BF16, 128>(a, s);
+  }
+  if (d->head_dim == 96)
+    return f32 ? launch_linear_fwd_wide<ttt::F32, 96>(a, s) : launch_linear_fwd_wide<ttt::BF16, 96>(a, s);
+  return f32 ? launch_linear_fwd_wide<ttt::F32, 128>(a, s) : launch_linear_fwd_wide<ttt::BF16, 128>(a, s);
 }
 
 int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
