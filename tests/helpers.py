@@ -13,7 +13,7 @@ def to_np(t):
     return np.asarray(t, dtype=np.float64)
 
 
-def assert_close(got, ref, tol, name=""):
+def assert_close(got, ref, tol, name="", min_frac=0.999):
     got, ref = to_np(got), to_np(ref)
     assert got.shape == ref.shape, (name, got.shape, ref.shape)
     assert np.isfinite(got).all(), f"{name}: non-finite values"
@@ -23,7 +23,7 @@ def assert_close(got, ref, tol, name=""):
     assert rel <= tol, f"{name}: max-norm relative error {rel:.3e} > {tol:g}"
     ok = err <= tol * np.abs(ref) + 0.1 * tol * scale
     frac = ok.mean()
-    assert frac >= 0.999, f"{name}: only {frac:.5f} of elements within elementwise bound"
+    assert frac >= min_frac, f"{name}: only {frac:.5f} of elements within elementwise bound"
     return rel
 
 

@@ -41,12 +41,17 @@ def test_mlp_fwd_matches_oracle(P, B, H, d, K, N, style, dtype):
     n = np_inputs(c)
     ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
                           n["lr"], n["gamma"], n["beta"], K=K)
-    # bf16 I/O with d <= 96 runs the register-resident kernel, whose products take bf16 operands
-    # (f32 accumulation and state): everything is held to the bf16 bar.  The other cases compute in
-    # f32 throughout and only round the stored output.
-    f32_products = dtype == torch.float32 or d > 96
+    # bf16 I/O runs the register-resident kernels (one CU for d <= 96, a pair of CUs for d = 128),
+    # whose products take bf16 operands (f32 accumulation and state): everything is held to the bf16
+    # bar.  f32 I/O computes in f32 throughout.
+    f32_products = dtype == torch.float32
+    # With bf16 products the biases, which start at zero in the baseline style and are pure sums of
+    # rounded update rows, carry a tail just above the elementwise floor (0.2 % of the largest entry):
+    # for them the share of elements inside the elementwise bound is asked to be 99 %, not 99.9 %.
     for name, g, r in zip(("out", "W1", "b1", "W2", "b2"), got, ref):
-        assert_close(g, r, 1e-4 if (f32_products and name != "out") else TOL[dtype], name)
+        loose = not f32_products and name in ("b1", "b2")
+        assert_close(g, r, 1e-4 if (f32_products and name != "out") else TOL[dtype], name,
+                     min_frac=0.99 if loose else 0.999)
 
 
 def test_mlp_fwd_bf16_lds_kernel_keeps_f32_products(P, monkeypatch):

@@ -16,6 +16,7 @@
 #include "ttt_linear_fwd_mw.hip.h"
 #include "ttt_linear_fwd_sk.hip.h"
 #include "ttt_mlp_bwd.hip.h"
+#include "ttt_mlp_fwd_cl2.hip.h"
 #include "ttt_mlp_fwd_rr.hip.h"
 
 namespace {
@@ -158,6 +159,19 @@ int launch_mlp_fwd_rr(const ttt::MlpFwdArgs& a, hipStream_t s) {
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_mlp_fwd (register-resident kernel) launch");
+}
+
+// head_dim 128, bf16 I/O: a pair of workgroups per (batch, head); the exchange flags live in W2_out,
+// which is zeroed first (a fill kernel, not a memset node)
+int launch_mlp_fwd_cl2(const ttt::MlpFwdArgs& a, hipStream_t s) {
+  auto kern = ttt::ttt_mlp_fwd_cl2_kernel<ttt::BF16, 128>;
+  constexpr size_t bytes = ttt::MlpCl2Lds<128, 2>::BYTES;
+  int rc = opt_in_lds(kern, bytes);
+  if (rc != TTT_OK) return rc;
+  const size_t units = (size_t)a.B * a.H, n = units * 128 * 512;
+  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a.W2, n);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(((units + 7) / 8) * 16)), dim3(512), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_mlp_fwd (two-CU kernel) launch");
 }
 
 template <class T, int D>
@@ -367,6 +381,7 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   // bf16 I/O, d <= 96: the state fits the register file of one CU.  TTT_MLP_FWD_KERNEL=lds forces
   // the LDS-tile kernel (f32 products, state in global memory) that the other cases use.
   const char* force = getenv("TTT_MLP_FWD_KERNEL");
+  if (!f32 && d->head_dim == 128 && !(force && strcmp(force, "lds") == 0)) return launch_mlp_fwd_cl2(a, s);
   if (!f32 && d->head_dim <= 96 && !(force && strcmp(force, "lds") == 0)) {
     switch (d->head_dim) {
       case 32: return launch_mlp_fwd_rr<ttt::BF16, 32>(a, s);
