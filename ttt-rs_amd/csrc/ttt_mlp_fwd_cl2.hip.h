@@ -61,20 +61,37 @@ __device__ __forceinline__ void send_tagged(unsigned long long* slot, f32x4 v, u
     __hip_atomic_store(slot + r, ((unsigned long long)tag << 32) | __float_as_uint(v[r]), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
 }
-// Polls until all four words carry `tag`.  The wait is bounded; after one wait has run out (`alive`
-// cleared) no further wait is attempted: a lost partner costs one time-out per wave, not one per
-// mini-batch, and ends in wrong numbers, never in a hang.
-__device__ __forceinline__ f32x4 recv_tagged(const unsigned long long* slot, unsigned tag, bool& alive) {
-  unsigned long long wd[4];
+// Receives N tiles at once: polls until the four words of every slot carry that slot's tag, all
+// loads of a round in flight together (one memory round trip per round, not one per tile).  The wait
+// is bounded; after one wait has run out (`alive` cleared) no further wait is attempted: a lost
+// partner costs one time-out per wave, not one per mini-batch, and ends in wrong numbers, never in a hang.
+template <int N>
+__device__ __forceinline__ void recv_tagged(const unsigned long long* const (&slot)[N], const unsigned (&tag)[N],
+                                            f32x4 (&out)[N], bool& alive) {
+  unsigned long long wd[N][4];
   int it = 0;
+  // light first stage: one lane watches the word stored last of the first slot, so that sixteen
+  // waiting waves do not flood the memory system with polls; the full check then usually passes at once
+  if (alive && (threadIdx.x & 63) == 0) {
+    const unsigned long long* last = slot[0] + 4 * 63 + 3;  // lane 63's fourth word (slot[] is lane 0's here)
+    while ((unsigned)(__hip_atomic_load(last, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) != tag[0]) {
+      if (++it >= (1 << 21)) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  it = 0;
   while (true) {
     bool ok = true;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      wd[r] = __hip_atomic_load(slot + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      ok = ok && (unsigned)(wd[r] >> 32) == tag;
-    }
-    // the whole wave leaves together: its lanes poll neighbouring words of the same tile
+    for (int n = 0; n < N; ++n)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        wd[n][r] = __hip_atomic_load(slot[n] + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ok = ok && (unsigned)(wd[n][r] >> 32) == tag[n];
+    // the whole wave leaves together: its lanes poll neighbouring words of the same tiles
     if (__all(ok) || !alive) break;
     if (++it >= (1 << 21)) {
       alive = false;
@@ -82,8 +99,10 @@ __device__ __forceinline__ f32x4 recv_tagged(const unsigned long long* slot, uns
     }
     __builtin_amdgcn_s_sleep(1);
   }
-  return f32x4{__uint_as_float((unsigned)wd[0]), __uint_as_float((unsigned)wd[1]),
-               __uint_as_float((unsigned)wd[2]), __uint_as_float((unsigned)wd[3])};
+#pragma unroll
+  for (int n = 0; n < N; ++n)
+    out[n] = f32x4{__uint_as_float((unsigned)wd[n][0]), __uint_as_float((unsigned)wd[n][1]),
+                   __uint_as_float((unsigned)wd[n][2]), __uint_as_float((unsigned)wd[n][3])};
 }
 
 #define RELANE() asm volatile("" : "+v"(lane))
@@ -223,36 +242,38 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
   auto send_tile = [&](int par_, int idx, f32x4 v, unsigned tag) {
     send_tagged(reinterpret_cast<unsigned long long*>(xout + par_ * L::XSLOT + idx * L::XTILE) + 4 * lane, v, tag);
   };
-  auto recv_tile = [&](int par_, int idx, unsigned tag) -> f32x4 {
-    return recv_tagged(reinterpret_cast<const unsigned long long*>(xin + par_ * L::XSLOT + idx * L::XTILE) + 4 * lane,
-                       tag, alive);
+  auto slot_in = [&](int par_, int idx) -> const unsigned long long* {
+    return reinterpret_cast<const unsigned long long*>(xin + par_ * L::XSLOT + idx * L::XTILE) + 4 * lane;
   };
 
   // ---- output path (previous mini-batch), wave w owns d-feature tile w.  CU 1 reduces its half and
   // sends it; CU 0 adds both halves, applies the causal correction and finishes the LayerNorm.
   f32x4 zb = {0.f, 0.f, 0.f, 0.f};
   frag qo_pend = IO::zero();  // xq tile of the mini-batch whose output is pending
-  auto output_reduce = [&](int st_out) {  // st_out: the mini-batch the output belongs to
-    const int xp = st_out & 1;
-    const unsigned tag = (unsigned)st_out + 1;
-    f32x4 at = {0.f, 0.f, 0.f, 0.f};
+  f32x4 at2 = {0.f, 0.f, 0.f, 0.f};
+  // local half of the pending output: this CU's split-k sums; CU 1 sends them off at once
+  auto output_local = [&](int st_out) {  // st_out: the mini-batch the output belongs to
+    at2 = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ww = 0; ww < NW; ++ww) at += PA[ww * 64 + lane];
-    pin(at);
+    for (int ww = 0; ww < NW; ++ww) at2 += PA[ww * 64 + lane];
+    pin(at2);
     zb = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ww = 0; ww < NW; ++ww) zb += IO::to_f32(P2[(ww * NT + w) * 64 + lane]);
     pin(zb);
     if (cu == 1) {
-      send_tile(xp, NT + w, zb, tag);
-      if (w == 0) send_tile(xp, 2 * NT, at, tag);
-      return;
+      send_tile(st_out & 1, NT + w, zb, (unsigned)st_out + 1);
+      if (w == 0) send_tile(st_out & 1, 2 * NT, at2, (unsigned)st_out + 1);
     }
-    zb += recv_tile(xp, NT + w, tag);
-    at += recv_tile(xp, 2 * NT, tag);
+  };
+  // CU 0: add CU 1's half, causal correction, row moments
+  auto output_finish = [&](f32x4 zb_part, f32x4 at_part) {
+    if (cu == 1) return;
+    zb += zb_part;
+    at2 += at_part;
     f32x4 m;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + at[r]) : 0.f;
+    for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + at2[r]) : 0.f;
     IO::mma(zb, GD[w * 64 + lane], IO::to_frag(m));  // GD still holds the previous mini-batch's G2
     float s0 = 0.f, s1 = 0.f;
 #pragma unroll
@@ -331,11 +352,11 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
     }
     lds_barrier();  // ---- B1
     RELANE();
-    fetch(st + 1);
 
     // ================= phase B: this CU's half of Z2 tile w, exchange with the partner, row moments;
     //                          then the output path of the previous mini-batch
-    f32x4 z, bq;
+    f32x4 z, bq, zq[HT];
+    frag Mf;
     {
       f32x4 zloc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -344,10 +365,55 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
         if ((ww & 3) == 3) pin(zloc);
       }
       send_tile(par, w, zloc, (unsigned)st + 1);
+      // everything that does not need the partner goes between the send and the wait
+      if (st > 0) output_local(st - 1);
+      // (XQ W1 + b1)^T for this wave's hidden units and the causal matrix M1: independent of the partner
+#pragma unroll
+      for (int j = 0; j < HT; ++j)
+#pragma unroll
+        for (int I = 0; I < NT; ++I) forget(W1c[I][j]);
+#pragma unroll
+      for (int j = 0; j < HT; ++j) zq[j] = *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g);
+      {
+        f32x4 At = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < NT / 2; ++q) {
+          frag k0, k1, q0, q1;
+          IO::load8(row(buf, 1) + 32 * q + 8 * g, true, k0, k1);
+          IO::load8(row(buf, 0) + 32 * q + 8 * g, true, q0, q1);
+#pragma unroll
+          for (int j = 0; j < HT; ++j)
+            IO::mma2(zq[j], IO::to_frag(W1c[2 * q][j]), IO::to_frag(W1c[2 * q + 1][j]), q0, q1);
+          IO::mma2(At, k0, k1, q0, q1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        f32x4 m;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + At[r]) : 0.f;
+        Mf = IO::to_frag(m);
+      }
       const frag ko = load4<T>(row(buf, 1) + own), vo = load4<T>(row(buf, 2) + own);
       const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + own), bet = *reinterpret_cast<const f32x4*>(BET + own);
       bq = gam * (bet - (IO::to_f32(vo) - IO::to_f32(ko)));
-      const f32x4 zpart = recv_tile(par, w, (unsigned)st + 1);
+      // one wait for everything the partner sends this mini-batch: its half of Z2 tile w and (to CU 0)
+      // its half of the pending output
+      f32x4 zpart, zb_part = {0.f, 0.f, 0.f, 0.f}, at_part = zb_part;
+      if (cu == 0 && st > 0) {
+        const unsigned long long* const sl[3] = {slot_in(par, w), slot_in(par ^ 1, NT + w), slot_in(par ^ 1, 2 * NT)};
+        const unsigned tg[3] = {(unsigned)st + 1, (unsigned)st, (unsigned)st};
+        f32x4 rv[3];
+        recv_tagged<3>(sl, tg, rv, alive);
+        zpart = rv[0];
+        zb_part = rv[1];
+        at_part = rv[2];
+      } else {
+        const unsigned long long* const sl[1] = {slot_in(par, w)};
+        const unsigned tg[1] = {(unsigned)st + 1};
+        f32x4 rv[1];
+        recv_tagged<1>(sl, tg, rv, alive);
+        zpart = rv[0];
+      }
+      fetch(st + 1);
       z = b2T + (cu == 0 ? zloc + zpart : zpart + zloc);  // same order of the halves on both CUs
       float S[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       const f32x4 az = gam * gam * z;
@@ -361,8 +427,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
         S[5] += bq[r] * z[r];
       }
       publish(S);
+      if (st > 0) output_finish(zb_part, at_part);
     }
-    if (st > 0) output_reduce(st - 1);
     lds_barrier();  // ---- B2
     RELANE();
 
@@ -414,31 +480,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int j = 0; j < HT; ++j)
-#pragma unroll
-      for (int I = 0; I < NT; ++I) forget(W1c[I][j]);
-    f32x4 zq[HT], At = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < HT; ++j) zq[j] = *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g);
-#pragma unroll
-    for (int q = 0; q < NT / 2; ++q) {
-      frag k0, k1, q0, q1;
-      IO::load8(row(buf, 1) + 32 * q + 8 * g, true, k0, k1);
-      IO::load8(row(buf, 0) + 32 * q + 8 * g, true, q0, q1);
-#pragma unroll
-      for (int j = 0; j < HT; ++j)
-        IO::mma2(zq[j], IO::to_frag(W1c[2 * q][j]), IO::to_frag(W1c[2 * q + 1][j]), q0, q1);
-      IO::mma2(At, k0, k1, q0, q1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    {
-      f32x4 m;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + At[r]) : 0.f;
-      const frag Mf = IO::to_frag(m);
-#pragma unroll
-      for (int j = 0; j < HT; ++j) IO::mma(zq[j], G1d[j], Mf);
-    }
+    for (int j = 0; j < HT; ++j) IO::mma(zq[j], G1d[j], Mf);
     frag xbf[HT];
 #pragma unroll
     for (int j = 0; j < HT; ++j) {
@@ -497,7 +539,15 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
 
   // ---- the last mini-batch's output
   lds_barrier();
-  output_reduce(a.n_stages - 1);
+  output_local(a.n_stages - 1);
+  if (cu == 0) {
+    const int lp = (a.n_stages - 1) & 1;
+    const unsigned long long* const sl[2] = {slot_in(lp, NT + w), slot_in(lp, 2 * NT)};
+    const unsigned tg[2] = {(unsigned)a.n_stages, (unsigned)a.n_stages};
+    f32x4 rv[2];
+    recv_tagged<2>(sl, tg, rv, alive);
+    output_finish(rv[0], rv[1]);
+  }
   lds_barrier();
   output_emit(a.n_stages - 1);
 
