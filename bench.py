@@ -266,10 +266,10 @@ def main():
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     else:
         flops = th * (6 * (6 * d * d + 4 * K * d) + 2 * (56 * d * d + 20 * K * d))
-        out["dtype"] = "f32"
+        out["dtype"] = "bf16"   # register-resident kernels: bf16 MFMA operands, f32 accumulation and state
         out["config"]["inner_model"] = "6 x TTT-Linear + 2 x TTT-MLP"
-        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
-                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
+        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": BF16_MFMA_PEAK_TF,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / BF16_MFMA_PEAK_TF, "traffic": None,
                            "kernel": "8 layer launches + input adds (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     tpath = os.path.join(ROOT, "profiles", "traffic.json")

@@ -64,7 +64,7 @@ __device__ __forceinline__ void send_tagged(unsigned long long* slot, f32x4 v, u
 // Receives N tiles at once: polls until the four words of every slot carry that slot's tag, all
 // loads of a round in flight together (one memory round trip per round, not one per tile).  The wait
 // is bounded; after one wait has run out (`alive` cleared) no further wait is attempted: a lost
-// partner costs one time-out per wave, not one per mini-batch, and ends in wrong numbers, never in a hang.
+// partner costs one time-out per wave, not one per mini-batch, and ends in NaNs in b1_out, never in a hang.
 template <int N>
 __device__ __forceinline__ void recv_tagged(const unsigned long long* const (&slot)[N], const unsigned (&tag)[N],
                                             f32x4 (&out)[N], bool& alive) {
@@ -567,7 +567,11 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
           W1[(size_t)feat(I, 4 * g + r) * F + hb + c] = W1c[I][j][r];
           W2[(size_t)(hb + 4 * g + r) * D + feat(I, c)] = W2c[j][I][r];
         }
-      if (c == 0) store4<F32>(a.b1 + bh * F + hb + 4 * g, *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g));
+      // a wait that ran out is made visible: this wave's slice of b1 becomes NaN (the partner, should it
+      // still arrive, writes only its own half of the state and cannot cover it up)
+      const float poison = alive ? 0.f : __builtin_nanf("");
+      if (c == 0)
+        store4<F32>(a.b1 + bh * F + hb + 4 * g, *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g) + poison);
     }
     if (cu == 0 && c == 0) store4<F32>(a.b2 + bh * D + own, b2T);
   }
