@@ -53,7 +53,11 @@ NAMES = [("grad_xq", "d_xq"), ("grad_xk", "d_xk"), ("grad_xv", "d_xv"), ("grad_w
 
 def compare(g, r, tol):
     for gn, rn in NAMES:
-        assert_close(g[gn], r[rn], tol, gn)
+        # bf16 I/O, products with bf16 operands: in a tensor of fewer than 1000 elements a single element
+        # outside the elementwise band is already more than 0.1 %, so one such element is let through there
+        n = np.asarray(r[rn]).size
+        min_frac = 0.999 if tol < 1e-3 else min(0.999, 1.0 - 1.5 / n)
+        assert_close(g[gn], r[rn], tol, gn, min_frac=min_frac)
 
 
 # (B, H, d, K, stages, checkpoint_interval)
@@ -84,15 +88,28 @@ def test_bwd_matches_oracle_baseline_style_inputs(P, dtype):
     compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])
 
 
-def test_bwd_with_upstream_state_gradients(P):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("d,K", [(32, 8), (64, 16)])
+def test_bwd_with_upstream_state_gradients(P, d, K, dtype):
     """d_W_out / d_b_out (the reference assumes zero, launch.rs:188-194; the ABI accepts them)."""
-    print("case bwd state grads", flush=True)
-    B, H, d, K, N = 2, 2, 32, 8, 3
-    c = P.synthetic.reference_test_inputs(77, B, H, N * K, d, K)
+    print(f"case bwd state grads d{d} K{K} {dtype}", flush=True)
+    B, H, N = 2, 2, 3
+    c = P.synthetic.reference_test_inputs(77, B, H, N * K, d, K, io_dtype=dtype)
     g = torch.Generator().manual_seed(6)
-    dO = torch.randn(B, H, N * K, d, generator=g)
+    dO = torch.randn(B, H, N * K, d, generator=g).to(dtype)
     sg = (torch.randn(B, H, d, d, generator=g), torch.randn(B, H, d, generator=g))
-    compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), 1e-4)
+    compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), TOL[dtype])
+
+
+def test_bwd_bf16_lds_kernel_on_request(P, monkeypatch):
+    """The LDS-tile kernel (f32 products) stays selectable for bf16 I/O."""
+    print("case bwd bf16 lds kernel", flush=True)
+    monkeypatch.setenv("TTT_LINEAR_BWD_KERNEL", "lds")
+    B, H, d, K, N = 1, 2, 64, 16, 3
+    c = P.synthetic.reference_test_inputs(79, B, H, N * K, d, K, io_dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(8)
+    dO = torch.randn(B, H, N * K, d, generator=g).to(torch.bfloat16)
+    compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[torch.bfloat16])
 
 
 def test_bwd_is_linear_in_upstream_gradient(P):

@@ -12,6 +12,7 @@
 #include "ttt_engine_fwd.hip.h"
 #include "ttt_layer_io.hip.h"
 #include "ttt_linear_bwd.hip.h"
+#include "ttt_linear_bwd_rr.hip.h"
 #include "ttt_linear_fwd.hip.h"
 #include "ttt_linear_fwd_mw.hip.h"
 #include "ttt_linear_fwd_sk.hip.h"
@@ -184,6 +185,17 @@ int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s)
   return hip_status(hipGetLastError(), "ttt_linear_bwd launch");
 }
 
+// bf16 I/O, one checkpoint per mini-batch: one wave per (batch, head), state gradient in registers
+template <int D>
+int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
+  auto kern = ttt::ttt_linear_bwd_rr_kernel<ttt::BF16, D>;
+  constexpr size_t bytes = ttt::LinBwdRrLds<D>::BYTES;
+  int rc = opt_in_lds(kern, bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_linear_bwd (register-resident kernel) launch");
+}
+
 template <class T, int D>
 int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
   auto kern = ttt::ttt_mlp_bwd_kernel<T, D>;
@@ -339,6 +351,14 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   if (d->io_dtype == TTT_F32) {
     if (d->head_dim == 64) return launch_linear_bwd<ttt::F32, 64>(a, grid, s);
     return launch_linear_bwd<ttt::F32, 32>(a, grid, s);
+  }
+  const char* ksel = std::getenv("TTT_LINEAR_BWD_KERNEL");
+  if (a.ckpt_interval == 1 && !(ksel && std::strcmp(ksel, "lds") == 0)) {
+    if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(d_out) || !aligned16(d_xq) ||
+        !aligned16(d_xk) || !aligned16(d_xv) || !aligned16(W_ckpt) || !aligned16(b_ckpt) || (a.seq_stride * d->head_dim) % 8 != 0)
+      return fail(TTT_ERR_SHAPE, "ttt_linear_bwd: tensors must be 16-byte aligned");
+    if (d->head_dim == 64) return launch_linear_bwd_rr<64>(a, grid, s);
+    return launch_linear_bwd_rr<32>(a, grid, s);
   }
   if (d->head_dim == 64) return launch_linear_bwd<ttt::BF16, 64>(a, grid, s);
   return launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
