@@ -27,6 +27,15 @@
 
 namespace ttt {
 
+// Sum over the 16 lanes of a row, in every lane: four rotations inside the row on the DPP path.
+__device__ __forceinline__ float row16_sum_dpp(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));  // row_ror:8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));  // row_ror:4
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));  // row_ror:2
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));  // row_ror:1
+  return v;
+}
+
 template <int D>
 struct LinBwdRrLds {
   static constexpr int NT = D / 16;
@@ -88,6 +97,13 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
   float pre_lrc = 0.f;
   f32x4 pre_lrs = {0.f, 0.f, 0.f, 0.f};
   auto fetch = [&](int stage) {
+    // the few register loads first: the copies to LDS must be the youngest loads of the batch (see the
+    // counted wait at the bottom of the loop)
+    const elem* lrp = static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K;
+    pre_lrc = (c < K) ? IO::load1(lrp + c) : 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) pre_lrs[r] = (4 * g + r < K) ? IO::load1(lrp + 4 * g + r) : 0.f;
+    __builtin_amdgcn_sched_barrier(0);
     unsigned char* dst = smem + (stage & 1) * L::STAGE;
     const size_t ci = bh * (size_t)a.n_ckpt + stage;
     const float* Wg = a.W_ckpt + ci * D * D;
@@ -112,10 +128,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
         dma(static_cast<const elem*>(a.d_out) + tok + 32 * q, L::X + (3 * NQ + q) * 1024);
       }
     }
-    const elem* lrp = static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K;
-    pre_lrc = (c < K) ? IO::load1(lrp + c) : 0.f;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) pre_lrs[r] = (4 * g + r < K) ? IO::load1(lrp + 4 * g + r) : 0.f;
+    __builtin_amdgcn_sched_barrier(0);
   };
   auto rowsum = [&](const f32x4 (&x)[NT]) {
     float s = 0.f;
@@ -140,9 +153,9 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
   fetch(a.n_stages - 1);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   for (int st = a.n_stages - 1; st >= 0; --st) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const float lr_c = pre_lrc;
     const f32x4 lr_s = pre_lrs;
     if (st > 0) fetch(st - 1);
@@ -378,7 +391,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
       }
       const float dlr = xg_sum(e2) + te_last * dl;
       float dte = xg_sum(e1);
-      const float tail = row16_sum(dl * lr_c);
+      const float tail = row16_sum_dpp(dl * lr_c);
       if (c == K - 1) dte += tail;
       if (g == 0 && tok_ok) {
         IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + c, dlr);
@@ -395,6 +408,15 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
       }
 #pragma unroll
     for (int J = 0; J < NT; ++J) IO::mma2(dbT[J], Zd[J], Z1d[J], ones, ones);
+    // The next mini-batch's copies to LDS must have landed; this mini-batch's stores and atomics, all issued
+    // after them, need not have (the atomics of all units meet on one cache line and take long).  Vector
+    // memory operations retire in order on this counter, so the wait leaves exactly those outstanding:
+    // 3 tensors x NQ stores, the d_lr store and the d_token_eta atomic.
+    static_assert(NQ == 1 || NQ == 2, "counted wait below");
+    if (NQ == 2)
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
   }
 
   // ---- results carried over the whole scan
