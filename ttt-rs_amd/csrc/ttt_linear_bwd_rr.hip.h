@@ -36,13 +36,37 @@ __device__ __forceinline__ float row16_sum_dpp(float v) {
   return v;
 }
 
+// 16 bytes per lane, global -> LDS at lds_base + 16 * lane, not passing registers.  Written as assembly
+// because the compiler makes every later LDS read wait for all copies it knows to be in flight (it cannot
+// tell the two stage buffers apart), which would turn the prefetch into a synchronous load; the waits
+// are placed by hand instead.  M0 (the LDS base of the copy) is restored.
+__device__ __forceinline__ void lds_dma16(const void* src, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src), "s"(lds_base)
+      : "memory");
+}
+
+// One 2-byte element per lane, zero-extended to a dword at lds_base + 4 * lane.
+__device__ __forceinline__ void lds_dma2(const void* src, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_ushort %1, off\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src), "s"(lds_base)
+      : "memory");
+}
+
 template <int D>
 struct LinBwdRrLds {
   static constexpr int NT = D / 16;
   static constexpr int W = 0;                       // NT*NT slots of 1 KiB: slot I*NT+J, lane (c,g): W[feat(I,c)][feat(J,4g..4g+3)]
   static constexpr int Bv = W + NT * NT * 1024;     // NT slots: b[feat(J,4g..4g+3)]
   static constexpr int X = Bv + NT * 1024;          // 4 tensors x NT/2 slots: X[token c][32q + 8g .. +7] (bf16)
-  static constexpr int STAGE = X + 4 * (NT / 2) * 1024;
+  static constexpr int LR = X + 4 * (NT / 2) * 1024;  // 16 dwords: lr of token c, zero-extended bf16
+  static constexpr int STAGE = LR + 256;
   static constexpr int BYTES = 2 * STAGE;
 };
 
@@ -94,41 +118,44 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
   for (int i = lane; i < L::BYTES / 16; i += 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
-  float pre_lrc = 0.f;
-  f32x4 pre_lrs = {0.f, 0.f, 0.f, 0.f};
-  auto fetch = [&](int stage) {
-    // the few register loads first: the copies to LDS must be the youngest loads of the batch (see the
-    // counted wait at the bottom of the loop)
-    const elem* lrp = static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K;
-    pre_lrc = (c < K) ? IO::load1(lrp + c) : 0.f;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) pre_lrs[r] = (4 * g + r < K) ? IO::load1(lrp + 4 * g + r) : 0.f;
-    __builtin_amdgcn_sched_barrier(0);
+  // The copies of one mini-batch are issued in NPART portions spread over the previous mini-batch's
+  // arithmetic: the memory pipeline accepts only so many requests at a time, and a wave that issues a
+  // whole mini-batch at once (29 KiB) sits in the issue for thousands of cycles while all other units do
+  // the same.  Everything goes through LDS, nothing through registers: a load the compiler knows of would
+  // make it place a wait for ALL outstanding memory operations, these copies included, before its first use.
+  constexpr int NPART = NT + 3;
+  auto fetch = [&](int stage, int part) {
+    if (stage < 0) return;
     unsigned char* dst = smem + (stage & 1) * L::STAGE;
     const size_t ci = bh * (size_t)a.n_ckpt + stage;
     const float* Wg = a.W_ckpt + ci * D * D;
     const float* bg = a.b_ckpt + ci * D;
-    auto dma = [&](const void* src, int off) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(dst + off), 16, 0, 0);
-    };
-#pragma unroll
-    for (int I = 0; I < NT; ++I)
+    const unsigned dst_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)dst;
+    auto dma = [&](const void* src, int off) { lds_dma16(src, dst_lds + off); };
+    const size_t tok = (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D + 8 * g;
+    if (part < NT) {
+      const int I = part;
 #pragma unroll
       for (int J = 0; J < NT; ++J) dma(Wg + feat(I, c) * D + own_offset<NT>(0, J, g), L::W + (I * NT + J) * 1024);
+    } else if (part == NT) {
 #pragma unroll
-    for (int J = 0; J < NT; ++J) dma(bg + own_offset<NT>(0, J, g), L::Bv + J * 1024);
-    const size_t tok = (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D + 8 * g;
-    if (c < K) {
+      for (int J = 0; J < NT; ++J) dma(bg + own_offset<NT>(0, J, g), L::Bv + J * 1024);
+      // lr of the 16 tokens (absent ones: a clamped position, zeroed at use), one 2-byte element per lane
+      if (lane < 16)
+        lds_dma2(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + (c < K ? c : K - 1),
+                 dst_lds + L::LR);
+    } else if (c < K) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
-        dma(static_cast<const elem*>(a.xq) + tok + 32 * q, L::X + (0 * NQ + q) * 1024);
-        dma(static_cast<const elem*>(a.xk) + tok + 32 * q, L::X + (1 * NQ + q) * 1024);
-        dma(static_cast<const elem*>(a.xv) + tok + 32 * q, L::X + (2 * NQ + q) * 1024);
-        dma(static_cast<const elem*>(a.d_out) + tok + 32 * q, L::X + (3 * NQ + q) * 1024);
+        if (part == NT + 1) {
+          dma(static_cast<const elem*>(a.xq) + tok + 32 * q, L::X + (0 * NQ + q) * 1024);
+          dma(static_cast<const elem*>(a.xk) + tok + 32 * q, L::X + (1 * NQ + q) * 1024);
+        } else {
+          dma(static_cast<const elem*>(a.xv) + tok + 32 * q, L::X + (2 * NQ + q) * 1024);
+          dma(static_cast<const elem*>(a.d_out) + tok + 32 * q, L::X + (3 * NQ + q) * 1024);
+        }
       }
     }
-    __builtin_amdgcn_sched_barrier(0);
   };
   auto rowsum = [&](const f32x4 (&x)[NT]) {
     float s = 0.f;
@@ -152,14 +179,22 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
   };
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
-  fetch(a.n_stages - 1);
+#pragma unroll
+  for (int part = 0; part < NPART; ++part) fetch(a.n_stages - 1, part);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   for (int st = a.n_stages - 1; st >= 0; --st) {
-    const float lr_c = pre_lrc;
-    const f32x4 lr_s = pre_lrs;
-    if (st > 0) fetch(st - 1);
+    fetch(st - 1, 0);
     const unsigned char* sb = smem + (st & 1) * L::STAGE + lane * 16;
+    float lr_c;
+    f32x4 lr_s;
+    {
+      const uint32_t* lrw = reinterpret_cast<const uint32_t*>(smem + (st & 1) * L::STAGE + L::LR);
+      lr_c = (c < K) ? __uint_as_float(lrw[c] << 16) : 0.f;
+      const u32x4 w4 = *reinterpret_cast<const u32x4*>(lrw + 4 * g);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) lr_s[r] = (4 * g + r < K) ? __uint_as_float(w4[r] << 16) : 0.f;
+    }
 
     // ---- this mini-batch's tiles and the state entering it
     frag q[NT], k[NT], v[NT], o[NT];
@@ -185,6 +220,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
       qd[I] = tokens_k(q[I]);
     }
 
+    if (1 < NPART) fetch(st - 1, 1);
     // ---- forward intermediates: Z1 = XK W + b, Zq = XQ W + b, attention block in both orientations
     f32x4 z1[NT], zb[NT], At = zero4, At2 = zero4;
 #pragma unroll
@@ -209,6 +245,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
       IO::mma2(At2, q[2 * qq], q[2 * qq + 1], k[2 * qq], k[2 * qq + 1]);  // [t = 4g+r][s = c]
     }
 
+    if (2 < NPART) fetch(st - 1, 2);
     // ---- first LayerNorm and the gradient of the reconstruction loss
     f32x4 xh[NT], G[NT], gO[NT];
     float rstd1, sgx;
@@ -240,6 +277,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
       onepA2[r] = low2 ? 1.f + At2[r] : 0.f;
       M2[r] = eta2[r] * onepA2[r];
     }
+    if (3 < NPART) fetch(st - 1, 3);
     // ---- Zb = XQ W + b - M G
     frag Gf[NT];
     {
@@ -250,6 +288,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
         IO::mma(zb[J], tokens_k(Gf[J]), nMf);
       }
     }
+    if (4 < NPART) fetch(st - 1, 4);
     // ---- output LayerNorm and its backward: dZb
     frag Zf[NT], Zd[NT];
     f32x4 DZB[NT];
@@ -274,6 +313,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
         Zd[J] = tokens_k(Zf[J]);
       }
     }
+    if (5 < NPART) fetch(st - 1, 5);
     // ---- P = dZb G^T in both orientations; dA = -P eta, d eta = -P (1 + A)
     f32x4 dA, dEta, dA2, dEta2;
     {
@@ -297,6 +337,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
       dA2 = -P2 * eta2;
       dEta2 = -P2 * onepA2;
     }
+    if (6 < NPART) fetch(st - 1, 6);
     const bool tok_ok = c < K;
     const size_t tok = (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D + 8 * g;
     // ---- dXQ = dO + dZb W^T + dA XK
