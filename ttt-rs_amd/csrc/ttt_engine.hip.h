@@ -104,15 +104,26 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
   }
 }
 
+// Sum over the 16 lanes of a row, in every lane: four rotations inside the row on the DPP path
+// (a shuffle goes through the LDS crossbar and costs an LDS round trip per step).
+__device__ __forceinline__ float row16_sum_dpp(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));  // row_ror:8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));  // row_ror:4
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));  // row_ror:2
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));  // row_ror:1
+  return v;
+}
 // sum over an aligned group of W lanes (W = 16 or 32) that share a token
 template <int W>
 __device__ __forceinline__ float rowgroup_sum(float v) {
-  if (W == 32) v += __shfl_xor(v, 16, 32);
-  v += __shfl_xor(v, 8, W);
-  v += __shfl_xor(v, 4, W);
-  v += __shfl_xor(v, 2, W);
-  v += __shfl_xor(v, 1, W);
-  return v;
+  if (W == 32) {
+    // rows 2k and 2k+1 exchanged: the two results add up to the sum of the pair in both rows
+    const uint32_t u = __float_as_uint(v);
+    const auto q = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const uint32_t q0 = q[0], q1 = q[1];
+    v = __uint_as_float(q0) + __uint_as_float(q1);
+  }
+  return row16_sum_dpp(v);
 }
 __device__ __forceinline__ float row16_sum(float v) { return rowgroup_sum<16>(v); }
 

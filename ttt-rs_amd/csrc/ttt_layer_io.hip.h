@@ -127,8 +127,7 @@ __global__ void __launch_bounds__(256) ttt_layer_epilogue_kernel(LayerEpilogueAr
     for (int r = 0; r < 4; ++r) s += v[j][0][r] + v[j][1][r];
   }
   auto wave_sum = [](float x) {
-    x = rowgroup_sum<32>(x);
-    return x + __shfl_xor(x, 32);
+    return xg_sum(row16_sum_dpp(x));
   };
   const float mu = wave_sum(s) / hidden;
   float q = 0.f;

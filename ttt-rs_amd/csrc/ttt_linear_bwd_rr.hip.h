@@ -27,15 +27,6 @@
 
 namespace ttt {
 
-// Sum over the 16 lanes of a row, in every lane: four rotations inside the row on the DPP path.
-__device__ __forceinline__ float row16_sum_dpp(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));  // row_ror:8
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));  // row_ror:4
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));  // row_ror:2
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));  // row_ror:1
-  return v;
-}
-
 // 16 bytes per lane, global -> LDS at lds_base + 16 * lane, not passing registers.  Written as assembly
 // because the compiler makes every later LDS read wait for all copies it knows to be in flight (it cannot
 // tell the two stage buffers apart), which would turn the prefetch into a synchronous load; the waits
