@@ -83,6 +83,12 @@ __device__ __forceinline__ float xg_sum4_scatter(float a, float b, float c, floa
   return __uint_as_float(r0) + __uint_as_float(r1);            // rows: a, b, c, d
 }
 
+// Workgroup barrier for LDS exchanges only: waits for this wave's LDS traffic, not for the
+// global prefetches in flight (a full __syncthreads() would drain those every mini-batch).
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <class T>
 struct Io;
 

@@ -15,7 +15,9 @@
 // db stay in LDS for the whole scan (the reference round-trips them through global memory
 // every stage).  Elementwise work uses thread (t = tid/16, cg = tid%16) for token t and
 // features cg, cg+16, ...; row statistics are 16-lane shuffles.  Arithmetic is f32 for both
-// I/O dtypes; bf16 tensors are converted at the tile loads and stores.
+// I/O dtypes; bf16 tensors are converted at the tile loads and stores.  The barriers inside the scan order
+// LDS traffic only (lds_barrier): a full __syncthreads() would also wait for every global store and for
+// the contended d_token_eta atomics of the mini-batch.
 #pragma once
 #include "ttt_engine.hip.h"
 
@@ -206,15 +208,15 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     const int ck = st / a.ckpt_interval;
     commit_state();
     for (int s2 = ck * a.ckpt_interval; s2 < st; ++s2) {
-      __syncthreads();
+      lds_barrier();
       load_tile(lds + L::XK, a.xk, s2);
       load_tile(lds + L::TG, a.xv, s2);
       load_lr(s2);
-      __syncthreads();
+      lds_barrier();
 #pragma unroll
       for (int j = 0; j < NJ; ++j) lds[L::TG + t * LD + cg + 16 * j] -= lds[L::XK + t * LD + cg + 16 * j];
       mm_lds<0>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane);
-      __syncthreads();
+      lds_barrier();
       {
         float xh[NJ], Gv[NJ], rstd;
         ln1(lds + L::XH, lds + L::TG, xh, Gv, rstd);
@@ -222,7 +224,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) lds[L::G + t * LD + cg + 16 * j] = Gv[j] * last;
       }
-      __syncthreads();
+      lds_barrier();
       // W -= XK^T (last * G) ; b -= colsum(last * G)      (linear.rs:134-144)
       mm_lds<2, 4, NJ, 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, 16, wave, lane);
       if (tid < D) {
@@ -231,11 +233,11 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
         sb[tid] -= s;
       }
     }
-    if (ck * a.ckpt_interval < st) __syncthreads();  // the re-simulation used the XK / target tiles
+    if (ck * a.ckpt_interval < st) lds_barrier();  // the re-simulation used the XK / target tiles
 
     // ================= this stage's tiles (target = XV - XK formed on the way), then prefetch the next
     commit_tiles();
-    __syncthreads();
+    lds_barrier();
     if (st > 0) fetch_stage(st - 1);
     // Z1 = XK W ; Zq = XQ W ; A = XQ XK^T
     // every product is cut into jobs of NB2 tile columns: two or more accumulator chains per wave keep the
@@ -243,7 +245,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     mm_lds<0, 4, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, 0);
     mm_lds<0, 4, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, 2);
     mm_lds<0>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, 1);
-    __syncthreads();
+    lds_barrier();
 
     // ================= forward intermediates: x_hat, rstd, G; eta, A (tril), M = eta (1 + A)
     float xh[NJ], Gv[NJ], rstd1;
@@ -262,10 +264,10 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       lds[L::ETA + t * LK + s] = et;
       lds[L::M + t * LK + s] = et * (1.f + at);
     }
-    __syncthreads();
+    lds_barrier();
     // Zb = XQ W - M G  (+ b added when read)
     mm_lds<2, 4, 1, 4>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NJ, 16, wave, lane);
-    __syncthreads();
+    lds_barrier();
 
     // ================= output LayerNorm and its backward (stage 4)
     {
@@ -300,14 +302,14 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
 #pragma unroll
       for (int j = 0; j < NJ; ++j) lds[L::DZB + t * LD + cg + 16 * j] = (gx2[j] - s1 - zv[j] * s2) * rstd2;
     }
-    __syncthreads();
+    lds_barrier();
 
     // ================= P = dZb G^T ; dQ = dZb W^T ; S = XK dW ; TMP = G dW^T
     mm_lds<0, 4, NB2>(lds + L::DQ, LD, lds + L::DZB, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 0);
     mm_lds<0, 4, NB2>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, LD, 1, NJ, D, wave, lane, 0);
     mm_lds<0, 4, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, LD, 1, 1, NJ, D, wave, lane, 2);
     mm_lds<0>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, 1, 1, D, wave, lane, 3);
-    __syncthreads();
+    lds_barrier();
 
     // ================= dA, d eta ; S += db ; dlast
     {
@@ -326,7 +328,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       dl = row16_sum(dl);
       if (cg == 0) lds[L::dlast + t] = -dl;
     }
-    __syncthreads();
+    lds_barrier();
 
     // ================= dQ += dA XK ; dK = dA^T XQ ; DGM = M^T dZb ; dW += XQ^T dZb ; db += colsum(dZb)
     mm_lds<1, 4, NJ, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NJ, 16, wave, lane, 0);
@@ -352,7 +354,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
         for (int r = 0; r < 16; ++r) s += lds[L::dlast + r] * slr[r];
       if (tt < K) atomicAdd(a.d_token_eta + (size_t)st * K + tt, s);
     }
-    __syncthreads();
+    lds_barrier();
 
     // ================= through G: second-order LayerNorm (stage 2), token-local
     {
@@ -396,7 +398,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
         lds[L::DK + t * LD + o] += dy[j] - last * lds[L::TMP + t * LD + o];
       }
     }
-    __syncthreads();
+    lds_barrier();
 
     // ================= dK += dZ1 W^T ; dW += XK^T dZ1 ; db += colsum(dZ1)
     mm_lds<1, 4, NB2>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 2);
@@ -406,7 +408,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       for (int r = 0; r < 16; ++r) s += lds[L::DZ1 + r * LD + tid];
       sdb[tid] += s;
     }
-    __syncthreads();
+    lds_barrier();
 
     // ================= store dXQ = dO + dQ, dXK
     if (t < K) {
@@ -419,7 +421,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
         IO::store1(pk + o, lds[L::DK + t * LD + o]);
       }
     }
-    __syncthreads();
+    lds_barrier();
   }
 
   // ---- results carried over the whole scan

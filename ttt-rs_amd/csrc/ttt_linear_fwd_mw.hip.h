@@ -23,12 +23,6 @@
 
 namespace ttt {
 
-// Workgroup barrier for LDS exchanges only: waits for this wave's LDS traffic, not for the
-// global prefetches in flight (a full __syncthreads() would drain those every mini-batch).
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 template <class T, int NT, int TPW>
 struct StageInMw {
   typename Io<T>::frag q[NT], k[NT];               // full rows: k-side operands
