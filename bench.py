@@ -232,6 +232,17 @@ def main():
                            "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
                            "kernel": "ttt_inner_inputs_kernel" if kind == "inner_inputs" else "ttt_layer_epilogue_kernel",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_bytes": alg}
+    elif kind == "linear_fwd_bwd" and io == "bf16" and ci == 1 and os.environ.get("TTT_LINEAR_BWD_KERNEL") != "lds":
+        # register-resident backward (bf16 MFMA operands): the pair of passes is bound by HBM in the limit
+        alg = linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)
+        out["dtype"] = "bf16"
+        out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci)
+        out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                           "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_rr_kernel (whole step)",
+                           "kernel_avg_us": dev_s * 1e6, "algorithmic_bytes": alg,
+                           "checkpoint_bytes": 2 * th * (d * d + d) * 4 // (ci * K),
+                           "algorithmic_flops": th * (24 * d * d + 26 * K * d)}
     elif kind == "linear_fwd_bwd":
         # the backward kernel dominates; it computes in f32 MFMA: 18 d^2 + 22 K d flop per token-head
         flops = th * (24 * d * d + 26 * K * d)

@@ -89,6 +89,53 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// 16 bytes per lane, global -> LDS at lds_base + 16 * lane, not passing registers.  Written as assembly
+// because the compiler makes every later LDS read wait for all copies it knows to be in flight (it cannot
+// tell the two stage buffers apart), which would turn the prefetch into a synchronous load; the waits
+// are placed by hand instead.  M0 (the LDS base of the copy) is restored.
+__device__ __forceinline__ void lds_dma16(const void* src, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src), "s"(lds_base)
+      : "memory");
+}
+
+// A wave-uniform pointer the compiler cannot prove uniform, moved to scalar registers.
+__device__ __forceinline__ const void* uniform_ptr(const void* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
+}
+// The same with the global address as wave-uniform base + 32-bit lane offset (one VGPR instead of two).
+__device__ __forceinline__ void lds_dma16(const void* base, unsigned lane_off, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(lane_off), "s"(uniform_ptr(base)), "s"(lds_base)
+      : "memory");
+}
+// One 2-byte element per lane, zero-extended to a dword at lds_base + 4 * lane.
+__device__ __forceinline__ void lds_dma2(const void* src, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_ushort %1, off\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src), "s"(lds_base)
+      : "memory");
+}
+
+__device__ __forceinline__ void lds_dma2(const void* base, unsigned lane_off, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(lane_off), "s"(uniform_ptr(base)), "s"(lds_base)
+      : "memory");
+}
+
 template <class T>
 struct Io;
 

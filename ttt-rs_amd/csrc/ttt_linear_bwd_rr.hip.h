@@ -27,29 +27,6 @@
 
 namespace ttt {
 
-// 16 bytes per lane, global -> LDS at lds_base + 16 * lane, not passing registers.  Written as assembly
-// because the compiler makes every later LDS read wait for all copies it knows to be in flight (it cannot
-// tell the two stage buffers apart), which would turn the prefetch into a synchronous load; the waits
-// are placed by hand instead.  M0 (the LDS base of the copy) is restored.
-__device__ __forceinline__ void lds_dma16(const void* src, unsigned lds_base) {
-  unsigned saved;
-  asm volatile(
-      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_nop 0\n\ts_mov_b32 m0, %0"
-      : "=&s"(saved)
-      : "v"(src), "s"(lds_base)
-      : "memory");
-}
-
-// One 2-byte element per lane, zero-extended to a dword at lds_base + 4 * lane.
-__device__ __forceinline__ void lds_dma2(const void* src, unsigned lds_base) {
-  unsigned saved;
-  asm volatile(
-      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_ushort %1, off\n\ts_nop 0\n\ts_mov_b32 m0, %0"
-      : "=&s"(saved)
-      : "v"(src), "s"(lds_base)
-      : "memory");
-}
-
 template <int D>
 struct LinBwdRrLds {
   static constexpr int NT = D / 16;

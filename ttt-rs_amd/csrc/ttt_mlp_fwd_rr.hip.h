@@ -99,7 +99,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
   frag* const GT = reinterpret_cast<frag*>(smem + L::GT);
   frag* const GD = reinterpret_cast<frag*>(smem + L::GD);
   frag* const KD = reinterpret_cast<frag*>(smem + L::KD);
-  float* const LRs = reinterpret_cast<float*>(smem + L::LR);
+  uint32_t* const LRs = reinterpret_cast<uint32_t*>(smem + L::LR);
   float* const GAM = reinterpret_cast<float*>(smem + L::PRM);
   float* const BET = GAM + D;
   float* const B1s = BET + D;  // b1: each wave reads and updates only its own slice
@@ -166,14 +166,14 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
         const unsigned char* src =
             static_cast<const unsigned char*>(ten == 0 ? a.xq : ten == 1 ? a.xk : a.xv) + tok0;
         if (goff[it] >= 0)
-          __builtin_amdgcn_global_load_lds(
-              (const __attribute__((address_space(1))) void*)(src + goff[it]),
-              (__attribute__((address_space(3))) void*)(dst + 1024 * b), 16, 0, 0);
+          lds_dma16(src, (unsigned)goff[it], (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(dst + 1024 * b));
       }
     }
-    if (tid < 16 && tid < K)
-      LRs[(stage % 3) * 16 + tid] =
-          IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid);
+    // lr as zero-extended bf16 words, copied like the tiles (a register load here would make the compiler
+    // wait for every copy in flight); absent tokens read a clamped position and are zeroed at use
+    if (tid < 16)
+      lds_dma2(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K, 2u * (unsigned)(tid < K ? tid : K - 1),
+               (unsigned)(size_t)(__attribute__((address_space(3))) uint32_t*)(LRs + (stage % 3) * 16));
   };
   // staged row of token c of tensor ten (0 xq, 1 xk, 2 xv)
   auto row = [&](int buf, int ten) -> const elem* {
@@ -287,7 +287,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
         IO::mma2(z1[j], IO::to_frag(W1c[2 * q][j]), IO::to_frag(W1c[2 * q + 1][j]), k0, k1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    const float lrc = LRs[buf * 16 + c];
+    const float lrc = (c < K) ? __uint_as_float(LRs[buf * 16 + c] << 16) : 0.f;
     // X2 = gelu(Z1), gelu'(Z1)
     frag x2f[HT];
     f32x4 dg[HT];
@@ -375,8 +375,12 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
       GD[w * 64 + lane] = IO::to_frag(t);
     }
     if (outw && st > 0) output_emit(st - 1);
-    // the next mini-batch's rows must have landed before anybody passes B3
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the next mini-batch's rows must have landed before anybody passes B3; the output store just issued
+    // (the only memory operation younger than the copies, which retire in order) may stay in flight
+    if (outw && st > 0)
+      asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();  // ---- B3
     RELANE();
 
