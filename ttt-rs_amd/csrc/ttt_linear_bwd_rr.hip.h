@@ -14,9 +14,9 @@
 //   W_t     read from the checkpoint as A operand (m = row i, k = column j) for dQ = dZb W^T and
 //           dK += dZ1 W^T; its transpose (m = j, k = i), for Z1 = XK W and Zq = XQ W, is made on the matrix
 //           pipe (identity multiplication, exact for bf16 values).
-//   dW      kept TWICE as f32 accumulator tiles: dWc[I][J] (rows i in registers) feeds S = XK dW as an A
-//           operand without moving data, DT[J][I] (rows j in registers) feeds G dW^T the same way; both get
-//           the rank-32 update [XQ; XK]^T [dZb; dZ1] with the operand roles swapped.
+//   dW      f32 accumulator tiles dWc[I][J] (rows i in registers), updated by one rank-32 product
+//           [XQ; XK]^T [dZb; dZ1] per mini-batch.  Its bf16 image is an A operand as it stands (m = j, k = i)
+//           for S = XK dW; for G dW^T the image is transposed tile by tile on the matrix pipe.
 //   [16 x 16] causal matrices are computed in both orientations (operands swapped) instead of transposed.
 // Staging: the checkpoint (16 KiB at d = 64), its bias and the four activation tiles of the next
 // mini-batch are copied global -> LDS without passing registers (global_load_lds_dwordx4), each lane
@@ -70,8 +70,8 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
     dgam[J] = dbet[J] = f32x4{0.f, 0.f, 0.f, 0.f};
     dbT[J] = a.d_b_out ? *reinterpret_cast<const f32x4*>(a.d_b_out + bh * D + f) : f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  // state gradient in both orientations
-  f32x4 dWc[NT][NT], DT[NT][NT];
+  // state gradient: dWc[I][J], rows i = feat(I, 4g+r) in registers, columns j = feat(J, c) on lanes
+  f32x4 dWc[NT][NT];
 #pragma unroll
   for (int I = 0; I < NT; ++I)
 #pragma unroll
@@ -79,7 +79,6 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         dWc[I][J][r] = a.d_W_out ? a.d_W_out[bh * D * D + feat(I, 4 * g + r) * D + feat(J, c)] : 0.f;
-        DT[J][I][r] = a.d_W_out ? a.d_W_out[bh * D * D + feat(I, c) * D + feat(J, 4 * g + r)] : 0.f;
       }
 
   // rows of absent tokens (c >= K) are never fetched: they stay zero
@@ -99,28 +98,31 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
     const float* Wg = a.W_ckpt + ci * D * D;
     const float* bg = a.b_ckpt + ci * D;
     const unsigned dst_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)dst;
-    auto dma = [&](const void* src, int off) { lds_dma16(src, dst_lds + off); };
-    const size_t tok = (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D + 8 * g;
+    // wave-uniform base + 32-bit lane offset: one address register per copy
+    auto dma = [&](const void* base, unsigned lane_off, int off) { lds_dma16(base, lane_off, dst_lds + off); };
+    const size_t tok0 = (bh * (size_t)a.seq_stride + (size_t)stage * K) * D;
+    const unsigned xoff = (unsigned)(c * D + 8 * g) * 2u;
     if (part < NT) {
       const int I = part;
 #pragma unroll
-      for (int J = 0; J < NT; ++J) dma(Wg + feat(I, c) * D + own_offset<NT>(0, J, g), L::W + (I * NT + J) * 1024);
+      for (int J = 0; J < NT; ++J)
+        dma(Wg, (unsigned)(feat(I, c) * D + own_offset<NT>(0, J, g)) * 4u, L::W + (I * NT + J) * 1024);
     } else if (part == NT) {
 #pragma unroll
-      for (int J = 0; J < NT; ++J) dma(bg + own_offset<NT>(0, J, g), L::Bv + J * 1024);
+      for (int J = 0; J < NT; ++J) dma(bg, (unsigned)own_offset<NT>(0, J, g) * 4u, L::Bv + J * 1024);
       // lr of the 16 tokens (absent ones: a clamped position, zeroed at use), one 2-byte element per lane
       if (lane < 16)
-        lds_dma2(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + (c < K ? c : K - 1),
-                 dst_lds + L::LR);
+        lds_dma2(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K,
+                 2u * (unsigned)(c < K ? c : K - 1), dst_lds + L::LR);
     } else if (c < K) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         if (part == NT + 1) {
-          dma(static_cast<const elem*>(a.xq) + tok + 32 * q, L::X + (0 * NQ + q) * 1024);
-          dma(static_cast<const elem*>(a.xk) + tok + 32 * q, L::X + (1 * NQ + q) * 1024);
+          dma(static_cast<const elem*>(a.xq) + tok0, xoff + 64u * q, L::X + (0 * NQ + q) * 1024);
+          dma(static_cast<const elem*>(a.xk) + tok0, xoff + 64u * q, L::X + (1 * NQ + q) * 1024);
         } else {
-          dma(static_cast<const elem*>(a.xv) + tok + 32 * q, L::X + (2 * NQ + q) * 1024);
-          dma(static_cast<const elem*>(a.d_out) + tok + 32 * q, L::X + (3 * NQ + q) * 1024);
+          dma(static_cast<const elem*>(a.xv) + tok0, xoff + 64u * q, L::X + (2 * NQ + q) * 1024);
+          dma(static_cast<const elem*>(a.d_out) + tok0, xoff + 64u * q, L::X + (3 * NQ + q) * 1024);
         }
       }
     }
@@ -337,13 +339,24 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
         IO::mma(dK[I], qd[I], dA2f);
         IO::mma(DGM[I], Zd[I], M2f);
       }
+      // dW tiles as A operands: as they are (m = column j, k = row i) for S, transposed on the matrix pipe
+      // (m = i, k = j) for G dW^T
 #pragma unroll
-      for (int qq = 0; qq < NQ; ++qq)
+      for (int qq = 0; qq < NQ; ++qq) {
+        frag t0[NT], t1[NT];
 #pragma unroll
         for (int J = 0; J < NT; ++J) {
-          IO::mma2(S[J], IO::to_frag(dWc[2 * qq][J]), IO::to_frag(dWc[2 * qq + 1][J]), k[2 * qq], k[2 * qq + 1]);
-          IO::mma2(TMP[J], IO::to_frag(DT[2 * qq][J]), IO::to_frag(DT[2 * qq + 1][J]), Gf[2 * qq], Gf[2 * qq + 1]);
+          const frag f0 = IO::to_frag(dWc[2 * qq][J]), f1 = IO::to_frag(dWc[2 * qq + 1][J]);
+          IO::mma2(S[J], f0, f1, k[2 * qq], k[2 * qq + 1]);
+          t0[J] = tokens_k(f0);
+          t1[J] = tokens_k(f1);
         }
+#pragma unroll
+        for (int pj = 0; pj < NQ; ++pj) {
+          IO::mma2(TMP[2 * qq], t0[2 * pj], t0[2 * pj + 1], Gf[2 * pj], Gf[2 * pj + 1]);
+          IO::mma2(TMP[2 * qq + 1], t1[2 * pj], t1[2 * pj + 1], Gf[2 * pj], Gf[2 * pj + 1]);
+        }
+      }
     }
     // ---- through G: second-order LayerNorm, token-local
     const float last = te_last * lr_c;
@@ -407,13 +420,12 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
         atomicAdd(a.d_token_eta + (size_t)st * K + c, dte);
       }
     }
-    // ---- state gradient: dW += XQ^T dZb + XK^T dZ1 (both orientations), db += colsum(dZb + dZ1)
+    // ---- state gradient: dW += XQ^T dZb + XK^T dZ1 (one rank-32 update), db += colsum(dZb + dZ1)
 #pragma unroll
     for (int I = 0; I < NT; ++I)
 #pragma unroll
       for (int J = 0; J < NT; ++J) {
         IO::mma2(dWc[I][J], qd[I], kd[I], Zd[J], Z1d[J]);
-        IO::mma2(DT[J][I], Zd[J], Z1d[J], qd[I], kd[I]);
       }
 #pragma unroll
     for (int J = 0; J < NT; ++J) IO::mma2(dbT[J], Zd[J], Z1d[J], ones, ones);
