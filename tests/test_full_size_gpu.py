@@ -106,6 +106,51 @@ def test_config2_linear_fwd_bwd_f32_full(P):
         assert_close(g1[gn], r[rn], 1e-4, gn)
 
 
+def test_config1_shape_linear_fwd_bwd_bf16_full(P, monkeypatch):
+    """The backward of config 1's shape (bf16 I/O, one checkpoint per mini-batch: the register-resident
+    backward kernel).  Products take bf16 operands, so all gradients are held to the bf16 bar; tensors
+    that are sums over thousands of bf16-rounded terms with a small result (the LayerNorm parameter
+    gradients, d_token_eta) are held to the max-norm bar only."""
+    B, H, d, seq, K = 32, 12, 64, 2048, 16
+    print("case config1-shape fwd+bwd bf16 full", flush=True)
+    c = P.synthetic.baseline_inputs(1, B, H, seq, d, K, io_dtype=torch.bfloat16, with_dout=True)
+    dv = dev(c)
+
+    def fwd_bwd(x):
+        out, W, b, Wc, bc = P.ttt_linear_forward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"],
+                                                     x["lr"], x["gamma"], x["beta"], K, 1e-6, 1,
+                                                     want_checkpoints=True)
+        g = P.ttt_linear_backward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"],
+                                      x["gamma"], x["beta"], Wc, bc, x["d_out"], K, 1e-6, 1)
+        torch.cuda.synchronize()
+        return out, g
+
+    out, g = fwd_bwd(dv)
+    for k, v in g.items():
+        assert torch.isfinite(v.float()).all(), k
+    # one batch entry alone: per-unit gradients are bit-identical
+    one = {k: (v[5:6].contiguous() if k in ("xq", "xk", "xv", "lr", "d_out") else v) for k, v in dv.items()}
+    o1, g1 = fwd_bwd(one)
+    assert torch.equal(o1, out[5:6])
+    for k in ("grad_xq", "grad_xk", "grad_xv", "grad_weight", "grad_bias", "grad_ttt_lr_eta"):
+        assert torch.equal(g1[k], g[k][5:6]), k
+    # the all-f32 LDS-tile kernel on the same launch agrees to the bf16 bar
+    monkeypatch.setenv("TTT_LINEAR_BWD_KERNEL", "lds")
+    _, gl = fwd_bwd(one)
+    monkeypatch.delenv("TTT_LINEAR_BWD_KERNEL")
+    for k in g1:
+        assert_close(g1[k], gl[k].double(), TOL[torch.bfloat16], "rr vs lds " + k, min_frac=0.0)
+    # oracle: all 128 mini-batches, all heads of that batch entry, all nine gradients
+    n = sub(c, [5], list(range(H)))
+    r = orc.linear_backward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                            n["gamma"], n["beta"], n["d_out"], K=K)
+    names = [("grad_xq", "d_xq", 0.999), ("grad_xk", "d_xk", 0.999), ("grad_xv", "d_xv", 0.999),
+             ("grad_weight", "d_W0", 0.99), ("grad_bias", "d_b0", 0.99), ("grad_ttt_lr_eta", "d_lr", 0.99),
+             ("grad_token_eta", "d_token_eta", 0.0), ("grad_ln_weight", "d_gamma", 0.0), ("grad_ln_bias", "d_beta", 0.0)]
+    for gn, rn, frac in names:
+        assert_close(g1[gn], r[rn], TOL[torch.bfloat16], gn, min_frac=frac)
+
+
 def test_config3_mlp_fwd_bf16_full(P):
     B, H, d, seq, K = 8, 16, 96, 2048, 16
     print("case config3 full", flush=True)
