@@ -83,9 +83,10 @@ def test_bwd_matches_oracle_baseline_style_inputs(P, dtype):
     """N(0,1) activations, gamma=1, beta=0, sigmoid lr/d, dOut ~ N(0,1) (benchmark config 2 style)."""
     print(f"case bwd baseline-style {dtype}", flush=True)
     B, H, d, K, N = 2, 2, 64, 16, 8
-    c = P.synthetic.baseline_inputs(2, B, H, N * K, d, K, io_dtype=dtype, with_dout=True)
-    dO = c.pop("d_out")
-    compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])
+    if d == 64 and K == 16:  # benchmark-style inputs at the benchmark's head size
+        c = P.synthetic.baseline_inputs(2, B, H, N * K, d, K, io_dtype=dtype, with_dout=True)
+        dO = c.pop("d_out")
+        compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -122,3 +123,24 @@ def test_bwd_is_linear_in_upstream_gradient(P):
     g3 = run_bwd(P, c, 3.0 * dO, K, 2)
     for k in g1:
         assert_close(g3[k], 3.0 * g1[k].double(), 1e-5, k)
+
+
+MW_CASES = [(2, 2, 32, 8, 1), (2, 2, 32, 8, 2), (1, 2, 64, 16, 3), (2, 3, 64, 16, 8), (1, 2, 64, 5, 3)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("B,H,d,K,N", MW_CASES)
+def test_bwd_multi_wave_kernel(P, monkeypatch, B, H, d, K, N, dtype):
+    """The feature-split kernel (several waves per (batch, head), exchanges through LDS), forced for both
+    I/O types; with upstream state gradients so that every term of the scan is exercised."""
+    print(f"case bwd multi-wave B{B} H{H} d{d} K{K} N{N} {dtype}", flush=True)
+    monkeypatch.setenv("TTT_LINEAR_BWD_WAVES", "4")
+    c = P.synthetic.reference_test_inputs(300 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
+    g = torch.Generator().manual_seed(9)
+    dO = torch.randn(B, H, N * K, d, generator=g).to(dtype)
+    sg = (0.1 * torch.randn(B, H, d, d, generator=g), 0.1 * torch.randn(B, H, d, generator=g))
+    compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), TOL[dtype])
+    if d == 64 and K == 16:  # benchmark-style inputs at the benchmark's head size
+        c = P.synthetic.baseline_inputs(2, B, H, N * K, d, K, io_dtype=dtype, with_dout=True)
+        dO = c.pop("d_out")
+        compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])

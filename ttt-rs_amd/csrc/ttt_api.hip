@@ -12,6 +12,7 @@
 #include "ttt_engine_fwd.hip.h"
 #include "ttt_layer_io.hip.h"
 #include "ttt_linear_bwd.hip.h"
+#include "ttt_linear_bwd_mw.hip.h"
 #include "ttt_linear_bwd_rr.hip.h"
 #include "ttt_linear_fwd.hip.h"
 #include "ttt_linear_fwd_mw.hip.h"
@@ -196,6 +197,17 @@ int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
   return hip_status(hipGetLastError(), "ttt_linear_bwd (register-resident kernel) launch");
 }
 
+// one checkpoint per mini-batch, NW waves per (batch, head): feature axis split, exchanges through LDS
+template <class T, int D, int NW>
+int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
+  auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW>;
+  constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem)>::BYTES;
+  int rc = opt_in_lds(kern, bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_linear_bwd (multi-wave register-resident kernel) launch");
+}
+
 template <class T, int D>
 int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
   auto kern = ttt::ttt_mlp_bwd_kernel<T, D>;
@@ -349,6 +361,11 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
                      d_beta, hd);
   const unsigned grid = (unsigned)(a.B * a.H);
   if (d->io_dtype == TTT_F32) {
+    const char* wsel = std::getenv("TTT_LINEAR_BWD_WAVES");
+    if (a.ckpt_interval == 1 && wsel && std::atoi(wsel) > 1) {
+      if (d->head_dim == 64) return launch_linear_bwd_mw<ttt::F32, 64, 4>(a, grid, s);
+      return launch_linear_bwd_mw<ttt::F32, 32, 2>(a, grid, s);
+    }
     if (d->head_dim == 64) return launch_linear_bwd<ttt::F32, 64>(a, grid, s);
     return launch_linear_bwd<ttt::F32, 32>(a, grid, s);
   }
@@ -357,6 +374,12 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
     if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(d_out) || !aligned16(d_xq) ||
         !aligned16(d_xk) || !aligned16(d_xv) || !aligned16(W_ckpt) || !aligned16(b_ckpt) || (a.seq_stride * d->head_dim) % 8 != 0)
       return fail(TTT_ERR_SHAPE, "ttt_linear_bwd: tensors must be 16-byte aligned");
+    const char* wsel = std::getenv("TTT_LINEAR_BWD_WAVES");
+    const int waves = wsel ? std::atoi(wsel) : 1;
+    if (waves > 1) {
+      if (d->head_dim == 64) return launch_linear_bwd_mw<ttt::BF16, 64, 4>(a, grid, s);
+      return launch_linear_bwd_mw<ttt::BF16, 32, 2>(a, grid, s);
+    }
     if (d->head_dim == 64) return launch_linear_bwd_rr<64>(a, grid, s);
     return launch_linear_bwd_rr<32>(a, grid, s);
   }

@@ -136,6 +136,16 @@ __device__ __forceinline__ void lds_dma2(const void* base, unsigned lane_off, un
       : "memory");
 }
 
+// One dword per lane at lds_base + 4 * lane.
+__device__ __forceinline__ void lds_dma4(const void* base, unsigned lane_off, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(lane_off), "s"(uniform_ptr(base)), "s"(lds_base)
+      : "memory");
+}
+
 template <class T>
 struct Io;
 

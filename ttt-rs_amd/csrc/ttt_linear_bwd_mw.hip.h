@@ -1,0 +1,561 @@
+// TTT-Linear fused backward for gfx950, checkpoint interval 1, NW wavefronts per (batch, head): the
+// register-resident scheme of ttt_linear_bwd_rr.hip.h with the feature axis cut into NW slices.
+//
+// Arithmetic: the reverse scan of ttt_linear_bwd.hip.h (reference
+// rust/fused/src/linear_fused_tile/backward/kernel.rs:253-429, backward/stage.rs:42-1006, second-order
+// LayerNorm layer_norm.rs:428-709).
+//
+// Wave w owns TPW = (d/16)/NW feature tiles.  Of every [16 x d] tile it holds its own features (transposed:
+// value r of lane (c, g) is feature feat(J, 4g+r) of token c); of the state gradient it holds the column
+// slice dW[:, own] (dWc) and the row slice dW[own, :] transposed (DT), each fed back as an A operand without
+// data movement.  What a wave needs of the other slices crosses through LDS at five points per mini-batch:
+//   X1  six raw moments of Z1 (mean, variance and both sums of the LN-L2 gradient follow from them), the
+//       partial attention blocks, XK^T / XQ^T fragments (tokens along k);
+//   X2  four raw moments of Zbar and of the output-LayerNorm backward; G fragments;
+//   X3  partial P = dZbar G^T; dZbar fragments in both forms;
+//   X4  six sums of the second-order LayerNorm (all its statistics are linear in them);
+//   X5  dZ1 fragments in both forms.
+// All matrix products with a d-deep contraction over the OTHER slices' features take those fragments as B
+// operands; products over tokens (rank-16) are local.  f32 I/O computes in true-f32 MFMA
+// (v_mfma_f32_16x16x4_f32), bf16 I/O in bf16 MFMA with f32 accumulation.
+// Staging: checkpoint, bias, lr and the four activation tiles of a mini-batch are copied global -> LDS
+// (one buffer: everything is moved to registers at the top of the mini-batch, the copies for the next one
+// are issued behind the first exchange).
+#pragma once
+#include "ttt_linear_bwd.hip.h"
+#include "ttt_linear_fwd_mw.hip.h"
+
+namespace ttt {
+
+template <int D, int NW, int ES>
+struct LinBwdMwLds {
+  static constexpr int NT = D / 16, TPW = NT / NW;
+  static constexpr int XS = (ES == 2) ? NT / 2 : NT;  // 1 KiB slots per activation tensor
+  static constexpr int FT = 64 * 4 * ES;              // bytes of one fragment tile
+  static constexpr int W = 0;                         // NT*NT slots: slot I*NT+J, lane (c,g): W[feat(I,c)][feat(J,4g..4g+3)]
+  static constexpr int Bv = W + NT * NT * 1024;       // NT slots: b[feat(J,4g..4g+3)]
+  static constexpr int X = Bv + NT * 1024;            // 4 tensors x XS slots
+  static constexpr int LR = X + 4 * XS * 1024;        // 16 dwords: lr of token c (bf16 zero-extended, or f32)
+  static constexpr int SUM = LR + 256;                // 3 exchanges x [8 sums][16 tokens][NW]
+  static constexpr int PT = SUM + 3 * 8 * 16 * NW * 4;  // 4 kinds x [NW][64] f32x4: partial [16 x 16] blocks
+  static constexpr int FR = PT + 4 * NW * 1024;       // 7 kinds x [NT][64] fragments
+  static constexpr int BYTES = FR + 7 * NT * FT;
+  static_assert(NT % NW == 0, "feature tiles must divide among the waves");
+  static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
+};
+
+template <class T, int D, int NW>
+__global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArgs a) {
+  using IO = Io<T>;
+  using frag = typename IO::frag;
+  using elem = typename IO::elem;
+  constexpr int ES = sizeof(elem);
+  constexpr bool BF = ES == 2;
+  using L = LinBwdMwLds<D, NW, ES>;
+  constexpr int NT = D / 16, TPW = NT / NW, NQ = NT / 2, XS = L::XS;
+  constexpr float inv_d = 1.0f / D;
+  enum { KD = 0, QD, GF, ZF, ZD, Z1F, Z1D };
+  enum { P_AT = 0, P_AT2, P_P, P_P2 };
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const size_t bh = blockIdx.x;
+  const int h = (int)(bh % a.H);
+  const int K = a.K;
+
+  float* const SUMp = reinterpret_cast<float*>(smem + L::SUM);
+  f32x4* const PTp = reinterpret_cast<f32x4*>(smem + L::PT);
+  frag* const FRp = reinterpret_cast<frag*>(smem + L::FR);
+  auto fr = [&](int kind, int J) -> frag& { return FRp[(kind * NT + J) * 64 + lane]; };
+  auto pt = [&](int kind, int ww) -> f32x4& { return PTp[(kind * NW + ww) * 64 + lane]; };
+
+  const float te_c = (c < K) ? a.token_eta[c] : 0.f;
+  const float te_last = a.token_eta[K - 1];
+  f32x4 te_s;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) te_s[r] = (4 * g + r < K) ? a.token_eta[4 * g + r] : 0.f;
+  const frag ident = identity_frag<T>(c, g);
+  const frag ones = splat_frag<T>(1.f);
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  f32x4 gam[TPW], bet[TPW], a2[TPW], dgam[TPW], dbet[TPW], dbT[TPW];
+  float sum_a = 0.f;
+  for (int f = 0; f < D; ++f) sum_a += a.gamma[h * D + f] * a.gamma[h * D + f];
+#pragma unroll
+  for (int jj = 0; jj < TPW; ++jj) {
+    const int f = own_offset<TPW>(w, jj, g);
+    gam[jj] = *reinterpret_cast<const f32x4*>(a.gamma + h * D + f);
+    bet[jj] = *reinterpret_cast<const f32x4*>(a.beta + h * D + f);
+    a2[jj] = gam[jj] * gam[jj];
+    dgam[jj] = dbet[jj] = zero4;
+    dbT[jj] = a.d_b_out ? *reinterpret_cast<const f32x4*>(a.d_b_out + bh * D + f) : zero4;
+  }
+  // dWc[I][jj]: rows i = feat(I, 4g+r), columns j = feat(own jj, c)
+  // DT[J][ii]:  rows j = feat(J, 4g+r), columns i = feat(own ii, c)   (= dW[own rows][all columns], transposed)
+  f32x4 dWc[NT][TPW], DT[NT][TPW];
+#pragma unroll
+  for (int I = 0; I < NT; ++I)
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      const int Jo = w * TPW + jj;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        dWc[I][jj][r] = a.d_W_out ? a.d_W_out[bh * D * D + feat(I, 4 * g + r) * D + feat(Jo, c)] : 0.f;
+        DT[I][jj][r] = a.d_W_out ? a.d_W_out[bh * D * D + feat(Jo, c) * D + feat(I, 4 * g + r)] : 0.f;
+      }
+    }
+
+  // rows of absent tokens (c >= K) are never fetched: they stay zero
+  for (int i = threadIdx.x; i < L::BYTES / 16; i += 64 * NW) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
+  __syncthreads();
+
+  // ---- copies of one mini-batch, dealt round-robin to the waves
+  const unsigned stg = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  auto fetch = [&](int stage) {
+    if (stage < 0) return;
+    const size_t ci = bh * (size_t)a.n_ckpt + stage;
+    const float* Wg = a.W_ckpt + ci * D * D;
+#pragma unroll
+    for (int it = 0; it < NT * NT / NW; ++it) {
+      const int n = w + NW * it, I = n / NT, J = n - I * NT;
+      lds_dma16(Wg, (unsigned)(feat(I, c) * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::W + n * 1024);
+    }
+    if (w == 0) {
+      const float* bg = a.b_ckpt + ci * D;
+#pragma unroll
+      for (int J = 0; J < NT; ++J) lds_dma16(bg, (unsigned)(32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::Bv + J * 1024);
+    }
+    const size_t tok0 = (bh * (size_t)a.seq_stride + (size_t)stage * K) * D;
+#pragma unroll
+    for (int ten = 0; ten < 4; ++ten) {
+      if (ten % NW != w) continue;
+      const elem* src = static_cast<const elem*>(ten == 0 ? a.xq : ten == 1 ? a.xk : ten == 2 ? a.xv : a.d_out) + tok0;
+      if (c < K) {
+#pragma unroll
+        for (int s = 0; s < XS; ++s) {
+          // bf16: 8 features of tiles 2s, 2s+1; f32: the 4 features of tile s
+          const unsigned off = BF ? (unsigned)(c * D + 32 * s + 8 * g) * 2u
+                                  : (unsigned)(c * D + 32 * (s >> 1) + 8 * g + 4 * (s & 1)) * 4u;
+          lds_dma16(src, off, stg + L::X + (ten * XS + s) * 1024);
+        }
+      }
+    }
+    if (w == NW - 1 && lane < 16) {
+      const elem* lrp = static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K;
+      const unsigned li = (unsigned)(c < K ? c : K - 1);
+      if (BF)
+        lds_dma2(lrp, 2u * li, stg + L::LR);
+      else
+        lds_dma4(lrp, 4u * li, stg + L::LR);
+    }
+  };
+  // partial sums of this wave's features -> totals in every wave; contains the exchange barrier
+  auto xsum = [&](int region, float (&S)[8]) {
+    const float v0 = xg_sum4_scatter(S[0], S[1], S[2], S[3]);
+    const float v1 = xg_sum4_scatter(S[4], S[5], S[6], S[7]);
+    float* e = SUMp + region * 8 * 16 * NW;
+    e[(g * 16 + c) * NW + w] = v0;
+    e[((g + 4) * 16 + c) * NW + w] = v1;
+    lds_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float s = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < NW; ++ww) s += e[(i * 16 + c) * NW + ww];
+      S[i] = s;
+    }
+  };
+  auto ptsum = [&](int kind) {
+    f32x4 s = pt(kind, 0);
+#pragma unroll
+    for (int ww = 1; ww < NW; ++ww) s += pt(kind, ww);
+    return s;
+  };
+  auto tokens_k = [&](frag x) {
+    f32x4 t = {0.f, 0.f, 0.f, 0.f};
+    IO::mma(t, x, ident);
+    return IO::to_frag(t);
+  };
+  // acc += sum over the NT tiles of A[J] B[J]
+  auto mma_all = [&](f32x4& acc, const frag (&A)[NT], const frag (&B)[NT]) {
+#pragma unroll
+    for (int qq = 0; qq < NQ; ++qq) IO::mma2(acc, A[2 * qq], A[2 * qq + 1], B[2 * qq], B[2 * qq + 1]);
+  };
+  // acc += sum over this wave's tiles
+  auto mma_own = [&](f32x4& acc, const frag (&A)[TPW], const frag (&B)[TPW]) {
+    if (TPW % 2 == 0) {
+#pragma unroll
+      for (int qq = 0; qq < TPW / 2; ++qq) IO::mma2(acc, A[2 * qq], A[2 * qq + 1], B[2 * qq], B[2 * qq + 1]);
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) IO::mma(acc, A[jj], B[jj]);
+    }
+  };
+  auto store_own = [&](void* base, size_t tokoff, const f32x4 (&x)[TPW]) {
+    elem* p = static_cast<elem*>(base) + tokoff;
+    if (TPW == 1) {
+      store4<T>(p + own_offset<TPW>(w, 0, g), x[0]);
+    } else {
+#pragma unroll
+      for (int qq = 0; qq < TPW / 2; ++qq) IO::store8(p + own_offset<TPW>(w, 2 * qq, g), x[2 * qq], x[2 * qq + 1]);
+    }
+  };
+
+  fetch(a.n_stages - 1);
+
+  for (int st = a.n_stages - 1; st >= 0; --st) {
+    // ---- the mini-batch's copies have landed (every wave waits for its own, then all meet)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+    const unsigned char* sl = smem + lane * 16;
+    frag q[NT], k[NT], qo[TPW], ko[TPW], vo[TPW], oo[TPW];  // full rows of xq, xk; own features of all four
+    if constexpr (BF) {
+#pragma unroll
+      for (int s = 0; s < XS; ++s) {
+        const u32x4 rq = *reinterpret_cast<const u32x4*>(sl + L::X + (0 * XS + s) * 1024);
+        const u32x4 rk = *reinterpret_cast<const u32x4*>(sl + L::X + (1 * XS + s) * 1024);
+        q[2 * s] = __builtin_bit_cast(frag, u32x2{rq[0], rq[1]});
+        q[2 * s + 1] = __builtin_bit_cast(frag, u32x2{rq[2], rq[3]});
+        k[2 * s] = __builtin_bit_cast(frag, u32x2{rk[0], rk[1]});
+        k[2 * s + 1] = __builtin_bit_cast(frag, u32x2{rk[2], rk[3]});
+      }
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const int Jo = w * TPW + jj;
+        qo[jj] = *reinterpret_cast<const frag*>(sl + L::X + (0 * XS + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
+        ko[jj] = *reinterpret_cast<const frag*>(sl + L::X + (1 * XS + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
+        vo[jj] = *reinterpret_cast<const frag*>(sl + L::X + (2 * XS + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
+        oo[jj] = *reinterpret_cast<const frag*>(sl + L::X + (3 * XS + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < NT; ++s) {
+        q[s] = *reinterpret_cast<const frag*>(sl + L::X + (0 * XS + s) * 1024);
+        k[s] = *reinterpret_cast<const frag*>(sl + L::X + (1 * XS + s) * 1024);
+      }
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        qo[jj] = *reinterpret_cast<const frag*>(sl + L::X + (0 * XS + w * TPW + jj) * 1024);
+        ko[jj] = *reinterpret_cast<const frag*>(sl + L::X + (1 * XS + w * TPW + jj) * 1024);
+        vo[jj] = *reinterpret_cast<const frag*>(sl + L::X + (2 * XS + w * TPW + jj) * 1024);
+        oo[jj] = *reinterpret_cast<const frag*>(sl + L::X + (3 * XS + w * TPW + jj) * 1024);
+      }
+    }
+    float lr_c;
+    f32x4 lr_s;
+    {
+      const uint32_t* lrw = reinterpret_cast<const uint32_t*>(smem + L::LR);
+      const u32x4 w4 = *reinterpret_cast<const u32x4*>(lrw + 4 * g);
+      auto cv = [&](uint32_t x) { return BF ? __uint_as_float(x << 16) : __uint_as_float(x); };
+      lr_c = (c < K) ? cv(lrw[c]) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) lr_s[r] = (4 * g + r < K) ? cv(w4[r]) : 0.f;
+    }
+    f32x4 bT[TPW];
+    frag Wn[TPW][NT], kdo[TPW], qdo[TPW];
+#pragma unroll
+    for (int ii = 0; ii < TPW; ++ii) {
+      const int Io = w * TPW + ii;
+      bT[ii] = *reinterpret_cast<const f32x4*>(sl + L::Bv + Io * 1024);
+#pragma unroll
+      for (int J = 0; J < NT; ++J)
+        Wn[ii][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + (Io * NT + J) * 1024));
+      kdo[ii] = tokens_k(ko[ii]);
+      qdo[ii] = tokens_k(qo[ii]);
+      fr(KD, Io) = kdo[ii];
+      fr(QD, Io) = qdo[ii];
+    }
+
+    // ---- forward intermediates of the own features: Z1 = XK W + b, Zq = XQ W + b; partial attention blocks
+    f32x4 z1[TPW], zb[TPW];
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      const int Jo = w * TPW + jj;
+      z1[jj] = zb[jj] = bT[jj];
+#pragma unroll
+      for (int qq = 0; qq < NQ; ++qq) {
+        // W tiles (rows 2qq / 2qq+1, own column tile), transposed on the matrix pipe: (m = j, k = i)
+        const frag wa0 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq) * NT + Jo) * 1024)));
+        const frag wa1 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq + 1) * NT + Jo) * 1024)));
+        IO::mma2(z1[jj], wa0, wa1, k[2 * qq], k[2 * qq + 1]);
+        IO::mma2(zb[jj], wa0, wa1, q[2 * qq], q[2 * qq + 1]);
+      }
+    }
+    {
+      f32x4 at = zero4, at2 = zero4;
+      mma_own(at, ko, qo);   // [s = 4g+r][t = c]
+      mma_own(at2, qo, ko);  // [t = 4g+r][s = c]
+      pt(P_AT, w) = at;
+      pt(P_AT2, w) = at2;
+    }
+    // ---- X1: raw moments of Z1
+    f32x4 bq[TPW];
+    float S1[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      bq[jj] = gam[jj] * (bet[jj] - (IO::to_f32(vo[jj]) - IO::to_f32(ko[jj])));
+      const f32x4 az = a2[jj] * z1[jj];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        S1[0] += z1[jj][r];
+        S1[1] += z1[jj][r] * z1[jj][r];
+        S1[2] += az[r];
+        S1[3] += az[r] * z1[jj][r];
+        S1[4] += bq[jj][r];
+        S1[5] += bq[jj][r] * z1[jj][r];
+      }
+    }
+    xsum(0, S1);
+    // every wave has moved the staged mini-batch to registers: the next one may be copied in
+    fetch(st - 1);
+
+    const float mu1 = S1[0] * inv_d;
+    const float rstd1 = __builtin_amdgcn_rsqf(S1[1] * inv_d - mu1 * mu1 + a.eps);
+    const float sa_xh = rstd1 * (S1[2] - mu1 * sum_a);                                    // sum a2 xh
+    const float sa_xh2 = rstd1 * rstd1 * (S1[3] - 2.f * mu1 * S1[2] + mu1 * mu1 * sum_a);  // sum a2 xh^2
+    const float s_gx = sa_xh + S1[4];                                                     // sum gx
+    const float s_gxxh = sa_xh2 + rstd1 * (S1[5] - mu1 * S1[4]);                          // sum gx xh
+    const float mgx = s_gx * inv_d, sgx = s_gxxh * inv_d;
+    f32x4 xh[TPW], gx[TPW], G[TPW];
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      xh[jj] = (z1[jj] - mu1) * rstd1;
+      gx[jj] = a2[jj] * xh[jj] + bq[jj];
+      G[jj] = (gx[jj] - mgx - xh[jj] * sgx) * rstd1;
+    }
+    // ---- eta, tril(A), M = eta (1 + A) in both orientations
+    f32x4 eta, onepA, eta2, onepA2, nM, M2;
+    {
+      const f32x4 At = ptsum(P_AT), At2 = ptsum(P_AT2);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const bool low = 4 * g + r <= c;
+        eta[r] = low ? te_c * lr_s[r] : 0.f;
+        onepA[r] = low ? 1.f + At[r] : 0.f;
+        nM[r] = -eta[r] * onepA[r];
+        const bool low2 = c <= 4 * g + r;
+        eta2[r] = low2 ? te_s[r] * lr_c : 0.f;
+        onepA2[r] = low2 ? 1.f + At2[r] : 0.f;
+        M2[r] = eta2[r] * onepA2[r];
+      }
+    }
+    // ---- Zb = XQ W + b - M G ; X2: raw moments of Zb and of the output-LayerNorm backward
+    frag Gf[TPW];
+    f32x4 gx2[TPW];
+    float S2[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    {
+      const frag nMf = IO::to_frag(nM);
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        Gf[jj] = IO::to_frag(G[jj]);
+        fr(GF, w * TPW + jj) = Gf[jj];
+        IO::mma(zb[jj], tokens_k(Gf[jj]), nMf);
+        gx2[jj] = IO::to_f32(oo[jj]) * gam[jj];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          S2[0] += zb[jj][r];
+          S2[1] += zb[jj][r] * zb[jj][r];
+          S2[2] += gx2[jj][r];
+          S2[3] += gx2[jj][r] * zb[jj][r];
+        }
+      }
+    }
+    xsum(1, S2);
+    frag Zf[TPW], Zd[TPW];
+    {
+      const float mu2 = S2[0] * inv_d;
+      const float rstd2 = __builtin_amdgcn_rsqf(S2[1] * inv_d - mu2 * mu2 + a.eps);
+      const float m1 = S2[2] * inv_d, m2 = rstd2 * (S2[3] - mu2 * S2[2]) * inv_d;
+      f32x4 P = zero4, P2 = zero4;
+      frag Gl[TPW], Zl[TPW];
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const f32x4 x2 = (zb[jj] - mu2) * rstd2;
+        const f32x4 dO = IO::to_f32(oo[jj]);
+        dgam[jj] += dO * x2;
+        dbet[jj] += dO;
+        const f32x4 dzb = (gx2[jj] - m1 - x2 * m2) * rstd2;
+        Zf[jj] = IO::to_frag(dzb);
+        Zd[jj] = tokens_k(Zf[jj]);
+        fr(ZF, w * TPW + jj) = Zf[jj];
+        fr(ZD, w * TPW + jj) = Zd[jj];
+        if (BF) {
+          // P feeds the gradients of eta (small differences of large sums): bf16 head + tail of both factors
+          Gl[jj] = IO::to_frag(G[jj] - IO::to_f32(Gf[jj]));
+          Zl[jj] = IO::to_frag(dzb - IO::to_f32(Zf[jj]));
+        }
+      }
+      // ---- X3: partial P = dZb G^T in both orientations
+      mma_own(P, Gf, Zf);   // [s][t]
+      mma_own(P2, Zf, Gf);  // [t][s]
+      if (BF) {
+        mma_own(P, Gl, Zf);
+        mma_own(P, Gf, Zl);
+        mma_own(P2, Zl, Gf);
+        mma_own(P2, Zf, Gl);
+      }
+      pt(P_P, w) = P;
+      pt(P_P2, w) = P2;
+    }
+    lds_barrier();
+    f32x4 dA, dEta, dA2, dEta2;
+    {
+      const f32x4 P = ptsum(P_P), P2 = ptsum(P_P2);
+      dA = -P * eta;
+      dEta = -P * onepA;
+      dA2 = -P2 * eta2;
+      dEta2 = -P2 * onepA2;
+    }
+    const bool tok_ok = c < K;
+    const size_t tokoff = (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
+    frag Zfa[NT], Gfa[NT];
+#pragma unroll
+    for (int J = 0; J < NT; ++J) {
+      Zfa[J] = fr(ZF, J);
+      Gfa[J] = fr(GF, J);
+    }
+    // ---- dXQ = dO + dZb W^T + dA XK   (own features)
+    {
+      const frag dAf = IO::to_frag(dA);
+      f32x4 dQ[TPW];
+#pragma unroll
+      for (int ii = 0; ii < TPW; ++ii) {
+        dQ[ii] = IO::to_f32(oo[ii]);
+        mma_all(dQ[ii], Wn[ii], Zfa);
+        // bf16: a k = 16 instruction accumulating straight onto the result of a k = 32 one has given wrong
+        // sums, so the rank-16 term is issued as k = 32 with a zero half
+        if (BF)
+          IO::mma2(dQ[ii], kdo[ii], IO::zero(), dAf, IO::zero());
+        else
+          IO::mma(dQ[ii], kdo[ii], dAf);
+      }
+      if (tok_ok) store_own(a.d_xq, tokoff, dQ);
+    }
+    // ---- dK = dA^T XQ ; DGM = M^T dZb ; S = XK dW + db ; TMP = G dW^T   (own features)
+    f32x4 dK[TPW], DGM[TPW], S[TPW], TMP[TPW];
+    {
+      const frag dA2f = IO::to_frag(dA2), M2f = IO::to_frag(M2);
+#pragma unroll
+      for (int ii = 0; ii < TPW; ++ii) {
+        dK[ii] = DGM[ii] = TMP[ii] = zero4;
+        S[ii] = dbT[ii];
+        IO::mma(dK[ii], qdo[ii], dA2f);
+        IO::mma(DGM[ii], Zd[ii], M2f);
+#pragma unroll
+        for (int qq = 0; qq < NQ; ++qq) {
+          IO::mma2(S[ii], IO::to_frag(dWc[2 * qq][ii]), IO::to_frag(dWc[2 * qq + 1][ii]), k[2 * qq], k[2 * qq + 1]);
+          IO::mma2(TMP[ii], IO::to_frag(DT[2 * qq][ii]), IO::to_frag(DT[2 * qq + 1][ii]), Gfa[2 * qq], Gfa[2 * qq + 1]);
+        }
+      }
+    }
+    // ---- X4: the six sums of the second-order LayerNorm
+    const float last = te_last * lr_c;
+    f32x4 u[TPW];
+    float S4[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      u[jj] = (DGM[jj] + last * S[jj]) * rstd1;  // u = -dG rstd1
+      const f32x4 au = a2[jj] * u[jj];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        S4[0] += u[jj][r];
+        S4[1] += u[jj][r] * xh[jj][r];
+        S4[2] += au[r];
+        S4[3] += au[r] * xh[jj][r];
+        S4[4] += u[jj][r] * gx[jj][r];
+        S4[5] += G[jj][r] * S[jj][r];
+      }
+    }
+    xsum(2, S4);
+    const float dl = -S4[5];
+    frag Z1f[TPW], Z1d[TPW];
+    {
+      const float s1 = S4[0] * inv_d, s2 = S4[1] * inv_d;
+      const float q1 = (s1 * sum_a + s2 * sa_xh - S4[2] + s2 * s_gx + sgx * S4[0]) * inv_d;
+      const float q2 = s1 * sa_xh + s2 * sa_xh2 - S4[3] + s2 * s_gxxh + sgx * S4[1];  // sum dxh xh
+      const float s_uG = rstd1 * (S4[4] - mgx * S4[0] - sgx * S4[1]);                  // sum u G
+      const float dsig = -(q2 * rstd1 - s_uG);
+      f32x4 ndy[TPW];
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const f32x4 dgx = s1 + xh[jj] * s2 - u[jj];
+        const f32x4 dy = gam[jj] * dgx;
+        // gO = gamma xh + beta - target = gx / gamma, kept as gamma-free form through bq
+        const f32x4 gO = gam[jj] * xh[jj] + bet[jj] - (IO::to_f32(vo[jj]) - IO::to_f32(ko[jj]));
+        dgam[jj] += gO * dgx + dy * xh[jj];
+        dbet[jj] += dy;
+        const f32x4 dxh = dy * gam[jj] + gx[jj] * s2 + u[jj] * sgx;
+        Z1f[jj] = IO::to_frag((dxh - q1) * rstd1 + xh[jj] * (dsig * inv_d));
+        Z1d[jj] = tokens_k(Z1f[jj]);
+        fr(Z1F, w * TPW + jj) = Z1f[jj];
+        fr(Z1D, w * TPW + jj) = Z1d[jj];
+        dK[jj] += dy - last * TMP[jj];
+        ndy[jj] = -dy;
+      }
+      if (tok_ok) store_own(a.d_xv, tokoff, ndy);
+    }
+    // ---- X5: dZ1 fragments
+    lds_barrier();
+    {
+      frag Z1fa[NT];
+#pragma unroll
+      for (int J = 0; J < NT; ++J) Z1fa[J] = fr(Z1F, J);
+#pragma unroll
+      for (int ii = 0; ii < TPW; ++ii) mma_all(dK[ii], Wn[ii], Z1fa);
+      if (tok_ok) store_own(a.d_xk, tokoff, dK);
+    }
+    // ---- d lr, d token_eta (one wave)
+    if (w == 0) {
+      float e2 = 0.f, e1 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        e2 += dEta2[r] * te_s[r];
+        e1 += dEta[r] * lr_s[r];
+      }
+      const float dlr = xg_sum(e2) + te_last * dl;
+      float dte = xg_sum(e1);
+      const float tail = row16_sum_dpp(dl * lr_c);
+      if (c == K - 1) dte += tail;
+      if (g == 0 && tok_ok) {
+        IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + c, dlr);
+        atomicAdd(a.d_token_eta + (size_t)st * K + c, dte);
+      }
+    }
+    // ---- state gradient: dW += XQ^T dZb + XK^T dZ1 (column slice and transposed row slice), db
+#pragma unroll
+    for (int I = 0; I < NT; ++I) {
+      const frag qa = fr(QD, I), ka = fr(KD, I), za = fr(ZD, I), z1a = fr(Z1D, I);
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        IO::mma2(dWc[I][jj], qa, ka, Zd[jj], Z1d[jj]);
+        IO::mma2(DT[I][jj], za, z1a, qdo[jj], kdo[jj]);
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) IO::mma2(dbT[jj], Zd[jj], Z1d[jj], ones, ones);
+  }
+
+  // ---- results carried over the whole scan
+#pragma unroll
+  for (int I = 0; I < NT; ++I)
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        a.d_W0[bh * D * D + feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = dWc[I][jj][r];
+#pragma unroll
+  for (int jj = 0; jj < TPW; ++jj) {
+    const int f = own_offset<TPW>(w, jj, g);
+    if (c == 0) store4<F32>(a.d_b0 + bh * D + f, dbT[jj]);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float sg = row16_sum_dpp(dgam[jj][r]), sbt = row16_sum_dpp(dbet[jj][r]);
+      if (c == 0) {
+        atomicAdd(a.d_gamma + h * D + f + r, sg);
+        atomicAdd(a.d_beta + h * D + f + r, sbt);
+      }
+    }
+  }
+}
+
+}  // namespace ttt
