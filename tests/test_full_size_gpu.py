@@ -83,11 +83,12 @@ def test_config2_linear_fwd_bwd_f32_full(P):
         return out, g
 
     out, g = fwd_bwd(dv, 1)
-    # a coarser checkpoint interval (re-simulated states) must give the same gradients
+    # a coarser checkpoint interval (states re-simulated, LDS-tile kernel instead of the register-resident
+    # one: a different summation order) must give the same gradients to the f32 bar
     _, g16 = fwd_bwd(dv, 16)
     torch.cuda.synchronize()
     for k in g:
-        assert_close(g16[k], g[k].double(), 1e-5, "ci16 " + k)
+        assert_close(g16[k], g[k].double(), 1e-4, "ci16 " + k)
     # one batch entry alone: per-unit gradients are identical, reduced ones are that entry's share
     one = {k: (v[3:4].contiguous() if k in ("xq", "xk", "xv", "lr", "d_out") else v) for k, v in dv.items()}
     o1, g1 = fwd_bwd(one, 1)

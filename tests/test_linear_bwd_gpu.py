@@ -144,3 +144,29 @@ def test_bwd_multi_wave_kernel(P, monkeypatch, B, H, d, K, N, dtype):
         c = P.synthetic.baseline_inputs(2, B, H, N * K, d, K, io_dtype=dtype, with_dout=True)
         dO = c.pop("d_out")
         compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("B,H,d,K,N", [(1, 2, 96, 16, 3), (2, 1, 96, 7, 2), (1, 2, 128, 16, 3)])
+def test_bwd_wide_heads(P, B, H, d, K, N, dtype):
+    """head_dim 96 and 128 (feature-split kernel only; 128 needs bf16 I/O: the f32 staging does not fit LDS)."""
+    print(f"case bwd wide B{B} H{H} d{d} K{K} N{N} {dtype}", flush=True)
+    c = P.synthetic.reference_test_inputs(400 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
+    g = torch.Generator().manual_seed(10)
+    dO = torch.randn(B, H, N * K, d, generator=g).to(dtype)
+    sg = (0.1 * torch.randn(B, H, d, d, generator=g), 0.1 * torch.randn(B, H, d, generator=g))
+    if d == 128 and dtype == torch.float32:
+        with pytest.raises(Exception, match="head_dim 128"):
+            run_bwd(P, c, dO, K, 1, sg)
+        return
+    compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), TOL[dtype])
+    if K == 16:
+        c = P.synthetic.baseline_inputs(4, B, H, N * K, d, K, io_dtype=dtype, with_dout=True)
+        dO = c.pop("d_out")
+        compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])
+
+
+def test_bwd_wide_heads_need_a_checkpoint_per_mini_batch(P):
+    c = P.synthetic.reference_test_inputs(1, 1, 1, 32, 96, 16)
+    with pytest.raises(Exception, match="checkpoint_interval 1"):
+        run_bwd(P, c, torch.ones(1, 1, 32, 96), 16, 2)

@@ -327,8 +327,6 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
                    void* stream) {
   int rc = ttt_linear_supported(d);
   if (rc != TTT_OK) return rc;
-  if (d->head_dim > 64)
-    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim %d has no kernel (32, 64)", d->head_dim);
   // W0/b0 are part of the saved state for interface parity; the state entering every stage is
   // rebuilt from the checkpoints (checkpoint 0 equals the initial state).
   (void)W0;
@@ -360,30 +358,47 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((hd + 255) / 256)), dim3(256), 0, s,
                      d_beta, hd);
   const unsigned grid = (unsigned)(a.B * a.H);
-  if (d->io_dtype == TTT_F32) {
-    const char* wsel = std::getenv("TTT_LINEAR_BWD_WAVES");
-    if (a.ckpt_interval == 1 && wsel && std::atoi(wsel) > 1) {
-      if (d->head_dim == 64) return launch_linear_bwd_mw<ttt::F32, 64, 4>(a, grid, s);
-      return launch_linear_bwd_mw<ttt::F32, 32, 2>(a, grid, s);
-    }
-    if (d->head_dim == 64) return launch_linear_bwd<ttt::F32, 64>(a, grid, s);
-    return launch_linear_bwd<ttt::F32, 32>(a, grid, s);
-  }
+  const bool f32 = d->io_dtype == TTT_F32;
+  const int D = d->head_dim;
+  // Kernel choice.  One checkpoint per mini-batch: the register-resident kernels (the state entering a
+  // mini-batch is read, not re-simulated).  Waves per (batch, head): f32 products are bound by the matrix
+  // pipe, so the feature axis is always split; bf16 runs one wave per unit when there are more units than
+  // two per CU and the split kernel otherwise.  TTT_LINEAR_BWD_KERNEL=lds and TTT_LINEAR_BWD_WAVES override.
   const char* ksel = std::getenv("TTT_LINEAR_BWD_KERNEL");
-  if (a.ckpt_interval == 1 && !(ksel && std::strcmp(ksel, "lds") == 0)) {
+  const bool want_lds = ksel && std::strcmp(ksel, "lds") == 0;
+  if (a.ckpt_interval == 1 && !(want_lds && D <= 64)) {
     if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(d_out) || !aligned16(d_xq) ||
-        !aligned16(d_xk) || !aligned16(d_xv) || !aligned16(W_ckpt) || !aligned16(b_ckpt) || (a.seq_stride * d->head_dim) % 8 != 0)
+        !aligned16(d_xk) || !aligned16(d_xv) || !aligned16(W_ckpt) || !aligned16(b_ckpt) ||
+        ((size_t)a.seq_stride * D) % 8 != 0)
       return fail(TTT_ERR_SHAPE, "ttt_linear_bwd: tensors must be 16-byte aligned");
     const char* wsel = std::getenv("TTT_LINEAR_BWD_WAVES");
-    const int waves = wsel ? std::atoi(wsel) : 1;
-    if (waves > 1) {
-      if (d->head_dim == 64) return launch_linear_bwd_mw<ttt::BF16, 64, 4>(a, grid, s);
-      return launch_linear_bwd_mw<ttt::BF16, 32, 2>(a, grid, s);
+    int waves = wsel ? std::atoi(wsel) : 0;
+    if (waves == 0) waves = (f32 || D > 64 || grid <= 512) ? 4 : 1;
+    if (f32) {
+      if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2>(a, grid, s);
+      if (D == 64) return waves == 2 ? launch_linear_bwd_mw<ttt::F32, 64, 2>(a, grid, s)
+                                     : launch_linear_bwd_mw<ttt::F32, 64, 4>(a, grid, s);
+      if (D == 96) return launch_linear_bwd_mw<ttt::F32, 96, 3>(a, grid, s);
+      return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
     }
-    if (d->head_dim == 64) return launch_linear_bwd_rr<64>(a, grid, s);
-    return launch_linear_bwd_rr<32>(a, grid, s);
+    if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2>(a, grid, s) : launch_linear_bwd_rr<32>(a, grid, s);
+    if (D == 64) {
+      if (waves == 1) return launch_linear_bwd_rr<64>(a, grid, s);
+      return waves == 2 ? launch_linear_bwd_mw<ttt::BF16, 64, 2>(a, grid, s)
+                        : launch_linear_bwd_mw<ttt::BF16, 64, 4>(a, grid, s);
+    }
+    if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3>(a, grid, s);
+    return launch_linear_bwd_mw<ttt::BF16, 128, 4>(a, grid, s);
   }
-  if (d->head_dim == 64) return launch_linear_bwd<ttt::BF16, 64>(a, grid, s);
+  // coarser checkpoints (states re-simulated from the last checkpoint), or on request: LDS-tile kernel
+  if (D > 64)
+    return fail(TTT_ERR_UNSUPPORTED,
+                "ttt_linear_bwd: head_dim %d needs checkpoint_interval 1 (got %d)", D, a.ckpt_interval);
+  if (f32) {
+    if (D == 64) return launch_linear_bwd<ttt::F32, 64>(a, grid, s);
+    return launch_linear_bwd<ttt::F32, 32>(a, grid, s);
+  }
+  if (D == 64) return launch_linear_bwd<ttt::BF16, 64>(a, grid, s);
   return launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
 }
 
