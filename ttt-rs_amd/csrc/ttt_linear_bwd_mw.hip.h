@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       const int n = w + NW * it, I = n / NT, J = n - I * NT;
       lds_dma16(Wg, (unsigned)(feat(I, c) * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::W + n * 1024);
     }
-    if (w == 0) {
+    if (w == 1 % NW) {
       const float* bg = a.b_ckpt + ci * D;
 #pragma unroll
       for (int J = 0; J < NT; ++J) lds_dma16(bg, (unsigned)(32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::Bv + J * 1024);
@@ -504,22 +504,23 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       for (int ii = 0; ii < TPW; ++ii) mma_all(dK[ii], Wn[ii], Z1fa);
       if (tok_ok) store_own(a.d_xk, tokoff, dK);
     }
-    // ---- d lr, d token_eta (one wave)
+    // ---- d lr (first wave), d token_eta (last wave): work of a single wave is skew at the next barrier
     if (w == 0) {
-      float e2 = 0.f, e1 = 0.f;
+      float e2 = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        e2 += dEta2[r] * te_s[r];
-        e1 += dEta[r] * lr_s[r];
-      }
+      for (int r = 0; r < 4; ++r) e2 += dEta2[r] * te_s[r];
       const float dlr = xg_sum(e2) + te_last * dl;
+      if (g == 0 && tok_ok)
+        IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + c, dlr);
+    }
+    if (w == NW - 1) {
+      float e1 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) e1 += dEta[r] * lr_s[r];
       float dte = xg_sum(e1);
       const float tail = row16_sum_dpp(dl * lr_c);
       if (c == K - 1) dte += tail;
-      if (g == 0 && tok_ok) {
-        IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + c, dlr);
-        atomicAdd(a.d_token_eta + (size_t)st * K + c, dte);
-      }
+      if (g == 0 && tok_ok) atomicAdd(a.d_token_eta + (size_t)st * K + c, dte);
     }
     // ---- state gradient: dW += XQ^T dZb + XK^T dZ1 (column slice and transposed row slice), db
 #pragma unroll
