@@ -239,7 +239,7 @@ def main():
         out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci)
         out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                           "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_rr_kernel (whole step)",
+                           "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_bytes": alg,
                            "checkpoint_bytes": 2 * th * (d * d + d) * 4 // (ci * K),
                            "algorithmic_flops": th * (24 * d * d + 26 * K * d)}
@@ -250,7 +250,7 @@ def main():
         out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci)
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
                            "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
-                           "kernel": "ttt_linear_fwd_kernel + ttt_linear_bwd_kernel (whole step)",
+                           "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops,
                            "algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)}
     elif kind == "mlp_fwd":
