@@ -178,13 +178,17 @@ def main():
                                              dv["d_out"], K)
                 return (fw[0], g["d_xq"])
         else:
+            # bf16 I/O, a checkpoint per mini-batch: checkpoints as bf16 operand fragments (same gradients bit
+            # for bit, half the checkpoint traffic); TTT_BENCH_CKPT=f32 keeps the reference's f32 matrices
+            packed = io == "bf16" and ci == 1 and os.environ.get("TTT_BENCH_CKPT") != "f32"
+
             def step():
                 out, W, b, Wc, bc = pkg.ttt_linear_forward_raw(
                     dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
-                    dv["gamma"], dv["beta"], K, 1e-6, ci, want_checkpoints=True)
+                    dv["gamma"], dv["beta"], K, 1e-6, ci, want_checkpoints=True, packed_checkpoints=packed)
                 g = pkg.ttt_linear_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
                                                 dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], Wc, bc,
-                                                dv["d_out"], K, 1e-6, ci)
+                                                dv["d_out"], K, 1e-6, ci, packed_checkpoints=packed)
                 return (out, g["grad_xq"])
 
     for _ in range(a.warmup):
@@ -236,12 +240,13 @@ def main():
         # register-resident backward (bf16 MFMA operands): the pair of passes is bound by HBM in the limit
         alg = linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)
         out["dtype"] = "bf16"
-        out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci)
+        out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci,
+                             checkpoint_format="f32" if os.environ.get("TTT_BENCH_CKPT") == "f32" else "packed bf16")
         out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
                            "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_bytes": alg,
-                           "checkpoint_bytes": 2 * th * (d * d + d) * 4 // (ci * K),
+                           "checkpoint_bytes": 2 * th * (d * d * (2 if os.environ.get("TTT_BENCH_CKPT") != "f32" else 4) + d * 4) // (ci * K),
                            "algorithmic_flops": th * (24 * d * d + 26 * K * d)}
     elif kind == "linear_fwd_bwd":
         # the backward kernel dominates; it computes in f32 MFMA: 18 d^2 + 22 K d flop per token-head

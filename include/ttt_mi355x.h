@@ -55,7 +55,19 @@ typedef struct ttt_desc {
                                   sequence (the reference's slice_seq, rust/core/src/inner.rs:70-77)
                                   is processed in place by pointing at its first token and passing
                                   the full length here. */
+  int32_t checkpoint_format;   /* 0: W checkpoints are f32 [d,d] row-major matrices (what the reference
+                                  saves, rust/fused/src/linear_fused_tile/forward/launch.rs:117-208),
+                                  any interval, readable by the caller.
+                                  1 (TTT_CKPT_PACKED): bf16 I/O with checkpoint_interval 1 only; a W
+                                  checkpoint is the bf16 image of the state in the kernels' own operand
+                                  order (the first d*d*2 bytes of its d*d*4-byte slot; same allocation),
+                                  written by ttt_linear_fwd and meaningful only to ttt_linear_bwd.  The
+                                  backward's products take bf16 operands anyway, so its results do not
+                                  change; half the checkpoint traffic, stored and fetched in whole
+                                  1 KiB rows.  No counterpart in the reference. */
 } ttt_desc;
+#define TTT_CKPT_F32 0
+#define TTT_CKPT_PACKED 1
 
 /* Library / build identification. */
 const char* ttt_version(void);

@@ -170,3 +170,43 @@ def test_bwd_wide_heads_need_a_checkpoint_per_mini_batch(P):
     c = P.synthetic.reference_test_inputs(1, 1, 1, 32, 96, 16)
     with pytest.raises(Exception, match="checkpoint_interval 1"):
         run_bwd(P, c, torch.ones(1, 1, 32, 96), 16, 2)
+
+
+@pytest.mark.parametrize("waves", ["1", "4"])
+@pytest.mark.parametrize("B,H,d,K,N", [(2, 2, 32, 8, 3), (2, 3, 64, 16, 8), (1, 2, 64, 5, 3), (1, 2, 96, 16, 3), (1, 2, 128, 16, 3)])
+def test_bwd_packed_checkpoints_change_nothing(P, monkeypatch, B, H, d, K, N, waves):
+    """bf16 I/O: checkpoints stored as bf16 operand fragments.  The backward rounds the state to bf16 before
+    its first product either way, so every gradient is bit-identical to the f32-checkpoint run; the forward's
+    outputs do not depend on the checkpoint format at all."""
+    if d > 64 and waves == "1":
+        pytest.skip("wide heads have the feature-split kernel only")
+    print(f"case bwd packed ckpt B{B} H{H} d{d} K{K} N{N} waves {waves}", flush=True)
+    monkeypatch.setenv("TTT_LINEAR_BWD_WAVES", waves)
+    c = P.synthetic.reference_test_inputs(500 + B + d + K + N, B, H, N * K, d, K, io_dtype=torch.bfloat16)
+    dv = to_dev(c)
+    g = torch.Generator().manual_seed(11)
+    dO = torch.randn(B, H, N * K, d, generator=g).to(torch.bfloat16).to("cuda:0")
+    res = []
+    for packed in (False, True):
+        out, W, b, Wc, bc = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"],
+                                                     dv["lr"], dv["gamma"], dv["beta"], K, 1e-6, 1,
+                                                     want_checkpoints=True, packed_checkpoints=packed)
+        gr = P.ttt_linear_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                                       dv["gamma"], dv["beta"], Wc, bc, dO, K, 1e-6, 1, packed_checkpoints=packed)
+        torch.cuda.synchronize()
+        res.append((out, W, b, gr))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][2], res[1][2])
+    for k in res[0][3]:
+        if k in ("grad_token_eta", "grad_ln_weight", "grad_ln_bias"):  # atomics: order of the additions varies
+            assert_close(res[1][3][k], res[0][3][k].double(), 1e-5, k)
+        else:
+            assert torch.equal(res[0][3][k], res[1][3][k]), k
+    compare(res[1][3], oracle_bwd(c, dO.cpu(), K), TOL[torch.bfloat16])
+
+
+def test_packed_checkpoints_rejected_where_unsupported(P):
+    c = P.synthetic.reference_test_inputs(2, 1, 1, 32, 32, 16)
+    dv = to_dev(c)
+    with pytest.raises(Exception, match="packed checkpoints"):
+        P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                                 dv["gamma"], dv["beta"], 16, 1e-6, 1, want_checkpoints=True, packed_checkpoints=True)

@@ -23,6 +23,7 @@ class TttDesc(C.Structure):
         ("batch", C.c_int32), ("heads", C.c_int32), ("seq", C.c_int32), ("head_dim", C.c_int32),
         ("mini_batch", C.c_int32), ("eps", C.c_float), ("checkpoint_interval", C.c_int32),
         ("io_dtype", C.c_int32), ("state_per_batch", C.c_int32), ("seq_stride", C.c_int32),
+        ("checkpoint_format", C.c_int32),
     ]
 
 

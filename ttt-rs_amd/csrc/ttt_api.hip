@@ -44,6 +44,8 @@ int check_common(const ttt_desc* d) {
   if (d->io_dtype != TTT_F32 && d->io_dtype != TTT_BF16)
     return fail(TTT_ERR_UNSUPPORTED, "io_dtype %d is neither TTT_F32 nor TTT_BF16", d->io_dtype);
   if (!(d->eps > 0.f)) return fail(TTT_ERR_SHAPE, "eps must be positive");
+  if (d->checkpoint_format != TTT_CKPT_F32 && d->checkpoint_format != TTT_CKPT_PACKED)
+    return fail(TTT_ERR_SHAPE, "checkpoint_format %d is neither TTT_CKPT_F32 nor TTT_CKPT_PACKED", d->checkpoint_format);
   if (d->seq_stride != 0 && d->seq_stride < d->seq)
     return fail(TTT_ERR_SHAPE, "seq_stride (%d) must be 0 or >= seq (%d)", d->seq_stride, d->seq);
   if ((int64_t)d->batch * d->heads > 0x7fffffffLL)
@@ -187,10 +189,10 @@ int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s)
 }
 
 // bf16 I/O, one checkpoint per mini-batch: one wave per (batch, head), state gradient in registers
-template <int D>
+template <int D, bool PK = false>
 int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  auto kern = ttt::ttt_linear_bwd_rr_kernel<ttt::BF16, D>;
-  constexpr size_t bytes = ttt::LinBwdRrLds<D>::BYTES;
+  auto kern = ttt::ttt_linear_bwd_rr_kernel<ttt::BF16, D, PK>;
+  constexpr size_t bytes = ttt::LinBwdRrLds<D, PK>::BYTES;
   int rc = opt_in_lds(kern, bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64), bytes, s, a);
@@ -198,10 +200,10 @@ int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
 }
 
 // one checkpoint per mini-batch, NW waves per (batch, head): feature axis split, exchanges through LDS
-template <class T, int D, int NW>
+template <class T, int D, int NW, bool PK = false>
 int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW>;
-  constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem)>::BYTES;
+  auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK>;
+  constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem), PK>::BYTES;
   int rc = opt_in_lds(kern, bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), bytes, s, a);
@@ -298,7 +300,13 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.ckpt_interval = d->checkpoint_interval;
   a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
   a.state_per_batch = d->state_per_batch ? 1 : 0;
+  a.ckpt_packed = (W_ckpt != nullptr && d->checkpoint_format == TTT_CKPT_PACKED) ? 1 : 0;
   a.eps = d->eps;
+  if (a.ckpt_packed) {
+    const char* k = std::getenv("TTT_LINEAR_FWD_KERNEL");
+    if (d->io_dtype != TTT_BF16 || d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
+      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need bf16 I/O, checkpoint_interval 1 and the register-resident kernels");
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   // register-resident kernels for every head_dim; the LDS-tile kernel (96/128) only on request
   const bool f32 = d->io_dtype == TTT_F32;
@@ -346,7 +354,13 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.n_stages = d->seq / d->mini_batch;
   a.ckpt_interval = d->checkpoint_interval;
   a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
+  a.ckpt_packed = d->checkpoint_format == TTT_CKPT_PACKED;
   a.eps = d->eps;
+  if (a.ckpt_packed) {
+    const char* k = std::getenv("TTT_LINEAR_BWD_KERNEL");
+    if (d->io_dtype != TTT_BF16 || d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
+      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need bf16 I/O, checkpoint_interval 1 and the register-resident kernels");
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   // accumulated outputs start from zero; a fill kernel (not a memset node) so the sequence
   // can be captured into a graph
@@ -380,6 +394,12 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
                                      : launch_linear_bwd_mw<ttt::F32, 64, 4>(a, grid, s);
       if (D == 96) return launch_linear_bwd_mw<ttt::F32, 96, 3>(a, grid, s);
       return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
+    }
+    if (a.ckpt_packed) {
+      if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2, true>(a, grid, s) : launch_linear_bwd_rr<32, true>(a, grid, s);
+      if (D == 64) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 64, 4, true>(a, grid, s) : launch_linear_bwd_rr<64, true>(a, grid, s);
+      if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3, true>(a, grid, s);
+      return launch_linear_bwd_mw<ttt::BF16, 128, 4, true>(a, grid, s);
     }
     if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2>(a, grid, s) : launch_linear_bwd_rr<32>(a, grid, s);
     if (D == 64) {

@@ -46,6 +46,7 @@ struct LinearBwdArgs {
   float* d_gamma;
   float* d_beta;
   int B, H, seq, seq_stride, K, n_stages, ckpt_interval, n_ckpt;
+  int ckpt_packed;  // W checkpoints as bf16 operand fragments (register-resident kernels, bf16 I/O)
   float eps;
 };
 

@@ -27,31 +27,35 @@
 
 namespace ttt {
 
-template <int D, int NW, int ES>
+// PK: the W checkpoint arrives packed (bf16 fragments in accumulator order, see store_ckpt_packed)
+template <int D, int NW, int ES, bool PK = false>
 struct LinBwdMwLds {
   static constexpr int NT = D / 16, TPW = NT / NW;
   static constexpr int XS = (ES == 2) ? NT / 2 : NT;  // 1 KiB slots per activation tensor
   static constexpr int FT = 64 * 4 * ES;              // bytes of one fragment tile
   static constexpr int W = 0;                         // NT*NT slots: slot I*NT+J, lane (c,g): W[feat(I,c)][feat(J,4g..4g+3)]
-  static constexpr int Bv = W + NT * NT * 1024;       // NT slots: b[feat(J,4g..4g+3)]
+                                                      // packed: NT*NT/2 slots: slot I*NT/2+q = tiles (I,2q), (I,2q+1)
+  static constexpr int WSLOTS = PK ? NT * NT / 2 : NT * NT;
+  static constexpr int Bv = W + WSLOTS * 1024;        // NT slots: b[feat(J,4g..4g+3)]
   static constexpr int X = Bv + NT * 1024;            // 4 tensors x XS slots
   static constexpr int LR = X + 4 * XS * 1024;        // 16 dwords: lr of token c (bf16 zero-extended, or f32)
   static constexpr int SUM = LR + 256;                // 3 exchanges x [8 sums][16 tokens][NW]
   static constexpr int PT = SUM + 3 * 8 * 16 * NW * 4;  // 4 kinds x [NW][64] f32x4: partial [16 x 16] blocks
   static constexpr int FR = PT + 4 * NW * 1024;       // 7 kinds x [NT][64] fragments
   static constexpr int BYTES = FR + 7 * NT * FT;
-  static_assert(NT % NW == 0, "feature tiles must divide among the waves");
+  static_assert(NT % NW == 0 && WSLOTS % NW == 0, "feature tiles must divide among the waves");
+  static_assert(!PK || ES == 2, "packed checkpoints are bf16");
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
 
-template <class T, int D, int NW>
+template <class T, int D, int NW, bool PK = false>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;
   constexpr int ES = sizeof(elem);
   constexpr bool BF = ES == 2;
-  using L = LinBwdMwLds<D, NW, ES>;
+  using L = LinBwdMwLds<D, NW, ES, PK>;
   constexpr int NT = D / 16, TPW = NT / NW, NQ = NT / 2, XS = L::XS;
   constexpr float inv_d = 1.0f / D;
   enum { KD = 0, QD, GF, ZF, ZD, Z1F, Z1D };
@@ -116,9 +120,12 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     const size_t ci = bh * (size_t)a.n_ckpt + stage;
     const float* Wg = a.W_ckpt + ci * D * D;
 #pragma unroll
-    for (int it = 0; it < NT * NT / NW; ++it) {
+    for (int it = 0; it < L::WSLOTS / NW; ++it) {
       const int n = w + NW * it, I = n / NT, J = n - I * NT;
-      lds_dma16(Wg, (unsigned)(feat(I, c) * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::W + n * 1024);
+      if (PK)  // whole 1 KiB rows
+        lds_dma16(Wg, (unsigned)(n * 1024 + lane * 16), stg + L::W + n * 1024);
+      else
+        lds_dma16(Wg, (unsigned)(feat(I, c) * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::W + n * 1024);
     }
     if (w == 1 % NW) {
       const float* bg = a.b_ckpt + ci * D;
@@ -258,8 +265,12 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       const int Io = w * TPW + ii;
       bT[ii] = *reinterpret_cast<const f32x4*>(sl + L::Bv + Io * 1024);
 #pragma unroll
-      for (int J = 0; J < NT; ++J)
-        Wn[ii][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + (Io * NT + J) * 1024));
+      for (int J = 0; J < NT; ++J) {
+        if constexpr (PK)  // stored as (m = j, k = i): transposed on the matrix pipe
+          Wn[ii][J] = tokens_k(*reinterpret_cast<const frag*>(sl + L::W + (Io * NQ + (J >> 1)) * 1024 + 8 * (J & 1)));
+        else
+          Wn[ii][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + (Io * NT + J) * 1024));
+      }
       kdo[ii] = tokens_k(ko[ii]);
       qdo[ii] = tokens_k(qo[ii]);
       fr(KD, Io) = kdo[ii];
@@ -275,8 +286,14 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
 #pragma unroll
       for (int qq = 0; qq < NQ; ++qq) {
         // W tiles (rows 2qq / 2qq+1, own column tile), transposed on the matrix pipe: (m = j, k = i)
-        const frag wa0 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq) * NT + Jo) * 1024)));
-        const frag wa1 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq + 1) * NT + Jo) * 1024)));
+        frag wa0, wa1;
+        if constexpr (PK) {
+          wa0 = *reinterpret_cast<const frag*>(sl + L::W + ((2 * qq) * NQ + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
+          wa1 = *reinterpret_cast<const frag*>(sl + L::W + ((2 * qq + 1) * NQ + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
+        } else {
+          wa0 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq) * NT + Jo) * 1024)));
+          wa1 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq + 1) * NT + Jo) * 1024)));
+        }
         IO::mma2(z1[jj], wa0, wa1, k[2 * qq], k[2 * qq + 1]);
         IO::mma2(zb[jj], wa0, wa1, q[2 * qq], q[2 * qq + 1]);
       }

@@ -27,23 +27,25 @@
 
 namespace ttt {
 
-template <int D>
+// PK: the W checkpoint arrives packed (bf16 fragments in accumulator order, see store_ckpt_packed)
+template <int D, bool PK = false>
 struct LinBwdRrLds {
   static constexpr int NT = D / 16;
   static constexpr int W = 0;                       // NT*NT slots of 1 KiB: slot I*NT+J, lane (c,g): W[feat(I,c)][feat(J,4g..4g+3)]
-  static constexpr int Bv = W + NT * NT * 1024;     // NT slots: b[feat(J,4g..4g+3)]
+                                                    // packed: NT*NT/2 slots: slot I*NT/2+q = tiles (I,2q), (I,2q+1)
+  static constexpr int Bv = W + (PK ? NT * NT / 2 : NT * NT) * 1024;  // NT slots: b[feat(J,4g..4g+3)]
   static constexpr int X = Bv + NT * 1024;          // 4 tensors x NT/2 slots: X[token c][32q + 8g .. +7] (bf16)
   static constexpr int LR = X + 4 * (NT / 2) * 1024;  // 16 dwords: lr of token c, zero-extended bf16
   static constexpr int STAGE = LR + 256;
   static constexpr int BYTES = 2 * STAGE;
 };
 
-template <class T, int D>
+template <class T, int D, bool PK = false>
 __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;
-  using L = LinBwdRrLds<D>;
+  using L = LinBwdRrLds<D, PK>;
   static_assert(sizeof(elem) == 2, "bf16 I/O only");
   constexpr int NT = D / 16, NQ = NT / 2;
   constexpr float inv_d = 1.0f / D;
@@ -104,9 +106,14 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
     const unsigned xoff = (unsigned)(c * D + 8 * g) * 2u;
     if (part < NT) {
       const int I = part;
+      if (PK) {
 #pragma unroll
-      for (int J = 0; J < NT; ++J)
-        dma(Wg, (unsigned)(feat(I, c) * D + own_offset<NT>(0, J, g)) * 4u, L::W + (I * NT + J) * 1024);
+        for (int q = 0; q < NQ; ++q) dma(Wg, (unsigned)((I * NQ + q) * 1024 + lane * 16), L::W + (I * NQ + q) * 1024);
+      } else {
+#pragma unroll
+        for (int J = 0; J < NT; ++J)
+          dma(Wg, (unsigned)(feat(I, c) * D + own_offset<NT>(0, J, g)) * 4u, L::W + (I * NT + J) * 1024);
+      }
     } else if (part == NT) {
 #pragma unroll
       for (int J = 0; J < NT; ++J) dma(bg, (unsigned)own_offset<NT>(0, J, g) * 4u, L::Bv + J * 1024);
@@ -203,8 +210,13 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
 #pragma unroll
         for (int J = 0; J < NT; ++J) {
           const int I = 2 * qq + e;
-          Wn[I][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sb + L::W + (I * NT + J) * 1024));
-          Wa[e][J] = tokens_k(Wn[I][J]);  // tile transpose: (m = j, k = i)
+          if constexpr (PK) {
+            Wa[e][J] = *reinterpret_cast<const frag*>(sb + L::W + (I * NQ + (J >> 1)) * 1024 + 8 * (J & 1));
+            Wn[I][J] = tokens_k(Wa[e][J]);
+          } else {
+            Wn[I][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sb + L::W + (I * NT + J) * 1024));
+            Wa[e][J] = tokens_k(Wn[I][J]);  // tile transpose: (m = j, k = i)
+          }
         }
 #pragma unroll
       for (int J = 0; J < NT; ++J) {

@@ -22,6 +22,7 @@ struct LinearFwdArgs {
   float* W_ckpt;
   float* b_ckpt;
   int B, H, seq, seq_stride, K, n_stages, ckpt_interval, n_ckpt, state_per_batch;
+  int ckpt_packed;  // W checkpoints as bf16 operand fragments (see store_ckpt_packed)
   float eps;
 };
 

@@ -59,6 +59,32 @@ __device__ __forceinline__ int own_offset(int w, int jj, int g) {
   return 32 * (J >> 1) + 8 * g + 4 * (J & 1);
 }
 
+// Packed W checkpoint: the bf16 image of the state in accumulator order.  Tile (I, J) is the fragment a
+// lane holds of it (value r of lane (c, g) is W[feat(I, 4g+r)][feat(J, c)]); the tiles (I, 2q) and (I, 2q+1)
+// share the 1 KiB row I * (d/32) + q, 16 bytes per lane.  This wave writes its TPW column tiles of every I.
+template <int NT, int TPW>
+__device__ __forceinline__ void store_ckpt_packed(float* slot, const f32x4 (&Wc)[NT][TPW], int w, int lane) {
+  unsigned char* base = reinterpret_cast<unsigned char*>(slot) + lane * 16;
+#pragma unroll
+  for (int I = 0; I < NT; ++I) {
+    if (TPW % 2 == 0) {
+#pragma unroll
+      for (int qq = 0; qq < TPW / 2; ++qq) {
+        const u32x2 lo = __builtin_bit_cast(u32x2, Io<BF16>::to_frag(Wc[I][2 * qq]));
+        const u32x2 hi = __builtin_bit_cast(u32x2, Io<BF16>::to_frag(Wc[I][2 * qq + 1]));
+        *reinterpret_cast<u32x4*>(base + (I * (NT / 2) + w * (TPW / 2) + qq) * 1024) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const int J = w * TPW + jj;
+        *reinterpret_cast<u32x2*>(base + (I * (NT / 2) + (J >> 1)) * 1024 + 8 * (J & 1)) =
+            __builtin_bit_cast(u32x2, Io<BF16>::to_frag(Wc[I][jj]));
+      }
+    }
+  }
+}
+
 template <class T, int D, int NW, bool FULL>
 __device__ __forceinline__ void load_stage_mw(StageInMw<T, D / 16, D / 16 / NW>& s, const LinearFwdArgs& a,
                                               size_t bh, int stage, int c, int g, int w) {
@@ -186,12 +212,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
       if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
         const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
         float* Wd = a.W_ckpt + ci * D * D;
+        if (a.ckpt_packed) {
+          store_ckpt_packed<NT, TPW>(Wd, Wc, w, lane);
+        } else {
 #pragma unroll
-        for (int I = 0; I < NT; ++I)
+          for (int I = 0; I < NT; ++I)
 #pragma unroll
-          for (int jj = 0; jj < TPW; ++jj)
+            for (int jj = 0; jj < TPW; ++jj)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+              for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+        }
         if (c == 0)
 #pragma unroll
           for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);

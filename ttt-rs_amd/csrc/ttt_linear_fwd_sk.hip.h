@@ -135,12 +135,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
       if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
         const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
         float* Wd = a.W_ckpt + ci * D * D;
+        if (a.ckpt_packed) {
+          store_ckpt_packed<NT, TPW>(Wd, Wc, w, lane);
+        } else {
 #pragma unroll
-        for (int I = 0; I < NT; ++I)
+          for (int I = 0; I < NT; ++I)
 #pragma unroll
-          for (int jj = 0; jj < TPW; ++jj)
+            for (int jj = 0; jj < TPW; ++jj)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+              for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+        }
         if (c == 0)
 #pragma unroll
           for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);

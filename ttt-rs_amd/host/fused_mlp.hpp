@@ -73,6 +73,7 @@ class FusedMlp {
     d.io_dtype = dtype;
     d.state_per_batch = state_per_batch ? 1 : 0;
     d.seq_stride = 0;
+    d.checkpoint_format = TTT_CKPT_F32;
     return d;
   }
 

@@ -124,6 +124,7 @@ class FusedTileMulti {
     d.io_dtype = dtype;
     d.state_per_batch = state_per_batch ? 1 : 0;
     d.seq_stride = 0;
+    d.checkpoint_format = TTT_CKPT_F32;
     return d;
   }
 

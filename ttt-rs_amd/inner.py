@@ -125,12 +125,14 @@ def _need_win(t: torch.Tensor, shape, dtype, name, pitch: int):
 
 def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
                            mini_batch: int, eps: float = 1e-6, checkpoint_interval: int = 1,
-                           want_checkpoints: bool = False, out: Optional[torch.Tensor] = None):
+                           want_checkpoints: bool = False, out: Optional[torch.Tensor] = None, packed_checkpoints: bool = False):
     """One call of ttt_linear_fwd on the current stream.
 
     Counterpart of fused_ttt_tile_forward_multi (rust/fused/src/linear_fused_tile/api.rs:52-83):
     weight [B,H,d,d] or [H,d,d], bias [B,H,d] or [H,d], token_eta [>=K] (first K entries used).
     Returns (output, weight_out, bias_out[, weight_ckpt, bias_ckpt]).
+    packed_checkpoints (bf16 I/O, interval 1): W checkpoints as bf16 operand fragments in kernel order, to be
+    handed to ttt_linear_backward_raw with the same flag; the tensor keeps its f32 [B,H,n,d,d] allocation.
     """
     B, H, seq, d = xq.shape
     io = xq.dtype
@@ -149,7 +151,8 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
     if token_eta.numel() < mini_batch:
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
     te = token_eta.to(torch.float32).contiguous()
-    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), pitch)
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), pitch,
+                   int(packed_checkpoints))
     check(lib().ttt_linear_supported(C.byref(desc)))
     dev = xq.device
     if out is None or (pitch == 0 and not out.is_contiguous()):
@@ -179,7 +182,7 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
 
 def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
                             weight_ckpt, bias_ckpt, grad_output, mini_batch: int, eps: float = 1e-6,
-                            checkpoint_interval: int = 1, grad_weight_out=None, grad_bias_out=None):
+                            checkpoint_interval: int = 1, grad_weight_out=None, grad_bias_out=None, packed_checkpoints: bool = False):
     """One call of ttt_linear_bwd on the current stream.
 
     Counterpart of backward_multi (rust/fused/src/linear_fused_tile/backward/launch.rs:332-438).
@@ -200,7 +203,8 @@ def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_
     ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
     ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
     te = token_eta.to(torch.float32).contiguous()
-    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), 0)
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), 0,
+                   int(packed_checkpoints))
     check(lib().ttt_linear_supported(C.byref(desc)))
     n = lib().ttt_linear_num_checkpoints(C.byref(desc))
     w_ck = _need(weight_ckpt, (B, H, n, d, d), torch.float32, "weight_ckpt")
