@@ -178,9 +178,9 @@ def main():
                                              dv["d_out"], K)
                 return (fw[0], g["d_xq"])
         else:
-            # bf16 I/O, a checkpoint per mini-batch: checkpoints as bf16 operand fragments (same gradients bit
-            # for bit, half the checkpoint traffic); TTT_BENCH_CKPT=f32 keeps the reference's f32 matrices
-            packed = io == "bf16" and ci == 1 and os.environ.get("TTT_BENCH_CKPT") != "f32"
+            # a checkpoint per mini-batch: checkpoints as operand fragments in kernel order (same gradients bit
+            # for bit; bf16 I/O: half the checkpoint traffic); TTT_BENCH_CKPT=f32 keeps the reference's f32 matrices
+            packed = ci == 1 and os.environ.get("TTT_BENCH_CKPT") != "f32"
 
             def step():
                 out, W, b, Wc, bc = pkg.ttt_linear_forward_raw(
@@ -252,7 +252,8 @@ def main():
         # the backward kernel dominates; it computes in f32 MFMA: 18 d^2 + 22 K d flop per token-head
         flops = th * (24 * d * d + 26 * K * d)
         out["dtype"] = "f32"
-        out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci)
+        out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci,
+                             checkpoint_format="f32 row-major" if (ci != 1 or os.environ.get("TTT_BENCH_CKPT") == "f32") else "packed")
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
                            "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
                            "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)",

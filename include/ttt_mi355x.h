@@ -58,13 +58,14 @@ typedef struct ttt_desc {
   int32_t checkpoint_format;   /* 0: W checkpoints are f32 [d,d] row-major matrices (what the reference
                                   saves, rust/fused/src/linear_fused_tile/forward/launch.rs:117-208),
                                   any interval, readable by the caller.
-                                  1 (TTT_CKPT_PACKED): bf16 I/O with checkpoint_interval 1 only; a W
-                                  checkpoint is the bf16 image of the state in the kernels' own operand
-                                  order (the first d*d*2 bytes of its d*d*4-byte slot; same allocation),
-                                  written by ttt_linear_fwd and meaningful only to ttt_linear_bwd.  The
+                                  1 (TTT_CKPT_PACKED): checkpoint_interval 1 only; a W checkpoint is the
+                                  state in the kernels' own operand order and operand type, written by
+                                  ttt_linear_fwd and meaningful only to ttt_linear_bwd (same allocation).
+                                  bf16 I/O: bf16 (the first d*d*2 bytes of each d*d*4-byte slot); the
                                   backward's products take bf16 operands anyway, so its results do not
-                                  change; half the checkpoint traffic, stored and fetched in whole
-                                  1 KiB rows.  No counterpart in the reference. */
+                                  change; half the checkpoint traffic.  f32 I/O: f32.  Either way stored
+                                  and fetched in whole 1 KiB rows instead of scattered 4-byte pieces.
+                                  No counterpart in the reference. */
 } ttt_desc;
 #define TTT_CKPT_F32 0
 #define TTT_CKPT_PACKED 1

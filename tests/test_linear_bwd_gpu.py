@@ -172,20 +172,23 @@ def test_bwd_wide_heads_need_a_checkpoint_per_mini_batch(P):
         run_bwd(P, c, torch.ones(1, 1, 32, 96), 16, 2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("waves", ["1", "4"])
 @pytest.mark.parametrize("B,H,d,K,N", [(2, 2, 32, 8, 3), (2, 3, 64, 16, 8), (1, 2, 64, 5, 3), (1, 2, 96, 16, 3), (1, 2, 128, 16, 3)])
-def test_bwd_packed_checkpoints_change_nothing(P, monkeypatch, B, H, d, K, N, waves):
-    """bf16 I/O: checkpoints stored as bf16 operand fragments.  The backward rounds the state to bf16 before
-    its first product either way, so every gradient is bit-identical to the f32-checkpoint run; the forward's
-    outputs do not depend on the checkpoint format at all."""
-    if d > 64 and waves == "1":
-        pytest.skip("wide heads have the feature-split kernel only")
-    print(f"case bwd packed ckpt B{B} H{H} d{d} K{K} N{N} waves {waves}", flush=True)
+def test_bwd_packed_checkpoints_change_nothing(P, monkeypatch, B, H, d, K, N, waves, dtype):
+    """Checkpoints stored as operand fragments in kernel order (bf16 I/O: as bf16).  The backward rounds the
+    state to its operand type before the first product either way, so every gradient is bit-identical to the
+    run with f32 row-major checkpoints; the forward's outputs do not depend on the checkpoint format at all."""
+    if (d > 64 or dtype == torch.float32) and waves == "1":
+        pytest.skip("wide heads and f32 I/O have the feature-split kernel only")
+    if d == 128 and dtype == torch.float32:
+        pytest.skip("no f32 backward at head_dim 128")
+    print(f"case bwd packed ckpt B{B} H{H} d{d} K{K} N{N} waves {waves} {dtype}", flush=True)
     monkeypatch.setenv("TTT_LINEAR_BWD_WAVES", waves)
-    c = P.synthetic.reference_test_inputs(500 + B + d + K + N, B, H, N * K, d, K, io_dtype=torch.bfloat16)
+    c = P.synthetic.reference_test_inputs(500 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
     dv = to_dev(c)
     g = torch.Generator().manual_seed(11)
-    dO = torch.randn(B, H, N * K, d, generator=g).to(torch.bfloat16).to("cuda:0")
+    dO = torch.randn(B, H, N * K, d, generator=g).to(dtype).to("cuda:0")
     res = []
     for packed in (False, True):
         out, W, b, Wc, bc = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"],
@@ -201,12 +204,12 @@ def test_bwd_packed_checkpoints_change_nothing(P, monkeypatch, B, H, d, K, N, wa
             assert_close(res[1][3][k], res[0][3][k].double(), 1e-5, k)
         else:
             assert torch.equal(res[0][3][k], res[1][3][k]), k
-    compare(res[1][3], oracle_bwd(c, dO.cpu(), K), TOL[torch.bfloat16])
+    compare(res[1][3], oracle_bwd(c, dO.cpu(), K), TOL[dtype])
 
 
 def test_packed_checkpoints_rejected_where_unsupported(P):
-    c = P.synthetic.reference_test_inputs(2, 1, 1, 32, 32, 16)
+    c = P.synthetic.reference_test_inputs(2, 1, 1, 64, 32, 16)
     dv = to_dev(c)
     with pytest.raises(Exception, match="packed checkpoints"):
         P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
-                                 dv["gamma"], dv["beta"], 16, 1e-6, 1, want_checkpoints=True, packed_checkpoints=True)
+                                 dv["gamma"], dv["beta"], 16, 1e-6, 2, want_checkpoints=True, packed_checkpoints=True)

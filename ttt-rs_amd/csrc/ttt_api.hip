@@ -304,8 +304,8 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.eps = d->eps;
   if (a.ckpt_packed) {
     const char* k = std::getenv("TTT_LINEAR_FWD_KERNEL");
-    if (d->io_dtype != TTT_BF16 || d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
-      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need bf16 I/O, checkpoint_interval 1 and the register-resident kernels");
+    if (d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
+      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   // register-resident kernels for every head_dim; the LDS-tile kernel (96/128) only on request
@@ -358,8 +358,8 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.eps = d->eps;
   if (a.ckpt_packed) {
     const char* k = std::getenv("TTT_LINEAR_BWD_KERNEL");
-    if (d->io_dtype != TTT_BF16 || d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
-      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need bf16 I/O, checkpoint_interval 1 and the register-resident kernels");
+    if (d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
+      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   // accumulated outputs start from zero; a fill kernel (not a memset node) so the sequence
@@ -388,6 +388,12 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
     const char* wsel = std::getenv("TTT_LINEAR_BWD_WAVES");
     int waves = wsel ? std::atoi(wsel) : 0;
     if (waves == 0) waves = (f32 || D > 64 || grid <= 512) ? 4 : 1;
+    if (f32 && a.ckpt_packed) {
+      if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2, true>(a, grid, s);
+      if (D == 64) return launch_linear_bwd_mw<ttt::F32, 64, 4, true>(a, grid, s);
+      if (D == 96) return launch_linear_bwd_mw<ttt::F32, 96, 3, true>(a, grid, s);
+      return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
+    }
     if (f32) {
       if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2>(a, grid, s);
       if (D == 64) return waves == 2 ? launch_linear_bwd_mw<ttt::F32, 64, 2>(a, grid, s)

@@ -35,7 +35,7 @@ struct LinBwdMwLds {
   static constexpr int FT = 64 * 4 * ES;              // bytes of one fragment tile
   static constexpr int W = 0;                         // NT*NT slots: slot I*NT+J, lane (c,g): W[feat(I,c)][feat(J,4g..4g+3)]
                                                       // packed: NT*NT/2 slots: slot I*NT/2+q = tiles (I,2q), (I,2q+1)
-  static constexpr int WSLOTS = PK ? NT * NT / 2 : NT * NT;
+  static constexpr int WSLOTS = (PK && ES == 2) ? NT * NT / 2 : NT * NT;
   static constexpr int Bv = W + WSLOTS * 1024;        // NT slots: b[feat(J,4g..4g+3)]
   static constexpr int X = Bv + NT * 1024;            // 4 tensors x XS slots
   static constexpr int LR = X + 4 * XS * 1024;        // 16 dwords: lr of token c (bf16 zero-extended, or f32)
@@ -44,7 +44,6 @@ struct LinBwdMwLds {
   static constexpr int FR = PT + 4 * NW * 1024;       // 7 kinds x [NT][64] fragments
   static constexpr int BYTES = FR + 7 * NT * FT;
   static_assert(NT % NW == 0 && WSLOTS % NW == 0, "feature tiles must divide among the waves");
-  static_assert(!PK || ES == 2, "packed checkpoints are bf16");
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
 
@@ -178,6 +177,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     for (int ww = 1; ww < NW; ++ww) s += pt(kind, ww);
     return s;
   };
+  // byte offset (without the lane's 16) of tile (I, J) of a packed checkpoint in the staging area
+  auto pk_off = [&](int I, int J) { return BF ? L::W + (I * NQ + (J >> 1)) * 1024 + 8 * (J & 1) : L::W + (I * NT + J) * 1024; };
   auto tokens_k = [&](frag x) {
     f32x4 t = {0.f, 0.f, 0.f, 0.f};
     IO::mma(t, x, ident);
@@ -267,7 +268,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
 #pragma unroll
       for (int J = 0; J < NT; ++J) {
         if constexpr (PK)  // stored as (m = j, k = i): transposed on the matrix pipe
-          Wn[ii][J] = tokens_k(*reinterpret_cast<const frag*>(sl + L::W + (Io * NQ + (J >> 1)) * 1024 + 8 * (J & 1)));
+          Wn[ii][J] = tokens_k(*reinterpret_cast<const frag*>(sl + pk_off(Io, J)));
         else
           Wn[ii][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + (Io * NT + J) * 1024));
       }
@@ -288,8 +289,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         // W tiles (rows 2qq / 2qq+1, own column tile), transposed on the matrix pipe: (m = j, k = i)
         frag wa0, wa1;
         if constexpr (PK) {
-          wa0 = *reinterpret_cast<const frag*>(sl + L::W + ((2 * qq) * NQ + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
-          wa1 = *reinterpret_cast<const frag*>(sl + L::W + ((2 * qq + 1) * NQ + (Jo >> 1)) * 1024 + 8 * (Jo & 1));
+          wa0 = *reinterpret_cast<const frag*>(sl + pk_off(2 * qq, Jo));
+          wa1 = *reinterpret_cast<const frag*>(sl + pk_off(2 * qq + 1, Jo));
         } else {
           wa0 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq) * NT + Jo) * 1024)));
           wa1 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq + 1) * NT + Jo) * 1024)));

@@ -59,15 +59,19 @@ __device__ __forceinline__ int own_offset(int w, int jj, int g) {
   return 32 * (J >> 1) + 8 * g + 4 * (J & 1);
 }
 
-// Packed W checkpoint: the bf16 image of the state in accumulator order.  Tile (I, J) is the fragment a
+// Packed W checkpoint: the image of the state in accumulator order, in the operand type of the I/O mode (bf16).  Tile (I, J) is the fragment a
 // lane holds of it (value r of lane (c, g) is W[feat(I, 4g+r)][feat(J, c)]); the tiles (I, 2q) and (I, 2q+1)
 // share the 1 KiB row I * (d/32) + q, 16 bytes per lane.  This wave writes its TPW column tiles of every I.
-template <int NT, int TPW>
+// f32 I/O keeps f32: tile (I, J) is the 1 KiB row I * (d/16) + J, 16 bytes per lane.
+template <class T, int NT, int TPW>
 __device__ __forceinline__ void store_ckpt_packed(float* slot, const f32x4 (&Wc)[NT][TPW], int w, int lane) {
   unsigned char* base = reinterpret_cast<unsigned char*>(slot) + lane * 16;
 #pragma unroll
   for (int I = 0; I < NT; ++I) {
-    if (TPW % 2 == 0) {
+    if (sizeof(typename Io<T>::elem) == 4) {
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) *reinterpret_cast<f32x4*>(base + (I * NT + w * TPW + jj) * 1024) = Wc[I][jj];
+    } else if (TPW % 2 == 0) {
 #pragma unroll
       for (int qq = 0; qq < TPW / 2; ++qq) {
         const u32x2 lo = __builtin_bit_cast(u32x2, Io<BF16>::to_frag(Wc[I][2 * qq]));
@@ -213,7 +217,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
         const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
         float* Wd = a.W_ckpt + ci * D * D;
         if (a.ckpt_packed) {
-          store_ckpt_packed<NT, TPW>(Wd, Wc, w, lane);
+          store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
         } else {
 #pragma unroll
           for (int I = 0; I < NT; ++I)

@@ -136,7 +136,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
         const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
         float* Wd = a.W_ckpt + ci * D * D;
         if (a.ckpt_packed) {
-          store_ckpt_packed<NT, TPW>(Wd, Wc, w, lane);
+          store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
         } else {
 #pragma unroll
           for (int I = 0; I < NT; ++I)
