@@ -39,6 +39,9 @@ struct TTTConfig {
   float base_lr = 1.0f;
   float epsilon = 1e-6f;
   int checkpoint_interval = 1;
+  /// Checkpoints as operand fragments in kernel order (ttt_desc.checkpoint_format = TTT_CKPT_PACKED):
+  /// interval 1 only, same gradients, less traffic.  No counterpart in the reference's config.
+  bool packed_checkpoints = false;
 };
 
 struct ModelConfig {
@@ -124,7 +127,7 @@ class FusedTileMulti {
     d.io_dtype = dtype;
     d.state_per_batch = state_per_batch ? 1 : 0;
     d.seq_stride = 0;
-    d.checkpoint_format = TTT_CKPT_F32;
+    d.checkpoint_format = config_.ttt.packed_checkpoints ? TTT_CKPT_PACKED : TTT_CKPT_F32;
     return d;
   }
 
