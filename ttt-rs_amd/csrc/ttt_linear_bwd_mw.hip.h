@@ -8,13 +8,13 @@
 // Wave w owns TPW = (d/16)/NW feature tiles.  Of every [16 x d] tile it holds its own features (transposed:
 // value r of lane (c, g) is feature feat(J, 4g+r) of token c); of the state gradient it holds the column
 // slice dW[:, own] (dWc) and the row slice dW[own, :] transposed (DT), each fed back as an A operand without
-// data movement.  What a wave needs of the other slices crosses through LDS at five points per mini-batch:
+// data movement.  What a wave needs of the other slices crosses through LDS at four points per mini-batch:
 //   X1  six raw moments of Z1 (mean, variance and both sums of the LN-L2 gradient follow from them), the
 //       partial attention blocks, XK^T / XQ^T fragments (tokens along k);
 //   X2  four raw moments of Zbar and of the output-LayerNorm backward; G fragments;
-//   X3  partial P = dZbar G^T; dZbar fragments in both forms;
-//   X4  six sums of the second-order LayerNorm (all its statistics are linear in them);
-//   X5  dZ1 fragments in both forms.
+//   X3  partial P = dZbar G^T, dZbar fragments in both forms, and the six sums of the second-order LayerNorm
+//       (all its statistics are linear in them; none needs P, so one exchange carries both);
+//   X4  dZ1 fragments in both forms.
 // All matrix products with a d-deep contraction over the OTHER slices' features take those fragments as B
 // operands; products over tokens (rank-16) are local.  f32 I/O computes in true-f32 MFMA
 // (v_mfma_f32_16x16x4_f32), bf16 I/O in bf16 MFMA with f32 accumulation.
@@ -403,7 +403,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
           Zl[jj] = IO::to_frag(dzb - IO::to_f32(Zf[jj]));
         }
       }
-      // ---- X3: partial P = dZb G^T in both orientations
+      // ---- partial P = dZb G^T in both orientations
       mma_own(P, Gf, Zf);   // [s][t]
       mma_own(P2, Zf, Gf);  // [t][s]
       if (BF) {
@@ -415,7 +415,41 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       pt(P_P, w) = P;
       pt(P_P2, w) = P2;
     }
-    lds_barrier();
+    // ---- DGM = M^T dZb ; S = XK dW + db (own features) ; X3 + X4 in one exchange: the partial P blocks and
+    //      dZb / G fragments travel with the six sums of the second-order LayerNorm, none of which needs P
+    const bool tok_ok = c < K;
+    const size_t tokoff = (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
+    f32x4 dK[TPW], DGM[TPW], S[TPW], TMP[TPW];
+    {
+      const frag M2f = IO::to_frag(M2);
+#pragma unroll
+      for (int ii = 0; ii < TPW; ++ii) {
+        DGM[ii] = zero4;
+        S[ii] = dbT[ii];
+        IO::mma(DGM[ii], Zd[ii], M2f);
+#pragma unroll
+        for (int qq = 0; qq < NQ; ++qq)
+          IO::mma2(S[ii], IO::to_frag(dWc[2 * qq][ii]), IO::to_frag(dWc[2 * qq + 1][ii]), k[2 * qq], k[2 * qq + 1]);
+      }
+    }
+    const float last = te_last * lr_c;
+    f32x4 u[TPW];
+    float S4[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      u[jj] = (DGM[jj] + last * S[jj]) * rstd1;  // u = -dG rstd1
+      const f32x4 au = a2[jj] * u[jj];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        S4[0] += u[jj][r];
+        S4[1] += u[jj][r] * xh[jj][r];
+        S4[2] += au[r];
+        S4[3] += au[r] * xh[jj][r];
+        S4[4] += u[jj][r] * gx[jj][r];
+        S4[5] += G[jj][r] * S[jj][r];
+      }
+    }
+    xsum(2, S4);
     f32x4 dA, dEta, dA2, dEta2;
     {
       const f32x4 P = ptsum(P_P), P2 = ptsum(P_P2);
@@ -424,8 +458,6 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       dA2 = -P2 * eta2;
       dEta2 = -P2 * onepA2;
     }
-    const bool tok_ok = c < K;
-    const size_t tokoff = (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
     frag Zfa[NT], Gfa[NT];
 #pragma unroll
     for (int J = 0; J < NT; ++J) {
@@ -449,42 +481,18 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       }
       if (tok_ok) store_own(a.d_xq, tokoff, dQ);
     }
-    // ---- dK = dA^T XQ ; DGM = M^T dZb ; S = XK dW + db ; TMP = G dW^T   (own features)
-    f32x4 dK[TPW], DGM[TPW], S[TPW], TMP[TPW];
+    // ---- dK = dA^T XQ ; TMP = G dW^T   (own features)
     {
-      const frag dA2f = IO::to_frag(dA2), M2f = IO::to_frag(M2);
+      const frag dA2f = IO::to_frag(dA2);
 #pragma unroll
       for (int ii = 0; ii < TPW; ++ii) {
-        dK[ii] = DGM[ii] = TMP[ii] = zero4;
-        S[ii] = dbT[ii];
+        dK[ii] = TMP[ii] = zero4;
         IO::mma(dK[ii], qdo[ii], dA2f);
-        IO::mma(DGM[ii], Zd[ii], M2f);
 #pragma unroll
-        for (int qq = 0; qq < NQ; ++qq) {
-          IO::mma2(S[ii], IO::to_frag(dWc[2 * qq][ii]), IO::to_frag(dWc[2 * qq + 1][ii]), k[2 * qq], k[2 * qq + 1]);
+        for (int qq = 0; qq < NQ; ++qq)
           IO::mma2(TMP[ii], IO::to_frag(DT[2 * qq][ii]), IO::to_frag(DT[2 * qq + 1][ii]), Gfa[2 * qq], Gfa[2 * qq + 1]);
-        }
       }
     }
-    // ---- X4: the six sums of the second-order LayerNorm
-    const float last = te_last * lr_c;
-    f32x4 u[TPW];
-    float S4[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int jj = 0; jj < TPW; ++jj) {
-      u[jj] = (DGM[jj] + last * S[jj]) * rstd1;  // u = -dG rstd1
-      const f32x4 au = a2[jj] * u[jj];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        S4[0] += u[jj][r];
-        S4[1] += u[jj][r] * xh[jj][r];
-        S4[2] += au[r];
-        S4[3] += au[r] * xh[jj][r];
-        S4[4] += u[jj][r] * gx[jj][r];
-        S4[5] += G[jj][r] * S[jj][r];
-      }
-    }
-    xsum(2, S4);
     const float dl = -S4[5];
     frag Z1f[TPW], Z1d[TPW];
     {
@@ -512,7 +520,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       }
       if (tok_ok) store_own(a.d_xv, tokoff, ndy);
     }
-    // ---- X5: dZ1 fragments
+    // ---- X4: dZ1 fragments
     lds_barrier();
     {
       frag Z1fa[NT];
