@@ -51,6 +51,10 @@ def test_shape_validation(P):
     assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_interval=0))) == P.TTT_ERR_SHAPE
     assert L.ttt_linear_supported(C.byref(desc(P, io_dtype=7))) == P.TTT_ERR_UNSUPPORTED
     assert L.ttt_linear_supported(None) == P.TTT_ERR_NULL
+    # checkpoint formats: 0 (f32 row-major) and 1 (packed) exist
+    assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_format=1))) == P.TTT_OK
+    assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_format=2))) == P.TTT_ERR_SHAPE
+    assert b"checkpoint_format" in L.ttt_last_error()
 
 
 def test_num_checkpoints(P):
