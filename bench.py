@@ -93,7 +93,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (the path shards over "
-                 "batch*heads with no communication, see DESIGN.md)")
+                 "batch*heads with no communication inside the scan; only parameter gradients reduce)")
 
     import torch
     if a.workload == "hbm_copy_calibration":
