@@ -11,6 +11,8 @@
 // for the in-order issue to interleave.  The exchange buffer is double-buffered by parity because
 // one barrier per iteration does not separate a fast wave's next write from a slow wave's read.
 #pragma once
+#include <type_traits>
+
 #include "ttt_linear_fwd_mw.hip.h"
 
 namespace ttt {
@@ -119,36 +121,29 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
     }
   };
 
+  // token_eta[K-1] == 0 means "no state update": instead of a branch inside the loop the two operands
+  // that carry tokens into the update (XK^T, the ones column of the bias update) are made zero
+  const frag ident_upd = upd ? ident : IO::zero();
+  const frag ones_upd = upd ? ones : IO::zero();
+
   constexpr int R = PF + 1;
   StageInMw<T, NT, TPW> buf[R];
 #pragma unroll
   for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], a, bh, u, c, g, w);
 
-  for (int st0 = 0; st0 < a.n_stages; st0 += R) {
+  // One pass over R mini-batches (the ring of prefetch registers is indexed at compile time).  CHECKED:
+  // the first and the last pass, which test for "no pending output yet" and "past the end"; the passes in
+  // between run without any branch, so that everything between two barriers -- the tail of one mini-batch
+  // (pending output, G, state update) and the head of the next (products, moments) -- is one basic block and
+  // the compiler can interleave the two dependency chains.
+  auto pass = [&](auto checked_tag, int st0) {
+    constexpr bool CHECKED = decltype(checked_tag)::value;
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int st = st0 + u;
       load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], a, bh, st + PF, c, g, w);
-      if (st >= a.n_stages) continue;
+      if (CHECKED && st >= a.n_stages) continue;
       const StageInMw<T, NT, TPW>& cur = buf[u];
-
-      if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
-        const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
-        float* Wd = a.W_ckpt + ci * D * D;
-        if (a.ckpt_packed) {
-          store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
-        } else {
-#pragma unroll
-          for (int I = 0; I < NT; ++I)
-#pragma unroll
-            for (int jj = 0; jj < TPW; ++jj)
-#pragma unroll
-              for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
-        }
-        if (c == 0)
-#pragma unroll
-          for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
-      }
 
       // ---- XK with tokens along k for the state update: depends on nothing computed here, so it
       // is issued first and fills the gaps of the dependent chain below
@@ -156,7 +151,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
 #pragma unroll
       for (int I = 0; I < NT; ++I) {
         f32x4 t = {0.f, 0.f, 0.f, 0.f};
-        IO::mma(t, cur.k[I], ident);  // t[r] = XK[s = 4g+r][feat(I,c)]
+        IO::mma(t, cur.k[I], ident_upd);  // t[r] = XK[s = 4g+r][feat(I,c)]
         kd[I] = IO::to_frag(t);
       }
       // ---- Z1^T, Zbar^T (this wave's feature rows) and the attention block
@@ -202,10 +197,26 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
           S[7] += zbp[jj][r] * zbp[jj][r];
         }
       }
+      // ---- checkpoint of the state entering this mini-batch (W and b change only behind the barrier);
+      // placed at the barrier so that its branch does not cut the stretch in two
+      if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
+        const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
+        float* Wd = a.W_ckpt + ci * D * D;
+        if (a.ckpt_packed) {
+          store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
+        } else {
+#pragma unroll
+          for (int I = 0; I < NT; ++I)
+#pragma unroll
+            for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+        }
+        if (c == 0)
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
+      }
       exchange8(S, st & 1);
-
-      // ---- pending output (previous mini-batch): independent of everything below
-      if (st > 0) emit_output(S[6], S[7], st - 1);
 
       // ---- recurrence: G'' , causal correction, state update
       f32x4 G[TPW];
@@ -235,14 +246,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
 #pragma unroll
         for (int jj = 0; jj < TPW; ++jj) IO::mma(zb[jj], Gd[jj], Mf);
       }
-      if (upd) {
 #pragma unroll
-        for (int I = 0; I < NT; ++I)
+      for (int I = 0; I < NT; ++I)
 #pragma unroll
-          for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
+        for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
 #pragma unroll
-        for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones);
-      }
+      for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones_upd);
+      // ---- pending output (previous mini-batch): nothing waits for it, so it is issued behind the state
+      // update and runs in the shadow of those matrix instructions (issue is in order: placed ahead of G it
+      // would delay the recurrence by its own issue time)
+      if (!CHECKED || st > 0) emit_output(S[6], S[7], st - 1);
       // this mini-batch's Zbar and xq become the pending output
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) {
@@ -250,6 +263,143 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
         qop[jj] = cur.qo[jj];
       }
     }
+  };
+  if constexpr (NT <= 4) {
+    int st0 = 0;
+    pass(std::true_type{}, st0);
+    for (st0 = R; st0 + R <= a.n_stages; st0 += R) pass(std::false_type{}, st0);
+    if (st0 < a.n_stages) pass(std::true_type{}, st0);
+  } else {
+    // Wide heads (d = 96, 128) keep the loop with its branches: in one long basic block the scheduler overlaps
+    // so much that the state tiles no longer fit the register file (d = 128: 30 spilled registers).
+    for (int st0 = 0; st0 < a.n_stages; st0 += R) {
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const int st = st0 + u;
+        load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], a, bh, st + PF, c, g, w);
+        if (st >= a.n_stages) continue;
+        const StageInMw<T, NT, TPW>& cur = buf[u];
+
+        if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
+          const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
+          float* Wd = a.W_ckpt + ci * D * D;
+          if (a.ckpt_packed) {
+            store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
+          } else {
+#pragma unroll
+            for (int I = 0; I < NT; ++I)
+#pragma unroll
+              for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+          }
+          if (c == 0)
+#pragma unroll
+            for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
+        }
+
+        // ---- XK with tokens along k for the state update: depends on nothing computed here, so it
+        // is issued first and fills the gaps of the dependent chain below
+        frag kd[NT];
+#pragma unroll
+        for (int I = 0; I < NT; ++I) {
+          f32x4 t = {0.f, 0.f, 0.f, 0.f};
+          IO::mma(t, cur.k[I], ident);  // t[r] = XK[s = 4g+r][feat(I,c)]
+          kd[I] = IO::to_frag(t);
+        }
+        // ---- Z1^T, Zbar^T (this wave's feature rows) and the attention block
+        f32x4 z1[TPW], zb[TPW], At = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          z1[jj] = bT[jj];
+          zb[jj] = bT[jj];
+        }
+#pragma unroll
+        for (int q = 0; q < NT / 2; ++q) {
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) {
+            const frag w0 = IO::to_frag(Wc[2 * q][jj]), w1 = IO::to_frag(Wc[2 * q + 1][jj]);
+            IO::mma2(z1[jj], w0, w1, cur.k[2 * q], cur.k[2 * q + 1]);
+            IO::mma2(zb[jj], w0, w1, cur.q[2 * q], cur.q[2 * q + 1]);
+          }
+          IO::mma2(At, cur.k[2 * q], cur.k[2 * q + 1], cur.q[2 * q], cur.q[2 * q + 1]);
+        }
+        // ---- row sums: six raw moments of Z1 (this mini-batch), two of the pending Zbar
+        f32x4 bq[TPW];
+        float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          f32x4 uu;  // beta - (xv - xk)
+          if (BF) {
+            uu = bet[jj];
+            IO::mma2(uu, nident, ident, cur.vo[jj], cur.ko[jj]);
+          } else {
+            uu = bet[jj] - (IO::to_f32(cur.vo[jj]) - IO::to_f32(cur.ko[jj]));
+          }
+          bq[jj] = gam[jj] * uu;
+          const f32x4 az = a2[jj] * z1[jj];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            S[0] += z1[jj][r];
+            S[1] += z1[jj][r] * z1[jj][r];
+            S[2] += az[r];
+            S[3] += az[r] * z1[jj][r];
+            S[4] += bq[jj][r];
+            S[5] += bq[jj][r] * z1[jj][r];
+            S[6] += zbp[jj][r];
+            S[7] += zbp[jj][r] * zbp[jj][r];
+          }
+        }
+        exchange8(S, st & 1);
+
+        // ---- pending output (previous mini-batch): independent of everything below
+        if (st > 0) emit_output(S[6], S[7], st - 1);
+
+        // ---- recurrence: G'' , causal correction, state update
+        f32x4 G[TPW];
+        {
+          const float mu = S[0] * inv_d;
+          const float var = S[1] * inv_d - mu * mu;
+          const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+          const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
+          const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
+          const float p = -sc * cur.lr * rstd;
+          const float c1 = p * rstd, c2 = -c1 * s2 * inv_d, c3 = -p * s1 * inv_d;
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) G[jj] = (z1[jj] - mu) * (a2[jj] * c1 + c2) + (bq[jj] * p + c3);
+        }
+        frag Gd[TPW];
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          f32x4 t = {0.f, 0.f, 0.f, 0.f};
+          IO::mma(t, IO::to_frag(G[jj]), ident);
+          Gd[jj] = IO::to_frag(t);
+        }
+        {
+          f32x4 m;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) m[r] = (4 * g + r <= c) ? rho_c * (1.f + At[r]) : 0.f;
+          const frag Mf = IO::to_frag(m);
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) IO::mma(zb[jj], Gd[jj], Mf);
+        }
+        if (upd) {
+#pragma unroll
+          for (int I = 0; I < NT; ++I)
+#pragma unroll
+            for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones);
+        }
+        // this mini-batch's Zbar and xq become the pending output
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          zbp[jj] = zb[jj];
+          qop[jj] = cur.qo[jj];
+        }
+      }
+    }
+
   }
 
   // ---- flush the last mini-batch's output
