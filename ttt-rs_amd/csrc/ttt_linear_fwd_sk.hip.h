@@ -67,23 +67,29 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
         for (int r = 0; r < 4; ++r) Wc[I][jj][r] = W0[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)];
   }
 
-  // pending output of the previous mini-batch
-  f32x4 zbp[TPW];
-  frag qop[TPW];
+  // pending output of the previous mini-batch (its LayerNorm sums travel in the next exchange) and, for
+  // d <= 64, of the one before (sums known: it is finished while the next exchange is in flight)
+  f32x4 zbp[TPW], zbo[TPW];
+  frag qop[TPW], qoo[TPW];
+  float so0 = 0.f, so1 = 0.f;
 #pragma unroll
   for (int jj = 0; jj < TPW; ++jj) {
-    zbp[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
-    qop[jj] = IO::zero();
+    zbp[jj] = zbo[jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+    qop[jj] = qoo[jj] = IO::zero();
   }
 
-  // publish this lane group's two sums, wait for the other waves, add up
-  auto exchange8 = [&](float (&S)[8], int parity) {
+  // publish this lane group's two sums ...
+  auto exchange8_publish = [&](const float (&S)[8], int parity) {
     // lane group g ends up with sums g and g+4 reduced over the wave, and publishes them
     const float v0 = xg_sum4_scatter(S[0], S[1], S[2], S[3]);
     const float v1 = xg_sum4_scatter(S[4], S[5], S[6], S[7]);
     float* e = ex[parity];
     e[(g * 16 + c) * NW + w] = v0;
     e[((g + 4) * 16 + c) * NW + w] = v1;
+  };
+  // ... wait for the other waves, add up
+  auto exchange8_collect = [&](float (&S)[8], int parity) {
+    const float* e = ex[parity];
     lds_barrier();
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -93,8 +99,24 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
       S[i] = s;
     }
   };
+  auto exchange8 = [&](float (&S)[8], int parity) {
+    exchange8_publish(S, parity);
+    exchange8_collect(S, parity);
+  };
+  // In-lane sums of a pending Zbar.  One routine with explicit fused multiply-adds for every place that forms
+  // them: a sequence processed in several calls must give the same bits as one call.
+  auto pend_sums = [&](const f32x4 (&z)[TPW], float& s0, float& s1) {
+    s0 = s1 = 0.f;
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s0 += z[jj][r];
+        s1 = __builtin_fmaf(z[jj][r], z[jj][r], s1);
+      }
+  };
   // out = xq + gamma (zbar - mu) rstd + beta for the pending mini-batch
-  auto emit_output = [&](float s0, float s1, int stage) {
+  auto emit_output = [&](float s0, float s1, int stage, const f32x4 (&zbp)[TPW], const frag (&qop)[TPW]) {
     const float mu = s0 * inv_d;
     const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
     if (FULL || c < K) {
@@ -136,6 +158,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
   // between run without any branch, so that everything between two barriers -- the tail of one mini-batch
   // (pending output, G, state update) and the head of the next (products, moments) -- is one basic block and
   // the compiler can interleave the two dependency chains.
+  float ps0 = 0.f, ps1 = 0.f;
   auto pass = [&](auto checked_tag, int st0) {
     constexpr bool CHECKED = decltype(checked_tag)::value;
 #pragma unroll
@@ -173,7 +196,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
       }
       // ---- row sums: six raw moments of Z1 (this mini-batch), two of the pending Zbar
       f32x4 bq[TPW];
-      float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, ps0, ps1};  // the pending Zbar's in-lane sums are ready
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) {
         f32x4 uu;  // beta - (xv - xk)
@@ -193,8 +216,6 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
           S[3] += az[r] * z1[jj][r];
           S[4] += bq[jj][r];
           S[5] += bq[jj][r] * z1[jj][r];
-          S[6] += zbp[jj][r];
-          S[7] += zbp[jj][r] * zbp[jj][r];
         }
       }
       // ---- checkpoint of the state entering this mini-batch (W and b change only behind the barrier);
@@ -216,7 +237,18 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
 #pragma unroll
           for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
       }
-      exchange8(S, st & 1);
+      exchange8_publish(S, st & 1);
+      // ---- the output pending since two mini-batches (sums known since the last exchange): nothing waits
+      // for it, and here it runs while this exchange is in flight (LDS write, barrier, LDS read)
+      if (!CHECKED || st > 1) emit_output(so0, so1, st - 2, zbo, qoo);
+      exchange8_collect(S, st & 1);
+      so0 = S[6];
+      so1 = S[7];
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        zbo[jj] = zbp[jj];
+        qoo[jj] = qop[jj];
+      }
 
       // ---- recurrence: G'' , causal correction, state update
       f32x4 G[TPW];
@@ -252,16 +284,14 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
         for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones_upd);
-      // ---- pending output (previous mini-batch): nothing waits for it, so it is issued behind the state
-      // update and runs in the shadow of those matrix instructions (issue is in order: placed ahead of G it
-      // would delay the recurrence by its own issue time)
-      if (!CHECKED || st > 0) emit_output(S[6], S[7], st - 1);
-      // this mini-batch's Zbar and xq become the pending output
+      // this mini-batch's Zbar and xq become the pending output; its in-lane sums are formed here, in the
+      // shadow of the state update, not between the next Z1 and its exchange
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) {
         zbp[jj] = zb[jj];
         qop[jj] = cur.qo[jj];
       }
+      pend_sums(zbp, ps0, ps1);
     }
   };
   if constexpr (NT <= 4) {
@@ -346,14 +376,13 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
             S[3] += az[r] * z1[jj][r];
             S[4] += bq[jj][r];
             S[5] += bq[jj][r] * z1[jj][r];
-            S[6] += zbp[jj][r];
-            S[7] += zbp[jj][r] * zbp[jj][r];
           }
         }
+        pend_sums(zbp, S[6], S[7]);
         exchange8(S, st & 1);
 
         // ---- pending output (previous mini-batch): independent of everything below
-        if (st > 0) emit_output(S[6], S[7], st - 1);
+        if (st > 0) emit_output(S[6], S[7], st - 1, zbp, qop);
 
         // ---- recurrence: G'' , causal correction, state update
         f32x4 G[TPW];
@@ -405,15 +434,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
   // ---- flush the last mini-batch's output
   {
     float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int jj = 0; jj < TPW; ++jj)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        S[6] += zbp[jj][r];
-        S[7] += zbp[jj][r] * zbp[jj][r];
-      }
+    pend_sums(zbp, S[6], S[7]);
     exchange8(S, a.n_stages & 1);
-    emit_output(S[6], S[7], a.n_stages - 1);
+    if (NT <= 4 && a.n_stages >= 2) emit_output(so0, so1, a.n_stages - 2, zbo, qoo);
+    emit_output(S[6], S[7], a.n_stages - 1, zbp, qop);
   }
   {
     float* Wd = a.W_out + bh * D * D;
