@@ -67,8 +67,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
         for (int r = 0; r < 4; ++r) Wc[I][jj][r] = W0[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)];
   }
 
-  // pending output of the previous mini-batch (its LayerNorm sums travel in the next exchange) and, for
-  // d <= 64, of the one before (sums known: it is finished while the next exchange is in flight)
+  // pending output of the previous mini-batch (its LayerNorm sums travel in the next exchange) and of the
+  // one before (sums known: it is finished while the next exchange is in flight)
   f32x4 zbp[TPW], zbo[TPW];
   frag qop[TPW], qoo[TPW];
   float so0 = 0.f, so1 = 0.f;
@@ -379,10 +379,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
           }
         }
         pend_sums(zbp, S[6], S[7]);
-        exchange8(S, st & 1);
-
-        // ---- pending output (previous mini-batch): independent of everything below
-        if (st > 0) emit_output(S[6], S[7], st - 1, zbp, qop);
+        exchange8_publish(S, st & 1);
+        if (st > 1) emit_output(so0, so1, st - 2, zbo, qoo);  // inside the exchange window, as above
+        exchange8_collect(S, st & 1);
+        so0 = S[6];
+        so1 = S[7];
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          zbo[jj] = zbp[jj];
+          qoo[jj] = qop[jj];
+        }
 
         // ---- recurrence: G'' , causal correction, state update
         f32x4 G[TPW];
@@ -436,7 +442,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
     float S[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     pend_sums(zbp, S[6], S[7]);
     exchange8(S, a.n_stages & 1);
-    if (NT <= 4 && a.n_stages >= 2) emit_output(so0, so1, a.n_stages - 2, zbo, qoo);
+    if (a.n_stages >= 2) emit_output(so0, so1, a.n_stages - 2, zbo, qoo);
     emit_output(S[6], S[7], a.n_stages - 1, zbp, qop);
   }
   {
