@@ -155,13 +155,18 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         lds_dma4(lrp, 4u * li, stg + L::LR);
     }
   };
-  // partial sums of this wave's features -> totals in every wave; contains the exchange barrier
-  auto xsum = [&](int region, float (&S)[8]) {
+  // partial sums of this wave's features -> totals in every wave, in two steps: publish, then (behind the
+  // exchange barrier) collect.  Issue is in order, so work that does not depend on the exchange is placed
+  // between the two: it runs while the LDS write, the barrier and the LDS reads are in flight.
+  auto xpub = [&](int region, const float (&S)[8]) {
     const float v0 = xg_sum4_scatter(S[0], S[1], S[2], S[3]);
     const float v1 = xg_sum4_scatter(S[4], S[5], S[6], S[7]);
     float* e = SUMp + region * 8 * 16 * NW;
     e[(g * 16 + c) * NW + w] = v0;
     e[((g + 4) * 16 + c) * NW + w] = v1;
+  };
+  auto xcol = [&](int region, float (&S)[8]) {
+    const float* e = SUMp + region * 8 * 16 * NW;
     lds_barrier();
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -323,7 +328,17 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         S1[5] += bq[jj][r] * z1[jj][r];
       }
     }
-    xsum(0, S1);
+    xpub(0, S1);
+    // window: S = XK dW + db (own features) needs nothing of this mini-batch but XK
+    f32x4 S[TPW];
+#pragma unroll
+    for (int ii = 0; ii < TPW; ++ii) {
+      S[ii] = dbT[ii];
+#pragma unroll
+      for (int qq = 0; qq < NQ; ++qq)
+        IO::mma2(S[ii], IO::to_frag(dWc[2 * qq][ii]), IO::to_frag(dWc[2 * qq + 1][ii]), k[2 * qq], k[2 * qq + 1]);
+    }
+    xcol(0, S1);
     // every wave has moved the staged mini-batch to registers: the next one may be copied in
     fetch(st - 1);
 
@@ -378,7 +393,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         }
       }
     }
-    xsum(1, S2);
+    xpub(1, S2);
+    xcol(1, S2);
     frag Zf[TPW], Zd[TPW];
     {
       const float mu2 = S2[0] * inv_d;
@@ -415,21 +431,17 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       pt(P_P, w) = P;
       pt(P_P2, w) = P2;
     }
-    // ---- DGM = M^T dZb ; S = XK dW + db (own features) ; X3 + X4 in one exchange: the partial P blocks and
-    //      dZb / G fragments travel with the six sums of the second-order LayerNorm, none of which needs P
+    // ---- DGM = M^T dZb (own features) ; X3: the partial P blocks and dZb / G fragments travel with the six
+    //      sums of the second-order LayerNorm, none of which needs P
     const bool tok_ok = c < K;
     const size_t tokoff = (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
-    f32x4 dK[TPW], DGM[TPW], S[TPW], TMP[TPW];
+    f32x4 dK[TPW], DGM[TPW], TMP[TPW];
     {
       const frag M2f = IO::to_frag(M2);
 #pragma unroll
       for (int ii = 0; ii < TPW; ++ii) {
         DGM[ii] = zero4;
-        S[ii] = dbT[ii];
         IO::mma(DGM[ii], Zd[ii], M2f);
-#pragma unroll
-        for (int qq = 0; qq < NQ; ++qq)
-          IO::mma2(S[ii], IO::to_frag(dWc[2 * qq][ii]), IO::to_frag(dWc[2 * qq + 1][ii]), k[2 * qq], k[2 * qq + 1]);
       }
     }
     const float last = te_last * lr_c;
@@ -449,7 +461,19 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         S4[5] += G[jj][r] * S[jj][r];
       }
     }
-    xsum(2, S4);
+    xpub(2, S4);
+    // window: TMP = G dW^T (own features) needs the G fragments of every wave, published one exchange ago
+    frag Gfa[NT];
+#pragma unroll
+    for (int J = 0; J < NT; ++J) Gfa[J] = fr(GF, J);
+#pragma unroll
+    for (int ii = 0; ii < TPW; ++ii) {
+      TMP[ii] = zero4;
+#pragma unroll
+      for (int qq = 0; qq < NQ; ++qq)
+        IO::mma2(TMP[ii], IO::to_frag(DT[2 * qq][ii]), IO::to_frag(DT[2 * qq + 1][ii]), Gfa[2 * qq], Gfa[2 * qq + 1]);
+    }
+    xcol(2, S4);
     f32x4 dA, dEta, dA2, dEta2;
     {
       const f32x4 P = ptsum(P_P), P2 = ptsum(P_P2);
@@ -458,12 +482,9 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       dA2 = -P2 * eta2;
       dEta2 = -P2 * onepA2;
     }
-    frag Zfa[NT], Gfa[NT];
+    frag Zfa[NT];
 #pragma unroll
-    for (int J = 0; J < NT; ++J) {
-      Zfa[J] = fr(ZF, J);
-      Gfa[J] = fr(GF, J);
-    }
+    for (int J = 0; J < NT; ++J) Zfa[J] = fr(ZF, J);
     // ---- dXQ = dO + dZb W^T + dA XK   (own features)
     {
       const frag dAf = IO::to_frag(dA);
@@ -481,16 +502,13 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       }
       if (tok_ok) store_own(a.d_xq, tokoff, dQ);
     }
-    // ---- dK = dA^T XQ ; TMP = G dW^T   (own features)
+    // ---- dK = dA^T XQ   (own features)
     {
       const frag dA2f = IO::to_frag(dA2);
 #pragma unroll
       for (int ii = 0; ii < TPW; ++ii) {
-        dK[ii] = TMP[ii] = zero4;
+        dK[ii] = zero4;
         IO::mma(dK[ii], qdo[ii], dA2f);
-#pragma unroll
-        for (int qq = 0; qq < NQ; ++qq)
-          IO::mma2(TMP[ii], IO::to_frag(DT[2 * qq][ii]), IO::to_frag(DT[2 * qq + 1][ii]), Gfa[2 * qq], Gfa[2 * qq + 1]);
       }
     }
     const float dl = -S4[5];
