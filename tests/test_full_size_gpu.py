@@ -117,16 +117,22 @@ def test_config1_shape_linear_fwd_bwd_bf16_full(P, monkeypatch):
     c = P.synthetic.baseline_inputs(1, B, H, seq, d, K, io_dtype=torch.bfloat16, with_dout=True)
     dv = dev(c)
 
-    def fwd_bwd(x):
+    def fwd_bwd(x, packed=False):
         out, W, b, Wc, bc = P.ttt_linear_forward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"],
                                                      x["lr"], x["gamma"], x["beta"], K, 1e-6, 1,
-                                                     want_checkpoints=True)
+                                                     want_checkpoints=True, packed_checkpoints=packed)
         g = P.ttt_linear_backward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"],
-                                      x["gamma"], x["beta"], Wc, bc, x["d_out"], K, 1e-6, 1)
+                                      x["gamma"], x["beta"], Wc, bc, x["d_out"], K, 1e-6, 1,
+                                      packed_checkpoints=packed)
         torch.cuda.synchronize()
         return out, g
 
     out, g = fwd_bwd(dv)
+    # packed checkpoints (what bench.py measures): same outputs and per-unit gradients, bit for bit
+    outp, gp = fwd_bwd(dv, packed=True)
+    assert torch.equal(outp, out)
+    for k in ("grad_xq", "grad_xk", "grad_xv", "grad_weight", "grad_bias", "grad_ttt_lr_eta"):
+        assert torch.equal(gp[k], g[k]), "packed " + k
     for k, v in g.items():
         assert torch.isfinite(v.float()).all(), k
     # one batch entry alone: per-unit gradients are bit-identical
