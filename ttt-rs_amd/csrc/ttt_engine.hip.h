@@ -65,8 +65,57 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
           acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u][j], acc[j], 0, 0, 0);
     };
     constexpr int KG = 4 * KU;
-    const int ngroups = Kd / KG;
-    int k = 0;
+    // Operand A contiguous along k (rows 16-byte aligned): the k values of a 16-deep step are re-assigned so
+    // that lane (c, g) supplies k = 4g .. 4g+3 to the four matrix instructions of the step (the pairing of
+    // slot and k only has to agree between A and B).  A is then one 16-byte load per step instead of four
+    // scalar ones, and so is B when it is contiguous along k too (a transposed weight matrix: its lanes
+    // would otherwise touch a different cache line each).
+    const bool fastA = a_cs == 1 && (a_rs & 3) == 0 && (Kd & 15) == 0 && (k0 & 3) == 0;
+    if (fastA) {
+      const bool vecB = b_rs == 1 && (b_cs & 3) == 0;
+      const int ao = (16 * tm + c) * a_rs + k0 + 4 * g;
+      const int bo = (k0 + 4 * g) * b_rs + (16 * tn0 + c) * b_cs;
+      auto loadA = [&](int kk) { return *reinterpret_cast<const f32x4*>(A + ao + kk); };
+      auto loadB = [&](int kk, int j) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (tn0 + j < Nt) {
+          const float* pb = B + bo + kk * b_rs + j * bcol;
+          if (vecB) {
+            v = *reinterpret_cast<const f32x4*>(pb);
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = pb[r * b_rs];
+          }
+        }
+        return v;
+      };
+      f32x4 a0 = loadA(0), b0[NB], a1, b1[NB];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) b0[j] = loadB(0, j);
+      auto step = [&](const f32x4& av, const f32x4 (&bv)[NB]) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int j = 0; j < NB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[r], bv[j][r], acc[j], 0, 0, 0);
+      };
+      int kk = 0;
+#pragma nounroll
+      for (; kk + 32 <= Kd; kk += 32) {
+        a1 = loadA(kk + 16);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) b1[j] = loadB(kk + 16, j);
+        step(a0, b0);
+        if (kk + 32 < Kd) {
+          a0 = loadA(kk + 32);
+#pragma unroll
+          for (int j = 0; j < NB; ++j) b0[j] = loadB(kk + 32, j);
+        }
+        step(a1, b1);
+      }
+      if (kk < Kd) step(a0, b0);
+    }
+    const int ngroups = fastA ? 0 : Kd / KG;
+    int k = fastA ? Kd : 0;
     if (ngroups > 0) {
       fetch(avA, bvA, 0);
       int gi = 0;

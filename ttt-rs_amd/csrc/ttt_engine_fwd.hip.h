@@ -83,7 +83,7 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a
   using elem = typename IO::elem;
   using L = LinFwdLds<D>;
   constexpr int LD = L::LD, LK = L::LK, NJ = D / 16, NT = D / 16;
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int t = tid >> 4, cg = tid & 15;
   const size_t bh = blockIdx.x;
@@ -231,7 +231,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
   constexpr int NW = 8, GW = 32, NJD = D / GW, NJM = M / GW, NTD = D / 16, NTM = M / 16;
   constexpr int NBM = NTM / NW;  // hidden-side tile columns per job: one job per wave
   constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int t = tid >> 5, cg = tid & 31;
   const size_t bh = blockIdx.x;

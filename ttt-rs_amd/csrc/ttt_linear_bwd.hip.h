@@ -78,7 +78,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   constexpr int LD = L::LD, LK = L::LK, NJ = D / 16;
   constexpr int NB2 = NJ >= 2 ? 2 : 1;  // tile columns per job of a [16 x D] product
   constexpr float inv_d = 1.0f / D;
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int t = tid >> 4, cg = tid & 15;  // elementwise mapping: token t, features cg + 16 j

@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
   constexpr int NBM = NTM / NW;  // [16 x 4d] products: one job of NBM tile columns per wave
   constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
   constexpr float inv_d = 1.0f / D;
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int t = tid >> 5, cg = tid & 31;  // elementwise mapping: token t, columns cg + 32 j
   const size_t bh = blockIdx.x;
