@@ -6,6 +6,7 @@
 // true-f32 MFMA (v_mfma_f32_16x16x4_f32): lane (c = lane%16, g = lane/16) supplies A(16tm+c, k+g)
 // and B(k+g, 16tn+c) for k = 0, 4, 8, ... and owns C(16tm+4g+r, 16tn+c), r = 0..3.
 #pragma once
+#include <type_traits>
 #include "ttt_frag.hip.h"
 
 namespace ttt {
@@ -34,11 +35,11 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
     const int coff = (16 * tm + 4 * g) * ldc + 16 * tn0 + c;
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-      const bool live = tn0 + j < Nt;
+      const bool live = Nt % NB == 0 || tn0 + j < Nt;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float v = 0.f;
-        if ((MODE == 1 || MODE == 2) && live) v = C[coff + r * ldc + 16 * j];
+        if (MODE == 1 || MODE == 2) v = C[coff + r * ldc + 16 * (live ? j : 0)];
         acc[j][r] = (MODE == 2) ? -v : v;
       }
     }
@@ -54,7 +55,13 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
       for (int u = 0; u < KU; ++u) {
         av[u] = A[ak + u * astep];
 #pragma unroll
-        for (int j = 0; j < NB; ++j) bv[u][j] = (tn0 + j < Nt) ? B[bk + u * bstep + j * bcol] : 0.f;
+        for (int j = 0; j < NB; ++j) {
+          // a tile column past the edge re-reads column tn0 and is zeroed afterwards: a load under a
+          // branch would make every wait that follows it count as if the load had not been issued
+          const bool live = Nt % NB == 0 || tn0 + j < Nt;
+          const float v = B[bk + u * bstep + (live ? j : 0) * bcol];
+          bv[u][j] = live ? v : 0.f;
+        }
       }
     };
     auto fma_group = [&](const float (&av)[KU], const float (&bv)[KU][NB]) {
@@ -77,53 +84,84 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
       const int bo = (k0 + 4 * g) * b_rs + (16 * tn0 + c) * b_cs;
       auto loadA = [&](int kk) { return *reinterpret_cast<const f32x4*>(A + ao + kk); };
       auto loadB = [&](int kk, int j) {
-        f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        if (tn0 + j < Nt) {
-          const float* pb = B + bo + kk * b_rs + j * bcol;
-          if (vecB) {
-            v = *reinterpret_cast<const f32x4*>(pb);
-          } else {
+        // a tile column past the edge re-reads column tn0 and is zeroed afterwards (no load under a branch)
+        const bool live = Nt % NB == 0 || tn0 + j < Nt;
+        const float* pb = B + bo + kk * b_rs + (live ? j : 0) * bcol;
+        f32x4 v;
+        if (vecB) {
+          v = *reinterpret_cast<const f32x4*>(pb);
+        } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] = pb[r * b_rs];
-          }
+          for (int r = 0; r < 4; ++r) v[r] = pb[r * b_rs];
         }
+        if (!live) v = f32x4{0.f, 0.f, 0.f, 0.f};
         return v;
       };
-      f32x4 a0 = loadA(0), b0[NB], a1, b1[NB];
-#pragma unroll
-      for (int j = 0; j < NB; ++j) b0[j] = loadB(0, j);
       auto step = [&](const f32x4& av, const f32x4 (&bv)[NB]) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
           for (int j = 0; j < NB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[r], bv[j][r], acc[j], 0, 0, 0);
       };
-      int kk = 0;
-#pragma nounroll
-      for (; kk + 32 <= Kd; kk += 32) {
-        a1 = loadA(kk + 16);
+      // PF 16-deep steps of operands are in flight at any time (a ring of PF register buffers, refilled
+      // right after use): the operands come from global memory, and with one step in flight a product
+      // over 4d would pay 24 memory latencies in a row.  PF divides the step count, so no refill is
+      // conditional; the scheduling barriers keep the refills where they are written.
+      auto run = [&](auto pf_tag) {
+        constexpr int PF = decltype(pf_tag)::value;
+        f32x4 av[PF], bv[PF][NB];
 #pragma unroll
-        for (int j = 0; j < NB; ++j) b1[j] = loadB(kk + 16, j);
-        step(a0, b0);
-        if (kk + 32 < Kd) {
-          a0 = loadA(kk + 32);
+        for (int u = 0; u < PF; ++u) {
+          av[u] = loadA(16 * u);
 #pragma unroll
-          for (int j = 0; j < NB; ++j) b0[j] = loadB(kk + 32, j);
+          for (int j = 0; j < NB; ++j) bv[u][j] = loadB(16 * u, j);
         }
-        step(a1, b1);
-      }
-      if (kk < Kd) step(a0, b0);
+        __builtin_amdgcn_sched_barrier(0);
+        int kk = 0;
+#pragma nounroll
+        for (; kk + 16 * PF < Kd; kk += 16 * PF) {
+#pragma unroll
+          for (int u = 0; u < PF; ++u) {
+            step(av[u], bv[u]);
+            av[u] = loadA(kk + 16 * (PF + u));
+#pragma unroll
+            for (int j = 0; j < NB; ++j) bv[u][j] = loadB(kk + 16 * (PF + u), j);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < PF; ++u) step(av[u], bv[u]);
+      };
+      constexpr int PFMAX = NB >= 4 ? 4 : NB == 3 ? 6 : 8;
+      const int nsteps = Kd >> 4;
+      if (PFMAX >= 8 && nsteps % 8 == 0)
+        run(std::integral_constant<int, 8>{});
+      else if (PFMAX >= 6 && nsteps % 6 == 0)
+        run(std::integral_constant<int, 6>{});
+      else if (nsteps % 4 == 0)
+        run(std::integral_constant<int, 4>{});
+      else if (nsteps % 3 == 0)
+        run(std::integral_constant<int, 3>{});
+      else if (nsteps % 2 == 0)
+        run(std::integral_constant<int, 2>{});
+      else
+        run(std::integral_constant<int, 1>{});
     }
     const int ngroups = fastA ? 0 : Kd / KG;
     int k = fastA ? Kd : 0;
     if (ngroups > 0) {
       fetch(avA, bvA, 0);
+      // the loads of a group are issued together: left to itself the scheduler, short of registers, issues
+      // them one at a time through a single register, and a product pays one memory latency per k-step
+      __builtin_amdgcn_sched_barrier(0);
       int gi = 0;
 #pragma nounroll
       for (; gi + 2 <= ngroups; gi += 2) {
         fetch(avB, bvB, (gi + 1) * KG);
+        __builtin_amdgcn_sched_barrier(0);
         fma_group(avA, bvA);
         if (gi + 2 < ngroups) fetch(avA, bvA, (gi + 2) * KG);
+        __builtin_amdgcn_sched_barrier(0);
         fma_group(avB, bvB);
       }
       if (gi < ngroups) fma_group(avA, bvA);
@@ -151,6 +189,29 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
       }
     }
   }
+}
+
+// Sum over r of p[r * stride] (+ q[r * stride]), r = 0..15, with all loads issued before the first add: written as
+// a plain loop the loads are issued one at a time, each waiting for the one before.
+__device__ __forceinline__ float col16_sum(const float* p, int stride) {
+  float v[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) v[r] = p[r * stride];
+  __builtin_amdgcn_sched_barrier(0);
+  float s = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s += v[r];
+  return s;
+}
+__device__ __forceinline__ float col16_sum2(const float* p, const float* q, int stride) {
+  float v[16], w[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) v[r] = p[r * stride], w[r] = q[r * stride];
+  __builtin_amdgcn_sched_barrier(0);
+  float s = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s += v[r] + w[r];
+  return s;
 }
 
 // Sum over the 16 lanes of a row, in every lane: four rotations inside the row on the DPP path

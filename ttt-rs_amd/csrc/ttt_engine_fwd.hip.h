@@ -232,8 +232,10 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
   constexpr int NBM = NTM / NW;  // hidden-side tile columns per job: one job per wave
   constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int t = tid >> 5, cg = tid & 31;
+  // re-derived from an opaque copy at the top of every mini-batch, so that the address arithmetic of the
+  // tile products is recomputed there instead of being hoisted out of the scan into (spilled) registers
+  int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int t = tid >> 5, cg = tid & 31;
   const size_t bh = blockIdx.x;
   const int h = (int)(bh % a.H), K = a.K;
   float *sb1 = lds + L::b1, *sb2 = lds + L::b2, *sgam = lds + L::gam, *sbet = lds + L::bet,
@@ -275,6 +277,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
   fetch(0);
 
   for (int st = 0; st < a.n_stages; ++st) {
+    asm volatile("" : "+v"(tid));
+    lane = tid & 63, wave = tid >> 6, t = tid >> 5, cg = tid & 31;
     const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
     // ---- XQ, XK, target = XV - XK from the prefetch registers
 #pragma unroll

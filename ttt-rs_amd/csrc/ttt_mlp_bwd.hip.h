@@ -84,7 +84,9 @@ __device__ __forceinline__ void gelu_tanh_all(float x, float& y, float& dy, floa
 }
 
 template <class T, int D>
-__global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
+// One workgroup per CU (the LDS use decides that), two waves per SIMD: said explicitly, because the scheduler
+// otherwise aims at a higher occupancy and, to save registers, issues independent loads one at a time.
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = MlpBwdLds<D>;
@@ -94,8 +96,11 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
   constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
   constexpr float inv_d = 1.0f / D;
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int t = tid >> 5, cg = tid & 31;  // elementwise mapping: token t, columns cg + 32 j
+  // The thread indices are re-derived from an opaque copy at the top of every mini-batch (below): the
+  // address arithmetic of the ~30 tile products is cheap, but hoisted out of the scan as loop invariants
+  // it would occupy several hundred registers and spill.
+  int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int t = tid >> 5, cg = tid & 31;  // elementwise mapping: token t, columns cg + 32 j
   const size_t bh = blockIdx.x;
   const int h = (int)(bh % a.H), K = a.K, N = a.n_stages;
   float *sb1 = lds + L::b1, *sb2 = lds + L::b2, *sdb1 = lds + L::db1, *sdb2 = lds + L::db2,
@@ -148,13 +153,22 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
   // this thread's NJM elements of a [16 x 4d] tile, all loads issued before any use (the tiles are
   // in global memory and may alias as far as the compiler knows, so a load-compute-store loop would
   // pay the full memory latency per element)
+  // One address per tile and immediate offsets for its NJM elements: the element offset is made opaque per
+  // call, or the compiler shares NJM 64-bit element indices between all tiles and spends a register pair and
+  // a 64-bit add on every access.
   auto ldm = [&](const float* tile, float (&v)[NJM]) {
+    int o = t * M + cg;
+    asm volatile("" : "+v"(o));
+    const float* p = tile + o;
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) v[j] = tile[t * M + cg + GW * j];
+    for (int j = 0; j < NJM; ++j) v[j] = p[GW * j];
   };
   auto stm = [&](float* tile, const float (&v)[NJM]) {
+    int o = t * M + cg;
+    asm volatile("" : "+v"(o));
+    float* p = tile + o;
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) tile[t * M + cg + GW * j] = v[j];
+    for (int j = 0; j < NJM; ++j) p[GW * j] = v[j];
   };
   auto part_sum = [&](int tt, int s) {
     float v = 0.f;
@@ -164,6 +178,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
   };
 
   for (int st = N - 1; st >= 0; --st) {
+    asm volatile("" : "+v"(tid));
+    lane = tid & 63, wave = tid >> 6, t = tid >> 5, cg = tid & 31;
     const float* G1l = a.G1s + ((bh * N + st) * (size_t)16) * M;
     const float* G2l = a.G2s + ((bh * N + st) * (size_t)16) * D;
     const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
@@ -180,12 +196,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     for (int j = 0; j < NJD; ++j) lds[L::TG + t * LD + cg + GW * j] -= lds[L::XK + t * LD + cg + GW * j];
     const float last = te_last * slr[t];
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
-    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, 16, wave, lane);
-    if (tid < M) {
-      float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += G1l[r * M + tid];
-      sb1[tid] += s;
-    }
+    mm_lds<1, NW, NBM, 4>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, 16, wave, lane);
+    if (tid < M) sb1[tid] += col16_sum(G1l + tid, M);
     __syncthreads();
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
     mm_lds<0, NW, NBM>(mZ1, M, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
@@ -204,12 +216,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     }
     __syncthreads();
     // ---- 4. roll W2, b2 back
-    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, 16, wave, lane);
-    if (tid < D) {
-      float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += G2l[r * D + tid];
-      sb2[tid] += s;
-    }
+    mm_lds<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, 16, wave, lane);
+    if (tid < D) sb2[tid] += col16_sum(G2l + tid, D);
     __syncthreads();
     // ---- 5. Z2 = X2 W2 ; A1 = XQ XK^T ; eta
     mm_lds<0, NW>(lds + L::XH, LD, mX2, M, 1, W2, D, 1, 1, NTD, M, wave, lane);
@@ -264,7 +272,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     }
     __syncthreads();
     // ---- 9. Zbar1 -= M1 G1 ; then + b1, Xbar2 = gelu
-    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(mZB1, M, lds + L::M1, LK, 1, mG1, M, 1, 1, NTM, 16, wave, lane);
+    mm_lds<2, NW, NBM, 4>(mZB1, M, lds + L::M1, LK, 1, mG1, M, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
     {
       float z[NJM], y[NJM];
@@ -338,9 +346,9 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     }
     __syncthreads();
     // ---- 14. dXbar2 += dA2 X2 ; dG2 -= M2^T dZbar2 ; dX2 = dA2^T Xbar2
-    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(mDXB, M, lds + L::DA, LK, 1, mX2, M, 1, 1, NTM, 16, wave, lane);
+    mm_lds<1, NW, NBM, 4>(mDXB, M, lds + L::DA, LK, 1, mX2, M, 1, 1, NTM, 16, wave, lane);
     mm_lds<2, NW, 1, 4>(lds + L::DG2, LD, lds + L::M2, 1, LK, lds + L::DZB2, LD, 1, 1, NTD, 16, wave, lane);
-    mm_lds<0, NW, NBM, (NBM >= 3 ? 1 : 2)>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
+    mm_lds<0, NW, NBM, 4>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
     // ---- 15. dX2 -= (last G2) dW2^T ; dZbar1 = dXbar2 gelu'(Zbar1)
     mm_lds<2, NW, NBM>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
@@ -385,7 +393,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     }
     __syncthreads();
     // ---- 18. dG1 -= M1^T dZbar1 ; dQ += dA1 XK ; dK = dA1^T XQ
-    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(mS1, M, lds + L::M1, 1, LK, mDXB, M, 1, 1, NTM, 16, wave, lane);
+    mm_lds<2, NW, NBM, 4>(mS1, M, lds + L::M1, 1, LK, mDXB, M, 1, 1, NTM, 16, wave, lane);
     mm_lds<1, NW, 1, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NTD, 16, wave, lane);
     mm_lds<0, NW, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NTD, 16, wave, lane, NTD % NW);
     __syncthreads();
@@ -469,15 +477,11 @@ __global__ void __launch_bounds__(512) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
     __syncthreads();
     // ---- 23. gradient accumulation; dK += dZ1 W1^T
     // dW2 += X2^T dZ2 + dU^T G2 + Xbar2^T dZbar2 as ONE rank-48 pass over dW2 (operands consecutive)
-    mm_lds<1, NW, NBD, (NBD >= 3 ? 1 : 2)>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, 48, wave, lane);
+    mm_lds<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, 48, wave, lane);
     // dW1 += XQ^T dZbar1 + XK^T dZ1 as one rank-32 pass
-    mm_lds<1, NW, NBM, (NBM >= 3 ? 1 : 2)>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, 32, wave, lane);
+    mm_lds<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, 32, wave, lane);
     mm_lds<1, NW>(lds + L::DK, LD, mDX2, M, 1, W1, 1, M, 1, NTD, M, wave, lane);
-    if (tid < M) {
-      float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += mDXB[r * M + tid] + mDX2[r * M + tid];
-      sdb1[tid] += s;
-    }
+    if (tid < M) sdb1[tid] += col16_sum2(mDXB + tid, mDX2 + tid, M);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < 16; ++r) s += lds[L::DZB2 + r * LD + tid] + lds[L::DZ2 + r * LD + tid];
