@@ -191,6 +191,90 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
   }
 }
 
+// Rank-K update of a matrix in global memory, K = 4 * KS small (16, 32, 48):
+//   C[16*Mt x 16*Nt] (+/-)= A * B   with A(m,k) = A[m*a_rs + k*a_cs], B(k,n) = B[k*b_rs + n*b_cs],
+// MODE 1: C += AB, 2: C -= AB; Nt a multiple of NB.  Jobs (tile row, NB tile columns) are dealt round-robin to the
+// waves as in mm_lds.  A job is a read-modify-write of its C tiles with only 4*KS*NB matrix instructions
+// in between, so a wave that handled its jobs one after the other would sit through a load latency and a
+// store latency per job.  Here the C tiles and operands of a wave's NEXT job are requested before the matrix
+// instructions of the current one (two register sets in ping-pong).  Every load is unconditional: past a
+// wave's last job the last job is re-read (and dropped), because a load under a branch makes the waits that
+// follow count as if it had not been issued.
+template <int MODE, int NW, int NB, int KS>
+__device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
+                                        int b_rs, int b_cs, int Mt, int Nt, int wave, int lane) {
+  static_assert(MODE == 1 || MODE == 2, "read-modify-write modes only");
+  const int c = lane & 15, g = lane >> 4;
+  const int nblk = Nt / NB, njobs = Mt * nblk;
+  // When the number of column blocks divides the number of waves, all jobs of a wave lie in one column block
+  // and share their B operand: it is loaded once and kept in registers.
+  const bool bfix = NW % nblk == 0;
+  float bf[KS][NB];
+  if (bfix) {
+    const int boff = g * b_rs + (16 * (wave % nblk) * NB + c) * b_cs;
+#pragma unroll
+    for (int u = 0; u < KS; ++u)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) bf[u][j] = B[boff + 4 * u * b_rs + 16 * j * b_cs];
+  }
+  struct Set {
+    f32x4 acc[NB];
+    float av[KS], bv[KS][NB];
+  };
+  auto request = [&](int job, Set& s) {
+    const int tm = job / nblk, tn0 = (job - tm * nblk) * NB;
+    const int coff = (16 * tm + 4 * g) * ldc + 16 * tn0 + c;
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s.acc[j][r] = C[coff + r * ldc + 16 * j];
+    const int aoff = (16 * tm + c) * a_rs + g * a_cs, boff = g * b_rs + (16 * tn0 + c) * b_cs;
+#pragma unroll
+    for (int u = 0; u < KS; ++u) {
+      s.av[u] = A[aoff + 4 * u * a_cs];
+      if (!bfix) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) s.bv[u][j] = B[boff + 4 * u * b_rs + 16 * j * b_cs];
+      }
+    }
+  };
+  auto finish = [&](int job, Set& s) {
+    const int tm = job / nblk, tn0 = (job - tm * nblk) * NB;
+    const int coff = (16 * tm + 4 * g) * ldc + 16 * tn0 + c;
+    if (MODE == 2) {
+#pragma unroll
+      for (int u = 0; u < KS; ++u) s.av[u] = -s.av[u];
+    }
+#pragma unroll
+    for (int u = 0; u < KS; ++u)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        s.acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(s.av[u], bfix ? bf[u][j] : s.bv[u][j], s.acc[j], 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) C[coff + r * ldc + 16 * j] = s.acc[j][r];
+  };
+  int job = wave;
+  if (job >= njobs) return;
+  const int last = job + ((njobs - 1 - job) / NW) * NW;  // this wave's last job
+  Set s0, s1;
+  request(job, s0);
+#pragma nounroll
+  for (;;) {
+    const int j1 = job + NW, j2 = job + 2 * NW;
+    request(j1 <= last ? j1 : last, s1);
+    __builtin_amdgcn_sched_barrier(0);
+    finish(job, s0);
+    if (j1 > last) break;
+    request(j2 <= last ? j2 : last, s0);
+    __builtin_amdgcn_sched_barrier(0);
+    finish(j1, s1);
+    if (j2 > last) break;
+    job = j2;
+  }
+}
+
 // Sum over r of p[r * stride] (+ q[r * stride]), r = 0..15, with all loads issued before the first add: written as
 // a plain loop the loads are issued one at a time, each waiting for the one before.
 __device__ __forceinline__ float col16_sum(const float* p, int stride) {

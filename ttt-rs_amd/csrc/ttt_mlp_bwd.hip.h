@@ -196,7 +196,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < NJD; ++j) lds[L::TG + t * LD + cg + GW * j] -= lds[L::XK + t * LD + cg + GW * j];
     const float last = te_last * slr[t];
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
-    mm_lds<1, NW, NBM, 4>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, 16, wave, lane);
+    mm_rank<1, NW, NBM, 4>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane);
     if (tid < M) sb1[tid] += col16_sum(G1l + tid, M);
     __syncthreads();
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
@@ -216,7 +216,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 4. roll W2, b2 back
-    mm_lds<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, 16, wave, lane);
+    mm_rank<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, wave, lane);
     if (tid < D) sb2[tid] += col16_sum(G2l + tid, D);
     __syncthreads();
     // ---- 5. Z2 = X2 W2 ; A1 = XQ XK^T ; eta
@@ -477,9 +477,9 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 23. gradient accumulation; dK += dZ1 W1^T
     // dW2 += X2^T dZ2 + dU^T G2 + Xbar2^T dZbar2 as ONE rank-48 pass over dW2 (operands consecutive)
-    mm_lds<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, 48, wave, lane);
+    mm_rank<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, wave, lane);
     // dW1 += XQ^T dZbar1 + XK^T dZ1 as one rank-32 pass
-    mm_lds<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, 32, wave, lane);
+    mm_rank<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, wave, lane);
     mm_lds<1, NW>(lds + L::DK, LD, mDX2, M, 1, W1, 1, M, 1, NTD, M, wave, lane);
     if (tid < M) sdb1[tid] += col16_sum2(mDXB + tid, mDX2 + tid, M);
     if (tid < D) {
