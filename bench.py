@@ -256,7 +256,9 @@ def main():
                              checkpoint_format="f32 row-major" if (ci != 1 or os.environ.get("TTT_BENCH_CKPT") == "f32") else "packed")
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
                            "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
-                           "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)",
+                           "kernel": ("ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)"
+                                      if ci == 1 and os.environ.get("TTT_LINEAR_BWD_KERNEL") != "lds" else
+                                      "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_kernel (whole step)"),
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops,
                            "algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)}
     elif kind == "mlp_fwd":
