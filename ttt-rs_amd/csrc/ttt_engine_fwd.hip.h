@@ -223,7 +223,8 @@ struct MlpLds {
 };
 
 template <class T, int D>
-__global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
+// one workgroup per CU (LDS), two waves per SIMD: stated so that the scheduler does not serialise loads to save registers
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = MlpLds<D>;
@@ -327,7 +328,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
     mm_lds<3, NW, NBM>(lds + L::BA, LM, lds + L::Z2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- Zbar1 -= M1 G1                                       (mlp.rs:164-169)
-    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(lds + L::BC, LM, lds + L::M1, LK, 1, lds + L::BA, LM, 1, 1, NTM, 16, wave, lane);
+    mm_lds<2, NW, NBM, 4>(lds + L::BC, LM, lds + L::M1, LK, 1, lds + L::BA, LM, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
     // ---- Xbar2 = gelu(Zbar1 + b1)                             (mlp.rs:171)
 #pragma unroll
@@ -388,8 +389,8 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
     }
     __syncthreads();
     // ---- W1 -= XK^T G1l ; W2 -= X2^T G2l ; b1 -= colsum(G1l) ; b2 -= colsum(G2l)
-    mm_lds<2, NW, NBM, (NBM >= 3 ? 1 : 2)>(W1, M, lds + L::XK, 1, LD, lds + L::BA, LM, 1, NTD, NTM, 16, wave, lane);
-    mm_lds<2, NW, NBD, (NBD >= 3 ? 1 : 2)>(W2, D, lds + L::BB, 1, LM, lds + L::Z2, LD, 1, NTM, NTD, 16, wave, lane);
+    mm_rank<2, NW, NBM, 4>(W1, M, lds + L::XK, 1, LD, lds + L::BA, LM, 1, NTD, NTM, wave, lane);
+    mm_rank<2, NW, NBD, 4>(W2, D, lds + L::BB, 1, LM, lds + L::Z2, LD, 1, NTM, NTD, wave, lane);
     if (tid < M) {
       float s = 0.f;
       for (int r = 0; r < 16; ++r) s += lds[L::BA + r * LM + tid];
