@@ -275,6 +275,61 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
   }
 }
 
+// C[16 x 16*NT] (LDS, row stride ldc) op= A[16 x Kd] * B[Kd x 16*NT] with Kd = NW * 16 * KSTEPS split over the waves:
+// wave w takes k in [w*16*KSTEPS, (w+1)*16*KSTEPS) for ALL NT tile columns, leaves its partial product in
+// part[w] (LDS, NW tiles of 16 rows, stride ldc), and after a barrier the partials are summed in wave order
+// (deterministic).  MODE 0: C = AB, 1: C += AB, 2: C -= AB.  A is contiguous along k (rows 16-byte aligned); B is
+// read 16 bytes at a time where it is contiguous along k too.  Against one job per tile column (mm_lds) every
+// element of A is fetched once instead of NT times, all NW waves work, and every operand of a wave is requested
+// before its first matrix instruction.  Contains a barrier: call from all threads; the caller's next barrier
+// publishes C.
+template <int MODE, int NW, int NT, int KSTEPS>
+__device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const float* A, int a_rs, const float* B,
+                                          int b_rs, int b_cs, int wave, int lane, int tid) {
+  const int c = lane & 15, g = lane >> 4;
+  const int k0 = wave * 16 * KSTEPS + 4 * g;
+  const bool vecB = b_rs == 1 && (b_cs & 3) == 0;
+  f32x4 av[KSTEPS], bv[KSTEPS][NT];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    av[s] = *reinterpret_cast<const f32x4*>(A + c * a_rs + k0 + 16 * s);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const float* pb = B + (k0 + 16 * s) * b_rs + (16 * j + c) * b_cs;
+      if (vecB) {
+        bv[s][j] = *reinterpret_cast<const f32x4*>(pb);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) bv[s][j][r] = pb[r * b_rs];
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  f32x4 acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s][r], bv[s][j][r], acc[j], 0, 0, 0);
+  float* mine = part + wave * 16 * ldc;
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) mine[(4 * g + r) * ldc + 16 * j + c] = acc[j][r];
+  __syncthreads();
+  for (int i = tid; i < 16 * 16 * NT; i += NW * 64) {
+    const int row = i / (16 * NT), col = i - row * (16 * NT);
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) v += part[(w * 16 + row) * ldc + col];
+    float* pc = C + row * ldc + col;
+    *pc = MODE == 0 ? v : MODE == 1 ? *pc + v : *pc - v;
+  }
+}
+
 // Sum over r of p[r * stride] (+ q[r * stride]), r = 0..15, with all loads issued before the first add: written as
 // a plain loop the loads are issued one at a time, each waiting for the one before.
 __device__ __forceinline__ float col16_sum(const float* p, int stride) {

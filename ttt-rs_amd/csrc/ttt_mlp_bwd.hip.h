@@ -68,7 +68,10 @@ struct MlpBwdLds {
                        DA = P + KK, DETA = DA + KK, PART = DETA + KK;
   static constexpr int b1 = PART + 8 * 256, b2 = b1 + M, db1 = b2 + D, db2 = db1 + M, gam = db2 + D,
                        bet = gam + D, lr = bet + D, te = lr + 16, rstd1 = te + 16, dlast = rstd1 + 16,
-                       END = dlast + 16;
+                       SKP = dlast + 16;
+  // partial products of the split-k [16 x d] products, one tile per wave: where LDS has the room (d <= 96)
+  static constexpr bool SPLITK = D <= 96;
+  static constexpr int END = SKP + (SPLITK ? 8 * TD : 0);
   static constexpr size_t BYTES = sizeof(float) * END;
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
@@ -170,6 +173,18 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
     for (int j = 0; j < NJM; ++j) p[GW * j] = v[j];
   };
+  // C[16 x d] (LDS) op= A[16 x 4d] (global tile) * B[4d x d]: split over k across the waves where LDS has room
+  // for the partial products, one job per tile column otherwise
+  auto prod_k = [&](auto mode, float* C, const float* A, const float* B, int b_rs, int b_cs) {
+    constexpr int MODE = decltype(mode)::value;
+    if constexpr (L::SPLITK)
+      mm_splitk<MODE, NW, NTD, M / (16 * NW)>(C, LD, lds + L::SKP, A, M, B, b_rs, b_cs, wave, lane, tid);
+    else
+      mm_lds<MODE, NW>(C, LD, A, M, 1, B, b_rs, b_cs, 1, NTD, M, wave, lane);
+  };
+  using M0 = std::integral_constant<int, 0>;
+  using M1 = std::integral_constant<int, 1>;
+  using M2 = std::integral_constant<int, 2>;
   auto part_sum = [&](int tt, int s) {
     float v = 0.f;
 #pragma unroll
@@ -220,7 +235,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (tid < D) sb2[tid] += col16_sum(G2l + tid, D);
     __syncthreads();
     // ---- 5. Z2 = X2 W2 ; A1 = XQ XK^T ; eta
-    mm_lds<0, NW>(lds + L::XH, LD, mX2, M, 1, W2, D, 1, 1, NTD, M, wave, lane);
+    prod_k(M0{}, lds + L::XH, mX2, W2, D, 1);
     mm_lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, NTD % NW);
     if (tid < 256) {
       const int tt = tid >> 4, s = tid & 15;
@@ -289,7 +304,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 10. A2 = Xbar2 X2^T (split-k) ; Zbar2 = Xbar2 W2
     splitk_xyT(mXB2, mX2);
-    mm_lds<0, NW>(lds + L::XH2, LD, mXB2, M, 1, W2, D, 1, 1, NTD, M, wave, lane);
+    prod_k(M0{}, lds + L::XH2, mXB2, W2, D, 1);
     __syncthreads();
     if (tid < 256) {
       const int tt = tid >> 4, s = tid & 15;
@@ -321,7 +336,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     // ---- 12. P2 = dZbar2 G2^T ; dXbar2 = dZbar2 W2^T ; S2 = X2 dW2
     mm_lds<0, NW>(lds + L::P, LK, lds + L::DZB2, LD, 1, lds + L::G2, 1, LD, 1, 1, D, wave, lane, NW - 1);
     mm_lds<0, NW, NBM>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
-    mm_lds<0, NW>(lds + L::DG2, LD, mX2, M, 1, dW2, D, 1, 1, NTD, M, wave, lane);
+    prod_k(M0{}, lds + L::DG2, mX2, dW2, D, 1);
     __syncthreads();
     // ---- 13. dA2, d eta ; dG2 = -last (S2 + db2) ; d last
     if (tid < 256) {
@@ -367,7 +382,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 16. P1 = dZbar1 G1^T (split-k) ; dQ = dZbar1 W1^T ; S1 = XK dW1
     splitk_xyT(mDXB, mG1);
-    mm_lds<0, NW>(lds + L::DQ, LD, mDXB, M, 1, W1, 1, M, 1, NTD, M, wave, lane);
+    prod_k(M0{}, lds + L::DQ, mDXB, W1, 1, M);
     mm_lds<0, NW, NBM>(mS1, M, lds + L::XK, LD, 1, dW1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 17. dA1, d eta ; dG1 = -last (S1 + db1) ; d last
@@ -398,7 +413,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     mm_lds<0, NW, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NTD, 16, wave, lane, NTD % NW);
     __syncthreads();
     // ---- 19. dK -= (last G1) dW1^T ; dU = dG1 gelu'(Z1) (kept in mU's place after saving U * gelu'')
-    mm_lds<2, NW>(lds + L::DK, LD, G1l, M, 1, dW1, 1, M, 1, NTD, M, wave, lane);
+    prod_k(M2{}, lds + L::DK, G1l, dW1, 1, M);
     {
       float z[NJM], dg1[NJM], u[NJM];
       ldm(mZ1, z);
@@ -416,7 +431,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 20. dG2 += dU W2
-    mm_lds<1, NW>(lds + L::DG2, LD, mU, M, 1, W2, D, 1, 1, NTD, M, wave, lane);
+    prod_k(M1{}, lds + L::DG2, mU, W2, D, 1);
     __syncthreads();
     // ---- 21. second-order LayerNorm: dZ2, dT, d gamma, d beta
     {
@@ -480,7 +495,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     mm_rank<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, wave, lane);
     // dW1 += XQ^T dZbar1 + XK^T dZ1 as one rank-32 pass
     mm_rank<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, wave, lane);
-    mm_lds<1, NW>(lds + L::DK, LD, mDX2, M, 1, W1, 1, M, 1, NTD, M, wave, lane);
+    prod_k(M1{}, lds + L::DK, mDX2, W1, 1, M);
     if (tid < M) sdb1[tid] += col16_sum2(mDXB + tid, mDX2 + tid, M);
     if (tid < D) {
       float s = 0.f;
