@@ -11,6 +11,26 @@
 
 namespace ttt {
 
+// 16 rows x 64 bytes of a row-major matrix in GLOBAL memory, delivered in matrix-operand order: lane (c = lane % 16,
+// g = lane / 16) receives the 16 bytes at row c, byte offset 16 g.  Loaded directly in that order, each quarter
+// wave (16 lanes with the same g) touches 16 cache lines and the load runs at 16 B per cycle and CU; here lane l
+// loads row l / 4, chunk l % 4, so a quarter wave touches 4 lines (the rate of a coalesced load), and the values
+// change lanes afterwards (ds_bpermute: lane 16 g + c takes from lane 4 c + g).  `load_rows_raw` issues the load,
+// `rows_to_operand` does the exchange, so that the exchange can sit where the value is used.
+__device__ __forceinline__ f32x4 load_rows_raw(const float* block, int row_stride, int lane) {
+  return *reinterpret_cast<const f32x4*>(block + (lane >> 2) * row_stride + 4 * (lane & 3));
+}
+__device__ __forceinline__ f32x4 rows_to_operand(const f32x4& v, int lane) {
+  const int src = 4 * (4 * (lane & 15) + (lane >> 4));
+  f32x4 o;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float x = v[r];  // through a scalar: a bit_cast applied to the vector element itself reads element 0
+    o[r] = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(x)));
+  }
+  return o;
+}
+
 // C[16*Mt x 16*Nt] (row-major, stride ldc)  op=  A * B over k in [k0, k0+Kd), Kd a multiple of 4.
 // A(m,k) = A[m*a_rs + k*a_cs], B(k,n) = B[k*b_rs + n*b_cs].
 // MODE 0: C = AB   1: C += AB   2: C -= AB   3: C *= AB (elementwise)
@@ -19,7 +39,9 @@ namespace ttt {
 // dealt round-robin to the NW waves of the workgroup, starting at wave `first`.  Inside a job the
 // A element of a k-step is loaded once and feeds NB MFMAs, and KU k-steps of operands are fetched
 // before the first MFMA of the group issues, so the loads of a group overlap its MFMAs.
-template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8)>
+// BG: B is in global memory and contiguous along k (a transposed weight matrix): loaded four lanes to a row and
+// exchanged between lanes before use (load_rows_raw / rows_to_operand).
+template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false>
 __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_rs, int a_cs,
                                        const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
                                        int wave, int lane, int first = 0, int k0 = 0) {
@@ -88,7 +110,9 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
         const bool live = Nt % NB == 0 || tn0 + j < Nt;
         const float* pb = B + bo + kk * b_rs + (live ? j : 0) * bcol;
         f32x4 v;
-        if (vecB) {
+        if (BG) {
+          v = load_rows_raw(B + (k0 + kk) * b_rs + 16 * (tn0 + (live ? j : 0)) * b_cs, b_cs, lane);
+        } else if (vecB) {
           v = *reinterpret_cast<const f32x4*>(pb);
         } else {
 #pragma unroll
@@ -122,6 +146,10 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
         for (; kk + 16 * PF < Kd; kk += 16 * PF) {
 #pragma unroll
           for (int u = 0; u < PF; ++u) {
+            if (BG) {
+#pragma unroll
+              for (int j = 0; j < NB; ++j) bv[u][j] = rows_to_operand(bv[u][j], lane);
+            }
             step(av[u], bv[u]);
             av[u] = loadA(kk + 16 * (PF + u));
 #pragma unroll
@@ -130,7 +158,13 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
           }
         }
 #pragma unroll
-        for (int u = 0; u < PF; ++u) step(av[u], bv[u]);
+        for (int u = 0; u < PF; ++u) {
+          if (BG) {
+#pragma unroll
+            for (int j = 0; j < NB; ++j) bv[u][j] = rows_to_operand(bv[u][j], lane);
+          }
+          step(av[u], bv[u]);
+        }
       };
       constexpr int PFMAX = NB >= 4 ? 4 : NB == 3 ? 6 : 8;
       const int nsteps = Kd >> 4;
@@ -278,8 +312,8 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
 // C[16 x 16*NT] (LDS, row stride ldc) op= A[16 x Kd] * B[Kd x 16*NT] with Kd = NW * 16 * KSTEPS split over the waves:
 // wave w takes k in [w*16*KSTEPS, (w+1)*16*KSTEPS) for ALL NT tile columns, leaves its partial product in
 // part[w] (LDS, NW tiles of 16 rows, stride ldc), and after a barrier the partials are summed in wave order
-// (deterministic).  MODE 0: C = AB, 1: C += AB, 2: C -= AB.  A is contiguous along k (rows 16-byte aligned); B is
-// read 16 bytes at a time where it is contiguous along k too.  Against one job per tile column (mm_lds) every
+// (deterministic).  MODE 0: C = AB, 1: C += AB, 2: C -= AB.  A is in global memory, contiguous along k (rows 16-byte
+// aligned), and so is B where b_rs == 1: both are then loaded four lanes to a row (load_rows_raw).  Against one job per tile column (mm_lds) every
 // element of A is fetched once instead of NT times, all NW waves work, and every operand of a wave is requested
 // before its first matrix instruction.  Contains a barrier: call from all threads; the caller's next barrier
 // publishes C.
@@ -287,17 +321,17 @@ template <int MODE, int NW, int NT, int KSTEPS>
 __device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const float* A, int a_rs, const float* B,
                                           int b_rs, int b_cs, int wave, int lane, int tid) {
   const int c = lane & 15, g = lane >> 4;
-  const int k0 = wave * 16 * KSTEPS + 4 * g;
+  const int kw = wave * 16 * KSTEPS, k0 = kw + 4 * g;
   const bool vecB = b_rs == 1 && (b_cs & 3) == 0;
   f32x4 av[KSTEPS], bv[KSTEPS][NT];
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) {
-    av[s] = *reinterpret_cast<const f32x4*>(A + c * a_rs + k0 + 16 * s);
+    av[s] = load_rows_raw(A + kw + 16 * s, a_rs, lane);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       const float* pb = B + (k0 + 16 * s) * b_rs + (16 * j + c) * b_cs;
       if (vecB) {
-        bv[s][j] = *reinterpret_cast<const f32x4*>(pb);
+        bv[s][j] = load_rows_raw(B + (kw + 16 * s) * b_rs + 16 * j * b_cs, b_cs, lane);
       } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r) bv[s][j][r] = pb[r * b_rs];
@@ -305,6 +339,15 @@ __device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const 
     }
   }
   __builtin_amdgcn_sched_barrier(0);
+  // A (and B where it is contiguous along k) arrived four lanes to a row: into operand order
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    av[s] = rows_to_operand(av[s], lane);
+    if (vecB) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) bv[s][j] = rows_to_operand(bv[s][j], lane);
+    }
+  }
   f32x4 acc[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};

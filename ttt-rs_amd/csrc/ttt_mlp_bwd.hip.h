@@ -269,7 +269,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 7. U = G2 W2^T ; Zbar1 = XQ W1
-    mm_lds<0, NW, NBM>(mU, M, lds + L::G2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<0, NW, NBM, 2, true>(mU, M, lds + L::G2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     mm_lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 8. G1 = U gelu'(Z1)
@@ -335,7 +335,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 12. P2 = dZbar2 G2^T ; dXbar2 = dZbar2 W2^T ; S2 = X2 dW2
     mm_lds<0, NW>(lds + L::P, LK, lds + L::DZB2, LD, 1, lds + L::G2, 1, LD, 1, 1, D, wave, lane, NW - 1);
-    mm_lds<0, NW, NBM>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<0, NW, NBM, 2, true>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     prod_k(M0{}, lds + L::DG2, mX2, dW2, D, 1);
     __syncthreads();
     // ---- 13. dA2, d eta ; dG2 = -last (S2 + db2) ; d last
@@ -366,7 +366,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     mm_lds<0, NW, NBM, 4>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
     // ---- 15. dX2 -= (last G2) dW2^T ; dZbar1 = dXbar2 gelu'(Zbar1)
-    mm_lds<2, NW, NBM>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<2, NW, NBM, 2, true>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
     {
       float z[NJM], v[NJM];
       ldm(mZB1, z);
@@ -474,7 +474,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 22. dX2 += dZ2 W2^T ; then dZ1 = dG1 U gelu''(Z1) + dX2 gelu'(Z1)
-    mm_lds<1, NW, NBM>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<1, NW, NBM, 2, true>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     {
       float z[NJM], f1[NJM], dx[NJM];
