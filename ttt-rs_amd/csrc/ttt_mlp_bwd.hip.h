@@ -144,12 +144,23 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   // C[16 x 16] (PART slices) = X Y^T over the 4d columns of two [16 x 4d] tiles, one k-slice per wave
   auto splitk_xyT = [&](const float* X, const float* Y) {
     const int c = lane & 15, g = lane >> 4;
-    constexpr int KS = M / NW;
+    constexpr int KS = M / NW, NS = KS / 16;
+    static_assert(KS % 16 == 0, "a wave's k-slice is a whole number of 16-deep steps");
+    // both tiles are contiguous along k: loaded four lanes to a row, then exchanged into operand order
+    f32x4 xa[NS], ya[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      xa[s] = load_rows_raw(X + wave * KS + 16 * s, M, lane);
+      ya[s] = load_rows_raw(Y + wave * KS + 16 * s, M, lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    const float* Ap = X + c * M + wave * KS + g;
-    const float* Bp = Y + c * M + wave * KS + g;
-#pragma unroll 4
-    for (int k = 0; k < KS; k += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ap[k], Bp[k], acc, 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const f32x4 xo = rows_to_operand(xa[s], lane), yo = rows_to_operand(ya[s], lane);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[r], yo[r], acc, 0, 0, 0);
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) lds[L::PART + wave * 256 + (4 * g + r) * 16 + c] = acc[r];
   };
