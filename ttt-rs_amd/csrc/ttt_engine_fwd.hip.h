@@ -325,7 +325,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- G1 = (G2 W2^T) * gelu'(Z1)                           (mlp.rs:151-152)
-    mm_lds<3, NW, NBM>(lds + L::BA, LM, lds + L::Z2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    mm_lds<3, NW, NBM, 2, true>(lds + L::BA, LM, lds + L::Z2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- Zbar1 -= M1 G1                                       (mlp.rs:164-169)
     mm_lds<2, NW, NBM, 4>(lds + L::BC, LM, lds + L::M1, LK, 1, lds + L::BA, LM, 1, 1, NTM, 16, wave, lane);
