@@ -277,6 +277,9 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   };
   fetch(0);
 
+  // without an output buffer (the sweep that the backward runs for the update factors and the final state) the
+  // output branch of every mini-batch is skipped: two of the five passes over the state and eight barriers
+  const bool want_out = a.out != nullptr;
   for (int st = 0; st < a.n_stages; ++st) {
     asm volatile("" : "+v"(tid));
     lane = tid & 63, wave = tid >> 6, t = tid >> 5, cg = tid & 31;
@@ -294,8 +297,10 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (st + 1 < a.n_stages) fetch(st + 1);
     // ---- Z1 = XK W1 ; Zbar1 = XQ W1 ; A1 = XQ XK^T            (mlp.rs:139,160,167)
     mm_lds<0, NW, NBM>(lds + L::BA, LM, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
-    mm_lds<0, NW, NBM>(lds + L::BC, LM, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
-    mm_lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane);
+    if (want_out) {
+      mm_lds<0, NW, NBM>(lds + L::BC, LM, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
+      mm_lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane);
+    }
     __syncthreads();
     // ---- X2 = gelu(Z1 + b1), keep gelu'(Z1 + b1) ; eta, M1 = eta (1 + A1)   (mlp.rs:141,154-162)
 #pragma unroll
@@ -306,7 +311,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       lds[L::BB + t * LM + o] = y;
       lds[L::BA + t * LM + o] = dy;
     }
-    if (tid < 256) {
+    if (want_out && tid < 256) {
       const int tt = tid >> 4, s = tid & 15;
       const float et = (s <= tt) ? ste[tt] * slr[s] : 0.f;
       lds[L::ETA + tt * LK + s] = et;
@@ -327,56 +332,61 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     // ---- G1 = (G2 W2^T) * gelu'(Z1)                           (mlp.rs:151-152)
     mm_lds<3, NW, NBM, 2, true>(lds + L::BA, LM, lds + L::Z2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
-    // ---- Zbar1 -= M1 G1                                       (mlp.rs:164-169)
-    mm_lds<2, NW, NBM, 4>(lds + L::BC, LM, lds + L::M1, LK, 1, lds + L::BA, LM, 1, 1, NTM, 16, wave, lane);
-    __syncthreads();
-    // ---- Xbar2 = gelu(Zbar1 + b1)                             (mlp.rs:171)
+    if (want_out) {  // the output branch: skipped when only the update factors and the final state are wanted
+      // ---- Zbar1 -= M1 G1                                       (mlp.rs:164-169)
+      mm_lds<2, NW, NBM, 4>(lds + L::BC, LM, lds + L::M1, LK, 1, lds + L::BA, LM, 1, 1, NTM, 16, wave, lane);
+      __syncthreads();
+      // ---- Xbar2 = gelu(Zbar1 + b1)                             (mlp.rs:171)
 #pragma unroll
-    for (int j = 0; j < NJM; ++j) {
-      const int o = cg + GW * j;
-      float y, dy;
-      gelu_tanh_pair(lds[L::BC + t * LM + o] + sb1[o], y, dy);
-      lds[L::BC + t * LM + o] = y;
-    }
-    __syncthreads();
-    // ---- A2 = Xbar2 X2^T (split over k, one slice per wave) ; Zbar2 = Xbar2 W2   (mlp.rs:173,178)
-    {
-      const int c = lane & 15, g = lane >> 4;
-      constexpr int KS = M / NW;  // k-slice per wave (multiple of 4)
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      const float* Ap = lds + L::BC + c * LM + wave * KS + g;
-      const float* Bp = lds + L::BB + c * LM + wave * KS + g;
+      for (int j = 0; j < NJM; ++j) {
+        const int o = cg + GW * j;
+        float y, dy;
+        gelu_tanh_pair(lds[L::BC + t * LM + o] + sb1[o], y, dy);
+        lds[L::BC + t * LM + o] = y;
+      }
+      __syncthreads();
+      // ---- A2 = Xbar2 X2^T (split over k, one slice per wave) ; Zbar2 = Xbar2 W2   (mlp.rs:173,178)
+      {
+        const int c = lane & 15, g = lane >> 4;
+        constexpr int KS = M / NW;  // k-slice per wave (multiple of 4)
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const float* Ap = lds + L::BC + c * LM + wave * KS + g;
+        const float* Bp = lds + L::BB + c * LM + wave * KS + g;
 #pragma unroll 4
-      for (int k = 0; k < KS; k += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ap[k], Bp[k], acc, 0, 0, 0);
+        for (int k = 0; k < KS; k += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ap[k], Bp[k], acc, 0, 0, 0);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) lds[L::PART + wave * 256 + (4 * g + r) * 16 + c] = acc[r];
-    }
-    mm_lds<0, NW>(lds + L::ZB2, LD, lds + L::BC, LM, 1, W2, D, 1, 1, NTD, M, wave, lane);
-    __syncthreads();
-    if (tid < 256) {
-      const int tt = tid >> 4, s = tid & 15;
-      float a2 = 0.f;
+        for (int r = 0; r < 4; ++r) lds[L::PART + wave * 256 + (4 * g + r) * 16 + c] = acc[r];
+      }
+      mm_lds<0, NW>(lds + L::ZB2, LD, lds + L::BC, LM, 1, W2, D, 1, 1, NTD, M, wave, lane);
+      __syncthreads();
+      if (tid < 256) {
+        const int tt = tid >> 4, s = tid & 15;
+        float a2 = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) a2 += lds[L::PART + w * 256 + tt * 16 + s];
-      lds[L::M2 + tt * LK + s] = lds[L::ETA + tt * LK + s] * (1.f + a2);
+        for (int w = 0; w < NW; ++w) a2 += lds[L::PART + w * 256 + tt * 16 + s];
+        lds[L::M2 + tt * LK + s] = lds[L::ETA + tt * LK + s] * (1.f + a2);
+      }
+      __syncthreads();
+      // ---- Zbar2 -= M2 G2                                       (mlp.rs:175-180)
+      mm_lds<2, NW, 1, 4>(lds + L::ZB2, LD, lds + L::M2, LK, 1, lds + L::Z2, LD, 1, 1, NTD, 16, wave, lane);
+      __syncthreads();
     }
-    __syncthreads();
-    // ---- Zbar2 -= M2 G2                                       (mlp.rs:175-180)
-    mm_lds<2, NW, 1, 4>(lds + L::ZB2, LD, lds + L::M2, LK, 1, lds + L::Z2, LD, 1, 1, NTD, 16, wave, lane);
-    __syncthreads();
     // ---- out = XQ + LN(Zbar2 + b2) ; scale G1, G2 by eta_last  (mlp.rs:182-207)
     {
-      float xh[NJD], rstd;
-      ln_stats<D, GW>(lds + L::ZB2 + t * LD, sb2, cg, a.eps, xh, rstd);
       const float last = te_last * slr[t];
+      if (want_out) {
+        float xh[NJD], rstd;
+        ln_stats<D, GW>(lds + L::ZB2 + t * LD, sb2, cg, a.eps, xh, rstd);
 #pragma unroll
-      for (int j = 0; j < NJD; ++j) {
-        const int o = cg + GW * j;
-        if (t < K && a.out != nullptr)
-          IO::store1(static_cast<elem*>(a.out) + row * D + o,
-                     lds[L::XQ + t * LD + o] + (sgam[o] * xh[j] + sbet[o]));
-        lds[L::Z2 + t * LD + o] *= last;
+        for (int j = 0; j < NJD; ++j) {
+          const int o = cg + GW * j;
+          if (t < K)
+            IO::store1(static_cast<elem*>(a.out) + row * D + o,
+                       lds[L::XQ + t * LD + o] + (sgam[o] * xh[j] + sbet[o]));
+        }
       }
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) lds[L::Z2 + t * LD + cg + GW * j] *= last;
 #pragma unroll
       for (int j = 0; j < NJM; ++j) lds[L::BA + t * LM + cg + GW * j] *= last;
       if (a.G1_save != nullptr) {
