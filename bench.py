@@ -226,7 +226,7 @@ def main():
         out["config"]["inner_model"] = "TTT-Linear"
         out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                           "kernel": "ttt_linear_fwd_kernel", "kernel_avg_us": dev_s * 1e6,
+                           "kernel": "ttt_linear_fwd_sk_kernel", "kernel_avg_us": dev_s * 1e6,
                            "algorithmic_bytes": alg}
     elif kind in ("inner_inputs", "layer_epilogue"):
         # inner_inputs: xq, xk, xv read and written once, logits in, lr out; epilogue: inner_out and gate in, out written
