@@ -234,12 +234,23 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
 // instructions of the current one (two register sets in ping-pong).  Every load is unconditional: past a
 // wave's last job the last job is re-read (and dropped), because a load under a branch makes the waits that
 // follow count as if it had not been issued.
-template <int MODE, int NW, int NB, int KS>
+//
+// FZ (needs one column block per wave, Nt / NB == NW): the product Z[16 x 16*Nt] = X[16 x 16*Mt] * C_new rides
+// along.  A wave meets every tile row of its column block, and an updated tile, still in accumulator layout (lane
+// (c, g), register r = C(16 tm + 4g + r, c)), is the B operand of a matrix instruction whose k slots are assigned
+// as k = 4g + r; with X (LDS, contiguous along k, row stride x_rs) read 16 bytes per lane as the matching A operand,
+// four more instructions per tile give the wave its complete columns of Z: the separate pass over C that the
+// product would need is saved.  Z (row stride ldz) is written once at the end.
+template <int MODE, int NW, int NB, int KS, bool FZ = false>
 __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
-                                        int b_rs, int b_cs, int Mt, int Nt, int wave, int lane) {
+                                        int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
+                                        const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
   static_assert(MODE == 1 || MODE == 2, "read-modify-write modes only");
   const int c = lane & 15, g = lane >> 4;
   const int nblk = Nt / NB, njobs = Mt * nblk;
+  f32x4 zacc[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) zacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   // When the number of column blocks divides the number of waves, all jobs of a wave lie in one column block
   // and share their B operand: it is loaded once and kept in registers.
   const bool bfix = NW % nblk == 0;
@@ -288,6 +299,13 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
     for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) C[coff + r * ldc + 16 * j] = s.acc[j][r];
+    if (FZ) {
+      const f32x4 xv = *reinterpret_cast<const f32x4*>(X + c * x_rs + 16 * tm + 4 * g);
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) zacc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[r], s.acc[j][r], zacc[j], 0, 0, 0);
+    }
   };
   int job = wave;
   if (job >= njobs) return;
@@ -306,6 +324,13 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
     finish(j1, s1);
     if (j2 > last) break;
     job = j2;
+  }
+  if (FZ) {
+    const int zoff = 4 * g * ldz + 16 * (wave % nblk) * NB + c;
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) Z[zoff + r * ldz + 16 * j] = zacc[j][r];
   }
 }
 

@@ -222,12 +222,11 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < NJD; ++j) lds[L::TG + t * LD + cg + GW * j] -= lds[L::XK + t * LD + cg + GW * j];
     const float last = te_last * slr[t];
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
-    mm_rank<1, NW, NBM, 4>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane);
+    // Z1 = XK W1 (step 3) rides along on the rolled-back tiles
+    mm_rank<1, NW, NBM, 4, true>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M);
     if (tid < M) sb1[tid] += col16_sum(G1l + tid, M);
     __syncthreads();
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
-    mm_lds<0, NW, NBM>(mZ1, M, lds + L::XK, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
-    __syncthreads();
     {
       float z[NJM], y[NJM];
       ldm(mZ1, z);
