@@ -514,6 +514,15 @@ def inner_loop_inputs(xq, xk, xv, lr_logits, lr_bias, base_lr, token_idx, learna
     return q, k, v, lr, te
 
 
+def lr_logit_grad(d_lr, lr_logits, base_lr, head_dim, dtype=np.float64):
+    """Gradient w.r.t. the lr-gate logits from the gradient w.r.t. ttt_lr_eta: the chain through
+    ttt_lr_eta = base_lr * sigmoid(logit) / head_dim (get_lr, ttt.rs:205-227).  d_lr and lr_logits have the same
+    shape ([B,H,seq]); the gate's bias is part of the logit."""
+    g, z = np.asarray(d_lr, dtype), np.asarray(lr_logits, dtype)
+    s = 1.0 / (1.0 + np.exp(-z))
+    return g * (base_lr / head_dim) * s * (1.0 - s)
+
+
 def layer_epilogue(inner_out, post_gamma, post_beta, gate=None, eps=1e-6):
     """TTT::forward after the inner model (ttt.rs:285-297): [B,H,seq,d] -> [B,seq,H*d], post_norm
     LayerNorm over the hidden axis (eps 1e-6), times gelu_tanh(gate) when the gate projection exists.

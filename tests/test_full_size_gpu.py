@@ -27,7 +27,7 @@ def dev(c):
     return {k: v.to("cuda:0") for k, v in c.items()}
 
 
-def sub(c, bs, hs, keys_bh=("xq", "xk", "xv", "lr", "d_out")):
+def sub(c, bs, hs, keys_bh=("xq", "xk", "xv", "lr", "d_out", "lr_logits")):
     """Slice of the inputs: batch entries bs, heads hs (numpy float64)."""
     o = {}
     for k, v in c.items():

@@ -213,3 +213,19 @@ def test_packed_checkpoints_rejected_where_unsupported(P):
     with pytest.raises(Exception, match="packed checkpoints"):
         P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
                                  dv["gamma"], dv["beta"], 16, 1e-6, 2, want_checkpoints=True, packed_checkpoints=True)
+
+
+def test_bwd_gives_eta_logit_gradients_as_the_fwd_bwd_configuration_asks(P):
+    """Benchmark-style inputs (lr = base_lr * sigmoid(logits) / d): the gradient w.r.t. the logits, i.e.
+    grad_ttt_lr_eta chained through the gate (rust/layer/src/ttt.rs:205-227), against the oracle's chain, which
+    tests/test_oracle_pins.py pins by finite differences through the forward."""
+    B, H, d, K, N = 2, 3, 64, 16, 4
+    print(f"case bwd eta logits B{B} H{H} d{d} K{K} N{N}", flush=True)
+    c = P.synthetic.baseline_inputs(2, B, H, N * K, d, K, io_dtype=torch.float32, with_dout=True)
+    logits = c.pop("lr_logits")
+    dO = c.pop("d_out")
+    g = run_bwd(P, c, dO, K, 1)
+    got = P.ttt_lr_eta_logit_grad(g["grad_ttt_lr_eta"], logits.to("cuda:0"), 1.0, d)
+    r = oracle_bwd(c, dO, K)
+    ref = orc.lr_logit_grad(r["d_lr"], logits.double().numpy(), 1.0, d)
+    assert_close(got, ref, 1e-4, "grad_lr_logits")

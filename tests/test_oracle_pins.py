@@ -414,3 +414,27 @@ def test_inner_loop_inputs_and_epilogue_pieces():
     np.testing.assert_allclose(orc.layer_epilogue(inner, g, b), ref.numpy(), rtol=1e-10, atol=1e-12)
     ref = F.gelu(torch.tensor(gate), approximate="tanh") * ref
     np.testing.assert_allclose(orc.layer_epilogue(inner, g, b, gate), ref.numpy(), rtol=1e-10, atol=1e-12)
+
+
+def test_lr_logit_grad_is_the_derivative_through_the_gate():
+    """d loss / d logit of the lr gate (ttt.rs:205-227) by central differences through the oracle forward, against
+    the oracle backward's d_lr chained through lr_logit_grad: pins the chain that BASELINE's forward+backward
+    configuration asks for (gradients w.r.t. the eta logits)."""
+    rng = np.random.default_rng(11)
+    B, H, seq, d, K, base = 1, 2, 8, 8, 4, 1.0
+    r = lambda *s, sc=1.0: rng.standard_normal(s) * sc
+    xq, xk, xv, dO = r(B, H, seq, d), r(B, H, seq, d), r(B, H, seq, d), r(B, H, seq, d)
+    W0, b0, gam, bet = r(H, d, d, sc=0.1), r(H, d, sc=0.1), 1 + r(H, d, sc=0.1), r(H, d, sc=0.1)
+    te = 1.0 / np.arange(1, K + 1)
+    z = r(B, H, seq)
+    lr_of = lambda zz: base / d / (1.0 + np.exp(-zz))
+    loss = lambda zz: (orc.linear_forward(W0, b0, xq, xk, xv, te, lr_of(zz), gam, bet, K=K)[0] * dO).sum()
+    g = orc.linear_backward(W0, b0, xq, xk, xv, te, lr_of(z), gam, bet, dO, K=K)
+    dz = orc.lr_logit_grad(g["d_lr"], z, base, d)
+    h = 1e-5
+    for idx in [(0, 0, 0), (0, 1, 3), (0, 0, 5), (0, 1, 7)]:
+        zp, zm = z.copy(), z.copy()
+        zp[idx] += h
+        zm[idx] -= h
+        fd = (loss(zp) - loss(zm)) / (2 * h)
+        assert abs(fd - dz[idx]) <= 1e-6 * max(1.0, abs(fd)), (idx, fd, dz[idx])

@@ -496,6 +496,15 @@ def rope_cos_sin(seq_len: int, offset: int, wrap: Optional[int], head_dim: int, 
     return freqs.cos().to(device), freqs.sin().to(device)
 
 
+def ttt_lr_eta_logit_grad(grad_ttt_lr_eta, lr_logits, base_lr: float, head_dim: int):
+    """Gradient w.r.t. the lr-gate logits from grad_ttt_lr_eta (an output of ttt_linear_backward_raw /
+    ttt_mlp_backward_raw): the chain through ttt_lr_eta = base_lr * sigmoid(logit) / head_dim (get_lr,
+    rust/layer/src/ttt.rs:205-227).  The reference leaves this step to Burn autodiff outside the fused kernel's
+    boundary; here it is one elementwise expression on the caller's device, in f32."""
+    s = torch.sigmoid(lr_logits.float())
+    return grad_ttt_lr_eta.float() * (base_lr / head_dim) * s * (1.0 - s)
+
+
 def inner_loop_inputs_raw(xq, xk, xv, lr_logits, lr_bias, base_lr: float, token_idx, learnable_token_idx,
                           mini_batch: int, rope=None, pos_offset: int = 0, pos_wrap: int = 0) -> TTTInputsInner:
     """One call of ttt_inner_inputs: TTT::get_inner_loop_inputs after the projections

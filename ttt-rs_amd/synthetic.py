@@ -32,7 +32,8 @@ def baseline_inputs(config_idx: int, B: int, H: int, seq: int, d: int, K: int = 
         c["W0"] = n(H, d, d) * 0.02
         c["b0"] = torch.zeros(H, d, dtype=torch.float32)
     c["gamma"], c["beta"] = torch.ones(H, d, dtype=torch.float32), torch.zeros(H, d, dtype=torch.float32)
-    c["lr"] = (base_lr / d) * torch.sigmoid(n(B, H, seq))
+    c["lr_logits"] = n(B, H, seq)  # kept for the chain d lr -> d logits (f32; not an input of the inner loop)
+    c["lr"] = (base_lr / d) * torch.sigmoid(c["lr_logits"])
     c["token_eta"] = 1.0 / torch.arange(1, K + 1, dtype=torch.float32)
     if with_dout:
         c["d_out"] = n(B, H, seq, d)
