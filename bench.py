@@ -274,9 +274,10 @@ def main():
                            "kernel": "ttt_mlp_fwd_rr_kernel" if rr else "ttt_mlp_fwd_kernel",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     elif kind == "mlp_fwd_bwd":
-        # forward (56 d^2 + 20 K d) plus the backward's own forward sweep and its 14 state-sized and
-        # 7 rank-16 products: (56 + 56 + 14*8 + 7*8) d^2 flop per token-head, K-sized terms aside
-        flops = th * (280 * d * d)
+        # forward (56 d^2 + 20 K d) plus the backward's own forward sweep (Z1, Z2, G1 and the two state updates:
+        # 40 d^2; its output branch is not run) and the reverse scan's 14 state-sized and 7 rank-16 products:
+        # (56 + 40 + 14*8 + 7*8) d^2 flop per token-head, K-sized terms aside
+        flops = th * (264 * d * d)
         out["dtype"] = "f32"
         out["config"]["inner_model"] = "TTT-MLP"
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
