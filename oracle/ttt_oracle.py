@@ -33,6 +33,13 @@ How each function is pinned (tests/test_oracle_*.py):
                        formulation, plus central finite differences of
                        linear_forward
   mlp_mini_batch    == primal per-token GD on both layers, written in the test
+  mlp_backward      == torch autograd (float64, double backward) through a torch restatement of the dual
+                       form whose forward is checked against mlp_forward, plus linearity
+  lr_logit_grad     == central finite differences of linear_forward through the gate
+  rope_apply        == complex rotation of adjacent pairs; inner_loop_inputs, layer_epilogue == their pieces
+                       (torch sigmoid / layer_norm / gelu) assembled independently in the test
+Frozen results of these functions for five small cases are kept in tests/golden (written by
+tests/golden/make_fixtures.py); tests/test_golden_cpu.py holds this module to them.
 The reference commits no golden vectors for this path (its fixtures are generated
 at test time), so absolute agreement with Burn-CPU's floating-point results is
 "parity unpinned"; agreement is to tolerance against this float64 restatement.
