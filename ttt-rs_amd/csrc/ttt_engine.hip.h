@@ -16,7 +16,8 @@ namespace ttt {
 // wave (16 lanes with the same g) touches 16 cache lines and the load runs at 16 B per cycle and CU; here lane l
 // loads row l / 4, chunk l % 4, so a quarter wave touches 4 lines (the rate of a coalesced load), and the values
 // change lanes afterwards (ds_bpermute: lane 16 g + c takes from lane 4 c + g).  `load_rows_raw` issues the load,
-// `rows_to_operand` does the exchange, so that the exchange can sit where the value is used.
+// `rows_to_operand` does the exchange, so that the exchange can sit where the value is used.  All 64 lanes of the
+// wave must be active in both.
 __device__ __forceinline__ f32x4 load_rows_raw(const float* block, int row_stride, int lane) {
   return *reinterpret_cast<const f32x4*>(block + (lane >> 2) * row_stride + 4 * (lane & 3));
 }
