@@ -67,3 +67,15 @@ def test_null_pointers_are_rejected_before_any_launch(P):
     L = P.lib()
     rc = L.ttt_linear_fwd(C.byref(desc(P)), *([None] * 15))
     assert rc == P.TTT_ERR_NULL
+
+
+def test_eta_logit_gradient_helper_matches_the_oracle_chain(P):
+    """Host logic, no GPU: the chain from grad_ttt_lr_eta to the lr-gate logits (rust/layer/src/ttt.rs:205-227)."""
+    import numpy as np
+    import torch
+    from oracle import ttt_oracle as orc
+    g = torch.Generator().manual_seed(3)
+    d_lr, z = torch.randn(2, 3, 32, generator=g), torch.randn(2, 3, 32, generator=g)
+    got = P.ttt_lr_eta_logit_grad(d_lr, z, 1.5, 64).double().numpy()
+    ref = orc.lr_logit_grad(d_lr.double().numpy(), z.double().numpy(), 1.5, 64)
+    assert np.abs(got - ref).max() <= 1e-6 * np.abs(ref).max()
