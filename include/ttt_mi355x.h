@@ -174,6 +174,26 @@ int ttt_mlp_bwd(const ttt_desc* desc, const void* xq, const void* xk, const void
                 float* d_gamma, float* d_beta, void* workspace, void* stream);
 
 /*
+ * ttt_mlp_bwd without a workspace argument and without any allocation.  No counterpart in the
+ * reference; it is for callers that cannot allocate device memory around the call (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same arguments, results
+ * and kernels as ttt_mlp_bwd; the workspace is a buffer of TTT_MLP_BWD_STATIC_MAX_BYTES that is part of
+ * the library's device image (each GPU the library runs on holds it until the process ends).
+ * A desc with ttt_mlp_bwd_workspace_bytes(desc) > TTT_MLP_BWD_STATIC_MAX_BYTES is refused with
+ * TTT_ERR_SHAPE (use ttt_mlp_bwd then).  All calls on one GPU share that buffer: calls that overlap on
+ * one GPU (different streams or threads) race; calls on one stream, or otherwise ordered, are safe.
+ * Nothing in the buffer has to survive between calls.
+ */
+#define TTT_MLP_BWD_STATIC_MAX_BYTES (32u << 20)
+int ttt_mlp_bwd_static(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                       const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                       const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                       const void* d_out, const float* d_W1_out, const float* d_b1_out,
+                       const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
+                       float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr,
+                       float* d_token_eta, float* d_gamma, float* d_beta, void* stream);
+
+/*
  * The elementwise work either side of the inner loop, one HBM-bound pass each (the GEMMs of the
  * projections stay with the BLAS the caller uses).  desc supplies batch, heads, seq, head_dim,
  * mini_batch and io_dtype; the other fields are ignored.

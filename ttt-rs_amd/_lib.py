@@ -14,7 +14,7 @@ TTT_F32, TTT_BF16 = 0, 1
 EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
-    "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_inner_inputs", "ttt_layer_epilogue",
+    "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_inner_inputs", "ttt_layer_epilogue",
 )
 
 
@@ -60,6 +60,7 @@ def lib() -> C.CDLL:
         L.ttt_mlp_bwd_workspace_bytes.argtypes = [dp]
         L.ttt_mlp_bwd_workspace_bytes.restype = C.c_int64
         L.ttt_mlp_bwd.argtypes = [dp] + [vp] * 29
+        L.ttt_mlp_bwd_static.argtypes = [dp] + [vp] * 28
         L.ttt_inner_inputs.argtypes = [dp] + [vp] * 5 + [C.c_float] + [vp] * 4 + [C.c_int, C.c_int] + [vp] * 6
         L.ttt_layer_epilogue.argtypes = [dp] + [vp] * 3 + [C.c_float] + [vp] * 3
         _lib = L

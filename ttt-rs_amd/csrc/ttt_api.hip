@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 
 #include "ttt_engine_fwd.hip.h"
 #include "ttt_layer_io.hip.h"
@@ -20,6 +21,9 @@
 #include "ttt_mlp_bwd.hip.h"
 #include "ttt_mlp_fwd_cl2.hip.h"
 #include "ttt_mlp_fwd_rr.hip.h"
+
+// Scratch of ttt_mlp_bwd_static (file scope, outside any namespace so that HIP_SYMBOL names it plainly).
+static __device__ __align__(256) unsigned char ttt_mlp_bwd_scratch_mem[TTT_MLP_BWD_STATIC_MAX_BYTES];
 
 namespace {
 
@@ -251,6 +255,103 @@ void launch_epilogue(const ttt::LayerEpilogueArgs& a, int nc, dim3 grid, hipStre
     case 1: hipLaunchKernelGGL((ttt::ttt_layer_epilogue_kernel<T, 1>), grid, dim3(256), 0, s, a); break;
     case 2: hipLaunchKernelGGL((ttt::ttt_layer_epilogue_kernel<T, 2>), grid, dim3(256), 0, s, a); break;
     default: hipLaunchKernelGGL((ttt::ttt_layer_epilogue_kernel<T, 4>), grid, dim3(256), 0, s, a); break;
+  }
+}
+
+
+// ---- built-in scratch of ttt_mlp_bwd_static ------------------------------------------------------
+// Device memory that belongs to the library's code object: every GPU the library runs on holds its own
+// copy at its own address until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels and fills get the looked-up device address.
+constexpr size_t kMlpBwdScratchBytes = TTT_MLP_BWD_STATIC_MAX_BYTES;
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_mlp_bwd_scratch[kMaxDevices];
+
+int mlp_bwd_scratch(void** out) {
+  int dev = -1;
+  int rc = hip_status(hipGetDevice(&dev), "hipGetDevice");
+  if (rc != TTT_OK) return rc;
+  if (dev < 0 || dev >= kMaxDevices) return fail(TTT_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  void* p = g_mlp_bwd_scratch[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    // first call on this device (it is the current one): every thread that gets here looks up the same address
+    rc = hip_status(hipGetSymbolAddress(&p, HIP_SYMBOL(ttt_mlp_bwd_scratch_mem)), "hipGetSymbolAddress(scratch)");
+    if (rc != TTT_OK) return rc;
+    if (p == nullptr) return fail(TTT_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+    g_mlp_bwd_scratch[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return TTT_OK;
+}
+
+int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                const void* d_out, const float* d_W1_out, const float* d_b1_out,
+                const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
+                float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
+                float* d_gamma, float* d_beta, void* workspace, void* stream) {
+  int rc = ttt_mlp_supported(d);
+  if (rc != TTT_OK) return rc;
+  if (!xq || !xk || !xv || !W1_0 || !b1_0 || !W2_0 || !b2_0 || !token_eta || !lr || !gamma || !beta ||
+      !d_out || !d_xq || !d_xk || !d_xv || !d_W1 || !d_b1 || !d_W2 || !d_b2 || !d_lr || !d_token_eta ||
+      !d_gamma || !d_beta || !workspace)
+    return fail(TTT_ERR_NULL, "ttt_mlp_bwd: a required pointer is NULL");
+  const bool up = d_W1_out || d_b1_out || d_W2_out || d_b2_out;
+  if (up && !(d_W1_out && d_b1_out && d_W2_out && d_b2_out))
+    return fail(TTT_ERR_NULL, "ttt_mlp_bwd: the four upstream state gradients must all be given or all be NULL");
+  if (!aligned16(workspace)) return fail(TTT_ERR_SHAPE, "ttt_mlp_bwd: workspace must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const MlpBwdWs w(d);
+  float* ws = static_cast<float*>(workspace);
+  const bool f32 = d->io_dtype == TTT_F32;
+  const size_t U = (size_t)d->batch * d->heads, D = d->head_dim, M = 4 * D;
+
+  // forward sweep with the LDS-tile kernel (f32 products): final state and, per mini-batch, the
+  // rank-16 factors of the state update
+  ttt::MlpFwdArgs fa;
+  fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
+  fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
+  fa.W1 = ws + w.W1; fa.b1 = ws + w.b1; fa.W2 = ws + w.W2; fa.b2 = ws + w.b2;
+  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s;
+  fa.B = d->batch; fa.H = d->heads; fa.seq = d->seq; fa.K = d->mini_batch;
+  fa.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
+  fa.n_stages = d->seq / d->mini_batch;
+  fa.state_per_batch = d->state_per_batch ? 1 : 0;
+  fa.eps = d->eps;
+  switch (d->head_dim) {
+    case 32: rc = f32 ? launch_mlp_fwd<ttt::F32, 32>(fa, s) : launch_mlp_fwd<ttt::BF16, 32>(fa, s); break;
+    case 64: rc = f32 ? launch_mlp_fwd<ttt::F32, 64>(fa, s) : launch_mlp_fwd<ttt::BF16, 64>(fa, s); break;
+    case 96: rc = f32 ? launch_mlp_fwd<ttt::F32, 96>(fa, s) : launch_mlp_fwd<ttt::BF16, 96>(fa, s); break;
+    default: rc = f32 ? launch_mlp_fwd<ttt::F32, 128>(fa, s) : launch_mlp_fwd<ttt::BF16, 128>(fa, s); break;
+  }
+  if (rc != TTT_OK) return rc;
+
+  // gradient accumulators start from the upstream state gradients (or zero); the reductions over
+  // batch / heads start from zero
+  copy_or_zero(d_W1, d_W1_out, U * D * M, s);
+  copy_or_zero(d_b1, d_b1_out, U * M, s);
+  copy_or_zero(d_W2, d_W2_out, U * M * D, s);
+  copy_or_zero(d_b2, d_b2_out, U * D, s);
+  copy_or_zero(d_token_eta, nullptr, (size_t)d->seq, s);
+  copy_or_zero(d_gamma, nullptr, (size_t)d->heads * D, s);
+  copy_or_zero(d_beta, nullptr, (size_t)d->heads * D, s);
+  rc = hip_status(hipGetLastError(), "ttt_mlp_bwd fills");
+  if (rc != TTT_OK) return rc;
+
+  ttt::MlpBwdArgs a;
+  a.xq = xq; a.xk = xk; a.xv = xv; a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta;
+  a.d_out = d_out; a.G1s = ws + w.G1s; a.G2s = ws + w.G2s; a.W1 = ws + w.W1; a.W2 = ws + w.W2;
+  a.b1f = ws + w.b1; a.b2f = ws + w.b2; a.mt = ws + w.mt;
+  a.d_xq = d_xq; a.d_xk = d_xk; a.d_xv = d_xv; a.d_W1 = d_W1; a.d_b1 = d_b1; a.d_W2 = d_W2; a.d_b2 = d_b2;
+  a.d_lr = d_lr; a.d_token_eta = d_token_eta; a.d_gamma = d_gamma; a.d_beta = d_beta;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
+  a.seq_stride = fa.seq_stride; a.n_stages = fa.n_stages; a.eps = d->eps;
+  switch (d->head_dim) {
+    case 32: return f32 ? launch_mlp_bwd<ttt::F32, 32>(a, s) : launch_mlp_bwd<ttt::BF16, 32>(a, s);
+    case 64: return f32 ? launch_mlp_bwd<ttt::F32, 64>(a, s) : launch_mlp_bwd<ttt::BF16, 64>(a, s);
+    case 96: return f32 ? launch_mlp_bwd<ttt::F32, 96>(a, s) : launch_mlp_bwd<ttt::BF16, 96>(a, s);
+    default: return f32 ? launch_mlp_bwd<ttt::F32, 128>(a, s) : launch_mlp_bwd<ttt::BF16, 128>(a, s);
   }
 }
 
@@ -493,68 +594,32 @@ int ttt_mlp_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
                 const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
                 float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
                 float* d_gamma, float* d_beta, void* workspace, void* stream) {
+  return mlp_bwd_impl(d, xq, xk, xv, W1_0, b1_0, W2_0, b2_0, token_eta, lr, gamma, beta, d_out, d_W1_out,
+                      d_b1_out, d_W2_out, d_b2_out, d_xq, d_xk, d_xv, d_W1, d_b1, d_W2, d_b2, d_lr,
+                      d_token_eta, d_gamma, d_beta, workspace, stream);
+}
+
+int ttt_mlp_bwd_static(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                       const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                       const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                       const void* d_out, const float* d_W1_out, const float* d_b1_out,
+                       const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
+                       float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr,
+                       float* d_token_eta, float* d_gamma, float* d_beta, void* stream) {
   int rc = ttt_mlp_supported(d);
   if (rc != TTT_OK) return rc;
-  if (!xq || !xk || !xv || !W1_0 || !b1_0 || !W2_0 || !b2_0 || !token_eta || !lr || !gamma || !beta ||
-      !d_out || !d_xq || !d_xk || !d_xv || !d_W1 || !d_b1 || !d_W2 || !d_b2 || !d_lr || !d_token_eta ||
-      !d_gamma || !d_beta || !workspace)
-    return fail(TTT_ERR_NULL, "ttt_mlp_bwd: a required pointer is NULL");
-  const bool up = d_W1_out || d_b1_out || d_W2_out || d_b2_out;
-  if (up && !(d_W1_out && d_b1_out && d_W2_out && d_b2_out))
-    return fail(TTT_ERR_NULL, "ttt_mlp_bwd: the four upstream state gradients must all be given or all be NULL");
-  if (!aligned16(workspace)) return fail(TTT_ERR_SHAPE, "ttt_mlp_bwd: workspace must be 16-byte aligned");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const MlpBwdWs w(d);
-  float* ws = static_cast<float*>(workspace);
-  const bool f32 = d->io_dtype == TTT_F32;
-  const size_t U = (size_t)d->batch * d->heads, D = d->head_dim, M = 4 * D;
-
-  // forward sweep with the LDS-tile kernel (f32 products): final state and, per mini-batch, the
-  // rank-16 factors of the state update
-  ttt::MlpFwdArgs fa;
-  fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
-  fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
-  fa.W1 = ws + w.W1; fa.b1 = ws + w.b1; fa.W2 = ws + w.W2; fa.b2 = ws + w.b2;
-  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s;
-  fa.B = d->batch; fa.H = d->heads; fa.seq = d->seq; fa.K = d->mini_batch;
-  fa.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
-  fa.n_stages = d->seq / d->mini_batch;
-  fa.state_per_batch = d->state_per_batch ? 1 : 0;
-  fa.eps = d->eps;
-  switch (d->head_dim) {
-    case 32: rc = f32 ? launch_mlp_fwd<ttt::F32, 32>(fa, s) : launch_mlp_fwd<ttt::BF16, 32>(fa, s); break;
-    case 64: rc = f32 ? launch_mlp_fwd<ttt::F32, 64>(fa, s) : launch_mlp_fwd<ttt::BF16, 64>(fa, s); break;
-    case 96: rc = f32 ? launch_mlp_fwd<ttt::F32, 96>(fa, s) : launch_mlp_fwd<ttt::BF16, 96>(fa, s); break;
-    default: rc = f32 ? launch_mlp_fwd<ttt::F32, 128>(fa, s) : launch_mlp_fwd<ttt::BF16, 128>(fa, s); break;
-  }
+  const int64_t need = ttt_mlp_bwd_workspace_bytes(d);
+  if (need < 0 || (uint64_t)need > kMlpBwdScratchBytes)
+    return fail(TTT_ERR_SHAPE,
+                "ttt_mlp_bwd_static: this shape needs %lld bytes of scratch, the built-in buffer holds %llu; "
+                "use ttt_mlp_bwd with a caller-owned workspace",
+                (long long)need, (unsigned long long)kMlpBwdScratchBytes);
+  void* ws = nullptr;
+  rc = mlp_bwd_scratch(&ws);
   if (rc != TTT_OK) return rc;
-
-  // gradient accumulators start from the upstream state gradients (or zero); the reductions over
-  // batch / heads start from zero
-  copy_or_zero(d_W1, d_W1_out, U * D * M, s);
-  copy_or_zero(d_b1, d_b1_out, U * M, s);
-  copy_or_zero(d_W2, d_W2_out, U * M * D, s);
-  copy_or_zero(d_b2, d_b2_out, U * D, s);
-  copy_or_zero(d_token_eta, nullptr, (size_t)d->seq, s);
-  copy_or_zero(d_gamma, nullptr, (size_t)d->heads * D, s);
-  copy_or_zero(d_beta, nullptr, (size_t)d->heads * D, s);
-  rc = hip_status(hipGetLastError(), "ttt_mlp_bwd fills");
-  if (rc != TTT_OK) return rc;
-
-  ttt::MlpBwdArgs a;
-  a.xq = xq; a.xk = xk; a.xv = xv; a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta;
-  a.d_out = d_out; a.G1s = ws + w.G1s; a.G2s = ws + w.G2s; a.W1 = ws + w.W1; a.W2 = ws + w.W2;
-  a.b1f = ws + w.b1; a.b2f = ws + w.b2; a.mt = ws + w.mt;
-  a.d_xq = d_xq; a.d_xk = d_xk; a.d_xv = d_xv; a.d_W1 = d_W1; a.d_b1 = d_b1; a.d_W2 = d_W2; a.d_b2 = d_b2;
-  a.d_lr = d_lr; a.d_token_eta = d_token_eta; a.d_gamma = d_gamma; a.d_beta = d_beta;
-  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
-  a.seq_stride = fa.seq_stride; a.n_stages = fa.n_stages; a.eps = d->eps;
-  switch (d->head_dim) {
-    case 32: return f32 ? launch_mlp_bwd<ttt::F32, 32>(a, s) : launch_mlp_bwd<ttt::BF16, 32>(a, s);
-    case 64: return f32 ? launch_mlp_bwd<ttt::F32, 64>(a, s) : launch_mlp_bwd<ttt::BF16, 64>(a, s);
-    case 96: return f32 ? launch_mlp_bwd<ttt::F32, 96>(a, s) : launch_mlp_bwd<ttt::BF16, 96>(a, s);
-    default: return f32 ? launch_mlp_bwd<ttt::F32, 128>(a, s) : launch_mlp_bwd<ttt::BF16, 128>(a, s);
-  }
+  return mlp_bwd_impl(d, xq, xk, xv, W1_0, b1_0, W2_0, b2_0, token_eta, lr, gamma, beta, d_out, d_W1_out,
+                      d_b1_out, d_W2_out, d_b2_out, d_xq, d_xk, d_xv, d_W1, d_b1, d_W2, d_b2, d_lr,
+                      d_token_eta, d_gamma, d_beta, ws, stream);
 }
 
 int ttt_inner_inputs(const ttt_desc* d, const void* xq, const void* xk, const void* xv,

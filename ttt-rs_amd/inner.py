@@ -275,13 +275,17 @@ def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_we
 
 
 def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias, d_out,
-                         mini_batch: int, eps: float = 1e-6, d_state_out=None):
+                         mini_batch: int, eps: float = 1e-6, d_state_out=None, static_scratch: bool = False,
+                         into=None):
     """One call of ttt_mlp_bwd on the current stream: gradients of the TTT-MLP inner loop
     (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50; the reference gets them
     from Burn autodiff).  Arguments as ttt_mlp_forward_raw plus d_out [B,H,seq,d] and the optional
     upstream gradients of the final state d_state_out = (dW1, db1, dW2, db2), per batch element.
     Returns a dict: d_xq, d_xk, d_xv, d_W1 [B,H,d,4d], d_b1, d_W2, d_b2 (per batch element), d_lr,
-    d_token_eta [seq], d_gamma, d_beta [H,d]."""
+    d_token_eta [seq], d_gamma, d_beta [H,d].
+    static_scratch: call ttt_mlp_bwd_static (the library's built-in scratch buffer instead of a workspace
+    allocated here); `into`: a dict returned by an earlier call of the same shape, whose tensors receive the
+    gradients (with both, the call allocates no device memory)."""
     B, H, seq, d = xq.shape
     m = w1.shape[-1]
     io = xq.dtype
@@ -311,23 +315,34 @@ def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_w
     up = [None] * 4
     if d_state_out is not None:
         up = [_need(g, sh, torch.float32, "d_state_out") for g, sh in zip(d_state_out, shapes)]
-    g_act = [torch.empty_like(xq) for _ in range(3)]
-    g_st = [torch.empty(sh, **f32) for sh in shapes]
-    g_lr = torch.empty_like(lr)
-    g_te = torch.empty(seq, **f32)
-    g_gam, g_bet = torch.empty((H, d), **f32), torch.empty((H, d), **f32)
-    nbytes = lib().ttt_mlp_bwd_workspace_bytes(C.byref(desc))
-    if nbytes < 0:
-        raise _lib.TttError(_lib.TTT_ERR_SHAPE, "ttt_mlp_bwd_workspace_bytes failed")
-    ws = torch.empty((nbytes + 3) // 4, **f32)
+    if into is not None:
+        g_act = [into["d_xq"], into["d_xk"], into["d_xv"]]
+        g_st = [into["d_W1"], into["d_b1"], into["d_W2"], into["d_b2"]]
+        g_lr, g_te, g_gam, g_bet = into["d_lr"], into["d_token_eta"], into["d_gamma"], into["d_beta"]
+        for t, sh in zip(g_act + g_st + [g_lr, g_te, g_gam, g_bet],
+                         [xq.shape] * 3 + shapes + [lr.shape, (seq,), (H, d), (H, d)]):
+            if tuple(t.shape) != tuple(sh) or not t.is_contiguous() or not t.is_cuda:
+                raise _lib.TttError(_lib.TTT_ERR_SHAPE, "into: a gradient tensor has the wrong shape or layout")
+    else:
+        g_act = [torch.empty_like(xq) for _ in range(3)]
+        g_st = [torch.empty(sh, **f32) for sh in shapes]
+        g_lr = torch.empty_like(lr)
+        g_te = torch.empty(seq, **f32)
+        g_gam, g_bet = torch.empty((H, d), **f32), torch.empty((H, d), **f32)
     stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     null = C.c_void_p(None)
+    args = [C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(w1), _ptr(b1), _ptr(w2), _ptr(b2), _ptr(te), _ptr(lr),
+            _ptr(ln_weight), _ptr(ln_bias), _ptr(d_out), *[null if g is None else _ptr(g) for g in up],
+            *[_ptr(g) for g in g_act], *[_ptr(g) for g in g_st], _ptr(g_lr), _ptr(g_te), _ptr(g_gam), _ptr(g_bet)]
     with torch.cuda.device(dev):
-        check(lib().ttt_mlp_bwd(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(w1), _ptr(b1), _ptr(w2),
-                                _ptr(b2), _ptr(te), _ptr(lr), _ptr(ln_weight), _ptr(ln_bias), _ptr(d_out),
-                                *[null if g is None else _ptr(g) for g in up],
-                                *[_ptr(g) for g in g_act], *[_ptr(g) for g in g_st], _ptr(g_lr), _ptr(g_te),
-                                _ptr(g_gam), _ptr(g_bet), _ptr(ws), stream))
+        if static_scratch:
+            check(lib().ttt_mlp_bwd_static(*args, stream))
+        else:
+            nbytes = lib().ttt_mlp_bwd_workspace_bytes(C.byref(desc))
+            if nbytes < 0:
+                raise _lib.TttError(_lib.TTT_ERR_SHAPE, "ttt_mlp_bwd_workspace_bytes failed")
+            ws = torch.empty((nbytes + 3) // 4, **f32)
+            check(lib().ttt_mlp_bwd(*args, _ptr(ws), stream))
     return dict(d_xq=g_act[0], d_xk=g_act[1], d_xv=g_act[2], d_W1=g_st[0], d_b1=g_st[1], d_W2=g_st[2],
                 d_b2=g_st[3], d_lr=g_lr, d_token_eta=g_te, d_gamma=g_gam, d_beta=g_bet)
 
