@@ -66,9 +66,26 @@ typedef struct ttt_desc {
                                   change; half the checkpoint traffic.  f32 I/O: f32.  Either way stored
                                   and fetched in whole 1 KiB rows instead of scattered 4-byte pieces.
                                   No counterpart in the reference. */
+  int32_t kernel_hint;         /* 0 (TTT_HINT_AUTO): the library chooses the kernel from the shape.  Otherwise a
+                                  tuning / testing request, read by the entry point the desc is passed to:
+                                  low byte = wavefronts per (batch, head) unit for the TTT-Linear kernels
+                                  (1, 2 or 4; clamped to what head_dim allows), TTT_HINT_LDS_TILES = the kernels
+                                  that keep state and tiles in LDS / global memory and compute every product in
+                                  f32 (TTT-Linear forward at head_dim 96/128, TTT-Linear backward at head_dim
+                                  <= 64, TTT-MLP forward).  A hint that names no existing kernel for the desc is
+                                  ignored.  The choice changes speed and, between bf16-operand and f32-operand
+                                  kernels, rounding; never the meaning of a result.  No counterpart in the
+                                  reference (its `threads` field, rust/fused/src/lib.rs:285-328, is the nearest). */
 } ttt_desc;
 #define TTT_CKPT_F32 0
 #define TTT_CKPT_PACKED 1
+#define TTT_HINT_AUTO 0
+#define TTT_HINT_WAVES_MASK 0xff
+#define TTT_HINT_LDS_TILES 0x100
+/* Testing only: the two workgroups that share a (batch, head) unit in ttt_mlp_fwd at head_dim 128 (bf16 I/O) give
+ * up waiting for each other at once, as if the partner had never become resident.  Exercises the failure path
+ * described at ttt_mlp_fwd: every output of the affected units is NaN.  All kernels still run to their end. */
+#define TTT_HINT_TEST_LOST_PARTNER 0x200
 
 /* Library / build identification. */
 const char* ttt_version(void);
@@ -80,6 +97,11 @@ int ttt_linear_supported(const ttt_desc* desc);
 /* Number of checkpoints per (batch, head): ceil((seq/mini_batch)/checkpoint_interval)
  * (rust/fused/src/linear_fused_tile/forward/launch.rs:221-226). */
 int64_t ttt_linear_num_checkpoints(const ttt_desc* desc);
+/* TTT_OK if ttt_linear_bwd has a kernel for this desc (it supports fewer combinations than the forward:
+ * checkpoint_interval > 1 only for head_dim <= 64, head_dim 128 only with bf16 I/O), else the status
+ * ttt_linear_bwd would return.  A training caller asks this before the forward, as the reference asks
+ * FusedTttConfig::is_supported (rust/fused/src/lib.rs:313-322) before it builds the layer. */
+int ttt_linear_bwd_supported(const ttt_desc* desc);
 
 /*
  * TTT-Linear multi-stage forward.  Replaces
@@ -133,6 +155,17 @@ int ttt_linear_bwd(const ttt_desc* desc, const void* xq, const void* xk, const v
  * (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50) behind the same
  * bundle convention.  W1_0 [H,d,4d] or [B,H,d,4d], b1_0 [H,4d] or [B,H,4d], W2_0 [H,4d,d] or
  * [B,H,4d,d], b2_0 [H,d] or [B,H,d] (state_per_batch selects); outputs are per batch element.
+ *
+ * head_dim 128 with bf16 I/O: a unit's state (512 KiB) is the whole register file of a CU, so a PAIR of
+ * workgroups on two CUs shares each unit and exchanges partial results once per mini-batch through global
+ * memory.  During the call W2_out is also that exchange area (the library zero-fills it first; its contents are
+ * meaningless until the call's work has finished).  The library launches at most as many workgroups at a time as
+ * the device has CUs, so on a GPU that is not shared both halves of every pair are resident together.  If a
+ * workgroup nevertheless waits for its partner in vain (about 0.1 s: CUs held by other processes or streams), the
+ * call cannot report it -- it returned TTT_OK when the work was enqueued -- so the failure is made impossible to
+ * miss in the data instead: EVERY output of that unit (its rows of out, W1_out, b1_out, W2_out, b2_out) is NaN.
+ * A caller that shares the GPU checks one output element per unit, or passes TTT_HINT_LDS_TILES to use the
+ * single-workgroup kernel (slower, f32 products).
  */
 int ttt_mlp_supported(const ttt_desc* desc);
 int ttt_mlp_fwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,

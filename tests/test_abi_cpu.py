@@ -63,6 +63,35 @@ def test_num_checkpoints(P):
     assert L.ttt_linear_num_checkpoints(C.byref(desc(P, seq=16 * 8, checkpoint_interval=1))) == 8
 
 
+def test_backward_support_query_and_kernel_hints(P):
+    """ttt_linear_bwd_supported answers what ttt_linear_bwd would (fewer combinations than the forward), and
+    desc.kernel_hint is part of the descriptor: the library reads no environment variable."""
+    L = P.lib()
+    ok = lambda **kw: L.ttt_linear_bwd_supported(C.byref(desc(P, **kw)))
+    assert ok() == P.TTT_OK
+    assert ok(head_dim=128, io_dtype=P.TTT_BF16) == P.TTT_OK
+    assert ok(head_dim=128, io_dtype=P.TTT_F32) == P.TTT_ERR_UNSUPPORTED       # forward only
+    assert L.ttt_linear_supported(C.byref(desc(P, head_dim=128))) == P.TTT_OK
+    assert ok(head_dim=96, checkpoint_interval=2) == P.TTT_ERR_UNSUPPORTED
+    assert b"checkpoint_interval 1" in L.ttt_last_error()
+    assert ok(head_dim=64, checkpoint_interval=2) == P.TTT_OK
+    assert ok(checkpoint_format=1, checkpoint_interval=2) == P.TTT_ERR_UNSUPPORTED
+    # packed checkpoints exist for the register-resident kernels only
+    assert ok(checkpoint_format=1, kernel_hint=P.TTT_HINT_LDS_TILES) == P.TTT_ERR_UNSUPPORTED
+    assert ok(kernel_hint=P.TTT_HINT_LDS_TILES) == P.TTT_OK
+    assert ok(kernel_hint=4) == P.TTT_OK and ok(kernel_hint=1, io_dtype=P.TTT_BF16) == P.TTT_OK
+    # a hint that names no kernel for the desc is ignored (no LDS-tile backward at head_dim 96)
+    assert ok(head_dim=96, kernel_hint=P.TTT_HINT_LDS_TILES) == P.TTT_OK
+    assert ok(seq=33) == P.TTT_ERR_SHAPE
+    # the struct the binding declares is the struct the header declares (field order and count)
+    text = open(os.path.join(ROOT, "include", "ttt_mi355x.h")).read()
+    body = re.sub(r"/\*.*?\*/", "", text[text.index("typedef struct ttt_desc {"):text.index("} ttt_desc;")], flags=re.S)
+    fields = re.findall(r"\b(?:int32_t|float)\s+(\w+)\s*;", body)
+    assert fields == [f[0] for f in P.TttDesc._fields_]
+    src = open(os.path.join(ROOT, "ttt-rs_amd", "csrc", "ttt_api.hip")).read()
+    assert "getenv" not in src
+
+
 def test_null_pointers_are_rejected_before_any_launch(P):
     L = P.lib()
     rc = L.ttt_linear_fwd(C.byref(desc(P)), *([None] * 15))

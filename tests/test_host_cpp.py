@@ -26,6 +26,12 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
           if (m.num_checkpoints(2, 64) != 4) return 2;
           ttt::TTTInputsInner in; in.batch = 2; in.seq_len = 33;   // not a multiple of 16, > 16
           ttt::TTTLinearState st; char out[4];
+          // a state without buffers is refused by the class itself
+          in.seq_len = 32;
+          try { m.forward(st, in, out, ttt::Checkpoints{}, nullptr); return 20; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 21; }
+          in.seq_len = 33;
+          st.weight = st.bias = st.next_weight = st.next_bias = dummy;
           try { m.forward_mini_batch(st, in, 0, 33, out, nullptr); return 3; }
           catch (const ttt::Error& e) { if (e.code != TTT_ERR_SHAPE) return 4; }
           in.seq_len = 32;                                          // valid shape, null tensors
@@ -39,6 +45,7 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
           const long long per_unit = 2LL * 96 * 384 + 384 + 96 + 2LL * 16 * (384 + 96) + 9LL * 16 * 384;
           if (mlp.backward_workspace_bytes(2, 32, TTT_BF16) != 4 * 2 * 2 * per_unit) return 8;
           ttt::TTTMLPState ms;
+          ms.w1 = ms.b1 = ms.w2 = ms.b2 = ms.next_w1 = ms.next_b1 = ms.next_w2 = ms.next_b2 = dummy;
           try { mlp.forward_mini_batch(ms, in, 0, 17, out, nullptr); return 9; }
           catch (const ttt::Error& e) { if (e.code != TTT_ERR_SHAPE) return 10; }
           try { mlp.backward(in, ms, out, nullptr, nullptr, nullptr, nullptr, ttt::TTTMLPGrads{}, out, nullptr); return 11; }
@@ -53,3 +60,80 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
     r = subprocess.run([str(exe)], capture_output=True, text=True)
     assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
     assert "NULL" in r.stdout
+
+
+def test_cpp_host_state_buffers_across_a_forward_with_remainder(tmp_path):
+    """The host classes against a stub of the C ABI that records what it is given: a forward with a remainder is
+    two launches; both must read a valid state and write a valid, different buffer (the first from the layer's
+    parameters when the state is not initialised), and the final state must end up where the class says."""
+    src = tmp_path / "s.cpp"
+    src.write_text(textwrap.dedent(r'''
+        #include <cstdio>
+        #include <vector>
+        #include "ttt-rs_amd/host/fused_tile_multi.hpp"
+        #include "ttt-rs_amd/host/fused_mlp.hpp"
+        struct Call { const float* w_in; float* w_out; int seq, K, per_batch, stride; const void* xq; };
+        static std::vector<Call> calls;
+        extern "C" {
+        const char* ttt_last_error(void) { return "stub"; }
+        int64_t ttt_linear_num_checkpoints(const ttt_desc*) { return 0; }
+        int64_t ttt_mlp_bwd_workspace_bytes(const ttt_desc*) { return 0; }
+        int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void*, const void*, const float* W0, const float* b0,
+                           const float*, const void*, const float*, const float*, void* out, float* W_out, float* b_out,
+                           float*, float*, void*) {
+          if (!W0 || !b0 || !W_out || !b_out || !out) return TTT_ERR_NULL;
+          calls.push_back({W0, W_out, d->seq, d->mini_batch, d->state_per_batch, d->seq_stride, xq});
+          return TTT_OK;
+        }
+        int ttt_linear_bwd(const ttt_desc*, const void*, const void*, const void*, const float*, const float*, const float*,
+                           const void*, const float*, const float*, const float*, const float*, const void*, const float*,
+                           const float*, void*, void*, void*, float*, float*, void*, float*, float*, float*, void*) { return TTT_OK; }
+        int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void*, const void*, const float* W1, const float* b1,
+                        const float* W2, const float* b2, const float*, const void*, const float*, const float*, void* out,
+                        float* W1o, float* b1o, float* W2o, float* b2o, void*) {
+          if (!W1 || !b1 || !W2 || !b2 || !W1o || !b1o || !W2o || !b2o || !out) return TTT_ERR_NULL;
+          calls.push_back({W1, W1o, d->seq, d->mini_batch, d->state_per_batch, d->seq_stride, xq});
+          return TTT_OK;
+        }
+        int ttt_mlp_bwd(const ttt_desc*, const void*, const void*, const void*, const float*, const float*, const float*,
+                        const float*, const float*, const void*, const float*, const float*, const void*, const float*,
+                        const float*, const float*, const float*, void*, void*, void*, float*, float*, float*, float*, void*,
+                        float*, float*, float*, void*, void*) { return TTT_OK; }
+        }
+        int main() {
+          ttt::ModelConfig cfg; cfg.num_heads = 2; cfg.head_dim = 64;
+          static float params[4], A[4], B[4], x[4 * 64 * 64];
+          ttt::FusedTileMulti m(cfg, params, params, params, params);
+          ttt::TTTInputsInner in; in.batch = 1; in.seq_len = 16 * 2 + 5; in.qkv = ttt::Qkv{x, x, x};
+          in.token_eta = params; in.ttt_lr_eta = x;
+          ttt::TTTLinearState st; st.weight = A; st.bias = A; st.next_weight = B; st.next_bias = B;
+          m.forward(st, in, x, ttt::Checkpoints{}, nullptr);
+          if (calls.size() != 2) return 1;
+          // launch 1: parameters in ([H,..] broadcast), buffer B out, 32 tokens in mini-batches of 16
+          if (calls[0].w_in != params || calls[0].w_out != B || calls[0].per_batch != 0 || calls[0].seq != 32 ||
+              calls[0].K != 16 || calls[0].stride != 37) return 2;
+          // launch 2: the remainder as one short mini-batch, reads B, writes A, window starts at token 32
+          if (calls[1].w_in != B || calls[1].w_out != A || calls[1].per_batch != 1 || calls[1].seq != 5 ||
+              calls[1].K != 5 || calls[1].stride != 37 || calls[1].xq != (const void*)(x + 32 * 64)) return 3;
+          if (st.weight != A || st.next_weight != B || !st.initialised) return 4;
+          // the next forward continues from the state (no re-read of the parameters)
+          calls.clear();
+          in.seq_len = 16;
+          m.forward(st, in, x, ttt::Checkpoints{}, nullptr);
+          if (calls.size() != 1 || calls[0].w_in != A || calls[0].w_out != B || calls[0].per_batch != 1) return 5;
+          // TTT-MLP: same protocol
+          calls.clear();
+          ttt::FusedMlp mlp(cfg, params, params, params, params, params, params);
+          ttt::TTTMLPState ms;
+          ms.w1 = ms.b1 = ms.w2 = ms.b2 = A; ms.next_w1 = ms.next_b1 = ms.next_w2 = ms.next_b2 = B;
+          in.seq_len = 16 + 3;
+          mlp.forward(ms, in, x, nullptr);
+          if (calls.size() != 2 || calls[0].w_in != params || calls[0].w_out != B || calls[1].w_in != B ||
+              calls[1].w_out != A || calls[1].seq != 3 || ms.w1 != A || !ms.initialised) return 6;
+          return 0;
+        }
+    '''))
+    exe = tmp_path / "s"
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-I", ROOT, str(src), "-o", str(exe)], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)

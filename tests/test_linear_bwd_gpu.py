@@ -23,7 +23,7 @@ def P():
     return importlib.import_module("ttt-rs_amd")
 
 
-def run_bwd(P, c, dO, K, ci, state_grads=None):
+def run_bwd(P, c, dO, K, ci, state_grads=None, bwd_hint=0):
     d = to_dev(c)
     out, W, b, Wc, bc = P.ttt_linear_forward_raw(d["xq"], d["xk"], d["xv"], d["W0"], d["b0"], d["token_eta"],
                                                  d["lr"], d["gamma"], d["beta"], K, 1e-6, ci,
@@ -32,7 +32,8 @@ def run_bwd(P, c, dO, K, ci, state_grads=None):
     if state_grads is not None:
         gw, gb = (x.to("cuda:0") for x in state_grads)
     g = P.ttt_linear_backward_raw(d["xq"], d["xk"], d["xv"], d["W0"], d["b0"], d["token_eta"], d["lr"],
-                                  d["gamma"], d["beta"], Wc, bc, dO.to("cuda:0"), K, 1e-6, ci, gw, gb)
+                                  d["gamma"], d["beta"], Wc, bc, dO.to("cuda:0"), K, 1e-6, ci, gw, gb,
+                                  kernel_hint=bwd_hint)
     torch.cuda.synchronize()
     return g
 
@@ -102,15 +103,14 @@ def test_bwd_with_upstream_state_gradients(P, d, K, dtype):
     compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), TOL[dtype])
 
 
-def test_bwd_bf16_lds_kernel_on_request(P, monkeypatch):
+def test_bwd_bf16_lds_kernel_on_request(P):
     """The LDS-tile kernel (f32 products) stays selectable for bf16 I/O."""
     print("case bwd bf16 lds kernel", flush=True)
-    monkeypatch.setenv("TTT_LINEAR_BWD_KERNEL", "lds")
     B, H, d, K, N = 1, 2, 64, 16, 3
     c = P.synthetic.reference_test_inputs(79, B, H, N * K, d, K, io_dtype=torch.bfloat16)
     g = torch.Generator().manual_seed(8)
     dO = torch.randn(B, H, N * K, d, generator=g).to(torch.bfloat16)
-    compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[torch.bfloat16])
+    compare(run_bwd(P, c, dO, K, 1, bwd_hint=P.TTT_HINT_LDS_TILES), oracle_bwd(c, dO, K), TOL[torch.bfloat16])
 
 
 def test_bwd_is_linear_in_upstream_gradient(P):
@@ -130,20 +130,19 @@ MW_CASES = [(2, 2, 32, 8, 1), (2, 2, 32, 8, 2), (1, 2, 64, 16, 3), (2, 3, 64, 16
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("B,H,d,K,N", MW_CASES)
-def test_bwd_multi_wave_kernel(P, monkeypatch, B, H, d, K, N, dtype):
+def test_bwd_multi_wave_kernel(P, B, H, d, K, N, dtype):
     """The feature-split kernel (several waves per (batch, head), exchanges through LDS), forced for both
     I/O types; with upstream state gradients so that every term of the scan is exercised."""
     print(f"case bwd multi-wave B{B} H{H} d{d} K{K} N{N} {dtype}", flush=True)
-    monkeypatch.setenv("TTT_LINEAR_BWD_WAVES", "4")
     c = P.synthetic.reference_test_inputs(300 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
     g = torch.Generator().manual_seed(9)
     dO = torch.randn(B, H, N * K, d, generator=g).to(dtype)
     sg = (0.1 * torch.randn(B, H, d, d, generator=g), 0.1 * torch.randn(B, H, d, generator=g))
-    compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), TOL[dtype])
+    compare(run_bwd(P, c, dO, K, 1, sg, bwd_hint=4), oracle_bwd(c, dO, K, sg), TOL[dtype])
     if d == 64 and K == 16:  # benchmark-style inputs at the benchmark's head size
         c = P.synthetic.baseline_inputs(2, B, H, N * K, d, K, io_dtype=dtype, with_dout=True)
         dO = c.pop("d_out")
-        compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])
+        compare(run_bwd(P, c, dO, K, 1, bwd_hint=4), oracle_bwd(c, dO, K), TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -175,16 +174,18 @@ def test_bwd_wide_heads_need_a_checkpoint_per_mini_batch(P):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("waves", ["1", "4"])
 @pytest.mark.parametrize("B,H,d,K,N", [(2, 2, 32, 8, 3), (2, 3, 64, 16, 8), (1, 2, 64, 5, 3), (1, 2, 96, 16, 3), (1, 2, 128, 16, 3)])
-def test_bwd_packed_checkpoints_change_nothing(P, monkeypatch, B, H, d, K, N, waves, dtype):
-    """Checkpoints stored as operand fragments in kernel order (bf16 I/O: as bf16).  The backward rounds the
-    state to its operand type before the first product either way, so every gradient is bit-identical to the
-    run with f32 row-major checkpoints; the forward's outputs do not depend on the checkpoint format at all."""
+def test_bwd_packed_checkpoints_change_nothing(P, B, H, d, K, N, waves, dtype):
+    """Checkpoints stored as operand fragments in kernel order (bf16 I/O: as bf16).  The forward's outputs do not
+    depend on the checkpoint format at all.  The backward works on the state minus its row means either way: a
+    packed checkpoint holds that difference as the forward had it, an f32 row-major checkpoint holds the state
+    itself and the backward subtracts the row means again, which reproduces the difference to an ulp of the
+    state.  So the two runs agree far inside the parity tolerance (f32: 1e-5; bf16 operands: where that ulp
+    moves a value across a bf16 rounding boundary a single operand changes by 2^-8, hence 5e-3), not bit for bit."""
     if (d > 64 or dtype == torch.float32) and waves == "1":
         pytest.skip("wide heads and f32 I/O have the feature-split kernel only")
     if d == 128 and dtype == torch.float32:
         pytest.skip("no f32 backward at head_dim 128")
     print(f"case bwd packed ckpt B{B} H{H} d{d} K{K} N{N} waves {waves} {dtype}", flush=True)
-    monkeypatch.setenv("TTT_LINEAR_BWD_WAVES", waves)
     c = P.synthetic.reference_test_inputs(500 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
     dv = to_dev(c)
     g = torch.Generator().manual_seed(11)
@@ -195,15 +196,13 @@ def test_bwd_packed_checkpoints_change_nothing(P, monkeypatch, B, H, d, K, N, wa
                                                      dv["lr"], dv["gamma"], dv["beta"], K, 1e-6, 1,
                                                      want_checkpoints=True, packed_checkpoints=packed)
         gr = P.ttt_linear_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
-                                       dv["gamma"], dv["beta"], Wc, bc, dO, K, 1e-6, 1, packed_checkpoints=packed)
+                                       dv["gamma"], dv["beta"], Wc, bc, dO, K, 1e-6, 1, packed_checkpoints=packed,
+                                       kernel_hint=int(waves))
         torch.cuda.synchronize()
         res.append((out, W, b, gr))
     assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][2], res[1][2])
     for k in res[0][3]:
-        if k in ("grad_token_eta", "grad_ln_weight", "grad_ln_bias"):  # atomics: order of the additions varies
-            assert_close(res[1][3][k], res[0][3][k].double(), 1e-5, k)
-        else:
-            assert torch.equal(res[0][3][k], res[1][3][k]), k
+        assert_close(res[1][3][k], res[0][3][k].double(), 1e-5 if dtype == torch.float32 else 5e-3, k, min_frac=0.99)
     compare(res[1][3], oracle_bwd(c, dO.cpu(), K), TOL[dtype])
 
 

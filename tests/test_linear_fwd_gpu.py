@@ -82,8 +82,11 @@ def test_checkpoints_hold_state_entering_stage(P, ci):
     assert_close(out, ro, 1e-4, "out")
     assert_close(Wc, rWc, 1e-4, "W_ckpt")
     assert_close(bc, rbc, 1e-4, "b_ckpt")
-    # first checkpoint is the initial state, bit for bit
-    assert torch.equal(Wc[:, :, 0].cpu(), c["W0"].unsqueeze(0).expand(B, H, d, d))
+    # first checkpoint is the initial state: the kernels carry the state minus its row means and add them back
+    # when they write a checkpoint, so it is reproduced to an ulp of the larger of the two, not bit for bit
+    w0 = c["W0"].unsqueeze(0).expand(B, H, d, d)
+    assert (Wc[:, :, 0].cpu() - w0).abs().max() <= 2.0 ** -22 * w0.abs().max()
+    # the final state of a sequence that never updates it IS the initial state bit for bit (test_lr_zero_...)
 
 
 def test_lr_zero_leaves_state_untouched(P):
@@ -115,8 +118,11 @@ def test_chained_single_stage_calls_equal_multi_stage(P):
                                              c["lr"][:, :, sl].contiguous(), c["gamma"], c["beta"], K)
         outs.append(o)
     torch.cuda.synchronize()
-    assert torch.equal(torch.cat(outs, 2), out)
-    assert torch.equal(Ws, W) and torch.equal(bs, b)
+    # every call splits its initial state into row means and the rest afresh, so the chain and the single call round
+    # differently in the last bits: they agree far inside the parity tolerance, not bit for bit
+    assert_close(torch.cat(outs, 2), out.double().cpu().numpy(), 1e-5, "chained out")
+    assert_close(Ws, W.double().cpu().numpy(), 1e-5, "chained W")
+    assert_close(bs, b.double().cpu().numpy(), 1e-5, "chained b")
 
 
 def test_inner_model_forward_with_remainder(P):

@@ -54,16 +54,16 @@ def test_mlp_fwd_matches_oracle(P, B, H, d, K, N, style, dtype):
                      min_frac=0.99 if loose else 0.999)
 
 
-def test_mlp_fwd_bf16_lds_kernel_keeps_f32_products(P, monkeypatch):
-    """TTT_MLP_FWD_KERNEL=lds selects the LDS-tile kernel for bf16 I/O too: f32 products, so the
+def test_mlp_fwd_bf16_lds_kernel_keeps_f32_products(P):
+    """kernel_hint TTT_HINT_LDS_TILES selects the LDS-tile kernel for bf16 I/O too: f32 products, so the
     state meets the f32 bar."""
     print("case mlp bf16 lds kernel", flush=True)
-    monkeypatch.setenv("TTT_MLP_FWD_KERNEL", "lds")
     B, H, d, K, N = 2, 2, 96, 16, 4
     c = mlp_case(P, 77, B, H, N * K, d, K, torch.bfloat16, "ref")
     dv = to_dev(c)
     got = P.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
-                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K,
+                                kernel_hint=P.TTT_HINT_LDS_TILES)
     torch.cuda.synchronize()
     n = np_inputs(c)
     ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
@@ -94,17 +94,16 @@ def test_mlp_inner_model_with_remainder(P):
 @pytest.mark.parametrize("kernel", ["registers", "lds"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("B,H,d,K,N,ci", [(2, 2, 96, 16, 4, 1), (1, 3, 128, 16, 5, 2), (1, 2, 128, 6, 3, 1)])
-def test_linear_fwd_wide_heads(P, B, H, d, K, N, ci, dtype, kernel, monkeypatch):
+def test_linear_fwd_wide_heads(P, B, H, d, K, N, ci, dtype, kernel):
     """head_dim 96 / 128: the register-resident kernel (default; bf16 I/O multiplies bf16 operands) and the
-    LDS-tile kernel (TTT_LINEAR_FWD_KERNEL=lds; f32 arithmetic for both I/O dtypes)."""
+    LDS-tile kernel (kernel_hint TTT_HINT_LDS_TILES; f32 arithmetic for both I/O dtypes)."""
     print(f"case linear wide B{B} H{H} d{d} K{K} N{N} ci{ci} {dtype} {kernel}", flush=True)
-    if kernel == "lds":
-        monkeypatch.setenv("TTT_LINEAR_FWD_KERNEL", "lds")
     c = P.synthetic.reference_test_inputs(300 + d, B, H, N * K, d, K, io_dtype=dtype)
     dv = to_dev(c)
     out, W, b, Wc, bc = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
                                                  dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K,
-                                                 1e-6, ci, want_checkpoints=True)
+                                                 1e-6, ci, want_checkpoints=True,
+                                                 kernel_hint=P.TTT_HINT_LDS_TILES if kernel == "lds" else 0)
     torch.cuda.synchronize()
     n = np_inputs(c)
     ro, rW, rb, rWc, rbc = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"],
@@ -113,3 +112,44 @@ def test_linear_fwd_wide_heads(P, B, H, d, K, N, ci, dtype, kernel, monkeypatch)
     state_tol = 1e-4 if (dtype == torch.float32 or kernel == "lds") else TOL[dtype]
     for name, g, r in (("W", W, rW), ("b", b, rb), ("W_ckpt", Wc, rWc), ("b_ckpt", bc, rbc)):
         assert_close(g, r, state_tol, name)
+
+
+def test_mlp_fwd_d128_lost_partner_is_loud(P):
+    """head_dim 128, bf16 I/O: two workgroups share a unit and wait for each other.  With the waits made to give up
+    at once (TTT_HINT_TEST_LOST_PARTNER; every kernel still runs to its end) the call still returns TTT_OK -- it
+    cannot know -- and every output of every unit is NaN, so the failure cannot pass for a result.  More units than
+    one launch holds (256 CUs: 128 units per launch) also exercises the batched launches."""
+    print("case mlp d128 lost partner", flush=True)
+    B, H, d, K, N = 1, 3, 128, 16, 3
+    c = mlp_case(P, 91, B, H, N * K, d, K, torch.bfloat16, "ref")
+    dv = to_dev(c)
+    args = (dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"],
+            dv["beta"], K)
+    got = P.ttt_mlp_forward_raw(*args, kernel_hint=P.TTT_HINT_TEST_LOST_PARTNER)
+    torch.cuda.synchronize()
+    for name, t in zip(("out", "W1", "b1", "W2", "b2"), got):
+        assert torch.isnan(t.float()).all(), f"{name}: a lost partner left finite values"
+    # and the same call without the hook is healthy afterwards (nothing sticky in the library)
+    ok = P.ttt_mlp_forward_raw(*args)
+    torch.cuda.synchronize()
+    for t in ok:
+        assert torch.isfinite(t.float()).all()
+
+
+def test_mlp_fwd_d128_more_units_than_one_launch(P):
+    """160 units of head_dim 128 need 320 workgroups: more than the CUs of the device, so the pairs go in two
+    launches; every unit must come out as when it is computed alone."""
+    print("case mlp d128 batched launches", flush=True)
+    B, H, d, K, N = 20, 8, 128, 16, 2
+    c = mlp_case(P, 92, B, H, N * K, d, K, torch.bfloat16, "ref")
+    dv = to_dev(c)
+    call = lambda x: P.ttt_mlp_forward_raw(x["xq"], x["xk"], x["xv"], x["W1"], x["b1"], x["W2"], x["b2"], x["token_eta"],
+                                           x["lr"], x["gamma"], x["beta"], K)
+    full = call(dv)
+    torch.cuda.synchronize()
+    for b in (0, 15, 16, 19):  # units on both sides of the launch boundary (128 units = 16 batch entries)
+        one = {k: (v[b:b + 1].contiguous() if k in ("xq", "xk", "xv", "lr") else v) for k, v in dv.items()}
+        r = call(one)
+        torch.cuda.synchronize()
+        for name, f, o in zip(("out", "W1", "b1", "W2", "b2"), full, r):
+            assert torch.equal(f[b:b + 1], o), (b, name)

@@ -10,9 +10,12 @@ LIB_PATH = os.path.join(HERE, "lib", "libttt_mi355x.so")
 
 TTT_OK, TTT_ERR_SHAPE, TTT_ERR_UNSUPPORTED, TTT_ERR_HIP, TTT_ERR_NULL = 0, -1, -2, -3, -4
 TTT_F32, TTT_BF16 = 0, 1
+TTT_HINT_AUTO, TTT_HINT_LDS_TILES = 0, 0x100  # kernel_hint: low byte = waves per unit (1, 2, 4)
+TTT_HINT_TEST_LOST_PARTNER = 0x200
 
 EXPORTS = (
-    "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_num_checkpoints",
+    "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_bwd_supported",
+    "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
     "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_inner_inputs", "ttt_layer_epilogue",
 )
@@ -23,7 +26,7 @@ class TttDesc(C.Structure):
         ("batch", C.c_int32), ("heads", C.c_int32), ("seq", C.c_int32), ("head_dim", C.c_int32),
         ("mini_batch", C.c_int32), ("eps", C.c_float), ("checkpoint_interval", C.c_int32),
         ("io_dtype", C.c_int32), ("state_per_batch", C.c_int32), ("seq_stride", C.c_int32),
-        ("checkpoint_format", C.c_int32),
+        ("checkpoint_format", C.c_int32), ("kernel_hint", C.c_int32),
     ]
 
 
@@ -51,6 +54,7 @@ def lib() -> C.CDLL:
         L.ttt_version.restype = C.c_char_p
         L.ttt_last_error.restype = C.c_char_p
         L.ttt_linear_supported.argtypes = [dp]
+        L.ttt_linear_bwd_supported.argtypes = [dp]
         L.ttt_linear_num_checkpoints.argtypes = [dp]
         L.ttt_linear_num_checkpoints.restype = C.c_int64
         L.ttt_linear_fwd.argtypes = [dp] + [vp] * 15

@@ -16,7 +16,6 @@ SOURCES = [os.path.join(HERE, "csrc", "ttt_api.hip")]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
-    "-DTTT_XG_SWAP=1",
     # keep the compiler from forming packed-f32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # let MFMA results live in ordinary VGPRs: the kernels consume them with VALU code right away,
@@ -41,5 +40,22 @@ def build_library(verbose: bool = False, extra_flags=()) -> str:
     return LIB_PATH
 
 
+DRIVER_PATH = os.path.join(LIB_DIR, "libttt_host_driver.so")
+
+
+def build_host_driver() -> str:
+    """The C++ host classes (host/*.hpp) behind C entry points, for the GPU test that drives them;
+    plain host code (g++), linked against the library."""
+    cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", "-Werror", "-fPIC", "-shared",
+           os.path.join(HERE, "host", "host_driver.cpp"), "-o", DRIVER_PATH,
+           "-L", LIB_DIR, "-lttt_mi355x", "-Wl,-rpath,$ORIGIN"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("g++ failed building " + DRIVER_PATH)
+    return DRIVER_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_host_driver())

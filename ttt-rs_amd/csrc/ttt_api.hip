@@ -68,17 +68,14 @@ int hip_status(hipError_t e, const char* what) {
 // A (batch, head) unit is a strictly sequential chain of mini-batches, so the launch is latency
 // bound until there are more units than SIMDs.  Few units: split each unit over several waves
 // (skewed workgroup kernel).  Many units: one wave per unit (no exchange at all).
-// TTT_LINEAR_FWD_WAVES = 1 | 2 | 4 overrides the number of waves per unit (tuning / tests).
-int fwd_waves_override() {
-  const char* e = std::getenv("TTT_LINEAR_FWD_WAVES");
-  return e ? std::atoi(e) : 0;
-}
-
+// desc.kernel_hint (low byte) = 1 | 2 | 4 overrides the number of waves per unit (tuning / tests).
 template <class T, int D, int NW>
 int launch_linear_fwd_nw(const ttt::LinearFwdArgs& a, hipStream_t s) {
-  constexpr int PF = 2;  // mini-batches prefetched ahead, in registers
+  // mini-batches prefetched ahead, in registers (f32 fragments are twice as large: the one-wave f32 kernel, which
+  // holds the whole state and all rows in one wave, has registers for one mini-batch ahead only)
+  constexpr int PF = (NW == 1 && sizeof(typename ttt::Io<T>::elem) == 4) ? 1 : 2;
   const dim3 grid((unsigned)(a.B * a.H)), block(64 * NW);
-  if (NW == 1) {
+  if constexpr (NW == 1) {
     if (a.K == 16)
       hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, true>), grid, block, 0, s, a);
     else
@@ -94,11 +91,14 @@ int launch_linear_fwd_nw(const ttt::LinearFwdArgs& a, hipStream_t s) {
 }
 
 template <class T, int D>
-int launch_linear_fwd(const ttt::LinearFwdArgs& a, hipStream_t s) {
-  constexpr int max_nw = D / 16;
+int launch_linear_fwd(const ttt::LinearFwdArgs& a, int waves_hint, hipStream_t s) {
   constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
+  // bf16 I/O: one or two waves per unit.  A four-wave bf16 variant (one feature tile per wave) is not offered: it
+  // was never faster than two, and its output LayerNorm came out wrong for one mini-batch in three of the
+  // branch-free passes (the k = 16 matrix instruction that adds the causal correction onto the k = 32 products).
+  constexpr int max_nw = f32 ? D / 16 : (D / 16 < 2 ? D / 16 : 2);
   const long units = (long)a.B * a.H;
-  int nw = fwd_waves_override();
+  int nw = waves_hint;
   if (nw <= 0) {
     // measured on MI355X (256 CUs x 4 SIMDs): bf16 is VALU-latency bound and likes 2 waves per unit
     // up to ~2 units per CU; f32 is MFMA bound (16x16x4 f32) and likes 4 until the CUs are shared
@@ -108,7 +108,9 @@ int launch_linear_fwd(const ttt::LinearFwdArgs& a, hipStream_t s) {
       nw = units <= 512 ? 2 : 1;
   }
   if (nw > max_nw) nw = max_nw;
-  if (nw >= 4) return launch_linear_fwd_nw<T, D, (max_nw >= 4 ? 4 : 2)>(a, s);
+  if constexpr (max_nw >= 4) {
+    if (nw >= 4) return launch_linear_fwd_nw<T, D, 4>(a, s);
+  }
   if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(a, s);
   return launch_linear_fwd_nw<T, D, 1>(a, s);
 }
@@ -130,19 +132,28 @@ int launch_linear_fwd_wide(const ttt::LinearFwdArgs& a, hipStream_t s) {
   return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
 }
 
-template <class K>
-int opt_in_lds(K kern, size_t bytes) {
-  // more than the default 64 KiB of LDS per workgroup has to be requested (per device)
-  return hip_status(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
-                    "hipFuncSetAttribute(LDS size)");
+// More than the default 64 KiB of LDS per workgroup has to be requested per kernel and device.  Done once:
+// one bit per device ordinal and kernel (the kernel is a template argument, so every kernel has its own mask).
+template <auto Kern>
+int opt_in_lds(size_t bytes) {
+  static std::atomic<uint64_t> done{0};
+  int dev = 0;
+  int rc = hip_status(hipGetDevice(&dev), "hipGetDevice");
+  if (rc != TTT_OK) return rc;
+  const uint64_t bit = (dev >= 0 && dev < 64) ? (uint64_t)1 << dev : 0;
+  if (bit != 0 && (done.load(std::memory_order_acquire) & bit) != 0) return TTT_OK;
+  rc = hip_status(hipFuncSetAttribute(reinterpret_cast<const void*>(Kern),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes),
+                  "hipFuncSetAttribute(LDS size)");
+  if (rc == TTT_OK) done.fetch_or(bit, std::memory_order_release);
+  return rc;
 }
 
 template <class T, int D>
 int launch_linear_fwd_lds(const ttt::LinearFwdArgs& a, hipStream_t s) {
-  auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D>;
+  constexpr auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D>;
   constexpr size_t bytes = ttt::LinFwdLds<D>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(256), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_fwd (LDS kernel) launch");
@@ -150,9 +161,9 @@ int launch_linear_fwd_lds(const ttt::LinearFwdArgs& a, hipStream_t s) {
 
 template <class T, int D>
 int launch_mlp_fwd(const ttt::MlpFwdArgs& a, hipStream_t s) {
-  auto kern = ttt::ttt_mlp_fwd_kernel<T, D>;
+  constexpr auto kern = ttt::ttt_mlp_fwd_kernel<T, D>;
   constexpr size_t bytes = ttt::MlpLds<D>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_mlp_fwd launch");
@@ -161,9 +172,9 @@ int launch_mlp_fwd(const ttt::MlpFwdArgs& a, hipStream_t s) {
 // register-resident kernel (d <= 96, bf16 operands on the matrix cores)
 template <class T, int D>
 int launch_mlp_fwd_rr(const ttt::MlpFwdArgs& a, hipStream_t s) {
-  auto kern = ttt::ttt_mlp_fwd_rr_kernel<T, D>;
+  constexpr auto kern = ttt::ttt_mlp_fwd_rr_kernel<T, D>;
   constexpr size_t bytes = ttt::MlpRrLds<D, sizeof(typename ttt::Io<T>::elem)>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_mlp_fwd (register-resident kernel) launch");
@@ -171,22 +182,35 @@ int launch_mlp_fwd_rr(const ttt::MlpFwdArgs& a, hipStream_t s) {
 
 // head_dim 128, bf16 I/O: a pair of workgroups per (batch, head); the exchange flags live in W2_out,
 // which is zeroed first (a fill kernel, not a memset node)
-int launch_mlp_fwd_cl2(const ttt::MlpFwdArgs& a, hipStream_t s) {
-  auto kern = ttt::ttt_mlp_fwd_cl2_kernel<ttt::BF16, 128>;
+int launch_mlp_fwd_cl2(ttt::MlpFwdArgs a, hipStream_t s) {
+  constexpr auto kern = ttt::ttt_mlp_fwd_cl2_kernel<ttt::BF16, 128>;
   constexpr size_t bytes = ttt::MlpCl2Lds<128, 2>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   const size_t units = (size_t)a.B * a.H, n = units * 128 * 512;
   hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a.W2, n);
-  hipLaunchKernelGGL(kern, dim3((unsigned)(((units + 7) / 8) * 16)), dim3(512), bytes, s, a);
+  // The two workgroups of a pair wait for each other, so both must be resident: a workgroup fills a CU (LDS,
+  // registers), hence no launch may hold more workgroups than the device has CUs.  The units are independent, so
+  // more units than that go in several launches on the stream.
+  int dev = 0, cus = 0;
+  rc = hip_status(hipGetDevice(&dev), "hipGetDevice");
+  if (rc != TTT_OK) return rc;
+  rc = hip_status(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute(CU count)");
+  if (rc != TTT_OK) return rc;
+  const size_t per_launch = (size_t)(cus / 16 > 0 ? cus / 16 : 1) * 8;  // groups of 16 workgroups = 8 units
+  for (size_t base = 0; base < units; base += per_launch) {
+    const size_t cnt = units - base < per_launch ? units - base : per_launch;
+    a.unit_base = (int)base;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(((cnt + 7) / 8) * 16)), dim3(512), bytes, s, a);
+  }
   return hip_status(hipGetLastError(), "ttt_mlp_fwd (two-CU kernel) launch");
 }
 
 template <class T, int D>
 int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  auto kern = ttt::ttt_linear_bwd_kernel<T, D>;
+  constexpr auto kern = ttt::ttt_linear_bwd_kernel<T, D>;
   constexpr size_t bytes = ttt::BwdLds<D>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_bwd launch");
@@ -195,9 +219,9 @@ int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s)
 // bf16 I/O, one checkpoint per mini-batch: one wave per (batch, head), state gradient in registers
 template <int D, bool PK = false>
 int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  auto kern = ttt::ttt_linear_bwd_rr_kernel<ttt::BF16, D, PK>;
+  constexpr auto kern = ttt::ttt_linear_bwd_rr_kernel<ttt::BF16, D, PK>;
   constexpr size_t bytes = ttt::LinBwdRrLds<D, PK>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_bwd (register-resident kernel) launch");
@@ -206,9 +230,9 @@ int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
 // one checkpoint per mini-batch, NW waves per (batch, head): feature axis split, exchanges through LDS
 template <class T, int D, int NW, bool PK = false>
 int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK>;
+  constexpr auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK>;
   constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem), PK>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_bwd (multi-wave register-resident kernel) launch");
@@ -216,12 +240,48 @@ int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
 
 template <class T, int D>
 int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
-  auto kern = ttt::ttt_mlp_bwd_kernel<T, D>;
+  constexpr auto kern = ttt::ttt_mlp_bwd_kernel<T, D>;
   constexpr size_t bytes = ttt::MlpBwdLds<D>::BYTES;
-  int rc = opt_in_lds(kern, bytes);
+  int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_mlp_bwd launch");
+}
+
+// Which TTT-Linear backward kernel serves a desc (and whether one does).
+// One checkpoint per mini-batch: the register-resident kernels (the state entering a mini-batch is read, not
+// re-simulated).  Waves per (batch, head): f32 products are bound by the matrix pipe, so the feature axis is
+// always split; bf16 runs one wave per unit when there are more units than two per CU and the split kernel
+// otherwise.  Coarser checkpoints (states re-simulated from the last checkpoint) or TTT_HINT_LDS_TILES: the
+// LDS-tile kernel, head_dim <= 64.  desc.kernel_hint's low byte overrides the number of waves.
+struct LinearBwdChoice {
+  enum Kind { LDS, REG } kind;
+  int waves;
+};
+int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
+  int rc = ttt_linear_supported(d);
+  if (rc != TTT_OK) return rc;
+  const int D = d->head_dim;
+  const bool f32 = d->io_dtype == TTT_F32;
+  const bool packed = d->checkpoint_format == TTT_CKPT_PACKED;
+  const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && D <= 64;
+  if (packed && (d->checkpoint_interval != 1 || want_lds))
+    return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
+  if (d->checkpoint_interval == 1 && !want_lds) {
+    if (f32 && D == 128)
+      return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
+    int waves = d->kernel_hint & TTT_HINT_WAVES_MASK;
+    if (waves == 0) waves = (f32 || D > 64 || (long)d->batch * d->heads <= 512) ? 4 : 1;
+    ch->kind = LinearBwdChoice::REG;
+    ch->waves = waves;
+    return TTT_OK;
+  }
+  if (D > 64)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim %d needs checkpoint_interval 1 (got %d)", D,
+                d->checkpoint_interval);
+  ch->kind = LinearBwdChoice::LDS;
+  ch->waves = 4;
+  return TTT_OK;
 }
 
 // dst = src, or zeros when src is null (a kernel, not a memcpy/memset node: capturable)
@@ -313,7 +373,7 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
   fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
   fa.W1 = ws + w.W1; fa.b1 = ws + w.b1; fa.W2 = ws + w.W2; fa.b2 = ws + w.b2;
-  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s;
+  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s; fa.unit_base = 0; fa.spin_limit = 1 << 21;
   fa.B = d->batch; fa.H = d->heads; fa.seq = d->seq; fa.K = d->mini_batch;
   fa.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   fa.n_stages = d->seq / d->mini_batch;
@@ -403,21 +463,19 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.state_per_batch = d->state_per_batch ? 1 : 0;
   a.ckpt_packed = (W_ckpt != nullptr && d->checkpoint_format == TTT_CKPT_PACKED) ? 1 : 0;
   a.eps = d->eps;
-  if (a.ckpt_packed) {
-    const char* k = std::getenv("TTT_LINEAR_FWD_KERNEL");
-    if (d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
-      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
-  }
+  const int waves_hint = d->kernel_hint & TTT_HINT_WAVES_MASK;
+  // the LDS-tile forward exists for head_dim 96/128 only; elsewhere the hint names no kernel and is ignored
+  const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
+  if (a.ckpt_packed && (d->checkpoint_interval != 1 || want_lds))
+    return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // register-resident kernels for every head_dim; the LDS-tile kernel (96/128) only on request
   const bool f32 = d->io_dtype == TTT_F32;
   switch (d->head_dim) {
-    case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, s) : launch_linear_fwd<ttt::BF16, 32>(a, s);
-    case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, s) : launch_linear_fwd<ttt::BF16, 64>(a, s);
+    case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, waves_hint, s) : launch_linear_fwd<ttt::BF16, 32>(a, waves_hint, s);
+    case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, waves_hint, s) : launch_linear_fwd<ttt::BF16, 64>(a, waves_hint, s);
     default: break;
   }
-  const char* force = getenv("TTT_LINEAR_FWD_KERNEL");
-  if (force && strcmp(force, "lds") == 0) {
+  if (want_lds) {
     if (d->head_dim == 96)
       return f32 ? launch_linear_fwd_lds<ttt::F32, 96>(a, s) : launch_linear_fwd_lds<ttt::BF16, 96>(a, s);
     return f32 ? launch_linear_fwd_lds<ttt::F32, 128>(a, s) : launch_linear_fwd_lds<ttt::BF16, 128>(a, s);
@@ -427,6 +485,11 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   return f32 ? launch_linear_fwd_wide<ttt::F32, 128>(a, s) : launch_linear_fwd_wide<ttt::BF16, 128>(a, s);
 }
 
+int ttt_linear_bwd_supported(const ttt_desc* d) {
+  LinearBwdChoice ch;
+  return choose_linear_bwd(d, &ch);
+}
+
 int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
                    const float* W0, const float* b0, const float* token_eta, const void* lr,
                    const float* gamma, const float* beta, const float* W_ckpt,
@@ -434,7 +497,9 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
                    const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
                    float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
                    void* stream) {
-  int rc = ttt_linear_supported(d);
+  // the kernel is chosen (and a desc without one refused) before anything is enqueued
+  LinearBwdChoice ch;
+  int rc = choose_linear_bwd(d, &ch);
   if (rc != TTT_OK) return rc;
   // W0/b0 are part of the saved state for interface parity; the state entering every stage is
   // rebuilt from the checkpoints (checkpoint 0 equals the initial state).
@@ -457,11 +522,12 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
   a.ckpt_packed = d->checkpoint_format == TTT_CKPT_PACKED;
   a.eps = d->eps;
-  if (a.ckpt_packed) {
-    const char* k = std::getenv("TTT_LINEAR_BWD_KERNEL");
-    if (d->checkpoint_interval != 1 || (k && std::strcmp(k, "lds") == 0))
-      return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
-  }
+  const int D = d->head_dim;
+  if (ch.kind != LinearBwdChoice::LDS &&
+      (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(d_out) || !aligned16(d_xq) ||
+       !aligned16(d_xk) || !aligned16(d_xv) || !aligned16(W_ckpt) || !aligned16(b_ckpt) ||
+       ((size_t)a.seq_stride * D) % 8 != 0))
+    return fail(TTT_ERR_SHAPE, "ttt_linear_bwd: tensors must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   // accumulated outputs start from zero; a fill kernel (not a memset node) so the sequence
   // can be captured into a graph
@@ -474,59 +540,36 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
                      d_beta, hd);
   const unsigned grid = (unsigned)(a.B * a.H);
   const bool f32 = d->io_dtype == TTT_F32;
-  const int D = d->head_dim;
-  // Kernel choice.  One checkpoint per mini-batch: the register-resident kernels (the state entering a
-  // mini-batch is read, not re-simulated).  Waves per (batch, head): f32 products are bound by the matrix
-  // pipe, so the feature axis is always split; bf16 runs one wave per unit when there are more units than
-  // two per CU and the split kernel otherwise.  TTT_LINEAR_BWD_KERNEL=lds and TTT_LINEAR_BWD_WAVES override.
-  const char* ksel = std::getenv("TTT_LINEAR_BWD_KERNEL");
-  const bool want_lds = ksel && std::strcmp(ksel, "lds") == 0;
-  if (a.ckpt_interval == 1 && !(want_lds && D <= 64)) {
-    if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(d_out) || !aligned16(d_xq) ||
-        !aligned16(d_xk) || !aligned16(d_xv) || !aligned16(W_ckpt) || !aligned16(b_ckpt) ||
-        ((size_t)a.seq_stride * D) % 8 != 0)
-      return fail(TTT_ERR_SHAPE, "ttt_linear_bwd: tensors must be 16-byte aligned");
-    const char* wsel = std::getenv("TTT_LINEAR_BWD_WAVES");
-    int waves = wsel ? std::atoi(wsel) : 0;
-    if (waves == 0) waves = (f32 || D > 64 || grid <= 512) ? 4 : 1;
-    if (f32 && a.ckpt_packed) {
-      if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2, true>(a, grid, s);
-      if (D == 64) return launch_linear_bwd_mw<ttt::F32, 64, 4, true>(a, grid, s);
-      if (D == 96) return launch_linear_bwd_mw<ttt::F32, 96, 3, true>(a, grid, s);
-      return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
-    }
-    if (f32) {
-      if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2>(a, grid, s);
-      if (D == 64) return waves == 2 ? launch_linear_bwd_mw<ttt::F32, 64, 2>(a, grid, s)
-                                     : launch_linear_bwd_mw<ttt::F32, 64, 4>(a, grid, s);
-      if (D == 96) return launch_linear_bwd_mw<ttt::F32, 96, 3>(a, grid, s);
-      return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
-    }
-    if (a.ckpt_packed) {
-      if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2, true>(a, grid, s) : launch_linear_bwd_rr<32, true>(a, grid, s);
-      if (D == 64) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 64, 4, true>(a, grid, s) : launch_linear_bwd_rr<64, true>(a, grid, s);
-      if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3, true>(a, grid, s);
-      return launch_linear_bwd_mw<ttt::BF16, 128, 4, true>(a, grid, s);
-    }
-    if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2>(a, grid, s) : launch_linear_bwd_rr<32>(a, grid, s);
-    if (D == 64) {
-      if (waves == 1) return launch_linear_bwd_rr<64>(a, grid, s);
-      return waves == 2 ? launch_linear_bwd_mw<ttt::BF16, 64, 2>(a, grid, s)
-                        : launch_linear_bwd_mw<ttt::BF16, 64, 4>(a, grid, s);
-    }
-    if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3>(a, grid, s);
-    return launch_linear_bwd_mw<ttt::BF16, 128, 4>(a, grid, s);
+  const int waves = ch.waves;
+  if (ch.kind == LinearBwdChoice::LDS) {
+    if (f32) return D == 64 ? launch_linear_bwd<ttt::F32, 64>(a, grid, s) : launch_linear_bwd<ttt::F32, 32>(a, grid, s);
+    return D == 64 ? launch_linear_bwd<ttt::BF16, 64>(a, grid, s) : launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
   }
-  // coarser checkpoints (states re-simulated from the last checkpoint), or on request: LDS-tile kernel
-  if (D > 64)
-    return fail(TTT_ERR_UNSUPPORTED,
-                "ttt_linear_bwd: head_dim %d needs checkpoint_interval 1 (got %d)", D, a.ckpt_interval);
+  if (f32 && a.ckpt_packed) {
+    if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2, true>(a, grid, s);
+    if (D == 64) return launch_linear_bwd_mw<ttt::F32, 64, 4, true>(a, grid, s);
+    return launch_linear_bwd_mw<ttt::F32, 96, 3, true>(a, grid, s);
+  }
   if (f32) {
-    if (D == 64) return launch_linear_bwd<ttt::F32, 64>(a, grid, s);
-    return launch_linear_bwd<ttt::F32, 32>(a, grid, s);
+    if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2>(a, grid, s);
+    if (D == 64) return waves == 2 ? launch_linear_bwd_mw<ttt::F32, 64, 2>(a, grid, s)
+                                   : launch_linear_bwd_mw<ttt::F32, 64, 4>(a, grid, s);
+    return launch_linear_bwd_mw<ttt::F32, 96, 3>(a, grid, s);
   }
-  if (D == 64) return launch_linear_bwd<ttt::BF16, 64>(a, grid, s);
-  return launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
+  if (a.ckpt_packed) {
+    if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2, true>(a, grid, s) : launch_linear_bwd_rr<32, true>(a, grid, s);
+    if (D == 64) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 64, 4, true>(a, grid, s) : launch_linear_bwd_rr<64, true>(a, grid, s);
+    if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3, true>(a, grid, s);
+    return launch_linear_bwd_mw<ttt::BF16, 128, 4, true>(a, grid, s);
+  }
+  if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2>(a, grid, s) : launch_linear_bwd_rr<32>(a, grid, s);
+  if (D == 64) {
+    if (waves == 1) return launch_linear_bwd_rr<64>(a, grid, s);
+    return waves == 2 ? launch_linear_bwd_mw<ttt::BF16, 64, 2>(a, grid, s)
+                      : launch_linear_bwd_mw<ttt::BF16, 64, 4>(a, grid, s);
+  }
+  if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3>(a, grid, s);
+  return launch_linear_bwd_mw<ttt::BF16, 128, 4>(a, grid, s);
 }
 
 int ttt_mlp_supported(const ttt_desc* d) {
@@ -555,7 +598,8 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   a.xq = xq; a.xk = xk; a.xv = xv; a.W1_0 = W1_0; a.b1_0 = b1_0; a.W2_0 = W2_0; a.b2_0 = b2_0;
   a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
   a.W1 = W1_out; a.b1 = b1_out; a.W2 = W2_out; a.b2 = b2_out;
-  a.G1_save = nullptr; a.G2_save = nullptr;
+  a.G1_save = nullptr; a.G2_save = nullptr; a.unit_base = 0;
+  a.spin_limit = (d->kernel_hint & TTT_HINT_TEST_LOST_PARTNER) ? 0 : (1 << 21);
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
   a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.n_stages = d->seq / d->mini_batch;
@@ -563,11 +607,11 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   a.eps = d->eps;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool f32 = d->io_dtype == TTT_F32;
-  // bf16 I/O, d <= 96: the state fits the register file of one CU.  TTT_MLP_FWD_KERNEL=lds forces
+  // bf16 I/O, d <= 96: the state fits the register file of one CU; d = 128: of two.  TTT_HINT_LDS_TILES forces
   // the LDS-tile kernel (f32 products, state in global memory) that the other cases use.
-  const char* force = getenv("TTT_MLP_FWD_KERNEL");
-  if (!f32 && d->head_dim == 128 && !(force && strcmp(force, "lds") == 0)) return launch_mlp_fwd_cl2(a, s);
-  if (!f32 && d->head_dim <= 96 && !(force && strcmp(force, "lds") == 0)) {
+  const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0;
+  if (!f32 && d->head_dim == 128 && !want_lds) return launch_mlp_fwd_cl2(a, s);
+  if (!f32 && d->head_dim <= 96 && !want_lds) {
     switch (d->head_dim) {
       case 32: return launch_mlp_fwd_rr<ttt::BF16, 32>(a, s);
       case 64: return launch_mlp_fwd_rr<ttt::BF16, 64>(a, s);

@@ -422,15 +422,6 @@ __device__ __forceinline__ float col16_sum2(const float* p, const float* q, int 
   return s;
 }
 
-// Sum over the 16 lanes of a row, in every lane: four rotations inside the row on the DPP path
-// (a shuffle goes through the LDS crossbar and costs an LDS round trip per step).
-__device__ __forceinline__ float row16_sum_dpp(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));  // row_ror:8
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));  // row_ror:4
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));  // row_ror:2
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));  // row_ror:1
-  return v;
-}
 // sum over an aligned group of W lanes (W = 16 or 32) that share a token
 template <int W>
 __device__ __forceinline__ float rowgroup_sum(float v) {

@@ -204,6 +204,8 @@ struct MlpFwdArgs {
   float* G2_save;
   int B, H, seq, seq_stride, K, n_stages, state_per_batch;
   float eps;
+  int unit_base;  // two-CU kernel only: first (batch, head) unit of this launch (the units are launched in batches)
+  int spin_limit;  // two-CU kernel only: polls before a wait for the partner gives up (0: give up at once; testing)
 };
 
 template <int D>

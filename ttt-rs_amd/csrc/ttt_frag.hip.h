@@ -45,26 +45,19 @@ __device__ __forceinline__ int feat(int J, int p) {
 
 // Sum over the four lane groups g (lanes c, c+16, c+32, c+48); result in every lane.
 __device__ __forceinline__ float xg_sum(float v) {
-#if TTT_XG_SWAP
   // permlane32_swap(a, b) exchanges a's upper 32 lanes with b's lower 32 lanes; with a == b == v
   // that leaves {lo,lo} in a and {hi,hi} in b, so a + b is lo + hi in every lane.
   // permlane16_swap does the same for odd/even rows of 16 lanes.  The two results are copied
   // into scalars before the float reinterpretation: bit-casting the vector elements in place
   // makes the front end read element 0 twice.
-  {
-    const uint32_t u = __float_as_uint(v);
-    const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    const uint32_t p0 = p[0], p1 = p[1];
-    v = __uint_as_float(p0) + __uint_as_float(p1);
-    const uint32_t w = __float_as_uint(v);
-    const auto q = __builtin_amdgcn_permlane16_swap(w, w, false, false);
-    const uint32_t q0 = q[0], q1 = q[1];
-    v = __uint_as_float(q0) + __uint_as_float(q1);
-  }
-#else
-  v += __shfl_xor(v, 16);
-  v += __shfl_xor(v, 32);
-#endif
+  const uint32_t u = __float_as_uint(v);
+  const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t p0 = p[0], p1 = p[1];
+  v = __uint_as_float(p0) + __uint_as_float(p1);
+  const uint32_t w = __float_as_uint(v);
+  const auto q = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+  const uint32_t q0 = q[0], q1 = q[1];
+  v = __uint_as_float(q0) + __uint_as_float(q1);
   return v;
 }
 
@@ -82,6 +75,20 @@ __device__ __forceinline__ float xg_sum4_scatter(float a, float b, float c, floa
   const uint32_t r0 = r[0], r1 = r[1];
   return __uint_as_float(r0) + __uint_as_float(r1);            // rows: a, b, c, d
 }
+
+// Sum over the 16 lanes of a row, in every lane: four rotations inside the row on the DPP path
+// (a shuffle goes through the LDS crossbar and costs an LDS round trip per step).
+__device__ __forceinline__ float row16_sum_dpp(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));  // row_ror:8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));  // row_ror:4
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));  // row_ror:2
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));  // row_ror:1
+  return v;
+}
+// The value of the first lane (c = 0) of each row of 16 lanes, in every lane of that row.  A rotation sum leaves
+// every lane with the same terms added in a different order, i.e. possibly different last bits; where all lanes
+// of a row must hold the SAME number (a pivot subtracted from a whole matrix row), one lane's result is shared.
+__device__ __forceinline__ float row16_first(float v) { return __shfl(v, (int)(threadIdx.x & 48u), 64); }
 
 // Workgroup barrier for LDS exchanges only: waits for this wave's LDS traffic, not for the
 // global prefetches in flight (a full __syncthreads() would drain those every mini-batch).

@@ -42,7 +42,8 @@ struct LinBwdMwLds {
   static constexpr int SUM = LR + 256;                // 3 exchanges x [8 sums][16 tokens][NW]
   static constexpr int PT = SUM + 3 * 8 * 16 * NW * 4;  // 4 kinds x [NW][64] f32x4: partial [16 x 16] blocks
   static constexpr int FR = PT + 4 * NW * 1024;       // 7 kinds x [NT][64] fragments
-  static constexpr int BYTES = FR + 7 * NT * FT;
+  static constexpr int M0 = FR + 7 * NT * FT;         // D row means of the initial W, then mean(b): the centred state
+  static constexpr int BYTES = M0 + (D + 4) * 4;
   static_assert(NT % NW == 0 && WSLOTS % NW == 0, "feature tiles must divide among the waves");
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
@@ -111,6 +112,40 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
   // rows of absent tokens (c >= K) are never fetched: they stay zero
   for (int i = threadIdx.x; i < L::BYTES / 16; i += 64 * NW) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
   __syncthreads();
+
+  // ---- the scan works on the centred state Wc = W - m 1^T, bc = b - mean(b), as the forward does (centre_state in
+  // ttt_linear_fwd_mw.hip.h): every product with W either feeds a LayerNorm (Z1, Zbar: a common shift of a row is
+  // discarded) or multiplies a LayerNorm gradient from the right (dZbar W^T, dZ1 W^T: the rows of dZbar and dZ1 sum
+  // to zero, so the m 1^T part contributes nothing).  m and mean(b) are those of the initial state (checkpoint 0):
+  // the forward's updates do not move them.  A packed checkpoint holds the centred matrix already.
+  float* const M0p = reinterpret_cast<float*>(smem + L::M0);
+  {
+    const size_t c0 = bh * (size_t)a.n_ckpt;
+    if (!PK) {
+      for (int i = threadIdx.x; i < D; i += 64 * NW) {
+        const f32x4* row = reinterpret_cast<const f32x4*>(a.W_ckpt + c0 * D * D + (size_t)i * D);
+        float sum = 0.f;
+        for (int j = 0; j < D / 4; ++j) {
+          const f32x4 v = row[j];
+          sum += (v[0] + v[1]) + (v[2] + v[3]);
+        }
+        M0p[i] = sum * inv_d;
+      }
+    }
+    if (threadIdx.x == 0) {
+      float sum = 0.f;
+      for (int f = 0; f < D; ++f) sum += a.b_ckpt[c0 * D + f];
+      M0p[D] = sum * inv_d;
+    }
+    __syncthreads();
+  }
+  float mrow[NT];  // m of row feat(I, c)
+#pragma unroll
+  for (int I = 0; I < NT; ++I) mrow[I] = PK ? 0.f : M0p[feat(I, c)];
+  float mrowo[TPW];  // the same for the wave's own row tiles
+#pragma unroll
+  for (int ii = 0; ii < TPW; ++ii) mrowo[ii] = PK ? 0.f : M0p[feat(w * TPW + ii, c)];
+  const float bbar = M0p[D];
 
   // ---- copies of one mini-batch, dealt round-robin to the waves
   const unsigned stg = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
@@ -269,13 +304,13 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
 #pragma unroll
     for (int ii = 0; ii < TPW; ++ii) {
       const int Io = w * TPW + ii;
-      bT[ii] = *reinterpret_cast<const f32x4*>(sl + L::Bv + Io * 1024);
+      bT[ii] = *reinterpret_cast<const f32x4*>(sl + L::Bv + Io * 1024) - bbar;
 #pragma unroll
       for (int J = 0; J < NT; ++J) {
         if constexpr (PK)  // stored as (m = j, k = i): transposed on the matrix pipe
           Wn[ii][J] = tokens_k(*reinterpret_cast<const frag*>(sl + pk_off(Io, J)));
         else
-          Wn[ii][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + (Io * NT + J) * 1024));
+          Wn[ii][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + (Io * NT + J) * 1024) - mrowo[ii]);
       }
       kdo[ii] = tokens_k(ko[ii]);
       qdo[ii] = tokens_k(qo[ii]);
@@ -297,8 +332,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
           wa0 = *reinterpret_cast<const frag*>(sl + pk_off(2 * qq, Jo));
           wa1 = *reinterpret_cast<const frag*>(sl + pk_off(2 * qq + 1, Jo));
         } else {
-          wa0 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq) * NT + Jo) * 1024)));
-          wa1 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq + 1) * NT + Jo) * 1024)));
+          wa0 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq) * NT + Jo) * 1024) - mrow[2 * qq]));
+          wa1 = tokens_k(IO::to_frag(*reinterpret_cast<const f32x4*>(sl + L::W + ((2 * qq + 1) * NT + Jo) * 1024) - mrow[2 * qq + 1]));
         }
         IO::mma2(z1[jj], wa0, wa1, k[2 * qq], k[2 * qq + 1]);
         IO::mma2(zb[jj], wa0, wa1, q[2 * qq], q[2 * qq + 1]);
@@ -343,7 +378,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     fetch(st - 1);
 
     const float mu1 = S1[0] * inv_d;
-    const float rstd1 = __builtin_amdgcn_rsqf(S1[1] * inv_d - mu1 * mu1 + a.eps);
+    const float rstd1 = __builtin_amdgcn_rsqf(fmaxf(S1[1] * inv_d - mu1 * mu1, 0.f) + a.eps);
     const float sa_xh = rstd1 * (S1[2] - mu1 * sum_a);                                    // sum a2 xh
     const float sa_xh2 = rstd1 * rstd1 * (S1[3] - 2.f * mu1 * S1[2] + mu1 * mu1 * sum_a);  // sum a2 xh^2
     const float s_gx = sa_xh + S1[4];                                                     // sum gx
@@ -398,7 +433,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     frag Zf[TPW], Zd[TPW];
     {
       const float mu2 = S2[0] * inv_d;
-      const float rstd2 = __builtin_amdgcn_rsqf(S2[1] * inv_d - mu2 * mu2 + a.eps);
+      const float rstd2 = __builtin_amdgcn_rsqf(fmaxf(S2[1] * inv_d - mu2 * mu2, 0.f) + a.eps);
       const float m1 = S2[2] * inv_d, m2 = rstd2 * (S2[3] - mu2 * S2[2]) * inv_d;
       f32x4 P = zero4, P2 = zero4;
       frag Gl[TPW], Zl[TPW];

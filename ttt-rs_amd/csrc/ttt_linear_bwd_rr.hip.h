@@ -37,7 +37,8 @@ struct LinBwdRrLds {
   static constexpr int X = Bv + NT * 1024;          // 4 tensors x NT/2 slots: X[token c][32q + 8g .. +7] (bf16)
   static constexpr int LR = X + 4 * (NT / 2) * 1024;  // 16 dwords: lr of token c, zero-extended bf16
   static constexpr int STAGE = LR + 256;
-  static constexpr int BYTES = 2 * STAGE;
+  static constexpr int M0 = 2 * STAGE;             // D row means of the initial W, then mean(b): the centred state
+  static constexpr int BYTES = M0 + (D + 4) * 4;
 };
 
 template <class T, int D, bool PK = false>
@@ -86,6 +87,36 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
   // rows of absent tokens (c >= K) are never fetched: they stay zero
   for (int i = lane; i < L::BYTES / 16; i += 64) reinterpret_cast<u32x4*>(smem)[i] = u32x4{0u, 0u, 0u, 0u};
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+  // The scan works on the centred state Wc = W - m 1^T, bc = b - mean(b), as the forward does (centre_state in
+  // ttt_linear_fwd_mw.hip.h): Z1 and Zbar feed LayerNorms, which discard a common shift of a row, and dZbar W^T,
+  // dZ1 W^T multiply LayerNorm gradients, whose rows sum to zero.  m, mean(b): those of checkpoint 0 (the forward's
+  // updates do not move them); a packed checkpoint holds the centred matrix already.
+  float* const M0p = reinterpret_cast<float*>(smem + L::M0);
+  {
+    const size_t c0 = bh * (size_t)a.n_ckpt;
+    if (!PK) {
+      for (int i = lane; i < D; i += 64) {
+        const f32x4* row = reinterpret_cast<const f32x4*>(a.W_ckpt + c0 * D * D + (size_t)i * D);
+        float sum = 0.f;
+        for (int j = 0; j < D / 4; ++j) {
+          const f32x4 v = row[j];
+          sum += (v[0] + v[1]) + (v[2] + v[3]);
+        }
+        M0p[i] = sum * inv_d;
+      }
+    }
+    if (lane == 0) {
+      float sum = 0.f;
+      for (int f = 0; f < D; ++f) sum += a.b_ckpt[c0 * D + f];
+      M0p[D] = sum * inv_d;
+    }
+    __syncthreads();
+  }
+  float mrow[NT];  // m of row feat(I, c)
+#pragma unroll
+  for (int I = 0; I < NT; ++I) mrow[I] = PK ? 0.f : M0p[feat(I, c)];
+  const float bbar = M0p[D];
 
   // The copies of one mini-batch are issued in NPART portions spread over the previous mini-batch's
   // arithmetic: the memory pipeline accepts only so many requests at a time, and a wave that issues a
@@ -189,7 +220,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
     }
     f32x4 bT[NT];
 #pragma unroll
-    for (int J = 0; J < NT; ++J) bT[J] = *reinterpret_cast<const f32x4*>(sb + L::Bv + J * 1024);
+    for (int J = 0; J < NT; ++J) bT[J] = *reinterpret_cast<const f32x4*>(sb + L::Bv + J * 1024) - bbar;
     frag Wn[NT][NT], kd[NT], qd[NT];
 #pragma unroll
     for (int I = 0; I < NT; ++I) {
@@ -214,7 +245,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
             Wa[e][J] = *reinterpret_cast<const frag*>(sb + L::W + (I * NQ + (J >> 1)) * 1024 + 8 * (J & 1));
             Wn[I][J] = tokens_k(Wa[e][J]);
           } else {
-            Wn[I][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sb + L::W + (I * NT + J) * 1024));
+            Wn[I][J] = IO::to_frag(*reinterpret_cast<const f32x4*>(sb + L::W + (I * NT + J) * 1024) - mrow[I]);
             Wa[e][J] = tokens_k(Wn[I][J]);  // tile transpose: (m = j, k = i)
           }
         }
@@ -234,7 +265,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
     {
       const float mu = rowsum(z1) * inv_d;
       const float var = rowdot(z1, z1) * inv_d - mu * mu;
-      rstd1 = __builtin_amdgcn_rsqf(var + a.eps);
+      rstd1 = __builtin_amdgcn_rsqf(fmaxf(var, 0.f) + a.eps);
 #pragma unroll
       for (int J = 0; J < NT; ++J) {
         xh[J] = (z1[J] - mu) * rstd1;
@@ -277,7 +308,7 @@ __global__ void __launch_bounds__(64) ttt_linear_bwd_rr_kernel(LinearBwdArgs a) 
     {
       const float mu = rowsum(zb) * inv_d;
       const float var = rowdot(zb, zb) * inv_d - mu * mu;
-      const float rstd2 = __builtin_amdgcn_rsqf(var + a.eps);
+      const float rstd2 = __builtin_amdgcn_rsqf(fmaxf(var, 0.f) + a.eps);
       f32x4 gx2[NT];
 #pragma unroll
       for (int J = 0; J < NT; ++J) {

@@ -59,7 +59,8 @@ __device__ __forceinline__ int own_offset(int w, int jj, int g) {
   return 32 * (J >> 1) + 8 * g + 4 * (J & 1);
 }
 
-// Packed W checkpoint: the image of the state in accumulator order, in the operand type of the I/O mode (bf16).  Tile (I, J) is the fragment a
+// Packed W checkpoint: the image of the CENTRED state (see centre_state; the backward works on the centred state
+// too, so the row means are not needed again) in accumulator order, in the operand type of the I/O mode (bf16).  Tile (I, J) is the fragment a
 // lane holds of it (value r of lane (c, g) is W[feat(I, 4g+r)][feat(J, c)]); the tiles (I, 2q) and (I, 2q+1)
 // share the 1 KiB row I * (d/32) + q, 16 bytes per lane.  This wave writes its TPW column tiles of every I.
 // f32 I/O keeps f32: tile (I, J) is the 1 KiB row I * (d/16) + J, 16 bytes per lane.
@@ -85,6 +86,133 @@ __device__ __forceinline__ void store_ckpt_packed(float* slot, const f32x4 (&Wc)
         *reinterpret_cast<u32x2*>(base + (I * (NT / 2) + (J >> 1)) * 1024 + 8 * (J & 1)) =
             __builtin_bit_cast(u32x2, Io<BF16>::to_frag(Wc[I][jj]));
       }
+    }
+  }
+}
+
+// ---- State centring -------------------------------------------------------------------------------------------
+// LayerNorm does not see a shift common to all d features of a row, and the inner loop looks at the state only
+// through LayerNorm: Z1 = XK W + b feeds the LN-L2 gradient, Zbar = XQ W + b - (...) G the output LayerNorm.  With
+//   W = Wc + m 1^T   (m_i = mean over the columns of row i)      b = bc + mean(b) 1
+// Z = X Wc + bc + (X m + mean b) 1^T, and the last term is a per-token constant that both LayerNorms discard.  The
+// update W += XK^T G'' keeps the split: the rows of G'' sum to zero (G is the gradient of a function that ignores a
+// common shift), and so do the columns it adds to b.  So m and mean(b) of the INITIAL state hold for the whole
+// sequence, and the kernels carry Wc and bc.  Z1 and Zbar then have row means at rounding level, which is what
+// makes the one-pass statistics (var = E z^2 - (E z)^2, where the reference takes two passes: var_mean_bias,
+// rust/core/src/util.rs:141-150) safe for states whose rows sit far from zero, and keeps the bf16 operand images of
+// W accurate whatever offset its rows carry.  No instruction is added to the loop.
+//
+// centre_state: centres the wave's column slice Wc[I][jj] and its bias features in place.  m0s (LDS, D + 1 floats)
+// receives m at index 16 I + p for row feat(I, p), and mean(b) at index D.  Every lane subtracts the numbers it
+// reads back from m0s, so a whole row is shifted by one and the same float.  xch: LDS scratch of NW * D floats.
+// Ends with a workgroup barrier.
+template <int D, int NW, int TPW>
+__device__ __forceinline__ void centre_state(f32x4 (&Wc)[D / 16][TPW], f32x4 (&bT)[TPW], const float* b0, float* m0s,
+                                             float* xch, int w, int c, int g) {
+  constexpr int NT = D / 16;
+#pragma unroll
+  for (int I = 0; I < NT; ++I)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float p = 0.f;
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) p += Wc[I][jj][r];
+      p = row16_sum_dpp(p);
+      if (c == 0) xch[(I * 16 + 4 * g + r) * NW + w] = p;
+    }
+  __syncthreads();
+  for (int i = threadIdx.x; i < D; i += 64 * NW) {
+    float s = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) s += xch[i * NW + ww];
+    m0s[i] = s * (1.0f / D);
+  }
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (int f = 0; f < D; ++f) s += b0[f];
+    m0s[D] = s * (1.0f / D);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int I = 0; I < NT; ++I) {
+    const f32x4 m = *reinterpret_cast<const f32x4*>(m0s + I * 16 + 4 * g);
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) Wc[I][jj] -= m;
+  }
+  const float bb = m0s[D];
+#pragma unroll
+  for (int jj = 0; jj < TPW; ++jj) bT[jj] -= bb;
+  __syncthreads();
+}
+
+// The state as f32 row-major matrices from the centred registers (checkpoints): W = Wc + m 1^T, b = bc + mean(b).
+template <int D, int TPW>
+__device__ __forceinline__ void store_state_f32(float* Wd, float* bd, const f32x4 (&Wc)[D / 16][TPW],
+                                                const f32x4 (&bT)[TPW], const float* m0s, int w, int c, int g) {
+  constexpr int NT = D / 16;
+#pragma unroll
+  for (int I = 0; I < NT; ++I) {
+    const f32x4 m = *reinterpret_cast<const f32x4*>(m0s + I * 16 + 4 * g);
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r] + m[r];
+  }
+  if (c == 0) {
+    const float bb = m0s[D];
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      f32x4 v = bT[jj];
+      v += bb;
+      *reinterpret_cast<f32x4*>(bd + own_offset<TPW>(w, jj, g)) = v;
+    }
+  }
+}
+
+// b = bc + mean(b) alone (the packed W checkpoint keeps the centred matrix; the bias checkpoint is always the true bias).
+template <int D, int TPW>
+__device__ __forceinline__ void store_bias_true(float* bd, const f32x4 (&bT)[TPW], const float* m0s, int w, int c, int g) {
+  if (c == 0) {
+    const float bb = m0s[D];
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      f32x4 v = bT[jj];
+      v += bb;
+      *reinterpret_cast<f32x4*>(bd + own_offset<TPW>(w, jj, g)) = v;
+    }
+  }
+}
+
+// The final state: initial state + (centred state now - centred state at the start).  The start value is formed
+// again exactly as centre_state formed it, so a sequence that never updates the state (lr = 0, token_eta[K-1] = 0)
+// returns the initial state bit for bit.
+template <int D, int TPW>
+__device__ __forceinline__ void store_state_final(float* Wd, float* bd, const float* W0, const float* b0,
+                                                  const f32x4 (&Wc)[D / 16][TPW], const f32x4 (&bT)[TPW],
+                                                  const float* m0s, int w, int c, int g) {
+  constexpr int NT = D / 16;
+#pragma unroll
+  for (int I = 0; I < NT; ++I) {
+    const f32x4 m = *reinterpret_cast<const f32x4*>(m0s + I * 16 + 4 * g);
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int at = feat(I, 4 * g + r) * D + feat(w * TPW + jj, c);
+        const float w0 = W0[at];
+        const float start = w0 - m[r];
+        Wd[at] = w0 + (Wc[I][jj][r] - start);
+      }
+  }
+  if (c == 0) {
+    const float bb = m0s[D];
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) {
+      const int f = own_offset<TPW>(w, jj, g);
+      const f32x4 v0 = *reinterpret_cast<const f32x4*>(b0 + f);
+      f32x4 start = v0;
+      start -= bb;
+      *reinterpret_cast<f32x4*>(bd + f) = v0 + (bT[jj] - start);
     }
   }
 }
@@ -196,6 +324,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
 #pragma unroll
         for (int r = 0; r < 4; ++r) Wc[I][jj][r] = W0[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)];
   }
+  // the kernel carries the centred state (see centre_state)
+  __shared__ __attribute__((aligned(16))) float m0s[D + 4];
+  __shared__ float cxch[NW * D];
+  centre_state<D, NW, TPW>(Wc, bT, a.b0 + sb * D, m0s, cxch, w, c, g);
 
   // Ring of R = PF+1 register sets, loop unrolled by R: step u consumes set u and refills the set
   // that step u-1 consumed, so every set has fixed registers and a load is never copied (a copy
@@ -218,17 +350,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
         float* Wd = a.W_ckpt + ci * D * D;
         if (a.ckpt_packed) {
           store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
+          store_bias_true<D, TPW>(a.b_ckpt + ci * D, bT, m0s, w, c, g);
         } else {
-#pragma unroll
-          for (int I = 0; I < NT; ++I)
-#pragma unroll
-            for (int jj = 0; jj < TPW; ++jj)
-#pragma unroll
-              for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+          store_state_f32<D, TPW>(Wd, a.b_ckpt + ci * D, Wc, bT, m0s, w, c, g);
         }
-        if (c == 0)
-#pragma unroll
-          for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
       }
 
       // ---- Z1^T, Zbar^T (this wave's feature rows) and the attention block
@@ -296,7 +421,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
       {
         const float mu = S[0] * inv_d;
         const float var = S[1] * inv_d - mu * mu;
-        const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+        const float rstd = __builtin_amdgcn_rsqf(fmaxf(var, 0.f) + a.eps);
         const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
         const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
         // G'' = p (gx - s1/d - xh s2/d), gx = a2 xh + bq, xh = (z - mu) rstd, p = -sc lr rstd
@@ -345,7 +470,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
           }
         }
         const float mu = s0 * inv_d;
-        const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
+        const float rstd = __builtin_amdgcn_rsqf(fmaxf(s1 * inv_d - mu * mu, 0.f) + a.eps);
         if (FULL || c < K) {
           elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
           f32x4 o[TPW];
@@ -386,18 +511,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArg
     }
   }
 
-  {
-    float* Wd = a.W_out + bh * D * D;
-#pragma unroll
-    for (int I = 0; I < NT; ++I)
-#pragma unroll
-      for (int jj = 0; jj < TPW; ++jj)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
-    if (c == 0)
-#pragma unroll
-      for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_out + bh * D + own_offset<TPW>(w, jj, g), bT[jj]);
-  }
+  store_state_final<D, TPW>(a.W_out + bh * D * D, a.b_out + bh * D, a.W0 + sb * D * D, a.b0 + sb * D, Wc, bT, m0s, w, c, g);
 }
 
 }  // namespace ttt

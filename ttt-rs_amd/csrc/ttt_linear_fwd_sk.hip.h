@@ -66,6 +66,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
 #pragma unroll
         for (int r = 0; r < 4; ++r) Wc[I][jj][r] = W0[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)];
   }
+  // the kernel carries the centred state (see centre_state): row means in LDS, the exchange buffer as scratch
+  __shared__ __attribute__((aligned(16))) float m0s[D + 4];
+  static_assert(NW * D <= 2 * 8 * 16 * NW, "the exchange buffer doubles as scratch of centre_state");
+  centre_state<D, NW, TPW>(Wc, bT, a.b0 + sb * D, m0s, &ex[0][0], w, c, g);
 
   // pending output of the previous mini-batch (its LayerNorm sums travel in the next exchange) and of the
   // one before (sums known: it is finished while the next exchange is in flight)
@@ -118,7 +122,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
   // out = xq + gamma (zbar - mu) rstd + beta for the pending mini-batch
   auto emit_output = [&](float s0, float s1, int stage, const f32x4 (&zbp)[TPW], const frag (&qop)[TPW]) {
     const float mu = s0 * inv_d;
-    const float rstd = __builtin_amdgcn_rsqf(s1 * inv_d - mu * mu + a.eps);
+    const float rstd = __builtin_amdgcn_rsqf(fmaxf(s1 * inv_d - mu * mu, 0.f) + a.eps);
     if (FULL || c < K) {
       elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D;
       f32x4 o[TPW];
@@ -225,17 +229,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
         float* Wd = a.W_ckpt + ci * D * D;
         if (a.ckpt_packed) {
           store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
+          store_bias_true<D, TPW>(a.b_ckpt + ci * D, bT, m0s, w, c, g);
         } else {
-#pragma unroll
-          for (int I = 0; I < NT; ++I)
-#pragma unroll
-            for (int jj = 0; jj < TPW; ++jj)
-#pragma unroll
-              for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+          store_state_f32<D, TPW>(Wd, a.b_ckpt + ci * D, Wc, bT, m0s, w, c, g);
         }
-        if (c == 0)
-#pragma unroll
-          for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
       }
       exchange8_publish(S, st & 1);
       // ---- the output pending since two mini-batches (sums known since the last exchange): nothing waits
@@ -255,7 +252,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
       {
         const float mu = S[0] * inv_d;
         const float var = S[1] * inv_d - mu * mu;
-        const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+        const float rstd = __builtin_amdgcn_rsqf(fmaxf(var, 0.f) + a.eps);
         const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
         const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
         const float p = -sc * cur.lr * rstd;
@@ -315,17 +312,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
           float* Wd = a.W_ckpt + ci * D * D;
           if (a.ckpt_packed) {
             store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
+            store_bias_true<D, TPW>(a.b_ckpt + ci * D, bT, m0s, w, c, g);
           } else {
-#pragma unroll
-            for (int I = 0; I < NT; ++I)
-#pragma unroll
-              for (int jj = 0; jj < TPW; ++jj)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
+            store_state_f32<D, TPW>(Wd, a.b_ckpt + ci * D, Wc, bT, m0s, w, c, g);
           }
-          if (c == 0)
-#pragma unroll
-            for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_ckpt + ci * D + own_offset<TPW>(w, jj, g), bT[jj]);
         }
 
         // ---- XK with tokens along k for the state update: depends on nothing computed here, so it
@@ -395,7 +385,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
         {
           const float mu = S[0] * inv_d;
           const float var = S[1] * inv_d - mu * mu;
-          const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+          const float rstd = __builtin_amdgcn_rsqf(fmaxf(var, 0.f) + a.eps);
           const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
           const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
           const float p = -sc * cur.lr * rstd;
@@ -445,18 +435,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArg
     if (a.n_stages >= 2) emit_output(so0, so1, a.n_stages - 2, zbo, qoo);
     emit_output(S[6], S[7], a.n_stages - 1, zbp, qop);
   }
-  {
-    float* Wd = a.W_out + bh * D * D;
-#pragma unroll
-    for (int I = 0; I < NT; ++I)
-#pragma unroll
-      for (int jj = 0; jj < TPW; ++jj)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) Wd[feat(I, 4 * g + r) * D + feat(w * TPW + jj, c)] = Wc[I][jj][r];
-    if (c == 0)
-#pragma unroll
-      for (int jj = 0; jj < TPW; ++jj) store4<F32>(a.b_out + bh * D + own_offset<TPW>(w, jj, g), bT[jj]);
-  }
+  store_state_final<D, TPW>(a.W_out + bh * D * D, a.b_out + bh * D, a.W0 + sb * D * D, a.b0 + sb * D, Wc, bT, m0s, w, c, g);
 }
 
 }  // namespace ttt

@@ -44,7 +44,8 @@ struct MlpCl2Lds {
   static constexpr int KD = GD + NT * 64 * 4 * ES;  // [2][NT][64] frag
   static constexpr int PRM = KD + 2 * NT * 64 * 4 * ES;  // gamma[d], beta[d], b1[FH] floats
   static constexpr int EXO = PRM + (2 * D + FH) * 4;
-  static constexpr int BYTES = EXO + 2 * 2 * 16 * 16;
+  static constexpr int LOST = EXO + 2 * 2 * 16 * 16;  // one word: a wait for the partner ran out
+  static constexpr int BYTES = LOST + 16;
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
   static_assert(NT == NW && D % 64 == 0 && ES == 2, "one reducer and one output tile per wave, bf16 I/O");
   static_assert(TILE % 1024 == 0 && P1 % 16 == 0, "input tiles are staged in 1 KiB wave blocks");
@@ -67,7 +68,7 @@ __device__ __forceinline__ void send_tagged(unsigned long long* slot, f32x4 v, u
 // partner costs one time-out per wave, not one per mini-batch, and ends in NaNs in b1_out, never in a hang.
 template <int N>
 __device__ __forceinline__ void recv_tagged(const unsigned long long* const (&slot)[N], const unsigned (&tag)[N],
-                                            f32x4 (&out)[N], bool& alive) {
+                                            f32x4 (&out)[N], bool& alive, int spin_limit) {
   unsigned long long wd[N][4];
   int it = 0;
   // light first stage: one lane watches the word stored last of the first slot, so that sixteen
@@ -75,7 +76,7 @@ __device__ __forceinline__ void recv_tagged(const unsigned long long* const (&sl
   if (alive && (threadIdx.x & 63) == 0) {
     const unsigned long long* last = slot[0] + 4 * 63 + 3;  // lane 63's fourth word (slot[] is lane 0's here)
     while ((unsigned)(__hip_atomic_load(last, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) != tag[0]) {
-      if (++it >= (1 << 21)) break;
+      if (++it >= spin_limit) break;
       __builtin_amdgcn_s_sleep(1);
     }
   }
@@ -93,7 +94,7 @@ __device__ __forceinline__ void recv_tagged(const unsigned long long* const (&sl
       for (int r = 0; r < 4; ++r) ok = ok && (unsigned)(wd[n][r] >> 32) == tag[n];
     // the whole wave leaves together: its lanes poll neighbouring words of the same tiles
     if (__all(ok) || !alive) break;
-    if (++it >= (1 << 21)) {
+    if (++it >= spin_limit) {
       alive = false;
       break;
     }
@@ -124,8 +125,10 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
   // blocks (i, i + 8) of every group of sixteen form a pair
   const int blk = blockIdx.x;
   const int cu = (blk >> 3) & 1;
-  const size_t bh = (size_t)(blk >> 4) * 8 + (blk & 7);
+  const size_t bh = (size_t)a.unit_base + (size_t)(blk >> 4) * 8 + (blk & 7);
   if (bh >= (size_t)a.B * a.H) return;
+  int& lost = *reinterpret_cast<int*>(smem + L::LOST);  // set by a wave whose wait for the partner ran out
+  if (tid == 0) lost = 0;
   const int h = (int)(bh % a.H), K = a.K;
   const int hoff = cu * FH;  // first hidden unit of this CU
 
@@ -176,6 +179,14 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
   float sum_a = 0.f;
 #pragma unroll
   for (int r = 0; r < 4; ++r) b2T[r] = a.b2_0[sb * D + own + r];
+  // the second layer is carried centred (see row_means16 in ttt_mlp_fwd_rr.hip.h)
+#pragma unroll
+  for (int j = 0; j < HT; ++j) {
+    const f32x4 m = row_means16<NT>(W2c[j], inv_d);
+#pragma unroll
+    for (int I = 0; I < NT; ++I) W2c[j][I] -= m;
+  }
+  b2T -= mean_of(a.b2_0 + sb * D, D, inv_d);
   for (int f = 0; f < D; ++f) sum_a += a.gamma[h * D + f] * a.gamma[h * D + f];
   for (int i = tid; i < D; i += 512) {
     GAM[i] = a.gamma[h * D + i];
@@ -238,7 +249,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
     return ((lo[0] + lo[1]) + (lo[2] + lo[3])) + ((hi[0] + hi[1]) + (hi[2] + hi[3]));
   };
   // tile slot `idx` of parity `par`: X1 tiles 0..NT-1, X2 tiles NT..2NT-1, the A2 tile 2NT
-  bool alive = true;
+  bool alive = a.spin_limit > 0;
   auto send_tile = [&](int par_, int idx, f32x4 v, unsigned tag) {
     send_tagged(reinterpret_cast<unsigned long long*>(xout + par_ * L::XSLOT + idx * L::XTILE) + 4 * lane, v, tag);
   };
@@ -291,7 +302,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
   auto output_emit = [&](int stage) {
     if (cu == 1) return;
     const float mu = collect(EXO, 0) * inv_d;
-    const float rstd = __builtin_amdgcn_rsqf(collect(EXO, 1) * inv_d - mu * mu + a.eps);
+    const float rstd = __builtin_amdgcn_rsqf(fmaxf(collect(EXO, 1) * inv_d - mu * mu, 0.f) + a.eps);
     if (c < K) {
       const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + own), bet = *reinterpret_cast<const f32x4*>(BET + own);
       elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D + own;
@@ -402,7 +413,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
         const unsigned long long* const sl[3] = {slot_in(par, w), slot_in(par ^ 1, NT + w), slot_in(par ^ 1, 2 * NT)};
         const unsigned tg[3] = {(unsigned)st + 1, (unsigned)st, (unsigned)st};
         f32x4 rv[3];
-        recv_tagged<3>(sl, tg, rv, alive);
+        recv_tagged<3>(sl, tg, rv, alive, a.spin_limit);
         zpart = rv[0];
         zb_part = rv[1];
         at_part = rv[2];
@@ -410,7 +421,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
         const unsigned long long* const sl[1] = {slot_in(par, w)};
         const unsigned tg[1] = {(unsigned)st + 1};
         f32x4 rv[1];
-        recv_tagged<1>(sl, tg, rv, alive);
+        recv_tagged<1>(sl, tg, rv, alive, a.spin_limit);
         zpart = rv[0];
       }
       fetch(st + 1);
@@ -439,7 +450,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
       for (int i = 0; i < 6; ++i) S[i] = collect(EX, i);
       const float mu = S[0] * inv_d;
       const float var = S[1] * inv_d - mu * mu;
-      const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+      const float rstd = __builtin_amdgcn_rsqf(fmaxf(var, 0.f) + a.eps);
       const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
       const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
       const float p = -sc * lrc * rstd;
@@ -550,7 +561,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
     const unsigned long long* const sl[2] = {slot_in(lp, NT + w), slot_in(lp, 2 * NT)};
     const unsigned tg[2] = {(unsigned)a.n_stages, (unsigned)a.n_stages};
     f32x4 rv[2];
-    recv_tagged<2>(sl, tg, rv, alive);
+    recv_tagged<2>(sl, tg, rv, alive, a.spin_limit);
     output_finish(rv[0], rv[1]);
   }
   lds_barrier();
@@ -558,27 +569,51 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
 
   // ---- final state: this CU's hidden half.  Its rows of W2_out held the exchange area; every read of
   // it by this workgroup is above, every write of the partner into it was awaited above.
+  if (!alive) lost = 1;
   __syncthreads();
+  // A wait for the partner that ran out (the two workgroups of a pair were not resident together long enough)
+  // must not pass for a result: the workgroup that saw it turns everything it owns of the unit into NaN -- its
+  // half of W1, b1, W2, b2 and the whole output of the unit (both workgroups do, as a rule: the partner then finds
+  // NaN tags where it polls and times out too).  The caller sees NaN in every output tensor of that unit.
+  const float poison = lost ? __builtin_nanf("") : 0.f;
   {
     float* W1 = a.W1 + bh * (size_t)D * F;
     float* W2 = a.W2 + bh * (size_t)D * F;
+    const float* W2i = a.W2_0 + sb * (size_t)D * F;
 #pragma unroll
     for (int j = 0; j < HT; ++j) {
       const int hb = hoff + 16 * (w * HT + j);
+      // second layer: initial value + (centred value now - centred value at the start); see ttt_mlp_fwd_rr.hip.h
+      f32x4 w0[NT];
 #pragma unroll
       for (int I = 0; I < NT; ++I)
 #pragma unroll
+        for (int r = 0; r < 4; ++r) w0[I][r] = W2i[(size_t)(hb + 4 * g + r) * D + feat(I, c)];
+      const f32x4 m = row_means16<NT>(w0, inv_d);
+#pragma unroll
+      for (int I = 0; I < NT; ++I) {
+        const f32x4 start = w0[I] - m;
+        const f32x4 fin = w0[I] + (W2c[j][I] - start);
+#pragma unroll
         for (int r = 0; r < 4; ++r) {
-          W1[(size_t)feat(I, 4 * g + r) * F + hb + c] = W1c[I][j][r];
-          W2[(size_t)(hb + 4 * g + r) * D + feat(I, c)] = W2c[j][I][r];
+          W1[(size_t)feat(I, 4 * g + r) * F + hb + c] = W1c[I][j][r] + poison;
+          W2[(size_t)(hb + 4 * g + r) * D + feat(I, c)] = fin[r] + poison;
         }
-      // a wait that ran out is made visible: this wave's slice of b1 becomes NaN (the partner, should it
-      // still arrive, writes only its own half of the state and cannot cover it up)
-      const float poison = alive ? 0.f : __builtin_nanf("");
+      }
       if (c == 0)
         store4<F32>(a.b1 + bh * F + hb + 4 * g, *reinterpret_cast<const f32x4*>(B1s + 16 * (w * HT + j) + 4 * g) + poison);
     }
-    if (cu == 0 && c == 0) store4<F32>(a.b2 + bh * D + own, b2T);
+    {
+      const float bb = mean_of(a.b2_0 + sb * D, D, inv_d);
+      const f32x4 v0 = *reinterpret_cast<const f32x4*>(a.b2_0 + sb * D + own);
+      const f32x4 start = v0 - bb;
+      if ((cu == 0 || lost) && c == 0) store4<F32>(a.b2 + bh * D + own, v0 + (b2T - start) + poison);
+    }
+    if (lost) {
+      elem* po = static_cast<elem*>(a.out) + bh * (size_t)a.seq_stride * D;
+      const size_t n = (size_t)a.n_stages * K * D;
+      for (size_t i = tid; i < n; i += 512) IO::store1(po + i, poison);
+    }
   }
 }
 

@@ -66,6 +66,39 @@ __device__ __forceinline__ void forget(f32x4& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void pin(f32x4& v) { asm volatile("" : "+v"(v)::"memory"); }
 __device__ __forceinline__ void pin(float& v) { asm volatile("" : "+v"(v)::"memory"); }
 
+// ---- Centred second layer.  The TTT-MLP loop looks at W2 and b2 only through LayerNorm (Z2 = X2 W2 + b2 feeds the
+// LN-L2 gradient, Zbar2 the output LayerNorm) and through G1 = (G2 W2^T) gelu'(Z1), where the rows of G2 sum to zero.
+// So, exactly as for the TTT-Linear state (centre_state in ttt_linear_fwd_mw.hip.h), the kernels carry
+// W2 - m 1^T (m_i = mean over the d columns of row i) and b2 - mean(b2): the dropped part shifts every feature of a
+// token by the same amount (discarded by both LayerNorms) and meets only zero row sums in G2 W2^T; the updates
+// W2 += X2^T G2'', b2 += colsum G2'' do not move m or mean(b2).  Z2 and Zbar2 then have row means at rounding
+// level, which keeps the one-pass statistics and the bf16 operand images of W2 accurate for any offset of its rows.
+//
+// Mean of each of the four rows (4g + r of a 16-row tile) of a [16 x d] tile held as NT accumulator tiles
+// (columns: tile I, lane c), the same float in all sixteen lanes of a row.  Made opaque so that the subtraction
+// that follows is a subtraction of this rounded number wherever it is repeated (no fused multiply-add).
+template <int NT>
+__device__ __forceinline__ f32x4 row_means16(const f32x4 (&t)[NT], float inv_d) {
+  f32x4 m;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float p = 0.f;
+#pragma unroll
+    for (int I = 0; I < NT; ++I) p += t[I][r];
+    m[r] = row16_first(row16_sum_dpp(p)) * inv_d;
+  }
+  asm volatile("" : "+v"(m));
+  return m;
+}
+// mean of d floats in global memory, the same float in every lane, opaque as above
+__device__ __forceinline__ float mean_of(const float* p, int d, float inv_d) {
+  float s = 0.f;
+  for (int f = 0; f < d; ++f) s += p[f];
+  s *= inv_d;
+  asm volatile("" : "+v"(s));
+  return s;
+}
+
 // The LDS addresses derived from the lane index are many (the regions span 150 KiB, beyond the
 // 64 KiB reach of an instruction offset) and all loop-invariant: hoisted out of the loop they are
 // spilled and reloaded from scratch.  Hiding the lane index from the optimiser at the start of each
@@ -135,6 +168,14 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
   float sum_a = 0.f;
 #pragma unroll
   for (int r = 0; r < 4; ++r) b2T[r] = a.b2_0[sb * D + own + r];
+  // the second layer is carried centred (see row_means16)
+#pragma unroll
+  for (int j = 0; j < HT; ++j) {
+    const f32x4 m = row_means16<NT>(W2c[j], inv_d);
+#pragma unroll
+    for (int I = 0; I < NT; ++I) W2c[j][I] -= m;
+  }
+  b2T -= mean_of(a.b2_0 + sb * D, D, inv_d);
   for (int f = 0; f < D; ++f) sum_a += a.gamma[h * D + f] * a.gamma[h * D + f];
   for (int i = tid; i < D; i += 512) {
     GAM[i] = a.gamma[h * D + i];
@@ -253,7 +294,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
   // part 2 (after B2): out = xq + gamma (zbar - mu) rstd + beta
   auto output_emit = [&](int stage) {
     const float mu = collect_o(0) * inv_d;
-    const float rstd = __builtin_amdgcn_rsqf(collect_o(1) * inv_d - mu * mu + a.eps);
+    const float rstd = __builtin_amdgcn_rsqf(fmaxf(collect_o(1) * inv_d - mu * mu, 0.f) + a.eps);
     if (c < K) {
       const f32x4 gam = *reinterpret_cast<const f32x4*>(GAM + ooff), bet = *reinterpret_cast<const f32x4*>(BET + ooff);
       const frag qo = load4<T>(row(stage % 3, 0) + ooff);
@@ -361,7 +402,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
       }
       const float mu = S[0] * inv_d;
       const float var = S[1] * inv_d - mu * mu;
-      const float rstd = __builtin_amdgcn_rsqf(var + a.eps);
+      const float rstd = __builtin_amdgcn_rsqf(fmaxf(var, 0.f) + a.eps);
       const float s1 = rstd * (S[2] - mu * sum_a) + S[4];
       const float s2 = rstd * rstd * (S[3] - 2.f * mu * S[2] + mu * mu * sum_a) + rstd * (S[5] - mu * S[4]);
       const float p = -sc * lrc * rstd;
@@ -494,23 +535,39 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
   lds_barrier();
   if (outw) output_emit(a.n_stages - 1);
 
-  // ---- final state
+  // ---- final state.  Second layer: initial value + (centred value now - centred value at the start), the start
+  // value formed again exactly as above, so a sequence that never updates the state returns it bit for bit.
   {
     float* W1 = a.W1 + bh * (size_t)D * F;
     float* W2 = a.W2 + bh * (size_t)D * F;
+    const float* W2i = a.W2_0 + sb * (size_t)D * F;
 #pragma unroll
     for (int j = 0; j < HT; ++j) {
       const int hb = 16 * (w * HT + j);
+      f32x4 w0[NT];
 #pragma unroll
       for (int I = 0; I < NT; ++I)
 #pragma unroll
+        for (int r = 0; r < 4; ++r) w0[I][r] = W2i[(size_t)(hb + 4 * g + r) * D + feat(I, c)];
+      const f32x4 m = row_means16<NT>(w0, inv_d);
+#pragma unroll
+      for (int I = 0; I < NT; ++I) {
+        const f32x4 start = w0[I] - m;
+        const f32x4 fin = w0[I] + (W2c[j][I] - start);
+#pragma unroll
         for (int r = 0; r < 4; ++r) {
           W1[(size_t)feat(I, 4 * g + r) * F + hb + c] = W1c[I][j][r];
-          W2[(size_t)(hb + 4 * g + r) * D + feat(I, c)] = W2c[j][I][r];
+          W2[(size_t)(hb + 4 * g + r) * D + feat(I, c)] = fin[r];
         }
+      }
       if (c == 0) store4<F32>(a.b1 + bh * F + hb + 4 * g, *reinterpret_cast<const f32x4*>(B1s + hb + 4 * g));
     }
-    if (red && c == 0) store4<F32>(a.b2 + bh * D + own, b2T);
+    if (red) {
+      const float bb = mean_of(a.b2_0 + sb * D, D, inv_d);
+      const f32x4 v0 = *reinterpret_cast<const f32x4*>(a.b2_0 + sb * D + own);
+      const f32x4 start = v0 - bb;
+      if (c == 0) store4<F32>(a.b2 + bh * D + own, v0 + (b2T - start));
+    }
   }
 }
 

@@ -13,8 +13,10 @@
 
 namespace ttt {
 
-/// mlp.rs:43-53: w1 [B,H,d,4d], b1 [B,H,4d], w2 [B,H,4d,d], b2 [B,H,d], f32.  `next_*` receive the
-/// updated state of a forward call; swap() makes them current.
+/// mlp.rs:43-53: w1 [B,H,d,4d], b1 [B,H,4d], w2 [B,H,4d,d], b2 [B,H,d], f32.  Two sets of caller-owned buffers,
+/// all eight always valid: a forward call reads the current set and writes `next_*`, then swap() makes those
+/// current.  `initialised == false`: the current set holds no state yet and the first launch reads the layer's
+/// [H,..] parameters instead (init_state without the copy), then sets the flag.
 struct TTTMLPState {
   float* w1 = nullptr;
   float* b1 = nullptr;
@@ -24,6 +26,7 @@ struct TTTMLPState {
   float* next_b1 = nullptr;
   float* next_w2 = nullptr;
   float* next_b2 = nullptr;
+  bool initialised = false;
   void swap() {
     float* t;
     t = w1; w1 = next_w1; next_w1 = t;
@@ -62,7 +65,7 @@ class FusedMlp {
   const ModelConfig& get_config() const { return config_; }
 
   ttt_desc desc(int batch, int seq, int mini_batch, ttt_dtype dtype, bool state_per_batch) const {
-    ttt_desc d;
+    ttt_desc d{};
     d.batch = batch;
     d.heads = config_.num_heads;
     d.seq = seq;
@@ -74,12 +77,13 @@ class FusedMlp {
     d.state_per_batch = state_per_batch ? 1 : 0;
     d.seq_stride = 0;
     d.checkpoint_format = TTT_CKPT_F32;
+    d.kernel_hint = config_.ttt.kernel_hint;
     return d;
   }
 
   /// inner.rs:25-50: all full mini-batches in one launch, then a trailing remainder as one short
-  /// mini-batch, as in-place windows of the [B,H,seq,d] tensors.  When state.w1 is null the first
-  /// launch reads the [H,..] parameters directly (init_state without the copy).
+  /// mini-batch, as in-place windows of the [B,H,seq,d] tensors.  A state that is not initialised yet
+  /// makes the first launch read the [H,..] parameters directly (see TTTMLPState).
   void forward(TTTMLPState& state, const TTTInputsInner& in, void* out, void* stream) const {
     const int K = config_.ttt.mini_batch_size;
     const int full = (in.seq_len / K) * K;
@@ -102,12 +106,12 @@ class FusedMlp {
   }
 
   /// Gradients of the whole sequence (seq a multiple of mini_batch_size) from the initial state
-  /// (state0.w1 null: the [H,..] parameters), grad_output [B,H,seq,d] and optional upstream gradients
+  /// (state0 not initialised: the [H,..] parameters), grad_output [B,H,seq,d] and optional upstream gradients
   /// of the final state (all four or none).
   void backward(const TTTInputsInner& in, const TTTMLPState& state0, const void* grad_output,
                 const float* grad_w1_out, const float* grad_b1_out, const float* grad_w2_out,
                 const float* grad_b2_out, const TTTMLPGrads& g, void* workspace, void* stream) const {
-    const bool per_batch = state0.w1 != nullptr;
+    const bool per_batch = state0.initialised;
     ttt_desc d = desc(in.batch, in.seq_len, config_.ttt.mini_batch_size, in.dtype, per_batch);
     check(ttt_mlp_bwd(&d, in.qkv.xq, in.qkv.xk, in.qkv.xv, per_batch ? state0.w1 : w1_,
                       per_batch ? state0.b1 : b1_, per_batch ? state0.w2 : w2_, per_batch ? state0.b2 : b2_,
@@ -123,7 +127,10 @@ class FusedMlp {
   }
   void launch(TTTMLPState& state, const TTTInputsInner& in, int first, int seq, int mini_batch, void* out,
               void* stream) const {
-    const bool per_batch = state.w1 != nullptr;
+    if (!state.w1 || !state.b1 || !state.w2 || !state.b2 || !state.next_w1 || !state.next_b1 || !state.next_w2 ||
+        !state.next_b2)
+      throw Error(TTT_ERR_NULL, "TTTMLPState: both sets of state buffers must be valid");
+    const bool per_batch = state.initialised;
     const std::size_t es = in.dtype == TTT_BF16 ? 2 : 4;
     const std::size_t row = (std::size_t)first * (std::size_t)config_.head_dim * es;
     ttt_desc d = desc(in.batch, seq, mini_batch, in.dtype, per_batch);
@@ -135,6 +142,7 @@ class FusedMlp {
                       const_cast<void*>(at(out, row)), state.next_w1, state.next_b1, state.next_w2,
                       state.next_b2, stream));
     state.swap();
+    state.initialised = true;
   }
 
   ModelConfig config_;

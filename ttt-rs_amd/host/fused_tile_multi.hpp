@@ -42,6 +42,8 @@ struct TTTConfig {
   /// Checkpoints as operand fragments in kernel order (ttt_desc.checkpoint_format = TTT_CKPT_PACKED):
   /// interval 1 only, same gradients, less traffic.  No counterpart in the reference's config.
   bool packed_checkpoints = false;
+  /// ttt_desc.kernel_hint (TTT_HINT_AUTO: the library chooses the kernels).
+  int kernel_hint = TTT_HINT_AUTO;
 };
 
 struct ModelConfig {
@@ -69,13 +71,17 @@ struct TTTInputsInner {
   std::size_t start_idx = 0;
 };
 
-/// linear.rs:27-33: weight [B,H,d,d], bias [B,H,d], f32.  `next_*` receive the updated state of a
-/// forward call (the library never writes a state in place); swap() makes them current.
+/// linear.rs:27-33: weight [B,H,d,d], bias [B,H,d], f32.  The library never writes a state in place, so a
+/// state is TWO pairs of caller-owned buffers, all four always valid: a forward call reads weight/bias and
+/// writes next_weight/next_bias, then swap() makes those current.  `initialised == false` means that
+/// weight/bias do not hold a state yet: the first launch then reads the layer's parameters directly
+/// ([H,..] broadcast over the batch: init_state of linear.rs:84-89 without the copy) and sets the flag.
 struct TTTLinearState {
   float* weight = nullptr;
   float* bias = nullptr;
   float* next_weight = nullptr;
   float* next_bias = nullptr;
+  bool initialised = false;
   void swap() {
     float* w = weight; weight = next_weight; next_weight = w;
     float* b = bias; bias = next_bias; next_bias = b;
@@ -116,7 +122,7 @@ class FusedTileMulti {
   const ModelConfig& get_config() const { return config_; }
 
   ttt_desc desc(int batch, int seq, int mini_batch, ttt_dtype dtype, bool state_per_batch) const {
-    ttt_desc d;
+    ttt_desc d{};
     d.batch = batch;
     d.heads = config_.num_heads;
     d.seq = seq;
@@ -128,6 +134,7 @@ class FusedTileMulti {
     d.state_per_batch = state_per_batch ? 1 : 0;
     d.seq_stride = 0;
     d.checkpoint_format = config_.ttt.packed_checkpoints ? TTT_CKPT_PACKED : TTT_CKPT_F32;
+    d.kernel_hint = config_.ttt.kernel_hint;
     return d;
   }
 
@@ -139,9 +146,8 @@ class FusedTileMulti {
   /// wrapper.rs:102-164 / inner.rs:25-50: all full mini-batches in one launch, then a trailing
   /// remainder as one short mini-batch, both as in-place windows of the [B,H,seq,d] tensors
   /// (desc.seq_stride).  state.weight/bias are read, state.next_* written, then swapped, so on
-  /// return `state` is the updated state.  When state.weight is null the first launch reads the
-  /// parameters directly ([H,..] broadcast: init_state of linear.rs:84-89 without the copy).
-  /// Checkpoints, if given, cover the full mini-batches.
+  /// return `state` is the updated state.  A state that is not initialised yet makes the first launch
+  /// read the parameters directly (see TTTLinearState).  Checkpoints, if given, cover the full mini-batches.
   void forward(TTTLinearState& state, const TTTInputsInner& in, void* out, const Checkpoints& ck,
                void* stream) const {
     const int K = config_.ttt.mini_batch_size;
@@ -180,7 +186,9 @@ class FusedTileMulti {
   // tokens [first, first+seq) of every (batch, head) unit, in place
   void launch(TTTLinearState& state, const TTTInputsInner& in, int first, int seq, int mini_batch,
               void* out, const Checkpoints& ck, void* stream) const {
-    const bool per_batch = state.weight != nullptr;
+    if (!state.weight || !state.bias || !state.next_weight || !state.next_bias)
+      throw Error(TTT_ERR_NULL, "TTTLinearState: weight, bias, next_weight and next_bias must all be valid buffers");
+    const bool per_batch = state.initialised;
     const std::size_t es = in.dtype == TTT_BF16 ? 2 : 4;
     const std::size_t row = (std::size_t)first * (std::size_t)config_.head_dim * es;
     ttt_desc d = desc(in.batch, seq, mini_batch, in.dtype, per_batch);
@@ -192,6 +200,7 @@ class FusedTileMulti {
                          const_cast<void*>(at(out, row)), state.next_weight, state.next_bias, ck.weight,
                          ck.bias, stream));
     state.swap();
+    state.initialised = true;
   }
 
   ModelConfig config_;

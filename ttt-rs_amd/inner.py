@@ -125,7 +125,8 @@ def _need_win(t: torch.Tensor, shape, dtype, name, pitch: int):
 
 def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
                            mini_batch: int, eps: float = 1e-6, checkpoint_interval: int = 1,
-                           want_checkpoints: bool = False, out: Optional[torch.Tensor] = None, packed_checkpoints: bool = False):
+                           want_checkpoints: bool = False, out: Optional[torch.Tensor] = None, packed_checkpoints: bool = False,
+                           kernel_hint: int = 0):
     """One call of ttt_linear_fwd on the current stream.
 
     Counterpart of fused_ttt_tile_forward_multi (rust/fused/src/linear_fused_tile/api.rs:52-83):
@@ -152,7 +153,7 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
     te = token_eta.to(torch.float32).contiguous()
     desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), pitch,
-                   int(packed_checkpoints))
+                   int(packed_checkpoints), kernel_hint)
     check(lib().ttt_linear_supported(C.byref(desc)))
     dev = xq.device
     if out is None or (pitch == 0 and not out.is_contiguous()):
@@ -182,7 +183,8 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
 
 def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
                             weight_ckpt, bias_ckpt, grad_output, mini_batch: int, eps: float = 1e-6,
-                            checkpoint_interval: int = 1, grad_weight_out=None, grad_bias_out=None, packed_checkpoints: bool = False):
+                            checkpoint_interval: int = 1, grad_weight_out=None, grad_bias_out=None, packed_checkpoints: bool = False,
+                            kernel_hint: int = 0):
     """One call of ttt_linear_bwd on the current stream.
 
     Counterpart of backward_multi (rust/fused/src/linear_fused_tile/backward/launch.rs:332-438).
@@ -204,8 +206,8 @@ def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_
     ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
     te = token_eta.to(torch.float32).contiguous()
     desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), int(per_batch), 0,
-                   int(packed_checkpoints))
-    check(lib().ttt_linear_supported(C.byref(desc)))
+                   int(packed_checkpoints), kernel_hint)
+    check(lib().ttt_linear_bwd_supported(C.byref(desc)))
     n = lib().ttt_linear_num_checkpoints(C.byref(desc))
     w_ck = _need(weight_ckpt, (B, H, n, d, d), torch.float32, "weight_ckpt")
     b_ck = _need(bias_ckpt, (B, H, n, d), torch.float32, "bias_ckpt")
@@ -234,7 +236,7 @@ def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_
 
 
 def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias,
-                        mini_batch: int, eps: float = 1e-6):
+                        mini_batch: int, eps: float = 1e-6, kernel_hint: int = 0):
     """One call of ttt_mlp_fwd on the current stream: the fused counterpart of
     TTTMLP::forward (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50).
     w1 [B,H,d,4d] or [H,d,4d], b1 [..,4d], w2 [..,4d,d], b2 [..,d].
@@ -259,7 +261,7 @@ def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_we
     if token_eta.numel() < mini_batch:
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
     te = token_eta.to(torch.float32).contiguous()
-    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), int(per_batch), 0)
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), int(per_batch), 0, 0, kernel_hint)
     check(lib().ttt_mlp_supported(C.byref(desc)))
     dev = xq.device
     f32 = dict(dtype=torch.float32, device=dev)
