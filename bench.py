@@ -51,79 +51,133 @@ def linear_bwd_bytes(B, H, seq, d, s):
     return B * H * seq * (7 * d * s + 2 * s)
 
 
-def cpu_baseline(c, K, kind, budget_s=20.0):
-    """Times the C/OpenMP port of the reference CPU path (oracle/ttt_oracle.c) on the host cores
-    on the same inputs (f32 arithmetic on the stored values), on a bounded batch slice."""
+def cpu_baseline(c, K, kind, budget_s=12.0):
+    """Times the C/OpenMP port of the reference CPU path (oracle/ttt_oracle.c) on the host cores on the same inputs
+    (f32 arithmetic on the stored values), on a bounded batch slice.  Forward workloads time the forward; the
+    TTT-Linear forward+backward workloads time forward and backward (what a training step of the reference's CPU
+    backend runs for this path); the C port has no TTT-MLP backward, so that workload times the forward only and
+    says so."""
     import numpy as np
     from oracle import c_oracle
     cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "9999")))
     n = {k: v.float().numpy() for k, v in c.items()}
     B, H, seq, d = n["xq"].shape
+    sl = lambda keys, nb: [n[k][:nb] if k in ("xq", "xk", "xv", "lr", "d_out") else n[k] for k in keys]
+    lin = ("W0", "b0", "xq", "xk", "xv", "token_eta", "lr", "gamma", "beta")
     if kind in ("mlp_fwd", "mlp_fwd_bwd"):
-        fn = c_oracle.mlp_fwd
         keys = ("W1", "b1", "W2", "b2", "xq", "xk", "xv", "token_eta", "lr", "gamma", "beta")
+        run = lambda nb: c_oracle.mlp_fwd(*sl(keys, nb), K=K, dtype=np.float32, nthreads=cores)
+        what = "forward" if kind == "mlp_fwd" else "forward only (the C port has no TTT-MLP backward)"
+    elif kind == "linear_fwd_bwd":
+        def run(nb):
+            c_oracle.linear_fwd(*sl(lin, nb), K=K, dtype=np.float32, nthreads=cores)
+            c_oracle.linear_bwd(*sl(lin + ("d_out",), nb), K=K, dtype=np.float32, nthreads=cores)
+        what = "forward + backward (all nine gradients)"
     else:
-        fn = c_oracle.linear_fwd
-        keys = ("W0", "b0", "xq", "xk", "xv", "token_eta", "lr", "gamma", "beta")
-    bsl = lambda nb: [n[k][:nb] if k in ("xq", "xk", "xv", "lr") else n[k] for k in keys]
+        run = lambda nb: c_oracle.linear_fwd(*sl(lin, nb), K=K, dtype=np.float32, nthreads=cores)
+        what = "forward"
     t0 = time.perf_counter()
-    fn(*bsl(1), K=K, dtype=np.float32, nthreads=cores)
+    run(1)
     t_one = time.perf_counter() - t0
     Bs = max(1, min(B, int(budget_s / 4 / max(t_one, 1e-4))))
     times = []
     for _ in range(3):
         t0 = time.perf_counter()
-        fn(*bsl(Bs), K=K, dtype=np.float32, nthreads=cores)
+        run(Bs)
         times.append(time.perf_counter() - t0)
     t = sum(times) / len(times)
-    what = "forward" if kind not in ("linear_fwd_bwd", "mlp_fwd_bwd") else "forward only (the C port has no backward)"
     return {"value": Bs * seq / t, "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"C/OpenMP f32 port of the reference CPU path, {what}, same inputs, batch {Bs} of "
                       f"{B} (tokens/s is batch-normalised), mean of 3 runs, {t:.3f} s per run"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="linear_fwd_125m_bf16", choices=sorted(WORKLOADS) + ["hbm_copy_calibration"])
-    ap.add_argument("--checkpoint-interval", type=int, default=1)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (the path shards over "
-                 "batch*heads with no communication inside the scan; only parameter gradients reduce)")
+class LinearCalls:
+    """The TTT-Linear entry points on preallocated buffers: what a step of the benchmark issues is the C-ABI call
+    and nothing else (no allocation, no copies), so the device time between the events around a call is the time of
+    its kernels."""
 
-    import torch
-    if a.workload == "hbm_copy_calibration":
-        # plain device-to-device copy of known size: reference point for the FETCH_SIZE / WRITE_SIZE
-        # counters (rocprofv3 --pmc) that the `traffic` figures are scaled by
-        nbytes = 512 << 20
-        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").random_(0, 255)
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        for _ in range(a.steps):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"workload": a.workload, "copy_bytes": nbytes, "steps": a.steps}))
-        return
-    pkg = importlib.import_module("ttt-rs_amd")
-    w = WORKLOADS[a.workload]
+    def __init__(self, pkg, dv, B, H, seq, d, K, dtype, ci, packed, with_bwd):
+        import ctypes as C
+        import torch
+        self.pkg, self.C = pkg, C
+        dev = dv["xq"].device
+        f32 = dict(dtype=torch.float32, device=dev)
+        self.desc = pkg.TttDesc(B, H, seq, d, K, 1e-6, ci, pkg.TTT_BF16 if dtype == torch.bfloat16 else pkg.TTT_F32,
+                                0, 0, int(packed), 0)
+        self.dv = dv
+        self.out = torch.empty_like(dv["xq"])
+        self.W, self.b = torch.empty((B, H, d, d), **f32), torch.empty((B, H, d), **f32)
+        self.Wc = self.bc = None
+        if with_bwd:
+            n = pkg.lib().ttt_linear_num_checkpoints(C.byref(self.desc))
+            self.Wc, self.bc = torch.empty((B, H, n, d, d), **f32), torch.empty((B, H, n, d), **f32)
+            self.g = dict(xq=torch.empty_like(dv["xq"]), xk=torch.empty_like(dv["xq"]), xv=torch.empty_like(dv["xq"]),
+                          W=torch.empty((B, H, d, d), **f32), b=torch.empty((B, H, d), **f32),
+                          lr=torch.empty_like(dv["lr"]), te=torch.empty(seq, **f32), gam=torch.empty((H, d), **f32),
+                          bet=torch.empty((H, d), **f32))
+        self.stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def _p(self, t):
+        return None if t is None else self.C.c_void_p(t.data_ptr())
+
+    def fwd(self):
+        d, p = self.dv, self._p
+        self.pkg._lib.check(self.pkg.lib().ttt_linear_fwd(
+            self.C.byref(self.desc), p(d["xq"]), p(d["xk"]), p(d["xv"]), p(d["W0"]), p(d["b0"]), p(d["token_eta"]),
+            p(d["lr"]), p(d["gamma"]), p(d["beta"]), p(self.out), p(self.W), p(self.b), p(self.Wc), p(self.bc),
+            self.stream))
+
+    def bwd(self):
+        d, p, g = self.dv, self._p, self.g
+        self.pkg._lib.check(self.pkg.lib().ttt_linear_bwd(
+            self.C.byref(self.desc), p(d["xq"]), p(d["xk"]), p(d["xv"]), p(d["W0"]), p(d["b0"]), p(d["token_eta"]),
+            p(d["lr"]), p(d["gamma"]), p(d["beta"]), p(self.Wc), p(self.bc), p(d["d_out"]), None, None, p(g["xq"]),
+            p(g["xk"]), p(g["xv"]), p(g["W"]), p(g["b"]), p(g["lr"]), p(g["te"]), p(g["gam"]), p(g["bet"]),
+            self.stream))
+
+
+def measured_counters(workload):
+    """HBM bytes per launch and matrix-pipe utilisation of a workload's dominant kernel, as measured with rocprofv3
+    counters and kept in profiles/traffic.json (not quantities of this run: counters cannot be read from inside it)."""
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(tpath):
+        return None, None
+    t = json.load(open(tpath))
+    return t.get(workload), t.get("mfma_util", {}).get(workload)
+
+
+def time_parts(parts, steps, torch):
+    """Average device time (s) of each named call, measured with HIP events on the launch stream around that call
+    alone, over `steps` repetitions of the whole sequence."""
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in parts]
+          for _ in range(steps)]
+    for row in ev:
+        for (e0, e1), (_, fn) in zip(row, parts):
+            e0.record()
+            fn()
+            e1.record()
+    torch.cuda.synchronize()
+    return {name: sum(row[i][0].elapsed_time(row[i][1]) for row in ev) / steps / 1e3
+            for i, (name, _) in enumerate(parts)}
+
+
+def run_workload(name, a, pkg, torch):
+    w = WORKLOADS[name]
     B, H, d, seq, K, io, kind = w["B"], w["H"], w["d"], w["seq"], w["K"], w["io"], w["kind"]
     dtype = {"bf16": torch.bfloat16, "f32": torch.float32}[io]
     s = 2 if io == "bf16" else 4
     ci = a.checkpoint_interval
     dev = torch.device("cuda:0")
     th = B * H * seq  # token-heads
+    parts = None      # [(kernel name, call)] when a step is a sequence of separately timed calls
+    c = None
 
     if kind == "stack":
         # 8 layers (6 TTT-Linear then 2 TTT-MLP); layer input = previous output + fresh projections
         layers = []
         for li in range(8):
-            c = pkg.synthetic.baseline_inputs(40 + li, B, H, seq, d, K, io_dtype=dtype, mlp=li >= 6)
-            layers.append({k: v.to(dev) for k, v in c.items()})
-        c = None
+            cl = pkg.synthetic.baseline_inputs(40 + li, B, H, seq, d, K, io_dtype=dtype, mlp=li >= 6)
+            layers.append({k: v.to(dev) for k, v in cl.items()})
 
         def step():
             x = None
@@ -137,7 +191,6 @@ def main():
                                                 L["lr"], L["gamma"], L["beta"], K)[0]
             return (x,)
     elif kind in ("inner_inputs", "layer_epilogue"):
-        c = None
         g = torch.Generator().manual_seed(1234 + w["cfg"])
         rn = lambda *sh: torch.randn(*sh, generator=g).to(dtype).to(dev)
         if kind == "inner_inputs":
@@ -161,15 +214,29 @@ def main():
                                           with_dout=kind in ("linear_fwd_bwd", "mlp_fwd_bwd"),
                                           mlp=kind in ("mlp_fwd", "mlp_fwd_bwd"))
         dv = {k: v.to(dev) for k, v in c.items()}
-        if kind == "linear_fwd":
-            def step():
-                return pkg.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
-                                                  dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+        if kind in ("linear_fwd", "linear_fwd_bwd"):
+            # a checkpoint per mini-batch: checkpoints as operand fragments in kernel order (bf16 I/O: half the
+            # checkpoint traffic); --checkpoint-format f32 keeps the reference's f32 matrices
+            packed = kind == "linear_fwd_bwd" and ci == 1 and a.checkpoint_format == "packed"
+            calls = LinearCalls(pkg, dv, B, H, seq, d, K, dtype, ci, packed, kind == "linear_fwd_bwd")
+            if kind == "linear_fwd":
+                parts = [("ttt_linear_fwd", calls.fwd)]
+
+                def step():
+                    calls.fwd()
+                    return (calls.out, calls.W)
+            else:
+                parts = [("ttt_linear_fwd (writes checkpoints)", calls.fwd), ("ttt_linear_bwd", calls.bwd)]
+
+                def step():
+                    calls.fwd()
+                    calls.bwd()
+                    return (calls.out, calls.g["xq"], calls.g["W"])
         elif kind == "mlp_fwd":
             def step():
                 return pkg.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
                                                dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
-        elif kind == "mlp_fwd_bwd":
+        else:
             def step():
                 fw = pkg.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
                                              dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
@@ -177,34 +244,21 @@ def main():
                                              dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"],
                                              dv["d_out"], K)
                 return (fw[0], g["d_xq"])
-        else:
-            # a checkpoint per mini-batch: checkpoints as operand fragments in kernel order (same gradients bit
-            # for bit; bf16 I/O: half the checkpoint traffic); TTT_BENCH_CKPT=f32 keeps the reference's f32 matrices
-            packed = ci == 1 and os.environ.get("TTT_BENCH_CKPT") != "f32"
-
-            def step():
-                out, W, b, Wc, bc = pkg.ttt_linear_forward_raw(
-                    dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
-                    dv["gamma"], dv["beta"], K, 1e-6, ci, want_checkpoints=True, packed_checkpoints=packed)
-                g = pkg.ttt_linear_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"],
-                                                dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], Wc, bc,
-                                                dv["d_out"], K, 1e-6, ci, packed_checkpoints=packed)
-                return (out, g["grad_xq"])
 
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for _ in range(a.steps)]
+    # the timed region: exactly `steps` steps between two synchronisations, nothing else on the stream
     t0 = time.perf_counter()
-    for e0, e1 in ev:
-        e0.record()          # events sit on the stream the kernels are launched on
+    for _ in range(a.steps):
         res = step()
-        e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    dev_s = sum(e0.elapsed_time(e1) for e0, e1 in ev) / len(ev) / 1e3  # device time of one step
     assert all(torch.isfinite(r.float()).all() for r in res)
+    # device times, in passes of their own: HIP events on the launch stream around a whole step, and around each
+    # call of a step that consists of several
+    dev_s = time_parts([("step", step)], a.steps, torch)["step"]
+    part_s = time_parts(parts, a.steps, torch) if parts else None
 
     pass_name = {"linear_fwd": "fwd", "linear_fwd_bwd": "fwd+bwd", "mlp_fwd": "fwd", "mlp_fwd_bwd": "fwd+bwd",
                  "stack": "fwd", "inner_inputs": "inner-loop inputs", "layer_epilogue": "layer epilogue"}[kind]
@@ -217,61 +271,70 @@ def main():
         "ms_per_step": wall / a.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "data": "synthetic",
-        "config": {"workload": a.workload, "batch": B, "heads": H, "head_dim": d, "seq_len": seq,
+        "config": {"workload": name, "batch": B, "heads": H, "head_dim": d, "seq_len": seq,
                    "mini_batch": K, "io_dtype": io, "pass": pass_name},
     }
+    traffic, mfma_util = measured_counters(name)
+    counters = {"traffic": traffic, "traffic_source": "profiles/traffic.json (rocprofv3 FETCH_SIZE/WRITE_SIZE runs)"
+                if traffic is not None else None}
+    if mfma_util is not None:
+        counters.update(mfma_util=mfma_util, mfma_util_source="profiles/traffic.json (rocprofv3 SQ_VALU_MFMA_BUSY_CYCLES "
+                        "over the cycles of the SIMDs that hold a wave)")
     if kind == "linear_fwd":
         alg = linear_fwd_bytes(B, H, seq, d, s)
-        out["dtype"] = "bf16" if io == "bf16" and d <= 64 else "f32"
+        k_s = part_s["ttt_linear_fwd"]
+        out["dtype"] = "bf16" if io == "bf16" else "f32"
         out["config"]["inner_model"] = "TTT-Linear"
-        out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                           "kernel": "ttt_linear_fwd_sk_kernel", "kernel_avg_us": dev_s * 1e6,
-                           "algorithmic_bytes": alg}
+        out["roofline"] = {"bound": "hbm", "achieved": alg / k_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": alg / k_s / 1e9 / HBM_PEAK_GBS, **counters,
+                           "kernel": "ttt_linear_fwd_sk_kernel", "kernel_avg_us": k_s * 1e6,
+                           "step_avg_us": dev_s * 1e6, "algorithmic_bytes": alg}
     elif kind in ("inner_inputs", "layer_epilogue"):
         # inner_inputs: xq, xk, xv read and written once, logits in, lr out; epilogue: inner_out and gate in, out written
         alg = th * (6 * d * s + 2 * s) if kind == "inner_inputs" else th * 3 * d * s
         out["dtype"] = "f32"
         out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                           "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, **counters,
                            "kernel": "ttt_inner_inputs_kernel" if kind == "inner_inputs" else "ttt_layer_epilogue_kernel",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_bytes": alg}
-    elif kind == "linear_fwd_bwd" and io == "bf16" and ci == 1 and os.environ.get("TTT_LINEAR_BWD_KERNEL") != "lds":
-        # register-resident backward (bf16 MFMA operands): the pair of passes is bound by HBM in the limit
-        alg = linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)
-        out["dtype"] = "bf16"
-        out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci,
-                             checkpoint_format="f32" if os.environ.get("TTT_BENCH_CKPT") == "f32" else "packed bf16")
-        out["roofline"] = {"bound": "hbm", "achieved": alg / dev_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": alg / dev_s / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                           "kernel": "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)",
-                           "kernel_avg_us": dev_s * 1e6, "algorithmic_bytes": alg,
-                           "checkpoint_bytes": 2 * th * (d * d * (2 if os.environ.get("TTT_BENCH_CKPT") != "f32" else 4) + d * 4) // (ci * K),
-                           "algorithmic_flops": th * (24 * d * d + 26 * K * d)}
     elif kind == "linear_fwd_bwd":
-        # the backward kernel dominates; it computes in f32 MFMA: 18 d^2 + 22 K d flop per token-head
-        flops = th * (24 * d * d + 26 * K * d)
-        out["dtype"] = "f32"
+        # dominant kernel: the backward.  bf16 I/O: bf16 matrix operands, the pair of passes is bound by HBM in the
+        # limit (7 d s + 2 s bytes per token-head for the backward); f32 I/O: true-f32 matrix products,
+        # 18 d^2 + 22 K d flop per token-head, bound by the f32 matrix pipe.
+        lds = ci != 1
+        bwd_s, fwd_s = part_s["ttt_linear_bwd"], part_s["ttt_linear_fwd (writes checkpoints)"]
+        ck_bytes = th * (d * d * (2 if (packed and io == "bf16") else 4) + d * 4) // (ci * K)  # written once, read once
+        out["dtype"] = io
         out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci,
-                             checkpoint_format="f32 row-major" if (ci != 1 or os.environ.get("TTT_BENCH_CKPT") == "f32") else "packed")
-        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
-                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
-                           "kernel": ("ttt_linear_fwd_sk_kernel + ttt_linear_bwd_mw_kernel (whole step)"
-                                      if ci == 1 and os.environ.get("TTT_LINEAR_BWD_KERNEL") != "lds" else
-                                      "ttt_linear_fwd_sk_kernel + ttt_linear_bwd_kernel (whole step)"),
-                           "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops,
-                           "algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s)}
+                             checkpoint_format="packed" if packed else "f32 row-major")
+        kname = "ttt_linear_bwd_kernel" if lds else "ttt_linear_bwd_mw_kernel"
+        if io == "bf16" and not lds:
+            alg = linear_bwd_bytes(B, H, seq, d, s)
+            roof = {"bound": "hbm", "achieved": alg / bwd_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": alg / bwd_s / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": alg}
+        else:
+            flops = th * (18 * d * d + 22 * K * d)
+            roof = {"bound": "mfma", "achieved": flops / bwd_s / 1e12, "peak": F32_MFMA_PEAK_TF, "unit": "TFLOP/s",
+                    "frac": flops / bwd_s / 1e12 / F32_MFMA_PEAK_TF, "algorithmic_flops": flops,
+                    "algorithmic_bytes": linear_bwd_bytes(B, H, seq, d, s)}
+        out["roofline"] = {**roof, **counters, "kernel": kname, "kernel_avg_us": bwd_s * 1e6,
+                           "step_avg_us": dev_s * 1e6, "checkpoint_bytes_each_way": ck_bytes,
+                           "other_kernels": [{"kernel": "ttt_linear_fwd_sk_kernel (writes checkpoints)",
+                                              "kernel_avg_us": fwd_s * 1e6,
+                                              "algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s)}],
+                           "step_algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s),
+                           "step_algorithmic_flops": th * (24 * d * d + 26 * K * d)}
     elif kind == "mlp_fwd":
         flops = th * (56 * d * d + 20 * K * d)
-        # bf16 I/O with d <= 96: register-resident kernel, bf16 MFMA operands with f32 accumulation and
-        # state; otherwise the LDS-tile kernel with f32 MFMA
-        rr = io == "bf16" and d <= 96 and os.environ.get("TTT_MLP_FWD_KERNEL") != "lds"
+        # bf16 I/O: register-resident kernels, bf16 matrix operands with f32 accumulation and state; f32 I/O: the
+        # LDS-tile kernel with f32 products
+        rr = io == "bf16"
         peak = BF16_MFMA_PEAK_TF if rr else F32_MFMA_PEAK_TF
         out["dtype"] = "bf16" if rr else "f32"
         out["config"]["inner_model"] = "TTT-MLP"
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": peak,
-                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / peak, "traffic": None,
-                           "kernel": "ttt_mlp_fwd_rr_kernel" if rr else "ttt_mlp_fwd_kernel",
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / peak, **counters,
+                           "kernel": ("ttt_mlp_fwd_rr_kernel" if d <= 96 else "ttt_mlp_fwd_cl2_kernel") if rr else "ttt_mlp_fwd_kernel",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     elif kind == "mlp_fwd_bwd":
         # forward (56 d^2 + 20 K d) plus the backward's own forward sweep (Z1, Z2, G1 and the two state updates:
@@ -281,7 +344,7 @@ def main():
         out["dtype"] = "f32"
         out["config"]["inner_model"] = "TTT-MLP"
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
-                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, "traffic": None,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, **counters,
                            "kernel": "ttt_mlp_fwd_rr_kernel + ttt_mlp_fwd_kernel + ttt_mlp_bwd_kernel (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     else:
@@ -289,14 +352,52 @@ def main():
         out["dtype"] = "bf16"   # register-resident kernels: bf16 MFMA operands, f32 accumulation and state
         out["config"]["inner_model"] = "6 x TTT-Linear + 2 x TTT-MLP"
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": BF16_MFMA_PEAK_TF,
-                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / BF16_MFMA_PEAK_TF, "traffic": None,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / BF16_MFMA_PEAK_TF, **counters,
                            "kernel": "8 layer launches + input adds (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        out["roofline"]["traffic"] = json.load(open(tpath)).get(a.workload)
     if not a.no_cpu_baseline and c is not None:
         out["cpu_baseline"] = cpu_baseline(c, K, kind)
+    return out
+
+
+# the headline metric names the forward AND the forward+backward at the 125M shape: the default run measures the
+# forward (BASELINE config 1) as the line's own value and these two forward+backward workloads as `extra` entries
+DEFAULT_EXTRA = ("linear_fwd_bwd_125m_bf16_b32", "linear_fwd_bwd_125m_f32_b8")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS) + ["hbm_copy_calibration"])
+    ap.add_argument("--checkpoint-interval", type=int, default=1)
+    ap.add_argument("--checkpoint-format", default="packed", choices=["packed", "f32"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="default run: only the forward, not the fwd+bwd entries")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (the path shards over "
+                 "batch*heads with no communication inside the scan; only parameter gradients reduce)")
+
+    import torch
+    if a.workload == "hbm_copy_calibration":
+        # plain device-to-device copy of known size: reference point for the FETCH_SIZE / WRITE_SIZE
+        # counters (rocprofv3 --pmc) that the `traffic` figures are scaled by
+        nbytes = 512 << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(a.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": a.workload, "copy_bytes": nbytes, "steps": a.steps}))
+        return
+    pkg = importlib.import_module("ttt-rs_amd")
+    default_run = a.workload is None
+    out = run_workload(a.workload or "linear_fwd_125m_bf16", a, pkg, torch)
+    if default_run and not a.no_extra:
+        out["extra"] = [run_workload(name, a, pkg, torch) for name in DEFAULT_EXTRA]
     print(json.dumps(out))
 
 

@@ -64,6 +64,18 @@ def test_c_port_matches_linear_fixture(path):
         assert rel(g, f[k]) <= 2e-4, k
 
 
+@pytest.mark.parametrize("path", LINEAR, ids=[os.path.basename(p)[:-4] for p in LINEAR])
+def test_c_port_backward_matches_linear_fixture(path):
+    """The C backward (f32) on the frozen cases, upstream state gradients included."""
+    f = np.load(path)
+    K = int(f["meta"][3])
+    a = [f["in_" + k].astype(np.float64) for k in LIN_IN]
+    got = c_oracle.linear_bwd(*a, f["in_d_out"], K=K, dtype=np.float32, nthreads=2, d_W_out=f["in_d_W_out"],
+                              d_b_out=f["in_d_b_out"])
+    for k, v in got.items():
+        assert rel(v, f["grad_" + k]) <= 5e-4, k
+
+
 @pytest.mark.parametrize("path", MLP, ids=[os.path.basename(p)[:-4] for p in MLP])
 def test_c_port_matches_mlp_fixture(path):
     f = np.load(path)

@@ -40,3 +40,21 @@ def test_c_mlp_fwd_matches_numpy_oracle(B, H, seq, d, K):
                                c["lr"], c["gamma"], c["beta"], K=K, dtype=dtype, nthreads=2)
         for g, r in zip(got, ref):
             assert np.abs(g - r).max() <= tol * np.abs(r).max()
+
+
+@pytest.mark.parametrize("B,H,N,d,K", [(2, 3, 4, 64, 16), (1, 2, 3, 32, 8), (1, 1, 1, 16, 4)])
+def test_c_linear_bwd_matches_numpy_oracle(B, H, N, d, K):
+    """The C backward (the timed CPU baseline of the forward+backward workloads) against the numpy oracle, which is
+    itself pinned to torch autograd through the primal per-token formulation (test_oracle_pins.py): all nine
+    gradients, float64 to rounding and float32 to 5e-4."""
+    seq = N * K
+    c = case(3, B, H, seq, d, K)
+    rng = np.random.default_rng(30)
+    d_out = rng.standard_normal((B, H, seq, d))
+    args = (c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"], c["gamma"], c["beta"], d_out)
+    ref = orc.linear_backward(*args, K=K)
+    for dtype, tol in ((np.float64, 1e-10), (np.float32, 5e-4)):
+        got = c_oracle.linear_bwd(*args, K=K, dtype=dtype, nthreads=2)
+        assert set(got) == set(ref)
+        for k in ref:
+            assert np.abs(got[k] - ref[k]).max() <= tol * np.abs(ref[k]).max(), (k, dtype)
