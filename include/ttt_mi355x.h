@@ -227,6 +227,39 @@ int ttt_mlp_bwd_static(const ttt_desc* desc, const void* xq, const void* xk, con
                        float* d_token_eta, float* d_gamma, float* d_beta, void* stream);
 
 /*
+ * A stack of inner models applied layer by layer (the long-context benchmark configuration: six TTT-Linear layers
+ * followed by two TTT-MLP layers): layer l runs its inner loop on
+ *     xq = x + pq_l,  xk = x + pk_l,  xv = x + pv_l      (x = output of layer l-1; layer 0: x = 0)
+ * where the sums are formed in f32 and rounded to io_dtype, and hands its output to layer l+1; the last layer's
+ * output is `out`.  One call enqueues everything: per layer one pass that forms the three sums (x is read once
+ * for all three) and the layer's ttt_linear_fwd / ttt_mlp_fwd launch, with desc (shape, eps, io_dtype,
+ * kernel_hint) shared by all layers and token_eta [mini_batch] shared too.  The reference has no single
+ * counterpart: it reaches the same chaining through one inner-model call per layer from its layer loop, and keeps
+ * a layer's kernel resident between calls in its streaming variant
+ * (rust/fused/src/linear_fused_tile/streaming/d2d/kernel.rs:98-232).
+ *
+ * kind: TTT_LAYER_LINEAR uses W1 = weight_init [H,d,d] (or [B,H,d,d]), b1 = bias_init; TTT_LAYER_MLP uses W1, b1,
+ * W2, b2 as ttt_mlp_fwd does (state_per_batch selects the leading dimension).  W1_out .. b2_out receive the
+ * layer's final state per batch element (Linear: W1_out [B,H,d,d], b1_out [B,H,d]; the other two unused).
+ * workspace: ttt_stack_fwd_workspace_bytes(desc) bytes, 16-byte aligned, caller-owned, free again when the
+ * call's work on `stream` has finished (the three input tensors of the current layer and two hand-over tensors).
+ * checkpoint fields of desc are ignored (forward only); seq_stride must be 0.
+ */
+#define TTT_LAYER_LINEAR 0
+#define TTT_LAYER_MLP 1
+typedef struct ttt_stack_layer {
+  int32_t kind;
+  const void *pq, *pk, *pv; /* [B,H,seq,d] io */
+  const float *W1, *b1, *W2, *b2;
+  const void* lr;           /* [B,H,seq] io (ttt_lr_eta of this layer) */
+  const float *gamma, *beta; /* [H,d] */
+  float *W1_out, *b1_out, *W2_out, *b2_out;
+} ttt_stack_layer;
+int64_t ttt_stack_fwd_workspace_bytes(const ttt_desc* desc);
+int ttt_stack_fwd(const ttt_desc* desc, int32_t n_layers, const ttt_stack_layer* layers /* host memory */,
+                  const float* token_eta, void* out, void* workspace, void* stream);
+
+/*
  * The elementwise work either side of the inner loop, one HBM-bound pass each (the GEMMs of the
  * projections stay with the BLAS the caller uses).  desc supplies batch, heads, seq, head_dim,
  * mini_batch and io_dtype; the other fields are ignored.

@@ -1,0 +1,123 @@
+"""GPU parity of ttt_stack_fwd (inner models applied layer by layer) through the C ABI.
+
+The long-context benchmark configuration is an 8-layer stack (6 TTT-Linear then 2 TTT-MLP layers, B=4, H=16,
+d=128, seq=8192, bf16 I/O) in which layer l runs on (previous output + fresh N(0,1) projections).  (batch, head)
+units never mix, so the float64 oracle carried through all eight layers on a two-unit slice is exact for those
+units.  Two comparisons:
+  * per layer, on the layer input the GPU actually produced (the oracle is fed the GPU's previous output): the
+    usual bf16 bar for every layer at full depth;
+  * free running: the oracle chains its own outputs (rounded to bf16 where the definition stores them).  Rounding
+    differences of one layer are inputs of the next, so the bar widens with depth; the last layer is held to
+    three times the single-layer bar.
+"""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import TOL, assert_close, to_np
+from oracle import ttt_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+def make_layers(P, B, H, seq, d, K, dtype, kinds, seed0=40):
+    layers = []
+    for li, mlp in enumerate(kinds):
+        c = P.synthetic.baseline_inputs(seed0 + li, B, H, seq, d, K, io_dtype=dtype, mlp=mlp)
+        c["pq"], c["pk"], c["pv"] = c.pop("xq"), c.pop("xk"), c.pop("xv")
+        layers.append(c)
+    return layers
+
+
+def bf16_round(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.float32)).to(torch.bfloat16).double().numpy()
+
+
+def oracle_layer(L, x, bs, hs, K, dtype):
+    """One layer of the float64 oracle on units (bs, hs); x: its input [len(bs), len(hs), seq, d] or None."""
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda v: np.asarray(v, dtype=np.float32).astype(np.float64))
+    sl = lambda t: to_np(t[bs][:, hs])
+    par = lambda t: to_np(t[hs])
+    q, k, v = sl(L["pq"]), sl(L["pk"]), sl(L["pv"])
+    if x is not None:
+        # the sums are formed in f32 and rounded to the I/O type
+        q, k, v = rnd(np.float32(x) + np.float32(q)), rnd(np.float32(x) + np.float32(k)), rnd(np.float32(x) + np.float32(v))
+    if "W2" in L:
+        return orc.mlp_forward(par(L["W1"]), par(L["b1"]), par(L["W2"]), par(L["b2"]), q, k, v, to_np(L["token_eta"]),
+                               sl(L["lr"]), par(L["gamma"]), par(L["beta"]), K=K)
+    return orc.linear_forward(par(L["W0"]), par(L["b0"]), q, k, v, to_np(L["token_eta"]), sl(L["lr"]), par(L["gamma"]),
+                              par(L["beta"]), K=K)
+
+
+def run_stack_layerwise(P, dl, K, n):
+    """The first n layers through ttt_stack_fwd: output and states of layer n-1."""
+    out, states = P.ttt_stack_forward_raw(dl[:n], dl[0]["token_eta"], K)
+    torch.cuda.synchronize()
+    return out, states[n - 1]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_small_stack_matches_oracle_layer_by_layer(P, dtype):
+    B, H, d, K, seq = 2, 2, 64, 16, 64
+    kinds = [False, False, True, False, True]
+    print(f"case stack small {dtype}", flush=True)
+    layers = make_layers(P, B, H, seq, d, K, dtype, kinds, seed0=70)
+    dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    bs, hs = [0, 1], [0, 1]
+    x_gpu = None
+    for n in range(1, len(kinds) + 1):
+        out, st = run_stack_layerwise(P, dl, K, n)
+        ref = oracle_layer(layers[n - 1], None if x_gpu is None else to_np(x_gpu), bs, hs, K, dtype)
+        tol = TOL[dtype]
+        assert_close(out, ref[0], tol, f"layer {n - 1} out")
+        for g, r, nm in zip(st, ref[1:], ("W1", "b1", "W2", "b2")):
+            f32_products = dtype == torch.float32
+            assert_close(g, r, 1e-4 if f32_products else tol, f"layer {n - 1} {nm}", min_frac=0.999 if f32_products else 0.99)
+        x_gpu = out.cpu()
+    # the stack call equals the chain of single-layer calls on explicitly formed sums, bit for bit
+    x = None
+    for L in dl:
+        q, k, v = (L["pq"], L["pk"], L["pv"]) if x is None else (x + L["pq"], x + L["pk"], x + L["pv"])
+        if "W2" in L:
+            x = P.ttt_mlp_forward_raw(q, k, v, L["W1"], L["b1"], L["W2"], L["b2"], L["token_eta"], L["lr"], L["gamma"],
+                                      L["beta"], K)[0]
+        else:
+            x = P.ttt_linear_forward_raw(q, k, v, L["W0"], L["b0"], L["token_eta"], L["lr"], L["gamma"], L["beta"], K)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(x, out)
+
+
+def test_config4_stack_chain_full_size(P):
+    B, H, d, K, seq = 4, 16, 128, 16, 8192
+    kinds = [False] * 6 + [True] * 2
+    dtype = torch.bfloat16
+    print("case stack config 4 (8 layers, B4 H16 d128 seq8192 bf16)", flush=True)
+    layers = make_layers(P, B, H, seq, d, K, dtype, kinds)
+    dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    bs, hs = [1], [3, 12]          # two units
+    x_gpu, x_free = None, None
+    tol = TOL[dtype]
+    for n in range(1, 9):
+        out, st = run_stack_layerwise(P, dl, K, n)
+        assert torch.isfinite(out.float()).all()
+        sub = out[bs][:, hs]
+        # (1) this layer alone, on the input the GPU produced
+        ref = oracle_layer(layers[n - 1], None if x_gpu is None else to_np(x_gpu), bs, hs, K, dtype)
+        assert_close(sub, ref[0], tol, f"layer {n - 1} out (given the GPU's input)")
+        for g, r, nm in zip(st, ref[1:], ("W1", "b1", "W2", "b2")):
+            # the biases are sums of 512 update rows of bf16-rounded factors that largely cancel: max-norm bar only
+            assert_close(g[bs][:, hs], r, tol, f"layer {n - 1} {nm}", min_frac=0.0 if nm.startswith("b") else 0.99)
+        # (2) free-running oracle chain
+        free = oracle_layer(layers[n - 1], x_free, bs, hs, K, dtype)
+        x_free = bf16_round(free[0])
+        rel = np.abs(to_np(sub) - free[0]).max() / np.abs(free[0]).max()
+        print(f"  layer {n - 1}: free-running max-norm relative difference {rel:.3e}", flush=True)
+        x_gpu = sub.cpu()
+    assert_close(sub, free[0], 3 * tol, "last layer, free-running chain", min_frac=0.99)

@@ -17,7 +17,7 @@ EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_bwd_supported",
     "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
-    "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_inner_inputs", "ttt_layer_epilogue",
+    "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue",
 )
 
 
@@ -28,6 +28,12 @@ class TttDesc(C.Structure):
         ("io_dtype", C.c_int32), ("state_per_batch", C.c_int32), ("seq_stride", C.c_int32),
         ("checkpoint_format", C.c_int32), ("kernel_hint", C.c_int32),
     ]
+
+
+class TttStackLayer(C.Structure):
+    """ttt_stack_layer of include/ttt_mi355x.h."""
+    _fields_ = [("kind", C.c_int32)] + [(n, C.c_void_p) for n in (
+        "pq", "pk", "pv", "W1", "b1", "W2", "b2", "lr", "gamma", "beta", "W1_out", "b1_out", "W2_out", "b2_out")]
 
 
 class TttError(RuntimeError):
@@ -65,6 +71,9 @@ def lib() -> C.CDLL:
         L.ttt_mlp_bwd_workspace_bytes.restype = C.c_int64
         L.ttt_mlp_bwd.argtypes = [dp] + [vp] * 29
         L.ttt_mlp_bwd_static.argtypes = [dp] + [vp] * 28
+        L.ttt_stack_fwd_workspace_bytes.argtypes = [dp]
+        L.ttt_stack_fwd_workspace_bytes.restype = C.c_int64
+        L.ttt_stack_fwd.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), vp, vp, vp, vp]
         L.ttt_inner_inputs.argtypes = [dp] + [vp] * 5 + [C.c_float] + [vp] * 4 + [C.c_int, C.c_int] + [vp] * 6
         L.ttt_layer_epilogue.argtypes = [dp] + [vp] * 3 + [C.c_float] + [vp] * 3
         _lib = L

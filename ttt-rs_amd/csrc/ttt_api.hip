@@ -666,6 +666,80 @@ int ttt_mlp_bwd_static(const ttt_desc* d, const void* xq, const void* xk, const 
                       d_token_eta, d_gamma, d_beta, ws, stream);
 }
 
+int64_t ttt_stack_fwd_workspace_bytes(const ttt_desc* d) {
+  if (check_common(d) != TTT_OK) return -1;
+  const int64_t es = d->io_dtype == TTT_BF16 ? 2 : 4;
+  const int64_t tensor = (((int64_t)d->batch * d->heads * d->seq * d->head_dim * es) + 255) / 256 * 256;
+  return 5 * tensor;
+}
+
+int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* layers, const float* token_eta,
+                  void* out, void* workspace, void* stream) {
+  int rc = check_common(d);
+  if (rc != TTT_OK) return rc;
+  if (n_layers <= 0) return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: n_layers must be positive (got %d)", n_layers);
+  if (!layers || !token_eta || !out || !workspace)
+    return fail(TTT_ERR_NULL, "ttt_stack_fwd: a required pointer is NULL");
+  if (d->seq_stride != 0 && d->seq_stride != d->seq)
+    return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: sequence windows (seq_stride) are not supported");
+  if (!aligned16(workspace) || !aligned16(out)) return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: out and workspace must be 16-byte aligned");
+  // everything is validated before anything is enqueued
+  for (int l = 0; l < n_layers; ++l) {
+    const ttt_stack_layer& L = layers[l];
+    if (L.kind != TTT_LAYER_LINEAR && L.kind != TTT_LAYER_MLP)
+      return fail(TTT_ERR_UNSUPPORTED, "ttt_stack_fwd: layer %d has kind %d", l, L.kind);
+    rc = L.kind == TTT_LAYER_LINEAR ? ttt_linear_supported(d) : ttt_mlp_supported(d);
+    if (rc != TTT_OK) return rc;
+    const bool mlp = L.kind == TTT_LAYER_MLP;
+    if (!L.pq || !L.pk || !L.pv || !L.W1 || !L.b1 || !L.lr || !L.gamma || !L.beta || !L.W1_out || !L.b1_out ||
+        (mlp && (!L.W2 || !L.b2 || !L.W2_out || !L.b2_out)))
+      return fail(TTT_ERR_NULL, "ttt_stack_fwd: layer %d: a required pointer is NULL", l);
+    if (!aligned16(L.pq) || !aligned16(L.pk) || !aligned16(L.pv))
+      return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: layer %d: pq/pk/pv must be 16-byte aligned", l);
+  }
+  ttt_desc ld = *d;
+  ld.seq_stride = 0;
+  ld.checkpoint_interval = 1;
+  ld.checkpoint_format = TTT_CKPT_F32;
+  const size_t es = d->io_dtype == TTT_BF16 ? 2 : 4;
+  const size_t elems = (size_t)d->batch * d->heads * d->seq * d->head_dim;
+  const size_t tensor = (elems * es + 255) / 256 * 256;
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  void* xq = ws;
+  void* xk = ws + tensor;
+  void* xv = ws + 2 * tensor;
+  void* hand[2] = {ws + 3 * tensor, ws + 4 * tensor};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const void* x = nullptr;
+  for (int l = 0; l < n_layers; ++l) {
+    const ttt_stack_layer& L = layers[l];
+    const void *q = L.pq, *k = L.pk, *v = L.pv;
+    if (x != nullptr) {
+      ttt::LayerInputsArgs a;
+      a.x = x; a.pq = L.pq; a.pk = L.pk; a.pv = L.pv; a.xq = xq; a.xk = xk; a.xv = xv;
+      a.n16 = elems * es / 16;
+      const dim3 grid((unsigned)((a.n16 + 255) / 256));
+      if (d->io_dtype == TTT_F32)
+        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::F32>, grid, dim3(256), 0, s, a);
+      else
+        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::BF16>, grid, dim3(256), 0, s, a);
+      rc = hip_status(hipGetLastError(), "ttt_stack_fwd (layer inputs) launch");
+      if (rc != TTT_OK) return rc;
+      q = xq; k = xk; v = xv;
+    }
+    void* o = (l == n_layers - 1) ? out : hand[l & 1];
+    if (L.kind == TTT_LAYER_LINEAR)
+      rc = ttt_linear_fwd(&ld, q, k, v, L.W1, L.b1, token_eta, L.lr, L.gamma, L.beta, o, L.W1_out, L.b1_out, nullptr,
+                          nullptr, stream);
+    else
+      rc = ttt_mlp_fwd(&ld, q, k, v, L.W1, L.b1, L.W2, L.b2, token_eta, L.lr, L.gamma, L.beta, o, L.W1_out, L.b1_out,
+                       L.W2_out, L.b2_out, stream);
+    if (rc != TTT_OK) return rc;
+    x = o;
+  }
+  return TTT_OK;
+}
+
 int ttt_inner_inputs(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
                      const void* lr_logits, const float* lr_bias, float base_lr, const float* token_idx,
                      const float* learnable_token_idx, const float* rope_cos, const float* rope_sin,

@@ -162,4 +162,41 @@ __global__ void __launch_bounds__(256) ttt_layer_epilogue_kernel(LayerEpilogueAr
   }
 }
 
+// Inputs of one layer of a stack: xq = x + pq, xk = x + pk, xv = x + pv (f32 sums rounded to the I/O type), x read
+// once for all three.  One thread per 16 bytes.
+struct LayerInputsArgs {
+  const void *x, *pq, *pk, *pv;
+  void *xq, *xk, *xv;
+  size_t n16;  // number of 16-byte chunks per tensor
+};
+template <class T>
+__global__ void __launch_bounds__(256) ttt_layer_inputs_kernel(LayerInputsArgs a) {
+  using IO = Io<T>;
+  constexpr int E = 16 / IO::kBytes;  // elements per chunk
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.n16) return;
+  const u32x4 rx = static_cast<const u32x4*>(a.x)[i];
+  const u32x4 rq = static_cast<const u32x4*>(a.pq)[i], rk = static_cast<const u32x4*>(a.pk)[i],
+              rv = static_cast<const u32x4*>(a.pv)[i];
+  auto add = [&](u32x4 p) {
+    u32x4 o;
+    if (E == 4) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = __float_as_uint(__uint_as_float(rx[e]) + __uint_as_float(p[e]));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(rx[e] << 16) + __uint_as_float(p[e] << 16);
+        const float hi = __uint_as_float(rx[e] & 0xffff0000u) + __uint_as_float(p[e] & 0xffff0000u);
+        const bf16x2 r = __builtin_convertvector(f32x2{lo, hi}, bf16x2);
+        o[e] = __builtin_bit_cast(uint32_t, r);
+      }
+    }
+    return o;
+  };
+  static_cast<u32x4*>(a.xq)[i] = add(rq);
+  static_cast<u32x4*>(a.xk)[i] = add(rk);
+  static_cast<u32x4*>(a.xv)[i] = add(rv);
+}
+
 }  // namespace ttt

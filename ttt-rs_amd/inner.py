@@ -500,6 +500,66 @@ class FusedTileMulti:
         return self._launch(state, inputs.slice_seq(r), len(r))
 
 
+def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6, kernel_hint: int = 0,
+                          workspace: Optional[torch.Tensor] = None):
+    """One call of ttt_stack_fwd on the current stream: inner models applied layer by layer, layer l on
+    xq = x + pq, xk = x + pk, xv = x + pv with x the previous layer's output (0 for the first layer).
+    layers: list of dicts with pq, pk, pv [B,H,seq,d], lr [B,H,seq], gamma, beta [H,d] and either W0, b0
+    (TTT-Linear) or W1, b1, W2, b2 (TTT-MLP), parameters [H,..].  Returns (out, states) with states[l] the final
+    state tensors of layer l (per batch element)."""
+    B, H, seq, d = layers[0]["pq"].shape
+    io = layers[0]["pq"].dtype
+    dev = layers[0]["pq"].device
+    f32 = dict(dtype=torch.float32, device=dev)
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(layers[0]["pq"]), 0, 0, 0, kernel_hint)
+    te = _need(token_eta.to(torch.float32), (token_eta.numel(),), torch.float32, "token_eta")
+    if te.numel() < mini_batch:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
+    arr = (_lib.TttStackLayer * len(layers))()
+    keep, states = [], []
+    for i, L in enumerate(layers):
+        mlp = "W2" in L
+        m = 4 * d
+        t = {k: _need(L[k], (B, H, seq, d), io, k) for k in ("pq", "pk", "pv")}
+        t["lr"] = _need(L["lr"], (B, H, seq), io, "lr")
+        t["gamma"] = _need(L["gamma"], (H, d), torch.float32, "gamma")
+        t["beta"] = _need(L["beta"], (H, d), torch.float32, "beta")
+        if mlp:
+            t["W1"] = _need(L["W1"], (H, d, m), torch.float32, "W1")
+            t["b1"] = _need(L["b1"], (H, m), torch.float32, "b1")
+            t["W2"] = _need(L["W2"], (H, m, d), torch.float32, "W2")
+            t["b2"] = _need(L["b2"], (H, d), torch.float32, "b2")
+            st = [torch.empty((B, H, d, m), **f32), torch.empty((B, H, m), **f32), torch.empty((B, H, m, d), **f32),
+                  torch.empty((B, H, d), **f32)]
+        else:
+            t["W1"] = _need(L["W0"], (H, d, d), torch.float32, "W0")
+            t["b1"] = _need(L["b0"], (H, d), torch.float32, "b0")
+            st = [torch.empty((B, H, d, d), **f32), torch.empty((B, H, d), **f32)]
+        keep.append(t)
+        states.append(st)
+        a = arr[i]
+        a.kind = 1 if mlp else 0
+        for k in ("pq", "pk", "pv", "W1", "b1", "lr", "gamma", "beta"):
+            setattr(a, k, t[k].data_ptr())
+        a.W2 = t["W2"].data_ptr() if mlp else None
+        a.b2 = t["b2"].data_ptr() if mlp else None
+        a.W1_out, a.b1_out = st[0].data_ptr(), st[1].data_ptr()
+        a.W2_out = st[2].data_ptr() if mlp else None
+        a.b2_out = st[3].data_ptr() if mlp else None
+    nbytes = lib().ttt_stack_fwd_workspace_bytes(C.byref(desc))
+    if nbytes < 0:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, lib().ttt_last_error().decode())
+    if workspace is None:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    elif workspace.numel() * workspace.element_size() < nbytes:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, "workspace too small")
+    out = torch.empty((B, H, seq, d), dtype=io, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_stack_fwd(C.byref(desc), len(layers), arr, _ptr(te), _ptr(out), _ptr(workspace), stream))
+    return out, states
+
+
 # --------------------------------------------------------------------------- either side of the inner loop
 def rope_cos_sin(seq_len: int, offset: int, wrap: Optional[int], head_dim: int, device, base: float = 10000.0):
     """RotaryEmbeddingConfig::init + RotaryEmbedding::get_cos_sin (rust/core/src/util.rs:266-322) in f32:
