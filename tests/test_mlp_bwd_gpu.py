@@ -98,3 +98,27 @@ def test_mlp_inner_model_backward_from_parameters(P):
     for k in GRADS:
         assert_close(got[k], ref[k], 1e-4, k)
     assert_close(got["d_W1"].sum(0), ref["d_W1"].sum(0), 1e-4, "parameter grad W1")
+
+
+def test_mlp_bwd_d128_is_deterministic(P):
+    """head_dim 128 is the variant at the register limit (the read-modify-write passes over the state prefetch one
+    job ahead in a second register set).  Nothing in it may depend on timing: the same call twice gives the same
+    bits in every output written by plain stores (the three outputs accumulated with floating-point atomics over
+    units are compared to 1e-5)."""
+    print("case mlp bwd d128 determinism", flush=True)
+    B, H, d, K, N = 2, 2, 128, 16, 3
+    for dtype in (torch.float32, torch.bfloat16):
+        c = mlp_case(P, 640, B, H, N * K, d, K, dtype, "ref")
+        dv = to_dev(c)
+        g = torch.Generator().manual_seed(13)
+        dO = torch.randn(B, H, N * K, d, generator=g).to(dtype).to("cuda:0")
+        runs = []
+        for _ in range(3):
+            runs.append(P.ttt_mlp_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
+                                               dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], dO, K))
+            torch.cuda.synchronize()
+        for r in runs[1:]:
+            for k in ("d_xq", "d_xk", "d_xv", "d_W1", "d_b1", "d_W2", "d_b2", "d_lr"):
+                assert torch.equal(r[k], runs[0][k]), (k, dtype)
+            for k in ("d_token_eta", "d_gamma", "d_beta"):
+                assert_close(r[k], runs[0][k].double().cpu().numpy(), 1e-5, k)

@@ -367,6 +367,28 @@ def test_mlp_backward_equals_autograd_through_dual(B, H, N, d, K, state_grads):
 
 
 # ------------------------------------------------------------------ either side of the inner loop
+def test_rope_frequencies_are_the_textbook_geometric_ladder():
+    """inv_freq[i] = base^(-2i/d) (RotaryEmbeddingConfig::init, rust/core/src/util.rs:270-275), checked at values
+    worked out by hand rather than by the formula: with base 10^4 and d = 64 the ladder is 10^(-i/8), so frequency
+    8 is 0.1, 16 is 0.01, 24 is 0.001 and the last (31) is 10^-3.875; with d = 16 frequency 4 is 0.01 and 2 is 0.1.
+    A wrong exponent (i/d instead of 2i/d), a wrong base or a ladder laid out over d instead of d/2 entries fails."""
+    import importlib
+    mirror = importlib.import_module("ttt-rs_amd").rope_cos_sin
+    for d, marks in ((64, {0: 1.0, 8: 0.1, 16: 0.01, 24: 0.001, 31: 1.333521432163324e-4}),
+                     (16, {0: 1.0, 2: 0.1, 4: 0.01, 7: 10.0 ** -3.5})):
+        cos, sin = orc.rope_cos_sin(6, 0, None, d)
+        assert cos.shape == (6, d // 2)
+        mc, ms = mirror(6, 0, None, d, "cpu")
+        for i, f in marks.items():
+            for pos in (1, 3, 5):
+                # the tables hold cos / sin of the f32 product pos * f32(inv_freq): 1e-6 relative to the angle
+                assert abs(cos[pos, i] - np.cos(pos * f)) <= 2e-6 and abs(sin[pos, i] - np.sin(pos * f)) <= 2e-6
+                assert abs(float(mc[pos, i]) - np.cos(pos * f)) <= 2e-6 and abs(float(ms[pos, i]) - np.sin(pos * f)) <= 2e-6
+    # wrap: position 21 with wrap 16 is position 5
+    cw, sw = orc.rope_cos_sin(1, 21, 16, 64)
+    assert abs(cw[0, 8] - np.cos(0.5)) <= 2e-6 and abs(sw[0, 8] - np.sin(0.5)) <= 2e-6
+
+
 def test_rope_is_complex_rotation_of_adjacent_pairs():
     """permute_qk -> rotate_half RoPE -> undo_permute_qk (ttt.rs:26-41, util.rs:349-392) is a rotation
     of the adjacent pairs (x[2i], x[2i+1]) by the angle pos * inv_freq[i]."""

@@ -242,6 +242,21 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
 // as k = 4g + r; with X (LDS, contiguous along k, row stride x_rs) read 16 bytes per lane as the matching A operand,
 // four more instructions per tile give the wave its complete columns of Z: the separate pass over C that the
 // product would need is saved.  Z (row stride ldz) is written once at the end.
+//
+// Ordering, as written (two named register sets s0 / s1 in ping-pong):
+//   * every job is one C tile row x NB tile columns and belongs to exactly one wave (job % NW), so no two waves
+//     ever touch the same element of C, and a lane reads and writes only its own elements of a tile;
+//   * a wave requests job n+1 into the idle set, then finishes job n (products, stores); the two jobs are different
+//     tiles, so the loads of n+1 and the stores of n never alias;
+//   * past its last job a wave requests that last job once more into the idle set, only so that the loop body is
+//     the same on every trip; that load may be overtaken by the last job's own stores, and nothing reads it.
+// So the result does not depend on how loads and stores of one wave interleave.  A variant that kept the sets in
+// an array indexed by the trip parity (`Set s[2]`) gave wrong head_dim-128 gradients that differed from run to run,
+// while the same array with three sets and this two-named-sets form never did.  Reading finds no ordering problem
+// in that source either; what differs is that the indexed array is not promoted to registers at 256 VGPRs (the
+// sets then live in per-lane scratch memory and are addressed with the loop-carried parity), i.e. the failure was
+// in code generated for that form, which is why it is not used.  The head_dim-128 instance (256 VGPRs, a handful of
+// registers spilled outside the loops) is held by a test that runs it three times and asks for identical bits.
 template <int MODE, int NW, int NB, int KS, bool FZ = false>
 __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                         int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
