@@ -180,13 +180,18 @@ def run_workload(name, a, pkg, torch):
             layers.append({k: v.to(dev) for k, v in cl.items()})
 
         stack = [dict(L, pq=L["xq"], pk=L["xk"], pv=L["xv"]) for L in layers]
-        nws = pkg.lib().ttt_stack_fwd_workspace_bytes(
-            __import__("ctypes").byref(pkg.TttDesc(B, H, seq, d, K, 1e-6, 1, pkg.TTT_BF16 if io == "bf16" else pkg.TTT_F32)))
+        # wavefront over sequence windows: layer l + 1 works on a window as soon as layer l has left it, windows
+        # that are ready together share a launch, and with --stack-streams 2 the TTT-MLP launches run beside the
+        # TTT-Linear ones (--stack-chunk 0: one launch per layer, one after the other)
+        chunk = a.stack_chunk
+        aux = torch.cuda.Stream(dev) if (chunk and a.stack_streams > 1) else None
+        nws = pkg.ttt_stack_workspace_bytes(B, H, seq, d, K, dtype, [li >= 6 for li in range(8)], chunk)
         ws = torch.empty(nws, dtype=torch.uint8, device=dev)
 
         def step():
-            # one call: per layer the input sums (x read once for xq, xk, xv) and the layer's inner loop
-            return (pkg.ttt_stack_forward_raw(stack, layers[0]["token_eta"], K, workspace=ws)[0],)
+            # one call: per layer and window the input sums (x read once for xq, xk, xv) and the inner loop
+            return (pkg.ttt_stack_forward_raw(stack, layers[0]["token_eta"], K, workspace=ws, chunk_tokens=chunk,
+                                              aux_stream=aux)[0],)
     elif kind in ("inner_inputs", "layer_epilogue"):
         g = torch.Generator().manual_seed(1234 + w["cfg"])
         rn = lambda *sh: torch.randn(*sh, generator=g).to(dtype).to(dev)
@@ -350,8 +355,11 @@ def run_workload(name, a, pkg, torch):
         out["config"]["inner_model"] = "6 x TTT-Linear + 2 x TTT-MLP"
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": BF16_MFMA_PEAK_TF,
                            "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / BF16_MFMA_PEAK_TF, **counters,
-                           "kernel": "ttt_stack_fwd: 8 layer launches + 7 input-sum passes (whole step)",
+                           "kernel": "ttt_stack_fwd: 8 layers x %d sequence windows, windows of a diagonal in one launch per kind, %d stream(s) (whole step)"
+                                     % (seq // a.stack_chunk if a.stack_chunk else 1, 2 if (a.stack_chunk and a.stack_streams > 1) else 1),
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
+        out["config"]["stack_chunk_tokens"] = a.stack_chunk
+        out["config"]["stack_streams"] = 2 if (a.stack_chunk and a.stack_streams > 1) else 1
     if not a.no_cpu_baseline and c is not None:
         out["cpu_baseline"] = cpu_baseline(c, K, kind)
     return out
@@ -371,6 +379,8 @@ def main():
     ap.add_argument("--checkpoint-interval", type=int, default=1)
     ap.add_argument("--checkpoint-format", default="packed", choices=["packed", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--stack-chunk", type=int, default=1024, help="stack workload: tokens per wavefront window (0: none)")
+    ap.add_argument("--stack-streams", type=int, default=2, choices=[1, 2], help="stack workload: 2 = TTT-MLP launches on a second stream")
     ap.add_argument("--no-extra", action="store_true", help="default run: only the forward, not the fwd+bwd entries")
     a = ap.parse_args()
     if a.gpus != 1:

@@ -231,18 +231,35 @@ int ttt_mlp_bwd_static(const ttt_desc* desc, const void* xq, const void* xk, con
  * followed by two TTT-MLP layers): layer l runs its inner loop on
  *     xq = x + pq_l,  xk = x + pk_l,  xv = x + pv_l      (x = output of layer l-1; layer 0: x = 0)
  * where the sums are formed in f32 and rounded to io_dtype, and hands its output to layer l+1; the last layer's
- * output is `out`.  One call enqueues everything: per layer one pass that forms the three sums (x is read once
- * for all three) and the layer's ttt_linear_fwd / ttt_mlp_fwd launch, with desc (shape, eps, io_dtype,
- * kernel_hint) shared by all layers and token_eta [mini_batch] shared too.  The reference has no single
- * counterpart: it reaches the same chaining through one inner-model call per layer from its layer loop, and keeps
- * a layer's kernel resident between calls in its streaming variant
- * (rust/fused/src/linear_fused_tile/streaming/d2d/kernel.rs:98-232).
+ * output is `out`.  One call enqueues everything: per layer and hand-over window one pass that forms the three
+ * sums (x is read once for all three) and the layer's ttt_linear_fwd / ttt_mlp_fwd launch, with desc (shape, eps,
+ * io_dtype, kernel_hint) shared by all layers and token_eta [mini_batch] shared too.
+ *
+ * Cross-layer wavefront.  A layer needs only tokens [0, t) of the layer below to process its own tokens [0, t),
+ * and one launch of a long-context shape fills a fraction of the GPU (a (batch, head) unit is one or two
+ * workgroups), so layers can run side by side: with chunk_tokens = c > 0 (a multiple of mini_batch that divides
+ * seq) every layer works window by window of c tokens, carrying its state from window to window, and window j of
+ * layer l is ready as soon as window j of layer l-1 and window j-1 of layer l are done.  The windows with
+ * l + j = t (a diagonal) are independent of each other; those of one kind go in ONE launch (up to eight
+ * argument blocks travel as kernel arguments and a workgroup picks its own), diagonal after diagonal, and so do
+ * their input sums.  aux_stream = NULL: everything on `stream`, in that order, with no events.  aux_stream = a second
+ * caller-owned stream (default priority, not the null stream): the TTT-MLP launches go there and run beside
+ * the TTT-Linear launches, ordered by events where a layer follows a layer of the other kind; `stream` is joined
+ * to it at the start and at the end, so for the caller the call is still one piece of work on `stream`.
+ * chunk_tokens = 0: one launch per layer on `stream`, bit-identical to calling ttt_linear_fwd / ttt_mlp_fwd layer
+ * by layer.  This is what the reference's streaming kernels are for (a layer's kernel stays resident and is fed
+ * window by window, rust/fused/src/linear_fused_tile/streaming/d2d/kernel.rs:98-232), done with ordinary launches
+ * in dependency order instead of a resident kernel polling a host-visible flag.
+ * Results do not depend on the plan beyond the last bits (a layer splits its state into row means and the rest at
+ * the start of every launch, see ttt_linear_fwd, so windows round differently from one long launch).
  *
  * kind: TTT_LAYER_LINEAR uses W1 = weight_init [H,d,d] (or [B,H,d,d]), b1 = bias_init; TTT_LAYER_MLP uses W1, b1,
  * W2, b2 as ttt_mlp_fwd does (state_per_batch selects the leading dimension).  W1_out .. b2_out receive the
  * layer's final state per batch element (Linear: W1_out [B,H,d,d], b1_out [B,H,d]; the other two unused).
- * workspace: ttt_stack_fwd_workspace_bytes(desc) bytes, 16-byte aligned, caller-owned, free again when the
- * call's work on `stream` has finished (the three input tensors of the current layer and two hand-over tensors).
+ * workspace: ttt_stack_fwd_workspace_bytes(...) bytes for the same plan, 16-byte aligned, caller-owned, free again
+ * when the call's work on `stream` has finished (three tensors of input sums; with a wavefront also one spare
+ * copy of every layer's state).  `out` doubles as the hand-over tensor between layers:
+ * it holds intermediate layers' outputs while the call runs.
  * checkpoint fields of desc are ignored (forward only); seq_stride must be 0.
  */
 #define TTT_LAYER_LINEAR 0
@@ -255,9 +272,11 @@ typedef struct ttt_stack_layer {
   const float *gamma, *beta; /* [H,d] */
   float *W1_out, *b1_out, *W2_out, *b2_out;
 } ttt_stack_layer;
-int64_t ttt_stack_fwd_workspace_bytes(const ttt_desc* desc);
+int64_t ttt_stack_fwd_workspace_bytes(const ttt_desc* desc, int32_t n_layers, const ttt_stack_layer* layers,
+                                      int32_t chunk_tokens);
 int ttt_stack_fwd(const ttt_desc* desc, int32_t n_layers, const ttt_stack_layer* layers /* host memory */,
-                  const float* token_eta, void* out, void* workspace, void* stream);
+                  const float* token_eta, void* out, void* workspace, int32_t chunk_tokens,
+                  void* aux_stream /* hipStream_t or NULL */, void* stream);
 
 /*
  * The elementwise work either side of the inner loop, one HBM-bound pass each (the GEMMs of the

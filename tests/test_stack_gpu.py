@@ -121,3 +121,91 @@ def test_config4_stack_chain_full_size(P):
         print(f"  layer {n - 1}: free-running max-norm relative difference {rel:.3e}", flush=True)
         x_gpu = sub.cpu()
     assert_close(sub, free[0], 3 * tol, "last layer, free-running chain", min_frac=0.99)
+
+
+def rel_max(a, b):
+    a, b = a.double(), b.double()
+    return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("d,chunk,n_aux", [(64, 32, 1), (64, 64, 0), (64, 16, 1), (64, 16, 0), (128, 32, 1), (128, 16, 0),
+                                           (32, 32, 1), (96, 32, 0)])
+def test_small_stack_wavefront(P, dtype, d, chunk, n_aux):
+    """Sequence windows, with and without the second stream: same results as one launch per layer (each window
+    re-centres and re-rounds the carried state once, so the bar is a tight tolerance, not bit equality), same bar
+    against the oracle, and the same bits on a second call (a missing wait would show as a difference)."""
+    B, H, K, seq = 2, 2, 16, 128
+    kinds = [False, True, False, False, True]
+    print(f"case stack wavefront small {dtype} d {d} chunk {chunk} streams {n_aux}", flush=True)
+    layers = make_layers(P, B, H, seq, d, K, dtype, kinds, seed0=90)
+    dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    te = dl[0]["token_eta"]
+    aux = torch.cuda.Stream("cuda:0") if n_aux else None
+    plain, plain_st = P.ttt_stack_forward_raw(dl, te, K)
+    wave, wave_st = P.ttt_stack_forward_raw(dl, te, K, chunk_tokens=chunk, aux_stream=aux)
+    again, again_st = P.ttt_stack_forward_raw(dl, te, K, chunk_tokens=chunk, aux_stream=aux)
+    torch.cuda.synchronize()
+    assert torch.equal(wave, again)
+    for a, b in zip(wave_st, again_st):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+    tol = TOL[dtype]
+    # against the plain plan: differences come from one more rounding of the state per window (f32) and from the
+    # bf16 roundings of outputs that those perturb (bf16)
+    assert rel_max(wave, plain) <= (2e-5 if dtype == torch.float32 else tol)
+    for a, b in zip(wave_st, plain_st):
+        for x, y in zip(a, b):
+            assert rel_max(x, y) <= (2e-5 if dtype == torch.float32 else tol)
+    # against the oracle, layer by layer on the input the GPU produced
+    bs, hs = [0, 1], [0, 1]
+    x_gpu = None
+    for n in range(1, len(kinds) + 1):
+        out, states = P.ttt_stack_forward_raw(dl[:n], te, K, chunk_tokens=chunk, aux_stream=aux)
+        torch.cuda.synchronize()
+        ref = oracle_layer(layers[n - 1], None if x_gpu is None else to_np(x_gpu), bs, hs, K, dtype)
+        assert_close(out, ref[0], tol, f"layer {n - 1} out")
+        for g, r, nm in zip(states[n - 1], ref[1:], ("W1", "b1", "W2", "b2")):
+            f32_products = dtype == torch.float32
+            assert_close(g, r, 1e-4 if f32_products else tol, f"layer {n - 1} {nm}", min_frac=0.999 if f32_products else 0.99)
+        x_gpu = out.cpu()
+
+
+def test_stack_wavefront_rejects_bad_plans(P):
+    B, H, d, K, seq = 1, 2, 64, 16, 64
+    layers = make_layers(P, B, H, seq, d, K, torch.bfloat16, [False, True], seed0=95)
+    dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    aux = torch.cuda.Stream("cuda:0")
+    for bad in (24, 48, 128):   # not a multiple of the mini-batch; not a divisor of seq; longer than seq
+        with pytest.raises(P.TttError):
+            P.ttt_stack_forward_raw(dl, dl[0]["token_eta"], K, chunk_tokens=bad, aux_stream=aux)
+    torch.cuda.synchronize()
+
+
+def test_config4_stack_wavefront_full_size(P):
+    """The long-context stack as bench.py runs it (windows of 1024 tokens, TTT-MLP launches on a second stream)
+    against the plain plan on all 64 units, at the bf16 bar widened for depth as in the chain test, and bit-equal
+    on a second call."""
+    B, H, d, K, seq = 4, 16, 128, 16, 8192
+    kinds = [False] * 6 + [True] * 2
+    dtype = torch.bfloat16
+    print("case stack config 4 wavefront (chunk 1024, 2 streams)", flush=True)
+    layers = make_layers(P, B, H, seq, d, K, dtype, kinds)
+    dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    te = dl[0]["token_eta"]
+    aux = torch.cuda.Stream("cuda:0")
+    plain, plain_st = P.ttt_stack_forward_raw(dl, te, K)
+    wave, wave_st = P.ttt_stack_forward_raw(dl, te, K, chunk_tokens=1024, aux_stream=aux)
+    again, _ = P.ttt_stack_forward_raw(dl, te, K, chunk_tokens=1024, aux_stream=aux)
+    torch.cuda.synchronize()
+    assert torch.isfinite(wave.float()).all()
+    assert torch.equal(wave, again)
+    tol = TOL[dtype]
+    r = rel_max(wave, plain)
+    print(f"  wavefront vs plain, last layer output: max-norm relative difference {r:.3e}", flush=True)
+    assert r <= 3 * tol
+    for li, (a, b) in enumerate(zip(wave_st, plain_st)):
+        for x, y, nm in zip(a, b, ("W1", "b1", "W2", "b2")):
+            rr = rel_max(x, y)
+            print(f"  layer {li} {nm}: {rr:.3e}", flush=True)
+            assert rr <= 3 * tol, (li, nm, rr)

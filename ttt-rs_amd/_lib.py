@@ -71,9 +71,9 @@ def lib() -> C.CDLL:
         L.ttt_mlp_bwd_workspace_bytes.restype = C.c_int64
         L.ttt_mlp_bwd.argtypes = [dp] + [vp] * 29
         L.ttt_mlp_bwd_static.argtypes = [dp] + [vp] * 28
-        L.ttt_stack_fwd_workspace_bytes.argtypes = [dp]
+        L.ttt_stack_fwd_workspace_bytes.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), C.c_int32]
         L.ttt_stack_fwd_workspace_bytes.restype = C.c_int64
-        L.ttt_stack_fwd.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), vp, vp, vp, vp]
+        L.ttt_stack_fwd.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), vp, vp, vp, C.c_int32, vp, vp]
         L.ttt_inner_inputs.argtypes = [dp] + [vp] * 5 + [C.c_float] + [vp] * 4 + [C.c_int, C.c_int] + [vp] * 6
         L.ttt_layer_epilogue.argtypes = [dp] + [vp] * 3 + [C.c_float] + [vp] * 3
         _lib = L

@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <atomic>
+#include <vector>
 
 #include "ttt_engine_fwd.hip.h"
 #include "ttt_layer_io.hip.h"
@@ -64,40 +65,51 @@ int hip_status(hipError_t e, const char* what) {
   return fail(TTT_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// up to ttt::kMaxProblems argument blocks as one kernel argument (unused slots zero)
+template <class A>
+ttt::Problems<A> pack_of(const A* probs, unsigned n) {
+  ttt::Problems<A> P{};
+  for (unsigned i = 0; i < n && i < (unsigned)ttt::kMaxProblems; ++i) P.p[i] = probs[i];
+  return P;
+}
+
 // ---- TTT-Linear forward, head_dim 32/64: kernel choice --------------------------------------
 // A (batch, head) unit is a strictly sequential chain of mini-batches, so the launch is latency
 // bound until there are more units than SIMDs.  Few units: split each unit over several waves
 // (skewed workgroup kernel).  Many units: one wave per unit (no exchange at all).
 // desc.kernel_hint (low byte) = 1 | 2 | 4 overrides the number of waves per unit (tuning / tests).
 template <class T, int D, int NW>
-int launch_linear_fwd_nw(const ttt::LinearFwdArgs& a, hipStream_t s) {
+int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s) {
+  const ttt::LinearFwdArgs& a = probs[0];
+  const auto P = pack_of(probs, ny);
   // mini-batches prefetched ahead, in registers (f32 fragments are twice as large: the one-wave f32 kernel, which
   // holds the whole state and all rows in one wave, has registers for one mini-batch ahead only)
   constexpr int PF = (NW == 1 && sizeof(typename ttt::Io<T>::elem) == 4) ? 1 : 2;
-  const dim3 grid((unsigned)(a.B * a.H)), block(64 * NW);
+  const dim3 grid((unsigned)(a.B * a.H), ny), block(64 * NW);
   if constexpr (NW == 1) {
     if (a.K == 16)
-      hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, true>), grid, block, 0, s, a);
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, true>), grid, block, 0, s, P);
     else
-      hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, false>), grid, block, 0, s, a);
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, false>), grid, block, 0, s, P);
   } else {
     constexpr int NWS = NW > 1 ? NW : 2;  // the skewed kernel needs at least two waves
     if (a.K == 16)
-      hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true>), grid, block, 0, s, a);
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true>), grid, block, 0, s, P);
     else
-      hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, false>), grid, block, 0, s, a);
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, false>), grid, block, 0, s, P);
   }
   return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
 }
 
 template <class T, int D>
-int launch_linear_fwd(const ttt::LinearFwdArgs& a, int waves_hint, hipStream_t s) {
+int launch_linear_fwd(const ttt::LinearFwdArgs* probs, int waves_hint, unsigned ny, hipStream_t s) {
+  const ttt::LinearFwdArgs& a = probs[0];
   constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
   // bf16 I/O: one or two waves per unit.  A four-wave bf16 variant (one feature tile per wave) is not offered: it
   // was never faster than two, and its output LayerNorm came out wrong for one mini-batch in three of the
   // branch-free passes (the k = 16 matrix instruction that adds the causal correction onto the k = 32 products).
   constexpr int max_nw = f32 ? D / 16 : (D / 16 < 2 ? D / 16 : 2);
-  const long units = (long)a.B * a.H;
+  const long units = (long)a.B * a.H * ny;
   int nw = waves_hint;
   if (nw <= 0) {
     // measured on MI355X (256 CUs x 4 SIMDs): bf16 is VALU-latency bound and likes 2 waves per unit
@@ -109,26 +121,28 @@ int launch_linear_fwd(const ttt::LinearFwdArgs& a, int waves_hint, hipStream_t s
   }
   if (nw > max_nw) nw = max_nw;
   if constexpr (max_nw >= 4) {
-    if (nw >= 4) return launch_linear_fwd_nw<T, D, 4>(a, s);
+    if (nw >= 4) return launch_linear_fwd_nw<T, D, 4>(probs, ny, s);
   }
-  if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(a, s);
-  return launch_linear_fwd_nw<T, D, 1>(a, s);
+  if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(probs, ny, s);
+  return launch_linear_fwd_nw<T, D, 1>(probs, ny, s);
 }
 
 // ---- TTT-Linear forward, head_dim 96/128: the same register-resident skewed kernel with two
 // feature tiles per wave (3 waves at d = 96, 4 at d = 128; one tile per wave was measured slower for
 // every shape tried: twice the waves exchange twice the row sums).  The LDS-tile kernel stays
-// available through TTT_LINEAR_FWD_KERNEL=lds.
+// available through TTT_HINT_LDS_TILES.
 template <class T, int D>
-int launch_linear_fwd_wide(const ttt::LinearFwdArgs& a, hipStream_t s) {
+int launch_linear_fwd_wide(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s) {
+  const ttt::LinearFwdArgs& a = probs[0];
+  const auto P = pack_of(probs, ny);
   constexpr int NW = D / 32;
   constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
   constexpr int PF = f32 ? 1 : 2;  // f32 fragments are twice as large: prefetch one mini-batch ahead
-  const dim3 grid((unsigned)(a.B * a.H)), block(64 * NW);
+  const dim3 grid((unsigned)(a.B * a.H), ny), block(64 * NW);
   if (a.K == 16)
-    hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, true>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, true>), grid, block, 0, s, P);
   else
-    hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, false>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, false>), grid, block, 0, s, P);
   return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
 }
 
@@ -150,58 +164,76 @@ int opt_in_lds(size_t bytes) {
 }
 
 template <class T, int D>
-int launch_linear_fwd_lds(const ttt::LinearFwdArgs& a, hipStream_t s) {
+int launch_linear_fwd_lds(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s) {
+  const ttt::LinearFwdArgs& a = probs[0];
   constexpr auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D>;
   constexpr size_t bytes = ttt::LinFwdLds<D>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(256), bytes, s, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H), ny), dim3(256), bytes, s, pack_of(probs, ny));
   return hip_status(hipGetLastError(), "ttt_linear_fwd (LDS kernel) launch");
 }
 
 template <class T, int D>
-int launch_mlp_fwd(const ttt::MlpFwdArgs& a, hipStream_t s) {
+int launch_mlp_fwd(const ttt::MlpFwdArgs* probs, unsigned ny, hipStream_t s) {
+  const ttt::MlpFwdArgs& a = probs[0];
   constexpr auto kern = ttt::ttt_mlp_fwd_kernel<T, D>;
   constexpr size_t bytes = ttt::MlpLds<D>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H), ny), dim3(512), bytes, s, pack_of(probs, ny));
   return hip_status(hipGetLastError(), "ttt_mlp_fwd launch");
 }
 
 // register-resident kernel (d <= 96, bf16 operands on the matrix cores)
 template <class T, int D>
-int launch_mlp_fwd_rr(const ttt::MlpFwdArgs& a, hipStream_t s) {
+int launch_mlp_fwd_rr(const ttt::MlpFwdArgs* probs, unsigned ny, hipStream_t s) {
+  const ttt::MlpFwdArgs& a = probs[0];
   constexpr auto kern = ttt::ttt_mlp_fwd_rr_kernel<T, D>;
   constexpr size_t bytes = ttt::MlpRrLds<D, sizeof(typename ttt::Io<T>::elem)>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H), ny), dim3(512), bytes, s, pack_of(probs, ny));
   return hip_status(hipGetLastError(), "ttt_mlp_fwd (register-resident kernel) launch");
 }
 
 // head_dim 128, bf16 I/O: a pair of workgroups per (batch, head); the exchange flags live in W2_out,
-// which is zeroed first (a fill kernel, not a memset node)
-int launch_mlp_fwd_cl2(ttt::MlpFwdArgs a, hipStream_t s) {
+// which is zeroed first (a fill kernel, not a memset node).
+// The two workgroups of a pair wait for each other, so both must be resident: a workgroup fills a CU (LDS,
+// registers), hence no launch may hold more workgroups than the device has CUs.  The units are independent, so
+// more units than that go in several launches on the stream.  Several problems travel together while they fit
+// that limit, otherwise one after the other.
+int launch_mlp_fwd_cl2(const ttt::MlpFwdArgs* probs, int n, hipStream_t s) {
   constexpr auto kern = ttt::ttt_mlp_fwd_cl2_kernel<ttt::BF16, 128>;
   constexpr size_t bytes = ttt::MlpCl2Lds<128, 2>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  const size_t units = (size_t)a.B * a.H, n = units * 128 * 512;
-  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a.W2, n);
-  // The two workgroups of a pair wait for each other, so both must be resident: a workgroup fills a CU (LDS,
-  // registers), hence no launch may hold more workgroups than the device has CUs.  The units are independent, so
-  // more units than that go in several launches on the stream.
   int dev = 0, cus = 0;
   rc = hip_status(hipGetDevice(&dev), "hipGetDevice");
   if (rc != TTT_OK) return rc;
   rc = hip_status(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute(CU count)");
   if (rc != TTT_OK) return rc;
+  const size_t units = (size_t)probs[0].B * probs[0].H, nz = units * 128 * 512;
+  for (int p = 0; p < n; ++p)
+    hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, s, probs[p].W2, nz);
   const size_t per_launch = (size_t)(cus / 16 > 0 ? cus / 16 : 1) * 8;  // groups of 16 workgroups = 8 units
-  for (size_t base = 0; base < units; base += per_launch) {
-    const size_t cnt = units - base < per_launch ? units - base : per_launch;
-    a.unit_base = (int)base;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(((cnt + 7) / 8) * 16)), dim3(512), bytes, s, a);
+  const size_t wg_per_problem = ((units + 7) / 8) * 16;
+  int together = (int)((size_t)cus / wg_per_problem);  // whole problems that fit the device at once
+  if (together > ttt::kMaxProblems) together = ttt::kMaxProblems;
+  for (int p = 0; p < n;) {
+    if (together >= 2 && n - p >= 2) {
+      const int cnt = n - p < together ? n - p : together;
+      hipLaunchKernelGGL(kern, dim3((unsigned)wg_per_problem, (unsigned)cnt), dim3(512), bytes, s, pack_of(probs + p, (unsigned)cnt));
+      p += cnt;
+      continue;
+    }
+    ttt::MlpFwdArgs a = probs[p];
+    for (size_t base = 0; base < units; base += per_launch) {
+      const size_t cnt = units - base < per_launch ? units - base : per_launch;
+      a.unit_base = (int)base;
+      hipLaunchKernelGGL(kern, dim3((unsigned)(((cnt + 7) / 8) * 16)), dim3(512), bytes, s, pack_of(&a, 1));
+    }
+    ++p;
   }
   return hip_status(hipGetLastError(), "ttt_mlp_fwd (two-CU kernel) launch");
 }
@@ -380,10 +412,10 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   fa.state_per_batch = d->state_per_batch ? 1 : 0;
   fa.eps = d->eps;
   switch (d->head_dim) {
-    case 32: rc = f32 ? launch_mlp_fwd<ttt::F32, 32>(fa, s) : launch_mlp_fwd<ttt::BF16, 32>(fa, s); break;
-    case 64: rc = f32 ? launch_mlp_fwd<ttt::F32, 64>(fa, s) : launch_mlp_fwd<ttt::BF16, 64>(fa, s); break;
-    case 96: rc = f32 ? launch_mlp_fwd<ttt::F32, 96>(fa, s) : launch_mlp_fwd<ttt::BF16, 96>(fa, s); break;
-    default: rc = f32 ? launch_mlp_fwd<ttt::F32, 128>(fa, s) : launch_mlp_fwd<ttt::BF16, 128>(fa, s); break;
+    case 32: rc = f32 ? launch_mlp_fwd<ttt::F32, 32>(&fa, 1, s) : launch_mlp_fwd<ttt::BF16, 32>(&fa, 1, s); break;
+    case 64: rc = f32 ? launch_mlp_fwd<ttt::F32, 64>(&fa, 1, s) : launch_mlp_fwd<ttt::BF16, 64>(&fa, 1, s); break;
+    case 96: rc = f32 ? launch_mlp_fwd<ttt::F32, 96>(&fa, 1, s) : launch_mlp_fwd<ttt::BF16, 96>(&fa, 1, s); break;
+    default: rc = f32 ? launch_mlp_fwd<ttt::F32, 128>(&fa, 1, s) : launch_mlp_fwd<ttt::BF16, 128>(&fa, 1, s); break;
   }
   if (rc != TTT_OK) return rc;
 
@@ -439,10 +471,15 @@ int64_t ttt_linear_num_checkpoints(const ttt_desc* d) {
   return (n + d->checkpoint_interval - 1) / d->checkpoint_interval;
 }
 
-int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
-                   const float* W0, const float* b0, const float* token_eta, const void* lr,
-                   const float* gamma, const float* beta, void* out, float* W_out, float* b_out,
-                   float* W_ckpt, float* b_ckpt, void* stream) {
+}  // extern "C"
+
+namespace {
+// ttt_linear_fwd in two steps, so that a caller with several problems of one shape (ttt_stack_fwd) can check and
+// describe each and launch them together: the argument block, then the launch of n of them.
+int prepare_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv, const float* W0,
+                       const float* b0, const float* token_eta, const void* lr, const float* gamma,
+                       const float* beta, void* out, float* W_out, float* b_out, float* W_ckpt, float* b_ckpt,
+                       ttt::LinearFwdArgs* pa) {
   int rc = ttt_linear_supported(d);
   if (rc != TTT_OK) return rc;
   if (!xq || !xk || !xv || !W0 || !b0 || !token_eta || !lr || !gamma || !beta || !out || !W_out || !b_out)
@@ -451,7 +488,7 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
     return fail(TTT_ERR_NULL, "W_ckpt and b_ckpt must both be given or both be NULL");
   if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(out))
     return fail(TTT_ERR_SHAPE, "xq/xk/xv/out must be 16-byte aligned");
-  ttt::LinearFwdArgs a;
+  ttt::LinearFwdArgs& a = *pa;
   a.xq = xq; a.xk = xk; a.xv = xv; a.W0 = W0; a.b0 = b0; a.token_eta = token_eta; a.lr = lr;
   a.gamma = gamma; a.beta = beta; a.out = out; a.W_out = W_out; a.b_out = b_out;
   a.W_ckpt = W_ckpt; a.b_ckpt = b_ckpt;
@@ -463,26 +500,53 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.state_per_batch = d->state_per_batch ? 1 : 0;
   a.ckpt_packed = (W_ckpt != nullptr && d->checkpoint_format == TTT_CKPT_PACKED) ? 1 : 0;
   a.eps = d->eps;
-  const int waves_hint = d->kernel_hint & TTT_HINT_WAVES_MASK;
   // the LDS-tile forward exists for head_dim 96/128 only; elsewhere the hint names no kernel and is ignored
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
   if (a.ckpt_packed && (d->checkpoint_interval != 1 || want_lds))
     return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+  return TTT_OK;
+}
+
+int dispatch_linear_fwd_pack(const ttt_desc* d, const ttt::LinearFwdArgs* a, unsigned ny, hipStream_t s) {
+  const int waves_hint = d->kernel_hint & TTT_HINT_WAVES_MASK;
+  const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
   const bool f32 = d->io_dtype == TTT_F32;
   switch (d->head_dim) {
-    case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, waves_hint, s) : launch_linear_fwd<ttt::BF16, 32>(a, waves_hint, s);
-    case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, waves_hint, s) : launch_linear_fwd<ttt::BF16, 64>(a, waves_hint, s);
+    case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, waves_hint, ny, s) : launch_linear_fwd<ttt::BF16, 32>(a, waves_hint, ny, s);
+    case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, waves_hint, ny, s) : launch_linear_fwd<ttt::BF16, 64>(a, waves_hint, ny, s);
     default: break;
   }
   if (want_lds) {
     if (d->head_dim == 96)
-      return f32 ? launch_linear_fwd_lds<ttt::F32, 96>(a, s) : launch_linear_fwd_lds<ttt::BF16, 96>(a, s);
-    return f32 ? launch_linear_fwd_lds<ttt::F32, 128>(a, s) : launch_linear_fwd_lds<ttt::BF16, 128>(a, s);
+      return f32 ? launch_linear_fwd_lds<ttt::F32, 96>(a, ny, s) : launch_linear_fwd_lds<ttt::BF16, 96>(a, ny, s);
+    return f32 ? launch_linear_fwd_lds<ttt::F32, 128>(a, ny, s) : launch_linear_fwd_lds<ttt::BF16, 128>(a, ny, s);
   }
   if (d->head_dim == 96)
-    return f32 ? launch_linear_fwd_wide<ttt::F32, 96>(a, s) : launch_linear_fwd_wide<ttt::BF16, 96>(a, s);
-  return f32 ? launch_linear_fwd_wide<ttt::F32, 128>(a, s) : launch_linear_fwd_wide<ttt::BF16, 128>(a, s);
+    return f32 ? launch_linear_fwd_wide<ttt::F32, 96>(a, ny, s) : launch_linear_fwd_wide<ttt::BF16, 96>(a, ny, s);
+  return f32 ? launch_linear_fwd_wide<ttt::F32, 128>(a, ny, s) : launch_linear_fwd_wide<ttt::BF16, 128>(a, ny, s);
+}
+
+// n problems of one shape: kMaxProblems per launch
+int dispatch_linear_fwd(const ttt_desc* d, const ttt::LinearFwdArgs* probs, int n, hipStream_t s) {
+  for (int p = 0; p < n; p += ttt::kMaxProblems) {
+    const int cnt = n - p < ttt::kMaxProblems ? n - p : ttt::kMaxProblems;
+    const int rc = dispatch_linear_fwd_pack(d, probs + p, (unsigned)cnt, s);
+    if (rc != TTT_OK) return rc;
+  }
+  return TTT_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                   const float* W0, const float* b0, const float* token_eta, const void* lr,
+                   const float* gamma, const float* beta, void* out, float* W_out, float* b_out,
+                   float* W_ckpt, float* b_ckpt, void* stream) {
+  ttt::LinearFwdArgs a;
+  int rc = prepare_linear_fwd(d, xq, xk, xv, W0, b0, token_eta, lr, gamma, beta, out, W_out, b_out, W_ckpt, b_ckpt, &a);
+  if (rc != TTT_OK) return rc;
+  return dispatch_linear_fwd(d, &a, 1, static_cast<hipStream_t>(stream));
 }
 
 int ttt_linear_bwd_supported(const ttt_desc* d) {
@@ -582,11 +646,14 @@ int ttt_mlp_supported(const ttt_desc* d) {
   return TTT_OK;
 }
 
-int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
-                const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
-                const float* token_eta, const void* lr, const float* gamma, const float* beta,
-                void* out, float* W1_out, float* b1_out, float* W2_out, float* b2_out,
-                void* stream) {
+}  // extern "C"
+
+namespace {
+// ttt_mlp_fwd in the same two steps as the Linear forward.
+int prepare_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv, const float* W1_0,
+                    const float* b1_0, const float* W2_0, const float* b2_0, const float* token_eta, const void* lr,
+                    const float* gamma, const float* beta, void* out, float* W1_out, float* b1_out, float* W2_out,
+                    float* b2_out, ttt::MlpFwdArgs* pa) {
   int rc = ttt_mlp_supported(d);
   if (rc != TTT_OK) return rc;
   if (!xq || !xk || !xv || !W1_0 || !b1_0 || !W2_0 || !b2_0 || !token_eta || !lr || !gamma || !beta ||
@@ -594,7 +661,7 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
     return fail(TTT_ERR_NULL, "ttt_mlp_fwd: a required pointer is NULL");
   if (W1_out == W1_0 || W2_out == W2_0)
     return fail(TTT_ERR_SHAPE, "ttt_mlp_fwd: W1_out/W2_out are the live state and must not alias W1_0/W2_0");
-  ttt::MlpFwdArgs a;
+  ttt::MlpFwdArgs& a = *pa;
   a.xq = xq; a.xk = xk; a.xv = xv; a.W1_0 = W1_0; a.b1_0 = b1_0; a.W2_0 = W2_0; a.b2_0 = b2_0;
   a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
   a.W1 = W1_out; a.b1 = b1_out; a.W2 = W2_out; a.b2 = b2_out;
@@ -605,25 +672,53 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   a.n_stages = d->seq / d->mini_batch;
   a.state_per_batch = d->state_per_batch ? 1 : 0;
   a.eps = d->eps;
-  hipStream_t s = static_cast<hipStream_t>(stream);
+  return TTT_OK;
+}
+
+int dispatch_mlp_fwd_pack(const ttt_desc* d, const ttt::MlpFwdArgs* a, unsigned ny, hipStream_t s) {
   const bool f32 = d->io_dtype == TTT_F32;
-  // bf16 I/O, d <= 96: the state fits the register file of one CU; d = 128: of two.  TTT_HINT_LDS_TILES forces
-  // the LDS-tile kernel (f32 products, state in global memory) that the other cases use.
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0;
-  if (!f32 && d->head_dim == 128 && !want_lds) return launch_mlp_fwd_cl2(a, s);
   if (!f32 && d->head_dim <= 96 && !want_lds) {
     switch (d->head_dim) {
-      case 32: return launch_mlp_fwd_rr<ttt::BF16, 32>(a, s);
-      case 64: return launch_mlp_fwd_rr<ttt::BF16, 64>(a, s);
-      default: return launch_mlp_fwd_rr<ttt::BF16, 96>(a, s);
+      case 32: return launch_mlp_fwd_rr<ttt::BF16, 32>(a, ny, s);
+      case 64: return launch_mlp_fwd_rr<ttt::BF16, 64>(a, ny, s);
+      default: return launch_mlp_fwd_rr<ttt::BF16, 96>(a, ny, s);
     }
   }
   switch (d->head_dim) {
-    case 32: return f32 ? launch_mlp_fwd<ttt::F32, 32>(a, s) : launch_mlp_fwd<ttt::BF16, 32>(a, s);
-    case 64: return f32 ? launch_mlp_fwd<ttt::F32, 64>(a, s) : launch_mlp_fwd<ttt::BF16, 64>(a, s);
-    case 96: return f32 ? launch_mlp_fwd<ttt::F32, 96>(a, s) : launch_mlp_fwd<ttt::BF16, 96>(a, s);
-    default: return f32 ? launch_mlp_fwd<ttt::F32, 128>(a, s) : launch_mlp_fwd<ttt::BF16, 128>(a, s);
+    case 32: return f32 ? launch_mlp_fwd<ttt::F32, 32>(a, ny, s) : launch_mlp_fwd<ttt::BF16, 32>(a, ny, s);
+    case 64: return f32 ? launch_mlp_fwd<ttt::F32, 64>(a, ny, s) : launch_mlp_fwd<ttt::BF16, 64>(a, ny, s);
+    case 96: return f32 ? launch_mlp_fwd<ttt::F32, 96>(a, ny, s) : launch_mlp_fwd<ttt::BF16, 96>(a, ny, s);
+    default: return f32 ? launch_mlp_fwd<ttt::F32, 128>(a, ny, s) : launch_mlp_fwd<ttt::BF16, 128>(a, ny, s);
   }
+}
+
+int dispatch_mlp_fwd(const ttt_desc* d, const ttt::MlpFwdArgs* probs, int n, hipStream_t s) {
+  // bf16 I/O, d <= 96: the state fits the register file of one CU; d = 128: of two.  TTT_HINT_LDS_TILES forces
+  // the LDS-tile kernel (f32 products, state in global memory) that the other cases use.
+  const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0;
+  if (d->io_dtype != TTT_F32 && d->head_dim == 128 && !want_lds) return launch_mlp_fwd_cl2(probs, n, s);
+  for (int p = 0; p < n; p += ttt::kMaxProblems) {
+    const int cnt = n - p < ttt::kMaxProblems ? n - p : ttt::kMaxProblems;
+    const int rc = dispatch_mlp_fwd_pack(d, probs + p, (unsigned)cnt, s);
+    if (rc != TTT_OK) return rc;
+  }
+  return TTT_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                void* out, float* W1_out, float* b1_out, float* W2_out, float* b2_out,
+                void* stream) {
+  ttt::MlpFwdArgs a;
+  int rc = prepare_mlp_fwd(d, xq, xk, xv, W1_0, b1_0, W2_0, b2_0, token_eta, lr, gamma, beta, out, W1_out, b1_out,
+                           W2_out, b2_out, &a);
+  if (rc != TTT_OK) return rc;
+  return dispatch_mlp_fwd(d, &a, 1, static_cast<hipStream_t>(stream));
 }
 
 int64_t ttt_mlp_bwd_workspace_bytes(const ttt_desc* d) {
@@ -666,78 +761,228 @@ int ttt_mlp_bwd_static(const ttt_desc* d, const void* xq, const void* xk, const 
                       d_token_eta, d_gamma, d_beta, ws, stream);
 }
 
-int64_t ttt_stack_fwd_workspace_bytes(const ttt_desc* d) {
-  if (check_common(d) != TTT_OK) return -1;
-  const int64_t es = d->io_dtype == TTT_BF16 ? 2 : 4;
-  const int64_t tensor = (((int64_t)d->batch * d->heads * d->seq * d->head_dim * es) + 255) / 256 * 256;
-  return 5 * tensor;
-}
+}  // extern "C"
 
-int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* layers, const float* token_eta,
-                  void* out, void* workspace, void* stream) {
+namespace {
+// How a ttt_stack_fwd call is laid out.  Windows (l, j) = layer l on tokens [j*chunk, (j+1)*chunk); window (l, j)
+// needs (l-1, j) and (l, j-1), so the windows of a diagonal l + j = t are independent.
+struct StackPlan {
+  int chunk, chunks;
+  size_t tensor;                  // bytes of one [B,H,seq,d] activation tensor, rounded up to 256
+  std::vector<size_t> state_off;  // byte offset of layer l's spare state copy (more than one window only)
+  int n_lin, n_mlp;               // windows of the two kinds
+  size_t total;
+};
+int plan_stack(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* layers, int32_t chunk_tokens, StackPlan* p) {
   int rc = check_common(d);
   if (rc != TTT_OK) return rc;
   if (n_layers <= 0) return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: n_layers must be positive (got %d)", n_layers);
-  if (!layers || !token_eta || !out || !workspace)
-    return fail(TTT_ERR_NULL, "ttt_stack_fwd: a required pointer is NULL");
+  if (!layers) return fail(TTT_ERR_NULL, "ttt_stack_fwd: layers is NULL");
   if (d->seq_stride != 0 && d->seq_stride != d->seq)
     return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: sequence windows (seq_stride) are not supported");
+  if (chunk_tokens < 0) return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: negative chunk_tokens");
+  const int chunk = chunk_tokens == 0 ? d->seq : chunk_tokens;
+  if (chunk % d->mini_batch != 0 || d->seq % chunk != 0)
+    return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: chunk_tokens (%d) must be a multiple of mini_batch (%d) that divides seq (%d)",
+                chunk, d->mini_batch, d->seq);
+  p->n_lin = p->n_mlp = 0;
+  for (int l = 0; l < n_layers; ++l) {
+    if (layers[l].kind != TTT_LAYER_LINEAR && layers[l].kind != TTT_LAYER_MLP)
+      return fail(TTT_ERR_UNSUPPORTED, "ttt_stack_fwd: layer %d has kind %d", l, layers[l].kind);
+    rc = layers[l].kind == TTT_LAYER_LINEAR ? ttt_linear_supported(d) : ttt_mlp_supported(d);
+    if (rc != TTT_OK) return rc;
+    (layers[l].kind == TTT_LAYER_LINEAR ? p->n_lin : p->n_mlp) += d->seq / chunk;
+  }
+  p->chunk = chunk;
+  p->chunks = d->seq / chunk;
+  const size_t es = d->io_dtype == TTT_BF16 ? 2 : 4;
+  const size_t D = d->head_dim, U = (size_t)d->batch * d->heads, M = 4 * D;
+  auto up = [](size_t n) { return (n + 255) / 256 * 256; };
+  p->tensor = up(U * d->seq * D * es);
+  size_t off = 3 * p->tensor;
+  p->state_off.assign(n_layers, 0);
+  if (p->chunks > 1) {
+    for (int l = 0; l < n_layers; ++l) {
+      p->state_off[l] = off;
+      const size_t floats = layers[l].kind == TTT_LAYER_MLP ? U * (2 * D * M + M + D) : U * (D * D + D);
+      off += up(floats * sizeof(float));
+    }
+  }
+  p->total = off;
+  return TTT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t ttt_stack_fwd_workspace_bytes(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* layers,
+                                      int32_t chunk_tokens) {
+  StackPlan p;
+  if (plan_stack(d, n_layers, layers, chunk_tokens, &p) != TTT_OK) return -1;
+  return (int64_t)p.total;
+}
+
+int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* layers, const float* token_eta,
+                  void* out, void* workspace, int32_t chunk_tokens, void* aux_stream, void* stream) {
+  StackPlan p;
+  int rc = plan_stack(d, n_layers, layers, chunk_tokens, &p);
+  if (rc != TTT_OK) return rc;
+  if (!token_eta || !out || !workspace) return fail(TTT_ERR_NULL, "ttt_stack_fwd: a required pointer is NULL");
   if (!aligned16(workspace) || !aligned16(out)) return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: out and workspace must be 16-byte aligned");
-  // everything is validated before anything is enqueued
+  if (aux_stream != nullptr && aux_stream == stream)
+    return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: aux_stream must differ from stream");
+  const size_t es = d->io_dtype == TTT_BF16 ? 2 : 4;
+  const size_t D = d->head_dim, U = (size_t)d->batch * d->heads, seq = d->seq, M = 4 * D;
+  const int C = p.chunks;
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  unsigned char* sums[3] = {ws, ws + p.tensor, ws + 2 * p.tensor};
+  hipStream_t main_s = static_cast<hipStream_t>(stream);
+  const bool two_lanes = aux_stream != nullptr && p.n_lin > 0 && p.n_mlp > 0;
+  hipStream_t lane_s[2] = {main_s, two_lanes ? static_cast<hipStream_t>(aux_stream) : main_s};
+
+  // ---- pass 1: check and describe every window; nothing is enqueued before all of them are accepted
+  struct Group { int t, kind, first, count, in_first, in_count; bool waits_other; };
+  std::vector<ttt::LinearFwdArgs> lin;
+  std::vector<ttt::MlpFwdArgs> mlp;
+  std::vector<ttt::LayerInputsArgs> ins;
+  std::vector<Group> groups;
   for (int l = 0; l < n_layers; ++l) {
     const ttt_stack_layer& L = layers[l];
-    if (L.kind != TTT_LAYER_LINEAR && L.kind != TTT_LAYER_MLP)
-      return fail(TTT_ERR_UNSUPPORTED, "ttt_stack_fwd: layer %d has kind %d", l, L.kind);
-    rc = L.kind == TTT_LAYER_LINEAR ? ttt_linear_supported(d) : ttt_mlp_supported(d);
-    if (rc != TTT_OK) return rc;
-    const bool mlp = L.kind == TTT_LAYER_MLP;
-    if (!L.pq || !L.pk || !L.pv || !L.W1 || !L.b1 || !L.lr || !L.gamma || !L.beta || !L.W1_out || !L.b1_out ||
-        (mlp && (!L.W2 || !L.b2 || !L.W2_out || !L.b2_out)))
-      return fail(TTT_ERR_NULL, "ttt_stack_fwd: layer %d: a required pointer is NULL", l);
+    if (!L.pq || !L.pk || !L.pv) return fail(TTT_ERR_NULL, "ttt_stack_fwd: layer %d: a required pointer is NULL", l);
     if (!aligned16(L.pq) || !aligned16(L.pk) || !aligned16(L.pv))
       return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: layer %d: pq/pk/pv must be 16-byte aligned", l);
   }
-  ttt_desc ld = *d;
-  ld.seq_stride = 0;
-  ld.checkpoint_interval = 1;
-  ld.checkpoint_format = TTT_CKPT_F32;
-  const size_t es = d->io_dtype == TTT_BF16 ? 2 : 4;
-  const size_t elems = (size_t)d->batch * d->heads * d->seq * d->head_dim;
-  const size_t tensor = (elems * es + 255) / 256 * 256;
-  unsigned char* ws = static_cast<unsigned char*>(workspace);
-  void* xq = ws;
-  void* xk = ws + tensor;
-  void* xv = ws + 2 * tensor;
-  void* hand[2] = {ws + 3 * tensor, ws + 4 * tensor};
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const void* x = nullptr;
-  for (int l = 0; l < n_layers; ++l) {
-    const ttt_stack_layer& L = layers[l];
-    const void *q = L.pq, *k = L.pk, *v = L.pv;
-    if (x != nullptr) {
-      ttt::LayerInputsArgs a;
-      a.x = x; a.pq = L.pq; a.pk = L.pk; a.pv = L.pv; a.xq = xq; a.xk = xk; a.xv = xv;
-      a.n16 = elems * es / 16;
-      const dim3 grid((unsigned)((a.n16 + 255) / 256));
-      if (d->io_dtype == TTT_F32)
-        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::F32>, grid, dim3(256), 0, s, a);
-      else
-        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::BF16>, grid, dim3(256), 0, s, a);
-      rc = hip_status(hipGetLastError(), "ttt_stack_fwd (layer inputs) launch");
-      if (rc != TTT_OK) return rc;
-      q = xq; k = xk; v = xv;
+  for (int t = 0; t < C + n_layers - 1; ++t) {
+    for (int kind = 0; kind < 2; ++kind) {
+      Group g{t, kind, kind == TTT_LAYER_LINEAR ? (int)lin.size() : (int)mlp.size(), 0, (int)ins.size(), 0, false};
+      for (int l = 0; l < n_layers; ++l) {
+        const int j = t - l;
+        const ttt_stack_layer& L = layers[l];
+        if (j < 0 || j >= C || L.kind != kind) continue;
+        const bool is_mlp = kind == TTT_LAYER_MLP;
+        const size_t tok0 = (size_t)j * p.chunk;
+        const size_t woff = tok0 * D * es;  // byte offset of the window inside a unit's rows
+        const unsigned char *q = static_cast<const unsigned char*>(L.pq) + woff, *k = static_cast<const unsigned char*>(L.pk) + woff,
+                            *v = static_cast<const unsigned char*>(L.pv) + woff;
+        unsigned char* ow = static_cast<unsigned char*>(out) + woff;  // `out` is the hand-over tensor too
+        if (l > 0) {
+          // window j of the sums tensors is free: its previous user (l-1, j) is done before this window starts
+          ttt::LayerInputsArgs a;
+          a.x = ow; a.pq = q; a.pk = k; a.pv = v;
+          a.xq = sums[0] + woff; a.xk = sums[1] + woff; a.xv = sums[2] + woff;
+          a.win16 = (size_t)p.chunk * D * es / 16;
+          a.pitch16 = seq * D * es / 16;
+          a.n16 = U * a.win16;
+          ins.push_back(a);
+          ++g.in_count;
+          q = sums[0] + woff; k = sums[1] + woff; v = sums[2] + woff;
+          if (layers[l - 1].kind != kind) g.waits_other = true;
+        }
+        ttt_desc ld = *d;
+        ld.seq = p.chunk;
+        ld.seq_stride = C > 1 ? d->seq : 0;
+        ld.checkpoint_interval = 1;
+        ld.checkpoint_format = TTT_CKPT_F32;
+        // state: window 0 starts from the layer's parameters; window j writes the caller's buffers when the
+        // number of windows still to come is even, the spare copy otherwise; window j + 1 reads what j wrote
+        float* spare = C > 1 ? reinterpret_cast<float*>(ws + p.state_off[l]) : nullptr;
+        float* sp[4] = {spare, nullptr, nullptr, nullptr};
+        if (spare) {
+          sp[1] = is_mlp ? spare + U * D * M : spare + U * D * D;
+          if (is_mlp) {
+            sp[2] = sp[1] + U * M;
+            sp[3] = sp[2] + U * M * D;
+          }
+        }
+        float* user[4] = {L.W1_out, L.b1_out, L.W2_out, L.b2_out};
+        float* const* to = ((C - 1 - j) % 2 == 0) ? user : sp;
+        float* const* from = ((C - j) % 2 == 0) ? user : sp;
+        const float *W1i = L.W1, *b1i = L.b1, *W2i = L.W2, *b2i = L.b2;
+        if (j > 0) {
+          ld.state_per_batch = 1;
+          W1i = from[0]; b1i = from[1]; W2i = from[2]; b2i = from[3];
+        }
+        const unsigned char* lr = L.lr ? static_cast<const unsigned char*>(L.lr) + tok0 * es : nullptr;
+        if (!is_mlp) {
+          ttt::LinearFwdArgs a;
+          rc = prepare_linear_fwd(&ld, q, k, v, W1i, b1i, token_eta, lr, L.gamma, L.beta, ow, to[0], to[1], nullptr, nullptr, &a);
+          if (rc != TTT_OK) return rc;
+          lin.push_back(a);
+        } else {
+          ttt::MlpFwdArgs a;
+          rc = prepare_mlp_fwd(&ld, q, k, v, W1i, b1i, W2i, b2i, token_eta, lr, L.gamma, L.beta, ow, to[0], to[1], to[2], to[3], &a);
+          if (rc != TTT_OK) return rc;
+          mlp.push_back(a);
+        }
+        ++g.count;
+      }
+      if (g.count > 0) groups.push_back(g);
     }
-    void* o = (l == n_layers - 1) ? out : hand[l & 1];
-    if (L.kind == TTT_LAYER_LINEAR)
-      rc = ttt_linear_fwd(&ld, q, k, v, L.W1, L.b1, token_eta, L.lr, L.gamma, L.beta, o, L.W1_out, L.b1_out, nullptr,
-                          nullptr, stream);
-    else
-      rc = ttt_mlp_fwd(&ld, q, k, v, L.W1, L.b1, L.W2, L.b2, token_eta, L.lr, L.gamma, L.beta, o, L.W1_out, L.b1_out,
-                       L.W2_out, L.b2_out, stream);
-    if (rc != TTT_OK) return rc;
-    x = o;
   }
-  return TTT_OK;
+
+  // ---- pass 2: the launches, diagonal by diagonal
+  // events (two lanes only): created here and destroyed before returning; the runtime keeps a recorded event
+  // alive until the work it marks has finished
+  std::vector<hipEvent_t> ev;
+  auto cleanup = [&](int r) {
+    for (hipEvent_t e : ev) (void)hipEventDestroy(e);
+    return r;
+  };
+  auto mark = [&](hipStream_t s, hipEvent_t* e) {
+    int r = hip_status(hipEventCreateWithFlags(e, hipEventDisableTiming), "hipEventCreateWithFlags");
+    if (r != TTT_OK) return r;
+    ev.push_back(*e);
+    return hip_status(hipEventRecord(*e, s), "hipEventRecord");
+  };
+  auto wait = [&](hipStream_t s, hipEvent_t e) { return hip_status(hipStreamWaitEvent(s, e, 0), "hipStreamWaitEvent"); };
+  if (two_lanes) {
+    hipEvent_t fork;
+    if ((rc = mark(main_s, &fork)) != TTT_OK) return cleanup(rc);
+    if ((rc = wait(lane_s[1], fork)) != TTT_OK) return cleanup(rc);
+  }
+  // done[kind][t & 1]: event after the lane's launches of diagonal t (done_t: which diagonal the slot holds)
+  hipEvent_t done[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+  int done_t[2][2] = {{-2, -2}, {-2, -2}};
+  for (const Group& g : groups) {
+    hipStream_t s = lane_s[g.kind];
+    const int other = 1 - g.kind;
+    // a window whose layer below is of the other kind waits for that lane's launches of the previous diagonal
+    // (the lane's later work is in stream order behind them, so its latest event would do as well, but would wait
+    // for more than is needed)
+    if (two_lanes && g.waits_other) {
+      const int slot = (g.t - 1) & 1;
+      if (done_t[other][slot] != g.t - 1) return cleanup(fail(TTT_ERR_SHAPE, "ttt_stack_fwd: internal: missing event of diagonal %d", g.t - 1));
+      if ((rc = wait(s, done[other][slot])) != TTT_OK) return cleanup(rc);
+    }
+    for (int i = 0; i < g.in_count; i += ttt::kMaxProblems) {
+      const unsigned cnt = (unsigned)(g.in_count - i < ttt::kMaxProblems ? g.in_count - i : ttt::kMaxProblems);
+      const ttt::LayerInputsArgs* a = &ins[g.in_first + i];
+      const dim3 grid((unsigned)((a->n16 + 255) / 256), cnt);
+      if (d->io_dtype == TTT_F32)
+        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::F32>, grid, dim3(256), 0, s, pack_of(a, cnt));
+      else
+        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::BF16>, grid, dim3(256), 0, s, pack_of(a, cnt));
+      if ((rc = hip_status(hipGetLastError(), "ttt_stack_fwd (layer inputs) launch")) != TTT_OK) return cleanup(rc);
+    }
+    ttt_desc ld = *d;
+    ld.seq = p.chunk;
+    if (g.kind == TTT_LAYER_LINEAR)
+      rc = dispatch_linear_fwd(&ld, &lin[g.first], g.count, s);
+    else
+      rc = dispatch_mlp_fwd(&ld, &mlp[g.first], g.count, s);
+    if (rc != TTT_OK) return cleanup(rc);
+    if (two_lanes) {
+      if ((rc = mark(s, &done[g.kind][g.t & 1])) != TTT_OK) return cleanup(rc);
+      done_t[g.kind][g.t & 1] = g.t;
+    }
+  }
+  if (two_lanes) {
+    hipEvent_t join;
+    if ((rc = mark(lane_s[1], &join)) != TTT_OK) return cleanup(rc);
+    if ((rc = wait(main_s, join)) != TTT_OK) return cleanup(rc);
+  }
+  return cleanup(TTT_OK);
 }
 
 int ttt_inner_inputs(const ttt_desc* d, const void* xq, const void* xk, const void* xv,

@@ -78,7 +78,8 @@ struct LinFwdLds {
 };
 
 template <class T, int D>
-__global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(LinearFwdArgs a) {
+__global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(Problems<LinearFwdArgs> problems) {
+  const LinearFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = LinFwdLds<D>;
@@ -226,7 +227,8 @@ struct MlpLds {
 
 template <class T, int D>
 // one workgroup per CU (LDS), two waves per SIMD: stated so that the scheduler does not serialise loads to save registers
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) ttt_mlp_fwd_kernel(MlpFwdArgs a) {
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) ttt_mlp_fwd_kernel(Problems<MlpFwdArgs> problems) {
+  const MlpFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = MlpLds<D>;

@@ -250,4 +250,15 @@ __device__ __forceinline__ typename Io<T>::frag splat_frag(float x) {
   return Io<T>::to_frag(f32x4{x, x, x, x});
 }
 
+// A launch may carry several independent problems of one shape, gridDim.y of them (windows of different layers of
+// a stack that are ready at the same time: one layer's 64 units alone leave three quarters of the CUs idle).  The
+// argument blocks of all of them travel as kernel arguments and workgroup (x, y) works on block y: the index is
+// uniform over the workgroup, so the fields are scalar loads from the kernel-argument segment exactly as for a
+// single block.
+constexpr int kMaxProblems = 8;
+template <class A>
+struct Problems {
+  A p[kMaxProblems];
+};
+
 }  // namespace ttt

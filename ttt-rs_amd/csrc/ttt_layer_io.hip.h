@@ -165,16 +165,20 @@ __global__ void __launch_bounds__(256) ttt_layer_epilogue_kernel(LayerEpilogueAr
 // Inputs of one layer of a stack: xq = x + pq, xk = x + pk, xv = x + pv (f32 sums rounded to the I/O type), x read
 // once for all three.  One thread per 16 bytes.
 struct LayerInputsArgs {
-  const void *x, *pq, *pk, *pv;
+  const void *x, *pq, *pk, *pv;  // all pointing at the first token of the window in unit 0
   void *xq, *xk, *xv;
-  size_t n16;  // number of 16-byte chunks per tensor
+  size_t n16;      // number of 16-byte chunks to process: units * win16
+  size_t win16;    // 16-byte chunks of one unit's window
+  size_t pitch16;  // 16-byte chunks between consecutive (batch, head) units
 };
 template <class T>
-__global__ void __launch_bounds__(256) ttt_layer_inputs_kernel(LayerInputsArgs a) {
+__global__ void __launch_bounds__(256) ttt_layer_inputs_kernel(Problems<LayerInputsArgs> problems) {
+  const LayerInputsArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   constexpr int E = 16 / IO::kBytes;  // elements per chunk
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= a.n16) return;
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= a.n16) return;
+  const size_t i = (t / a.win16) * a.pitch16 + t % a.win16;
   const u32x4 rx = static_cast<const u32x4*>(a.x)[i];
   const u32x4 rq = static_cast<const u32x4*>(a.pq)[i], rk = static_cast<const u32x4*>(a.pk)[i],
               rv = static_cast<const u32x4*>(a.pv)[i];

@@ -272,7 +272,8 @@ __device__ __forceinline__ float xg_reduce(float v) {
 }
 
 template <class T, int D, int NW, int PF, bool FULL>
-__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(LinearFwdArgs a) {
+__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<LinearFwdArgs> problems) {
+  const LinearFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;

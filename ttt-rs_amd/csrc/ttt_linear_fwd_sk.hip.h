@@ -18,7 +18,8 @@
 namespace ttt {
 
 template <class T, int D, int NW, int PF, bool FULL>
-__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(LinearFwdArgs a) {
+__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
+  const LinearFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;

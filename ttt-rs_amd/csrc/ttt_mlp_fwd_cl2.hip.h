@@ -109,7 +109,8 @@ __device__ __forceinline__ void recv_tagged(const unsigned long long* const (&sl
 #define RELANE() asm volatile("" : "+v"(lane))
 
 template <class T, int D>
-__global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(MlpFwdArgs a) {
+__global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArgs> problems) {
+  const MlpFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;

@@ -106,7 +106,8 @@ __device__ __forceinline__ float mean_of(const float* p, int d, float inv_d) {
 #define RELANE() asm volatile("" : "+v"(lane))
 
 template <class T, int D>
-__global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(MlpFwdArgs a) {
+__global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(Problems<MlpFwdArgs> problems) {
+  const MlpFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;

@@ -500,10 +500,27 @@ class FusedTileMulti:
         return self._launch(state, inputs.slice_seq(r), len(r))
 
 
+def ttt_stack_workspace_bytes(B: int, H: int, seq: int, d: int, mini_batch: int, io: torch.dtype, mlp_flags,
+                              chunk_tokens: int = 0) -> int:
+    """ttt_stack_fwd_workspace_bytes for a stack whose layer l is TTT-MLP where mlp_flags[l] is true."""
+    desc = TttDesc(B, H, seq, d, mini_batch, 1e-6, 1, _lib.TTT_BF16 if io == torch.bfloat16 else _lib.TTT_F32)
+    arr = (_lib.TttStackLayer * len(mlp_flags))()
+    for a, f in zip(arr, mlp_flags):
+        a.kind = 1 if f else 0
+    n = lib().ttt_stack_fwd_workspace_bytes(C.byref(desc), len(mlp_flags), arr, chunk_tokens)
+    if n < 0:
+        raise _lib.TttError(_lib.TTT_ERR_SHAPE, lib().ttt_last_error().decode())
+    return n
+
+
 def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6, kernel_hint: int = 0,
-                          workspace: Optional[torch.Tensor] = None):
+                          workspace: Optional[torch.Tensor] = None, chunk_tokens: int = 0,
+                          aux_stream: Optional[torch.cuda.Stream] = None):
     """One call of ttt_stack_fwd on the current stream: inner models applied layer by layer, layer l on
     xq = x + pq, xk = x + pk, xv = x + pv with x the previous layer's output (0 for the first layer).
+    chunk_tokens > 0 runs the layers as a wavefront over sequence windows of that many tokens (layer l + 1 works on
+    a window as soon as layer l has left it; windows that are ready together share a launch); aux_stream, a second
+    torch.cuda.Stream, lets the TTT-MLP launches run beside the TTT-Linear ones.
     layers: list of dicts with pq, pk, pv [B,H,seq,d], lr [B,H,seq], gamma, beta [H,d] and either W0, b0
     (TTT-Linear) or W1, b1, W2, b2 (TTT-MLP), parameters [H,..].  Returns (out, states) with states[l] the final
     state tensors of layer l (per batch element)."""
@@ -546,7 +563,7 @@ def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6,
         a.W1_out, a.b1_out = st[0].data_ptr(), st[1].data_ptr()
         a.W2_out = st[2].data_ptr() if mlp else None
         a.b2_out = st[3].data_ptr() if mlp else None
-    nbytes = lib().ttt_stack_fwd_workspace_bytes(C.byref(desc))
+    nbytes = lib().ttt_stack_fwd_workspace_bytes(C.byref(desc), len(layers), arr, chunk_tokens)
     if nbytes < 0:
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, lib().ttt_last_error().decode())
     if workspace is None:
@@ -556,7 +573,11 @@ def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6,
     out = torch.empty((B, H, seq, d), dtype=io, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     with torch.cuda.device(dev):
-        check(lib().ttt_stack_fwd(C.byref(desc), len(layers), arr, _ptr(te), _ptr(out), _ptr(workspace), stream))
+        check(lib().ttt_stack_fwd(C.byref(desc), len(layers), arr, _ptr(te), _ptr(out), _ptr(workspace),
+                                  chunk_tokens, C.c_void_p(aux_stream.cuda_stream) if aux_stream is not None else None,
+                                  stream))
+    # aux_stream reads and writes tensors that torch's allocator ties to the current stream only; the call joins
+    # it into the current stream before it returns, so later work on that stream is ordered after it
     return out, states
 
 
