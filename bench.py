@@ -379,7 +379,7 @@ def main():
     ap.add_argument("--checkpoint-interval", type=int, default=1)
     ap.add_argument("--checkpoint-format", default="packed", choices=["packed", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--stack-chunk", type=int, default=1024, help="stack workload: tokens per wavefront window (0: none)")
+    ap.add_argument("--stack-chunk", type=int, default=2048, help="stack workload: tokens per wavefront window (0: none)")
     ap.add_argument("--stack-streams", type=int, default=2, choices=[1, 2], help="stack workload: 2 = TTT-MLP launches on a second stream")
     ap.add_argument("--no-extra", action="store_true", help="default run: only the forward, not the fwd+bwd entries")
     a = ap.parse_args()

@@ -767,7 +767,8 @@ namespace {
 // How a ttt_stack_fwd call is laid out.  Windows (l, j) = layer l on tokens [j*chunk, (j+1)*chunk); window (l, j)
 // needs (l-1, j) and (l, j-1), so the windows of a diagonal l + j = t are independent.
 struct StackPlan {
-  int chunk, chunks;
+  int chunks;                     // number of windows
+  std::vector<int> tok0, len;     // first token and length of every window
   size_t tensor;                  // bytes of one [B,H,seq,d] activation tensor, rounded up to 256
   std::vector<size_t> state_off;  // byte offset of layer l's spare state copy (more than one window only)
   int n_lin, n_mlp;               // windows of the two kinds
@@ -791,10 +792,18 @@ int plan_stack(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* layer
       return fail(TTT_ERR_UNSUPPORTED, "ttt_stack_fwd: layer %d has kind %d", l, layers[l].kind);
     rc = layers[l].kind == TTT_LAYER_LINEAR ? ttt_linear_supported(d) : ttt_mlp_supported(d);
     if (rc != TTT_OK) return rc;
-    (layers[l].kind == TTT_LAYER_LINEAR ? p->n_lin : p->n_mlp) += d->seq / chunk;
   }
-  p->chunk = chunk;
-  p->chunks = d->seq / chunk;
+  // Windows of `chunk` tokens.  (Splitting the first window so that the upper layers start sooner was measured
+  // and did not pay: the two-CU TTT-MLP kernel at the top of the benchmark stack bounds the call, and more
+  // windows cost it more launches.)
+  p->tok0.clear();
+  p->len.clear();
+  for (int t0 = 0; t0 < d->seq; t0 += chunk) {
+    p->tok0.push_back(t0);
+    p->len.push_back(chunk);
+  }
+  p->chunks = (int)p->tok0.size();
+  for (int l = 0; l < n_layers; ++l) (layers[l].kind == TTT_LAYER_LINEAR ? p->n_lin : p->n_mlp) += p->chunks;
   const size_t es = d->io_dtype == TTT_BF16 ? 2 : 4;
   const size_t D = d->head_dim, U = (size_t)d->batch * d->heads, M = 4 * D;
   auto up = [](size_t n) { return (n + 255) / 256 * 256; };
@@ -842,10 +851,16 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
   hipStream_t lane_s[2] = {main_s, two_lanes ? static_cast<hipStream_t>(aux_stream) : main_s};
 
   // ---- pass 1: check and describe every window; nothing is enqueued before all of them are accepted
-  struct Group { int t, kind, first, count, in_first, in_count; bool waits_other; };
+  // A group = the windows of one kind on one diagonal.  before / after: input sums launched ahead of the group's
+  // kernels (for its own windows) and behind them (for windows of the other kind on the next diagonal whose layer
+  // below is in this group: formed on the producer's stream, they are off the consumer's).
+  struct Group {
+    int t, kind, first, count;
+    bool waits_other;
+    std::vector<ttt::LayerInputsArgs> before, after;
+  };
   std::vector<ttt::LinearFwdArgs> lin;
   std::vector<ttt::MlpFwdArgs> mlp;
-  std::vector<ttt::LayerInputsArgs> ins;
   std::vector<Group> groups;
   for (int l = 0; l < n_layers; ++l) {
     const ttt_stack_layer& L = layers[l];
@@ -855,13 +870,13 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
   }
   for (int t = 0; t < C + n_layers - 1; ++t) {
     for (int kind = 0; kind < 2; ++kind) {
-      Group g{t, kind, kind == TTT_LAYER_LINEAR ? (int)lin.size() : (int)mlp.size(), 0, (int)ins.size(), 0, false};
+      Group g{t, kind, kind == TTT_LAYER_LINEAR ? (int)lin.size() : (int)mlp.size(), 0, false, {}, {}};
       for (int l = 0; l < n_layers; ++l) {
         const int j = t - l;
         const ttt_stack_layer& L = layers[l];
         if (j < 0 || j >= C || L.kind != kind) continue;
         const bool is_mlp = kind == TTT_LAYER_MLP;
-        const size_t tok0 = (size_t)j * p.chunk;
+        const size_t tok0 = (size_t)p.tok0[j];
         const size_t woff = tok0 * D * es;  // byte offset of the window inside a unit's rows
         const unsigned char *q = static_cast<const unsigned char*>(L.pq) + woff, *k = static_cast<const unsigned char*>(L.pk) + woff,
                             *v = static_cast<const unsigned char*>(L.pv) + woff;
@@ -871,16 +886,25 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
           ttt::LayerInputsArgs a;
           a.x = ow; a.pq = q; a.pk = k; a.pv = v;
           a.xq = sums[0] + woff; a.xk = sums[1] + woff; a.xv = sums[2] + woff;
-          a.win16 = (size_t)p.chunk * D * es / 16;
+          a.win16 = (size_t)p.len[j] * D * es / 16;
           a.pitch16 = seq * D * es / 16;
           a.n16 = U * a.win16;
-          ins.push_back(a);
-          ++g.in_count;
           q = sums[0] + woff; k = sums[1] + woff; v = sums[2] + woff;
-          if (layers[l - 1].kind != kind) g.waits_other = true;
+          if (layers[l - 1].kind != kind) {
+            g.waits_other = true;
+            // the producer's group: the other kind on the previous diagonal (it holds window (l-1, j), so it exists
+            // and is one of the last two groups pushed)
+            Group* prod = nullptr;
+            for (size_t i = groups.size(); i-- > 0 && groups[i].t >= t - 1;)
+              if (groups[i].t == t - 1 && groups[i].kind != kind) prod = &groups[i];
+            if (prod == nullptr) return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: internal: no group for window (%d, %d)", l - 1, j);
+            (two_lanes ? prod->after : g.before).push_back(a);
+          } else {
+            g.before.push_back(a);
+          }
         }
         ttt_desc ld = *d;
-        ld.seq = p.chunk;
+        ld.seq = p.len[j];
         ld.seq_stride = C > 1 ? d->seq : 0;
         ld.checkpoint_interval = 1;
         ld.checkpoint_format = TTT_CKPT_F32;
@@ -941,6 +965,20 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
     if ((rc = mark(main_s, &fork)) != TTT_OK) return cleanup(rc);
     if ((rc = wait(lane_s[1], fork)) != TTT_OK) return cleanup(rc);
   }
+  auto input_sums = [&](const std::vector<ttt::LayerInputsArgs>& v, hipStream_t s) {
+    for (size_t i = 0; i < v.size(); i += ttt::kMaxProblems) {
+      const unsigned cnt = (unsigned)(v.size() - i < (size_t)ttt::kMaxProblems ? v.size() - i : (size_t)ttt::kMaxProblems);
+      const ttt::LayerInputsArgs* a = &v[i];
+      size_t n16 = 0;  // the grid covers the longest window, threads past the end of a shorter one exit
+      for (unsigned k = 0; k < cnt; ++k) n16 = a[k].n16 > n16 ? a[k].n16 : n16;
+      const dim3 grid((unsigned)((n16 + 255) / 256), cnt);
+      if (d->io_dtype == TTT_F32)
+        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::F32>, grid, dim3(256), 0, s, pack_of(a, cnt));
+      else
+        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::BF16>, grid, dim3(256), 0, s, pack_of(a, cnt));
+    }
+    return hip_status(hipGetLastError(), "ttt_stack_fwd (layer inputs) launch");
+  };
   // done[kind][t & 1]: event after the lane's launches of diagonal t (done_t: which diagonal the slot holds)
   hipEvent_t done[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
   int done_t[2][2] = {{-2, -2}, {-2, -2}};
@@ -955,23 +993,15 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
       if (done_t[other][slot] != g.t - 1) return cleanup(fail(TTT_ERR_SHAPE, "ttt_stack_fwd: internal: missing event of diagonal %d", g.t - 1));
       if ((rc = wait(s, done[other][slot])) != TTT_OK) return cleanup(rc);
     }
-    for (int i = 0; i < g.in_count; i += ttt::kMaxProblems) {
-      const unsigned cnt = (unsigned)(g.in_count - i < ttt::kMaxProblems ? g.in_count - i : ttt::kMaxProblems);
-      const ttt::LayerInputsArgs* a = &ins[g.in_first + i];
-      const dim3 grid((unsigned)((a->n16 + 255) / 256), cnt);
-      if (d->io_dtype == TTT_F32)
-        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::F32>, grid, dim3(256), 0, s, pack_of(a, cnt));
-      else
-        hipLaunchKernelGGL(ttt::ttt_layer_inputs_kernel<ttt::BF16>, grid, dim3(256), 0, s, pack_of(a, cnt));
-      if ((rc = hip_status(hipGetLastError(), "ttt_stack_fwd (layer inputs) launch")) != TTT_OK) return cleanup(rc);
-    }
-    ttt_desc ld = *d;
-    ld.seq = p.chunk;
+    if ((rc = input_sums(g.before, s)) != TTT_OK) return cleanup(rc);
+    ttt_desc ld = *d;  // only what chooses the kernel is read from it; the windows' lengths are in the argument blocks
+    ld.seq = d->mini_batch;
     if (g.kind == TTT_LAYER_LINEAR)
       rc = dispatch_linear_fwd(&ld, &lin[g.first], g.count, s);
     else
       rc = dispatch_mlp_fwd(&ld, &mlp[g.first], g.count, s);
     if (rc != TTT_OK) return cleanup(rc);
+    if ((rc = input_sums(g.after, s)) != TTT_OK) return cleanup(rc);
     if (two_lanes) {
       if ((rc = mark(s, &done[g.kind][g.t & 1])) != TTT_OK) return cleanup(rc);
       done_t[g.kind][g.t & 1] = g.t;
