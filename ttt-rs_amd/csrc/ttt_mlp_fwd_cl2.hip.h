@@ -56,11 +56,17 @@ struct MlpCl2Lds {
 };
 
 // One [16 x 16] f32 tile (this lane's four values) as four (value, tag) words.
+// The two workgroups of a pair sit on CUs of one XCD (see the block numbering in the kernel), which share an L2.
+// The stores therefore carry workgroup scope: they leave the CU (its L1 writes through) and stay in that L2, where
+// the partner's device-scope loads, which bypass its own L1, find them.  Device-scope stores would also be written
+// through to memory, every one of them: measured at 2.8 GB of writes per launch of 128 units x 2048 tokens, which
+// made the kernel 40 % slower on a full GPU than on a quarter of it.  Should a pair ever land on two XCDs, its
+// words never arrive, the waits run out and the unit's outputs are NaN (see recv_tagged): loud, not wrong.
 __device__ __forceinline__ void send_tagged(unsigned long long* slot, f32x4 v, unsigned tag) {
 #pragma unroll
   for (int r = 0; r < 4; ++r)
     __hip_atomic_store(slot + r, ((unsigned long long)tag << 32) | __float_as_uint(v[r]), __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
+                       __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 // Receives N tiles at once: polls until the four words of every slot carry that slot's tag, all
 // loads of a round in flight together (one memory round trip per round, not one per tile).  The wait
