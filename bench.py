@@ -281,7 +281,7 @@ def run_workload(name, a, pkg, torch):
                 if traffic is not None else None}
     if mfma_util is not None:
         counters.update(mfma_util=mfma_util, mfma_util_source="profiles/traffic.json (rocprofv3 SQ_VALU_MFMA_BUSY_CYCLES "
-                        "over the cycles of the SIMDs that hold a wave)")
+                        "of the dominant kernel over its traced duration x 2.4 GHz x 1024 SIMDs)")
     if kind == "linear_fwd":
         alg = linear_fwd_bytes(B, H, seq, d, s)
         k_s = part_s["ttt_linear_fwd"]
