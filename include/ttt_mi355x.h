@@ -157,11 +157,13 @@ int ttt_linear_bwd(const ttt_desc* desc, const void* xq, const void* xk, const v
  * [B,H,4d,d], b2_0 [H,d] or [B,H,d] (state_per_batch selects); outputs are per batch element.
  *
  * head_dim 128 with bf16 I/O: a unit's state (512 KiB) is the whole register file of a CU, so a PAIR of
- * workgroups on two CUs shares each unit and exchanges partial results once per mini-batch through global
- * memory.  During the call W2_out is also that exchange area (the library zero-fills it first; its contents are
- * meaningless until the call's work has finished).  The library launches at most as many workgroups at a time as
+ * workgroups on two CUs of one XCD shares each unit and exchanges partial results once per mini-batch through
+ * global memory, in the L2 cache those two CUs share.  During the call W2_out is also that exchange area (the
+ * library zero-fills it first; its contents are meaningless until the call's work has finished); it must be
+ * ordinary device memory (hipMalloc), not fine-grained or host memory.  The library launches at most as many workgroups at a time as
  * the device has CUs, so on a GPU that is not shared both halves of every pair are resident together.  If a
- * workgroup nevertheless waits for its partner in vain (about 0.1 s: CUs held by other processes or streams), the
+ * workgroup nevertheless waits for its partner in vain (2^21 polls, seconds: CUs held by other processes or
+ * streams, or a pair that was not placed on one XCD), the
  * call cannot report it -- it returned TTT_OK when the work was enqueued -- so the failure is made impossible to
  * miss in the data instead: EVERY output of that unit (its rows of out, W1_out, b1_out, W2_out, b2_out) is NaN.
  * A caller that shares the GPU checks one output element per unit, or passes TTT_HINT_LDS_TILES to use the
