@@ -48,10 +48,15 @@ def run_case(P, B, H, d, K, N, dtype, style, state_grads=False, seed=0):
 def test_mlp_bwd_matches_oracle(P, B, H, d, K, N, style, state_grads, dtype):
     print(f"case mlp bwd {style} B{B} H{H} d{d} K{K} N{N} {dtype} state_grads={state_grads}", flush=True)
     got, ref = run_case(P, B, H, d, K, N, dtype, style, state_grads)
-    # arithmetic is f32 for both I/O dtypes; bf16 rounds the stored activation gradients
+    # The reverse scan's arithmetic is f32 for both I/O dtypes; bf16 rounds the stored activation gradients.  With
+    # bf16 I/O up to head_dim 96 the update factors it rolls back and differentiates are those of the bf16-operand
+    # forward (rounded to bf16 as that forward applied them), so every gradient is held to the bf16 bar there;
+    # f32 I/O and head_dim 128 (f32 forward sweep) keep 1e-4 for the gradients stored in f32.
+    bf16_factors = dtype == torch.bfloat16 and d <= 96
     for k in GRADS:
         io_out = k in ("d_xq", "d_xk", "d_xv", "d_lr")
-        assert_close(got[k], ref[k], TOL[dtype] if io_out else 1e-4, k)
+        assert_close(got[k], ref[k], TOL[dtype] if (io_out or bf16_factors) else 1e-4, k,
+                     min_frac=0.99 if bf16_factors else 0.999)
 
 
 def test_mlp_bwd_is_linear_in_upstream_gradient(P):

@@ -399,8 +399,11 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   const bool f32 = d->io_dtype == TTT_F32;
   const size_t U = (size_t)d->batch * d->heads, D = d->head_dim, M = 4 * D;
 
-  // forward sweep with the LDS-tile kernel (f32 products): final state and, per mini-batch, the
-  // rank-16 factors of the state update
+  // forward sweep: final state and, per mini-batch, the rank-16 factors of the state update.  bf16 I/O up to
+  // head_dim 96: the register-resident forward itself (the factors are then the ones the forward of this step
+  // applied, rounded to bf16 as its matrix instructions took them); its output goes to d_xq, which the reverse
+  // scan overwrites afterwards.  Otherwise the LDS-tile kernel (f32 products, no output).
+  const bool rr_sweep = !f32 && d->head_dim <= 96 && !(d->kernel_hint & TTT_HINT_LDS_TILES);
   ttt::MlpFwdArgs fa;
   fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
   fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
@@ -411,6 +414,14 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   fa.n_stages = d->seq / d->mini_batch;
   fa.state_per_batch = d->state_per_batch ? 1 : 0;
   fa.eps = d->eps;
+  if (rr_sweep) {
+    fa.out = d_xq;
+    switch (d->head_dim) {
+      case 32: rc = launch_mlp_fwd_rr<ttt::BF16, 32>(&fa, 1, s); break;
+      case 64: rc = launch_mlp_fwd_rr<ttt::BF16, 64>(&fa, 1, s); break;
+      default: rc = launch_mlp_fwd_rr<ttt::BF16, 96>(&fa, 1, s); break;
+    }
+  } else
   switch (d->head_dim) {
     case 32: rc = f32 ? launch_mlp_fwd<ttt::F32, 32>(&fa, 1, s) : launch_mlp_fwd<ttt::BF16, 32>(&fa, 1, s); break;
     case 64: rc = f32 ? launch_mlp_fwd<ttt::F32, 64>(&fa, 1, s) : launch_mlp_fwd<ttt::BF16, 64>(&fa, 1, s); break;

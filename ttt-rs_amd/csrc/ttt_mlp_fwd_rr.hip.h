@@ -395,6 +395,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(Problems<MlpFwdArgs
     RELANE();
 
     // ================= phase C: reducers: G2'' in both orientations; output waves: store the output
+    frag g2_saved = IO::zero();
     if (red) {
       float S[6];
 #pragma unroll
@@ -415,6 +416,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(Problems<MlpFwdArgs
       IO::mma(t, gt, ident);
       GT[w * 64 + lane] = gt;
       GD[w * 64 + lane] = IO::to_frag(t);
+      g2_saved = gt;
     }
     if (outw && st > 0) output_emit(st - 1);
     // the next mini-batch's rows must have landed before anybody passes B3; the output store just issued
@@ -427,6 +429,15 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(Problems<MlpFwdArgs
     RELANE();
 
     // ================= phase D: G1, Zbar1, Xbar2, split-k partials of the output path, updates
+    // The factors of this mini-batch's state update for ttt_mlp_bwd, eta_last * G1 [16 x 4d] and eta_last * G2
+    // [16 x d] (row = token), exactly as the update applies them: rounded to the operand type, sign undone
+    // (G'' = -eta_last * lr * G); zeros when token_eta[K-1] = 0 switches the update off.  Stored behind B3 so
+    // that the counted waits of phase C see the same memory operations as without them.
+    const size_t save_row = (bh * (size_t)a.n_stages + st) * 16 + c;
+    if (a.G2_save != nullptr && red) {
+      const f32x4 v = upd ? -IO::to_f32(g2_saved) : f32x4{0.f, 0.f, 0.f, 0.f};
+      *reinterpret_cast<f32x4*>(a.G2_save + save_row * D + own) = v;
+    }
 #pragma unroll
     for (int j = 0; j < HT; ++j)
 #pragma unroll
@@ -443,8 +454,13 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_rr_kernel(Problems<MlpFwdArgs
         IO::mma2(acc, IO::to_frag(t0), IO::to_frag(t1), GT[(2 * q) * 64 + lane], GT[(2 * q + 1) * 64 + lane]);
       }
       f32x4 t = {0.f, 0.f, 0.f, 0.f};
-      IO::mma(t, IO::to_frag(acc * dg[j]), ident);
+      const frag g1b = IO::to_frag(acc * dg[j]);
+      IO::mma(t, g1b, ident);
       G1d[j] = IO::to_frag(t);
+      if (a.G1_save != nullptr) {
+        const f32x4 v = upd ? -IO::to_f32(g1b) : f32x4{0.f, 0.f, 0.f, 0.f};
+        *reinterpret_cast<f32x4*>(a.G1_save + save_row * F + 16 * (w * HT + j) + 4 * g) = v;
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     // Zbar1^T = (XQ W1 + b1)^T + G1''^T M1, with M1[s][t] = (token_eta[t] / sc)(1 + A1[t][s]) for s <= t.
