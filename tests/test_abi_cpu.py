@@ -98,6 +98,37 @@ def test_null_pointers_are_rejected_before_any_launch(P):
     assert rc == P.TTT_ERR_NULL
 
 
+def test_stack_plan_is_validated_without_a_gpu(P):
+    """ttt_stack_fwd_workspace_bytes / ttt_stack_fwd check the plan (layer kinds, window length, pointers) before any
+    HIP call: wrong plans answer with an error code here, on a machine without a GPU."""
+    L = P.lib()
+    d = desc(P, batch=1, heads=2, seq=64, head_dim=64, io_dtype=P.TTT_BF16)
+    layers = (P.TttStackLayer * 2)()
+    layers[0].kind, layers[1].kind = 0, 1
+    U, D, M, seq = 2, 64, 256, 64
+    tensor = (U * seq * D * 2 + 255) // 256 * 256
+    assert L.ttt_stack_fwd_workspace_bytes(C.byref(d), 2, layers, 0) == 3 * tensor
+    # with windows: one spare copy of every layer's state as well
+    up = lambda n: (n + 255) // 256 * 256
+    spare = up(U * (D * D + D) * 4) + up(U * (2 * D * M + M + D) * 4)
+    assert L.ttt_stack_fwd_workspace_bytes(C.byref(d), 2, layers, 32) == 3 * tensor + spare
+    for bad in (24, 48, 128, -16):      # not a multiple of mini_batch; not a divisor of seq; longer than seq; negative
+        assert L.ttt_stack_fwd_workspace_bytes(C.byref(d), 2, layers, bad) == -1
+        assert b"chunk_tokens" in L.ttt_last_error()
+    layers[1].kind = 7
+    assert L.ttt_stack_fwd_workspace_bytes(C.byref(d), 2, layers, 0) == -1
+    layers[1].kind = 1
+    assert L.ttt_stack_fwd_workspace_bytes(C.byref(d), 0, layers, 0) == -1
+    # NULL token_eta / out / workspace, then NULL layer tensors: refused before anything is enqueued
+    assert L.ttt_stack_fwd(C.byref(d), 2, layers, None, None, None, 0, None, None) == P.TTT_ERR_NULL
+    dummy = C.create_string_buffer(64)
+    ptr = C.c_void_p((C.addressof(dummy) + 15) // 16 * 16)
+    assert L.ttt_stack_fwd(C.byref(d), 2, layers, ptr, ptr, ptr, 0, None, None) == P.TTT_ERR_NULL
+    assert b"layer 0" in L.ttt_last_error()
+    # the second stream must be a different one
+    assert L.ttt_stack_fwd(C.byref(d), 2, layers, ptr, ptr, ptr, 32, ptr, ptr) == P.TTT_ERR_SHAPE
+
+
 def test_eta_logit_gradient_helper_matches_the_oracle_chain(P):
     """Host logic, no GPU: the chain from grad_ttt_lr_eta to the lr-gate logits (rust/layer/src/ttt.rs:205-227)."""
     import numpy as np
