@@ -172,6 +172,34 @@ def test_small_stack_wavefront(P, dtype, d, seq, chunk, n_aux):
         x_gpu = out.cpu()
 
 
+@pytest.mark.parametrize("kinds,d,seq,chunk,n_aux", [
+    ([False, True, False], 64, 96, 32, 1),      # three windows: the last one writes the caller's state buffers
+    ([True], 64, 96, 32, 1),                    # a single layer, still in windows
+    ([False] * 10, 32, 160, 16, 0),             # ten windows of one kind on a diagonal: two launches (eight per launch)
+    ([True] * 3 + [False] * 9, 32, 160, 16, 1),  # Linear layers above MLP layers, more than eight at once
+], ids=["odd-windows", "one-layer", "ten-linear", "mlp-below-linear"])
+def test_stack_wavefront_plans(P, kinds, d, seq, chunk, n_aux):
+    """Plans the other tests do not reach, against the one-launch-per-layer plan (itself held to the oracle above)."""
+    B, H, K = 1, 2, 16
+    dtype = torch.float32
+    print(f"case stack plan {kinds} d {d} seq {seq} chunk {chunk} streams {n_aux}", flush=True)
+    layers = make_layers(P, B, H, seq, d, K, dtype, kinds, seed0=120)
+    dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    te = dl[0]["token_eta"]
+    aux = torch.cuda.Stream("cuda:0") if n_aux else None
+    plain, plain_st = P.ttt_stack_forward_raw(dl, te, K)
+    wave, wave_st = P.ttt_stack_forward_raw(dl, te, K, chunk_tokens=chunk, aux_stream=aux)
+    again, _ = P.ttt_stack_forward_raw(dl, te, K, chunk_tokens=chunk, aux_stream=aux)
+    torch.cuda.synchronize()
+    assert torch.equal(wave, again)
+    # rounding differences of a layer are inputs of the next: the bar widens with depth
+    bar = 2e-5 * len(kinds)
+    assert rel_max(wave, plain) <= bar
+    for a, b in zip(wave_st, plain_st):
+        for x, y in zip(a, b):
+            assert rel_max(x, y) <= bar
+
+
 def test_stack_wavefront_rejects_bad_plans(P):
     B, H, d, K, seq = 1, 2, 64, 16, 64
     layers = make_layers(P, B, H, seq, d, K, torch.bfloat16, [False, True], seed0=95)
