@@ -166,10 +166,16 @@ int ttt_linear_bwd(const ttt_desc* desc, const void* xq, const void* xk, const v
  * streams, or a pair that was not placed on one XCD), the
  * call cannot report it -- it returned TTT_OK when the work was enqueued -- so the failure is made impossible to
  * miss in the data instead: EVERY output of that unit (its rows of out, W1_out, b1_out, W2_out, b2_out) is NaN.
- * A caller that shares the GPU checks one output element per unit, or passes TTT_HINT_LDS_TILES to use the
- * single-workgroup kernel (slower, f32 products).
+ * A caller that shares the GPU checks one output element per unit, reads the status word below, or passes
+ * TTT_HINT_LDS_TILES to use the single-workgroup kernel (slower, f32 products).
+ *
+ * ttt_mlp_fwd_lost_workgroups: the device's status word of that kernel, the number of workgroups whose wait for
+ * their partner ran out since the library was loaded on the current device (0 on a healthy run; it never
+ * decreases, compare with the value before the call).  A blocking copy from the device: call it after the
+ * stream's work has finished.  No counterpart in the reference.
  */
 int ttt_mlp_supported(const ttt_desc* desc);
+int ttt_mlp_fwd_lost_workgroups(int64_t* count);
 int ttt_mlp_fwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
                 const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
                 const float* token_eta, const void* lr, const float* gamma, const float* beta,

@@ -125,15 +125,25 @@ def test_mlp_fwd_d128_lost_partner_is_loud(P):
     dv = to_dev(c)
     args = (dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"],
             dv["beta"], K)
+    import ctypes
+    def lost_workgroups():
+        n = ctypes.c_int64(-1)
+        P.check(P.lib().ttt_mlp_fwd_lost_workgroups(ctypes.byref(n)))
+        return n.value
+    torch.cuda.synchronize()
+    before = lost_workgroups()
     got = P.ttt_mlp_forward_raw(*args, kernel_hint=P.TTT_HINT_TEST_LOST_PARTNER)
     torch.cuda.synchronize()
     for name, t in zip(("out", "W1", "b1", "W2", "b2"), got):
         assert torch.isnan(t.float()).all(), f"{name}: a lost partner left finite values"
+    # the device's status word counts the workgroups that gave up: both of every pair here
+    assert lost_workgroups() == before + 2 * B * H
     # and the same call without the hook is healthy afterwards (nothing sticky in the library)
     ok = P.ttt_mlp_forward_raw(*args)
     torch.cuda.synchronize()
     for t in ok:
         assert torch.isfinite(t.float()).all()
+    assert lost_workgroups() == before + 2 * B * H
 
 
 def test_mlp_fwd_d128_more_units_than_one_launch(P):

@@ -17,7 +17,7 @@ EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_bwd_supported",
     "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
-    "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue",
+    "ttt_mlp_fwd_lost_workgroups", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue",
 )
 
 
@@ -71,6 +71,7 @@ def lib() -> C.CDLL:
         L.ttt_mlp_bwd_workspace_bytes.restype = C.c_int64
         L.ttt_mlp_bwd.argtypes = [dp] + [vp] * 29
         L.ttt_mlp_bwd_static.argtypes = [dp] + [vp] * 28
+        L.ttt_mlp_fwd_lost_workgroups.argtypes = [C.POINTER(C.c_int64)]
         L.ttt_stack_fwd_workspace_bytes.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), C.c_int32]
         L.ttt_stack_fwd_workspace_bytes.restype = C.c_int64
         L.ttt_stack_fwd.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), vp, vp, vp, C.c_int32, vp, vp]

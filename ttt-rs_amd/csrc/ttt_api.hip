@@ -732,6 +732,16 @@ int ttt_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   return dispatch_mlp_fwd(d, &a, 1, static_cast<hipStream_t>(stream));
 }
 
+int ttt_mlp_fwd_lost_workgroups(int64_t* count) {
+  if (!count) return fail(TTT_ERR_NULL, "ttt_mlp_fwd_lost_workgroups: count is NULL");
+  unsigned int v = 0;
+  int rc = hip_status(hipMemcpyFromSymbol(&v, HIP_SYMBOL(ttt::g_mlp_fwd_lost_workgroups), sizeof(v), 0, hipMemcpyDeviceToHost),
+                      "hipMemcpyFromSymbol(status word)");
+  if (rc != TTT_OK) return rc;
+  *count = (int64_t)v;
+  return TTT_OK;
+}
+
 int64_t ttt_mlp_bwd_workspace_bytes(const ttt_desc* d) {
   if (ttt_mlp_supported(d) != TTT_OK) return -1;
   return (int64_t)(MlpBwdWs(d).total * sizeof(float));

@@ -112,6 +112,10 @@ __device__ __forceinline__ void recv_tagged(const unsigned long long* const (&sl
                    __uint_as_float((unsigned)wd[n][2]), __uint_as_float((unsigned)wd[n][3])};
 }
 
+// Status word of the two-CU kernel: workgroups whose wait for their partner ran out, counted since the library was
+// loaded (one copy per GPU).  Read by ttt_mlp_fwd_lost_workgroups.
+__device__ unsigned int g_mlp_fwd_lost_workgroups = 0u;
+
 #define RELANE() asm volatile("" : "+v"(lane))
 
 template <class T, int D>
@@ -617,6 +621,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArg
       if ((cu == 0 || lost) && c == 0) store4<F32>(a.b2 + bh * D + own, v0 + (b2T - start) + poison);
     }
     if (lost) {
+      if (tid == 0) atomicAdd(&g_mlp_fwd_lost_workgroups, 1u);
       elem* po = static_cast<elem*>(a.out) + bh * (size_t)a.seq_stride * D;
       const size_t n = (size_t)a.n_stages * K * D;
       for (size_t i = tid; i < n; i += 512) IO::store1(po + i, poison);
