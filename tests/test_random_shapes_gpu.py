@@ -1,0 +1,108 @@
+"""GPU parity on seeded random shapes: TTT-Linear forward + backward and TTT-MLP forward through the C ABI against
+the float64 oracle.  The other GPU tests use the reference's own shapes and the benchmark shapes; this one draws
+(batch, heads, head_dim, mini_batch, stages, per-batch state, style of inputs) from a fixed seed, so that shapes
+nobody thought of are covered too (odd head counts, every head_dim with short and long mini-batches, one stage).
+Bars: the max-norm bar of the other tests (1e-4 / 2e-2) for every tensor; the elementwise band on 99.9 % of the
+elements for f32 and on 99 % for bf16 I/O (products with bf16 operands: on these small tensors, mini-batches of one
+token included, a few elements in a thousand leave the band while the max-norm error stays far inside its bar)."""
+import importlib
+import random
+
+import pytest
+import torch
+
+from helpers import TOL, assert_close, np_inputs, to_dev
+from oracle import ttt_oracle as orc
+from test_linear_bwd_gpu import NAMES, compare, oracle_bwd
+from test_mlp_fwd_gpu import mlp_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+def draw(seed, n, dims):
+    rng = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        cs = dict(B=rng.choice([1, 2, 3]), H=rng.choice([1, 2, 3, 5]), d=rng.choice(dims),
+                  K=rng.choice([1, 3, 4, 8, 11, 16]), N=rng.choice([1, 2, 5, 9]),
+                  style=rng.choice(["ref", "baseline"]), seed=rng.randrange(1 << 20))
+        # at least 24 tokens, so that the 99.9 % rule of the elementwise band has more than a few hundred elements to
+        # speak of (in a tensor of 320 bf16 values one element outside the band is already 0.3 %)
+        cs["N"] = max(cs["N"], -(-24 // cs["K"]))
+        cases.append(cs)
+    return cases
+
+
+def linear_inputs(P, cs, dtype):
+    gen = P.synthetic.reference_test_inputs if cs["style"] == "ref" else P.synthetic.baseline_inputs
+    return gen(cs["seed"], cs["B"], cs["H"], cs["N"] * cs["K"], cs["d"], cs["K"], io_dtype=dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("cs", draw(2024, 10, [32, 64, 96, 128]), ids=lambda c: "B{B}H{H}d{d}K{K}N{N}{style}".format(**c))
+def test_linear_forward_random_shape(P, cs, dtype):
+    print(f"case random linear fwd {cs} {dtype}", flush=True)
+    K = cs["K"]
+    c = linear_inputs(P, cs, dtype)
+    d = to_dev(c)
+    out, W, b = P.ttt_linear_forward_raw(d["xq"], d["xk"], d["xv"], d["W0"], d["b0"], d["token_eta"], d["lr"],
+                                         d["gamma"], d["beta"], K)[:3]
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ro, rW, rb = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"], n["gamma"],
+                                    n["beta"], K=K)[:3]
+    tol = TOL[dtype]
+    frac = 0.99 if dtype == torch.bfloat16 else 0.999
+    few = cs["B"] * cs["H"] * cs["d"] < 1000   # one element of a small tensor is already more than 0.1 %
+    assert_close(out, ro, tol, "out", min_frac=frac)
+    assert_close(W, rW, tol, "W", min_frac=frac)
+    assert_close(b, rb, tol, "b", min_frac=0.99 if few else frac)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("cs", draw(7, 8, [32, 64]), ids=lambda c: "B{B}H{H}d{d}K{K}N{N}{style}".format(**c))
+def test_linear_backward_random_shape(P, cs, dtype):
+    print(f"case random linear bwd {cs} {dtype}", flush=True)
+    K = cs["K"]
+    c = linear_inputs(P, cs, dtype)
+    c.pop("d_out", None)
+    g = torch.Generator().manual_seed(cs["seed"] + 1)
+    dO = torch.randn(cs["B"], cs["H"], cs["N"] * K, cs["d"], generator=g).to(dtype)
+    d = to_dev(c)
+    fw = P.ttt_linear_forward_raw(d["xq"], d["xk"], d["xv"], d["W0"], d["b0"], d["token_eta"], d["lr"], d["gamma"],
+                                  d["beta"], K, want_checkpoints=True)
+    got = P.ttt_linear_backward_raw(d["xq"], d["xk"], d["xv"], d["W0"], d["b0"], d["token_eta"], d["lr"], d["gamma"],
+                                    d["beta"], fw[3], fw[4], dO.to("cuda:0"), K)
+    torch.cuda.synchronize()
+    ref = oracle_bwd(c, dO, K)
+    if dtype == torch.float32:
+        compare(got, ref, TOL[dtype])
+    else:
+        import numpy as np
+        for gn, rn in NAMES:
+            n = np.asarray(ref[rn]).size   # in a tensor of 64 elements one element outside the band is 1.6 %
+            assert_close(got[gn], ref[rn], TOL[dtype], gn, min_frac=min(0.99, 1.0 - 1.5 / n))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("cs", draw(99, 6, [32, 64, 96, 128]), ids=lambda c: "B{B}H{H}d{d}K{K}N{N}{style}".format(**c))
+def test_mlp_forward_random_shape(P, cs, dtype):
+    print(f"case random mlp fwd {cs} {dtype}", flush=True)
+    K = cs["K"]
+    c = mlp_case(P, cs["seed"], cs["B"], cs["H"], cs["N"] * K, cs["d"], K, dtype, cs["style"])
+    d = to_dev(c)
+    got = P.ttt_mlp_forward_raw(d["xq"], d["xk"], d["xv"], d["W1"], d["b1"], d["W2"], d["b2"], d["token_eta"], d["lr"],
+                                d["gamma"], d["beta"], K)
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                          n["gamma"], n["beta"], K=K)
+    tol = TOL[dtype]
+    frac = 0.99 if dtype == torch.bfloat16 else 0.999
+    for g, r, nm in zip(got, ref, ("out", "W1", "b1", "W2", "b2")):
+        assert_close(g, r, tol, nm, min_frac=0.99 if nm.startswith("b") else frac)
