@@ -90,6 +90,37 @@ __device__ __forceinline__ void store_ckpt_packed(float* slot, const f32x4 (&Wc)
   }
 }
 
+// Where the next checkpoint of a (batch, head) unit goes and when it is due.  A checkpoint is written before every
+// ckpt_interval-th mini-batch; the slot pointers advance by one checkpoint each time and a counter says how many
+// mini-batches are left until the next one, so the loop needs neither the division st / ckpt_interval nor the
+// products (bh * n_ckpt + st / ckpt_interval) * d * d.
+template <int D>
+struct CkptCursor {
+  float* W;      // next W slot (null: no checkpoints)
+  float* b;      // next b slot
+  int every;     // ckpt_interval
+  int left;      // mini-batches until the next checkpoint (0: due now)
+  bool packed;
+  __device__ __forceinline__ CkptCursor(const LinearFwdArgs& a, size_t bh) {
+    const bool on = a.W_ckpt != nullptr;
+    W = on ? a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D) : nullptr;
+    b = on ? a.b_ckpt + bh * (size_t)a.n_ckpt * D : nullptr;
+    every = on ? a.ckpt_interval : 1;
+    left = 0;
+    packed = a.ckpt_packed != 0;
+  }
+  // true when a checkpoint is due before this mini-batch; call once per mini-batch, then advance() if it was
+  __device__ __forceinline__ bool due() const { return W != nullptr && left == 0; }
+  __device__ __forceinline__ void advance() {
+    W += D * D;
+    b += D;
+    left = every;
+  }
+  __device__ __forceinline__ void next_stage() {
+    if (W != nullptr) --left;
+  }
+};
+
 // ---- State centring -------------------------------------------------------------------------------------------
 // LayerNorm does not see a shift common to all d features of a row, and the inner loop looks at the state only
 // through LayerNorm: Z1 = XK W + b feeds the LN-L2 gradient, Zbar = XQ W + b - (...) G the output LayerNorm.  With
@@ -171,9 +202,8 @@ __device__ __forceinline__ void store_state_f32(float* Wd, float* bd, const f32x
 
 // b = bc + mean(b) alone (the packed W checkpoint keeps the centred matrix; the bias checkpoint is always the true bias).
 template <int D, int TPW>
-__device__ __forceinline__ void store_bias_true(float* bd, const f32x4 (&bT)[TPW], const float* m0s, int w, int c, int g) {
+__device__ __forceinline__ void store_bias_true(float* bd, const f32x4 (&bT)[TPW], float bb, int w, int c, int g) {
   if (c == 0) {
-    const float bb = m0s[D];
 #pragma unroll
     for (int jj = 0; jj < TPW; ++jj) {
       f32x4 v = bT[jj];
@@ -337,6 +367,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
   StageInMw<T, NT, TPW> buf[R];
 #pragma unroll
   for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], a, bh, u, c, g, w);
+  CkptCursor<D> ck(a, bh);
+  const float b_mean = __builtin_amdgcn_readfirstlane(m0s[D]);  // mean of the initial bias (split off by centre_state)
 
   for (int st0 = 0; st0 < a.n_stages; st0 += R) {
 #pragma unroll
@@ -346,16 +378,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
       if (st >= a.n_stages) continue;
       const StageInMw<T, NT, TPW>& cur = buf[u];
 
-      if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
-        const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
-        float* Wd = a.W_ckpt + ci * D * D;
-        if (a.ckpt_packed) {
-          store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
-          store_bias_true<D, TPW>(a.b_ckpt + ci * D, bT, m0s, w, c, g);
+      if (ck.due()) {
+        if (ck.packed) {
+          store_ckpt_packed<T, NT, TPW>(ck.W, Wc, w, lane);
+          store_bias_true<D, TPW>(ck.b, bT, b_mean, w, c, g);
         } else {
-          store_state_f32<D, TPW>(Wd, a.b_ckpt + ci * D, Wc, bT, m0s, w, c, g);
+          store_state_f32<D, TPW>(ck.W, ck.b, Wc, bT, m0s, w, c, g);
         }
+        ck.advance();
       }
+      ck.next_stage();
 
       // ---- Z1^T, Zbar^T (this wave's feature rows) and the attention block
       f32x4 z1[TPW], zb[TPW], At = {0.f, 0.f, 0.f, 0.f};

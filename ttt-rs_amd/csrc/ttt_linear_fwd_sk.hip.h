@@ -164,6 +164,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
   // (pending output, G, state update) and the head of the next (products, moments) -- is one basic block and
   // the compiler can interleave the two dependency chains.
   float ps0 = 0.f, ps1 = 0.f;
+  CkptCursor<D> ck(a, bh);
+  const float b_mean = __builtin_amdgcn_readfirstlane(m0s[D]);  // mean of the initial bias (split off by centre_state)
   auto pass = [&](auto checked_tag, int st0) {
     constexpr bool CHECKED = decltype(checked_tag)::value;
 #pragma unroll
@@ -225,16 +227,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
       }
       // ---- checkpoint of the state entering this mini-batch (W and b change only behind the barrier);
       // placed at the barrier so that its branch does not cut the stretch in two
-      if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
-        const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
-        float* Wd = a.W_ckpt + ci * D * D;
-        if (a.ckpt_packed) {
-          store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
-          store_bias_true<D, TPW>(a.b_ckpt + ci * D, bT, m0s, w, c, g);
+      if (ck.due()) {
+        if (ck.packed) {
+          store_ckpt_packed<T, NT, TPW>(ck.W, Wc, w, lane);
+          store_bias_true<D, TPW>(ck.b, bT, b_mean, w, c, g);
         } else {
-          store_state_f32<D, TPW>(Wd, a.b_ckpt + ci * D, Wc, bT, m0s, w, c, g);
+          store_state_f32<D, TPW>(ck.W, ck.b, Wc, bT, m0s, w, c, g);
         }
+        ck.advance();
       }
+      ck.next_stage();
       exchange8_publish(S, st & 1);
       // ---- the output pending since two mini-batches (sums known since the last exchange): nothing waits
       // for it, and here it runs while this exchange is in flight (LDS write, barrier, LDS read)
@@ -308,16 +310,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
         if (st >= a.n_stages) continue;
         const StageInMw<T, NT, TPW>& cur = buf[u];
 
-        if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
-          const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
-          float* Wd = a.W_ckpt + ci * D * D;
-          if (a.ckpt_packed) {
-            store_ckpt_packed<T, NT, TPW>(Wd, Wc, w, lane);
-            store_bias_true<D, TPW>(a.b_ckpt + ci * D, bT, m0s, w, c, g);
+        if (ck.due()) {
+          if (ck.packed) {
+            store_ckpt_packed<T, NT, TPW>(ck.W, Wc, w, lane);
+            store_bias_true<D, TPW>(ck.b, bT, b_mean, w, c, g);
           } else {
-            store_state_f32<D, TPW>(Wd, a.b_ckpt + ci * D, Wc, bT, m0s, w, c, g);
+            store_state_f32<D, TPW>(ck.W, ck.b, Wc, bT, m0s, w, c, g);
           }
+          ck.advance();
         }
+        ck.next_stage();
 
         // ---- XK with tokens along k for the state update: depends on nothing computed here, so it
         // is issued first and fills the gaps of the dependent chain below
