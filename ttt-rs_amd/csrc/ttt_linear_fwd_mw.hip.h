@@ -247,18 +247,41 @@ __device__ __forceinline__ void store_state_final(float* Wd, float* bd, const fl
   }
 }
 
+// Where one (batch, head) unit's rows start, as wave-uniform byte pointers formed once; a token's row is then a
+// 32-bit byte offset from them (a unit spans at most seq_stride * d * 4 bytes), which is what the addressing of
+// global loads and stores takes directly: scalar base plus 32-bit lane offset, no 64-bit arithmetic and no renewed
+// fetch of the kernel arguments per mini-batch.
+template <class T, int D>
+struct UnitBase {
+  using elem = typename Io<T>::elem;
+  const unsigned char *xq, *xk, *xv, *lr;
+  unsigned char* out;
+  __device__ __forceinline__ UnitBase(const LinearFwdArgs& a, size_t bh) {
+    const size_t row0 = bh * (size_t)a.seq_stride;
+    xq = static_cast<const unsigned char*>(a.xq) + row0 * (D * sizeof(elem));
+    xk = static_cast<const unsigned char*>(a.xk) + row0 * (D * sizeof(elem));
+    xv = static_cast<const unsigned char*>(a.xv) + row0 * (D * sizeof(elem));
+    lr = static_cast<const unsigned char*>(a.lr) + row0 * sizeof(elem);
+    out = static_cast<unsigned char*>(a.out) + row0 * (D * sizeof(elem));
+  }
+  // byte offset of token (stage * K + c) of the unit
+  static __device__ __forceinline__ unsigned row_off(int stage, int K, int c) {
+    return ((unsigned)stage * (unsigned)K + (unsigned)c) * (unsigned)(D * sizeof(elem));
+  }
+};
+
 template <class T, int D, int NW, bool FULL>
-__device__ __forceinline__ void load_stage_mw(StageInMw<T, D / 16, D / 16 / NW>& s, const LinearFwdArgs& a,
-                                              size_t bh, int stage, int c, int g, int w) {
+__device__ __forceinline__ void load_stage_mw(StageInMw<T, D / 16, D / 16 / NW>& s, const UnitBase<T, D>& ub, int K,
+                                              int n_stages, int stage, int c, int g, int w) {
   using IO = Io<T>;
   using elem = typename IO::elem;
   constexpr int NT = D / 16, TPW = NT / NW;
-  if (FULL) stage = min(stage, a.n_stages - 1);
-  const bool ok = FULL || ((c < a.K) && (stage < a.n_stages));
-  const size_t tok = bh * (size_t)a.seq_stride + (size_t)stage * a.K + c;
-  const elem* pq = static_cast<const elem*>(a.xq) + tok * D;
-  const elem* pk = static_cast<const elem*>(a.xk) + tok * D;
-  const elem* pv = static_cast<const elem*>(a.xv) + tok * D;
+  if (FULL) stage = min(stage, n_stages - 1);
+  const bool ok = FULL || ((c < K) && (stage < n_stages));
+  const unsigned off = UnitBase<T, D>::row_off(stage, K, c);
+  const elem* pq = reinterpret_cast<const elem*>(ub.xq + off);
+  const elem* pk = reinterpret_cast<const elem*>(ub.xk + off);
+  const elem* pv = reinterpret_cast<const elem*>(ub.xv + off);
 #pragma unroll
   for (int q = 0; q < NT / 2; ++q) {
     IO::load8(pq + 32 * q + 8 * g, ok, s.q[2 * q], s.q[2 * q + 1]);
@@ -269,24 +292,25 @@ __device__ __forceinline__ void load_stage_mw(StageInMw<T, D / 16, D / 16 / NW>&
 #pragma unroll
     for (int q = 0; q < NT / 2; ++q) IO::load8(pv + 32 * q + 8 * g, ok, s.vo[2 * q], s.vo[2 * q + 1]);
   } else if (TPW == 1) {
-    const int off = own_offset<TPW>(w, 0, g);
+    const int off1 = own_offset<TPW>(w, 0, g);
     if (ok) {
-      s.qo[0] = load4<T>(pq + off);
-      s.ko[0] = load4<T>(pk + off);
-      s.vo[0] = load4<T>(pv + off);
+      s.qo[0] = load4<T>(pq + off1);
+      s.ko[0] = load4<T>(pk + off1);
+      s.vo[0] = load4<T>(pv + off1);
     } else {
       s.qo[0] = s.ko[0] = s.vo[0] = IO::zero();
     }
   } else {
 #pragma unroll
     for (int qq = 0; qq < TPW / 2; ++qq) {
-      const int off = own_offset<TPW>(w, 2 * qq, g);  // eight contiguous features: tiles 2qq, 2qq+1
-      IO::load8(pq + off, ok, s.qo[2 * qq], s.qo[2 * qq + 1]);
-      IO::load8(pk + off, ok, s.ko[2 * qq], s.ko[2 * qq + 1]);
-      IO::load8(pv + off, ok, s.vo[2 * qq], s.vo[2 * qq + 1]);
+      const int off2 = own_offset<TPW>(w, 2 * qq, g);  // eight contiguous features: tiles 2qq, 2qq+1
+      IO::load8(pq + off2, ok, s.qo[2 * qq], s.qo[2 * qq + 1]);
+      IO::load8(pk + off2, ok, s.ko[2 * qq], s.ko[2 * qq + 1]);
+      IO::load8(pv + off2, ok, s.vo[2 * qq], s.vo[2 * qq + 1]);
     }
   }
-  s.lr = ok ? IO::load1(static_cast<const elem*>(a.lr) + tok) : 0.f;
+  const unsigned tok = (unsigned)stage * (unsigned)K + (unsigned)c;
+  s.lr = ok ? IO::load1(reinterpret_cast<const elem*>(ub.lr + tok * (unsigned)sizeof(elem))) : 0.f;
 }
 
 // Sum over the four lane groups.  MF: one f32 MFMA against a ones operand (keeps the VALU free);
@@ -365,8 +389,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
   // at the loop back-edge would have to wait for the load, i.e. undo the prefetch).
   constexpr int R = PF + 1;
   StageInMw<T, NT, TPW> buf[R];
+  const UnitBase<T, D> ub(a, bh);
+  const int K_ = a.K, n_stages_ = a.n_stages;
 #pragma unroll
-  for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], a, bh, u, c, g, w);
+  for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], ub, K_, n_stages_, u, c, g, w);
   CkptCursor<D> ck(a, bh);
   const float b_mean = __builtin_amdgcn_readfirstlane(m0s[D]);  // mean of the initial bias (split off by centre_state)
 
@@ -374,7 +400,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int st = st0 + u;
-      load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], a, bh, st + PF, c, g, w);
+      load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], ub, K_, n_stages_, st + PF, c, g, w);
       if (st >= a.n_stages) continue;
       const StageInMw<T, NT, TPW>& cur = buf[u];
 
@@ -505,7 +531,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
         const float mu = s0 * inv_d;
         const float rstd = __builtin_amdgcn_rsqf(fmaxf(s1 * inv_d - mu * mu, 0.f) + a.eps);
         if (FULL || c < K) {
-          elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
+          elem* po = reinterpret_cast<elem*>(ub.out + UnitBase<T, D>::row_off(st, K, c));
           f32x4 o[TPW];
 #pragma unroll
           for (int jj = 0; jj < TPW; ++jj) {

@@ -33,7 +33,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
   const int c = lane & 15, g = lane >> 4;
   const size_t bh = blockIdx.x;
   const int h = (int)(bh % a.H);
-  const int K = a.K;
+  const int K = a.K, n_stages_ = a.n_stages;
+  const UnitBase<T, D> ub(a, bh);
 
   // same scale folding as the unskewed kernel: G'' = -sc lr G, M'' = (token_eta[t]/sc)(1 + A)
   const float te_last = a.token_eta[K - 1];
@@ -125,7 +126,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
     const float mu = s0 * inv_d;
     const float rstd = __builtin_amdgcn_rsqf(fmaxf(s1 * inv_d - mu * mu, 0.f) + a.eps);
     if (FULL || c < K) {
-      elem* po = static_cast<elem*>(a.out) + (bh * (size_t)a.seq_stride + (size_t)stage * K + c) * D;
+      elem* po = reinterpret_cast<elem*>(ub.out + UnitBase<T, D>::row_off(stage, K, c));
       f32x4 o[TPW];
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) {
@@ -156,7 +157,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
   constexpr int R = PF + 1;
   StageInMw<T, NT, TPW> buf[R];
 #pragma unroll
-  for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], a, bh, u, c, g, w);
+  for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], ub, K, n_stages_, u, c, g, w);
 
   // One pass over R mini-batches (the ring of prefetch registers is indexed at compile time).  CHECKED:
   // the first and the last pass, which test for "no pending output yet" and "past the end"; the passes in
@@ -171,7 +172,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int st = st0 + u;
-      load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], a, bh, st + PF, c, g, w);
+      load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], ub, K, n_stages_, st + PF, c, g, w);
       if (CHECKED && st >= a.n_stages) continue;
       const StageInMw<T, NT, TPW>& cur = buf[u];
 
@@ -306,7 +307,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         const int st = st0 + u;
-        load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], a, bh, st + PF, c, g, w);
+        load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], ub, K, n_stages_, st + PF, c, g, w);
         if (st >= a.n_stages) continue;
         const StageInMw<T, NT, TPW>& cur = buf[u];
 
