@@ -96,14 +96,14 @@ class LinearCalls:
     and nothing else (no allocation, no copies), so the device time between the events around a call is the time of
     its kernels."""
 
-    def __init__(self, pkg, dv, B, H, seq, d, K, dtype, ci, packed, with_bwd):
+    def __init__(self, pkg, dv, B, H, seq, d, K, dtype, ci, ckpt_format, with_bwd):
         import ctypes as C
         import torch
         self.pkg, self.C = pkg, C
         dev = dv["xq"].device
         f32 = dict(dtype=torch.float32, device=dev)
         self.desc = pkg.TttDesc(B, H, seq, d, K, 1e-6, ci, pkg.TTT_BF16 if dtype == torch.bfloat16 else pkg.TTT_F32,
-                                0, 0, int(packed), 0)
+                                0, 0, int(ckpt_format), 0)
         self.dv = dv
         self.out = torch.empty_like(dv["xq"])
         self.W, self.b = torch.empty((B, H, d, d), **f32), torch.empty((B, H, d), **f32)
@@ -217,10 +217,15 @@ def run_workload(name, a, pkg, torch):
                                           mlp=kind in ("mlp_fwd", "mlp_fwd_bwd"))
         dv = {k: v.to(dev) for k, v in c.items()}
         if kind in ("linear_fwd", "linear_fwd_bwd"):
-            # a checkpoint per mini-batch: checkpoints as operand fragments in kernel order (bf16 I/O: half the
-            # checkpoint traffic); --checkpoint-format f32 keeps the reference's f32 matrices
-            packed = kind == "linear_fwd_bwd" and ci == 1 and a.checkpoint_format == "packed"
-            calls = LinearCalls(pkg, dv, B, H, seq, d, K, dtype, ci, packed, kind == "linear_fwd_bwd")
+            # a checkpoint per mini-batch: what is saved for the backward is the library's cheapest form for the shape
+            # ("auto"): bf16 I/O up to 512 units and head_dim 96, the update factors and the final state (a quarter of
+            # the packed bytes; the feature-split backward walks the states back); otherwise the states as operand
+            # fragments in kernel order ("packed").  --checkpoint-format f32 keeps the reference's f32 matrices.
+            ckfmt = 0
+            if kind == "linear_fwd_bwd" and ci == 1:
+                fits = dtype == torch.bfloat16 and d <= 96 and B * H <= 512 and seq // K >= 2
+                ckfmt = {"f32": 0, "packed": 1, "factors": 2, "auto": 2 if fits else 1}[a.checkpoint_format]
+            calls = LinearCalls(pkg, dv, B, H, seq, d, K, dtype, ci, ckfmt, kind == "linear_fwd_bwd")
             if kind == "linear_fwd":
                 parts = [("ttt_linear_fwd", calls.fwd)]
 
@@ -305,10 +310,13 @@ def run_workload(name, a, pkg, torch):
         # 18 d^2 + 22 K d flop per token-head, bound by the f32 matrix pipe.
         lds = ci != 1
         bwd_s, fwd_s = part_s["ttt_linear_bwd"], part_s["ttt_linear_fwd (writes checkpoints)"]
-        ck_bytes = th * (d * d * (2 if (packed and io == "bf16") else 4) + d * 4) // (ci * K)  # written once, read once
+        if ckfmt == 2:  # a [16 x d] bf16 factor per mini-batch and the final state per unit
+            ck_bytes = th * (16 * d * 2) // K + B * H * (d * d + d) * 4
+        else:
+            ck_bytes = th * (d * d * (2 if (ckfmt == 1 and io == "bf16") else 4) + d * 4) // (ci * K)  # written once, read once
         out["dtype"] = io
         out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci,
-                             checkpoint_format="packed" if packed else "f32 row-major")
+                             checkpoint_format=("f32 row-major", "packed", "update factors")[ckfmt])
         kname = "ttt_linear_bwd_kernel" if lds else "ttt_linear_bwd_mw_kernel"
         if io == "bf16" and not lds:
             alg = linear_bwd_bytes(B, H, seq, d, s)
@@ -377,7 +385,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS) + ["hbm_copy_calibration"])
     ap.add_argument("--checkpoint-interval", type=int, default=1)
-    ap.add_argument("--checkpoint-format", default="packed", choices=["packed", "f32"])
+    ap.add_argument("--checkpoint-format", default="auto", choices=["auto", "factors", "packed", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stack-chunk", type=int, default=2048, help="stack workload: tokens per wavefront window (0: none)")
     ap.add_argument("--stack-streams", type=int, default=2, choices=[1, 2], help="stack workload: 2 = TTT-MLP launches on a second stream")

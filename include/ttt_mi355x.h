@@ -65,7 +65,17 @@ typedef struct ttt_desc {
                                   backward's products take bf16 operands anyway, so its results do not
                                   change; half the checkpoint traffic.  f32 I/O: f32.  Either way stored
                                   and fetched in whole 1 KiB rows instead of scattered 4-byte pieces.
-                                  No counterpart in the reference. */
+                                  No counterpart in the reference.
+                                  2 (TTT_CKPT_FACTORS): bf16 I/O, checkpoint_interval 1, head_dim <= 96.  No
+                                  states are saved: ttt_linear_fwd writes, into the same W_ckpt / b_ckpt
+                                  allocations, the state after the last mini-batch and per mini-batch the
+                                  [16 x d] factor of its state update (32*d bytes instead of 2*d*d), and
+                                  ttt_linear_bwd walks the state back from the end, W_t = W_{t+1} - XK_t^T G_t
+                                  with the operands the forward multiplied: each state is recovered up to one
+                                  f32 rounding per element and mini-batch, far below the bf16 rounding of the
+                                  operands it then becomes.  A quarter of the packed format's traffic.  A
+                                  sequence of one mini-batch is saved packed (the buffers are the same).
+                                  Meaningful only to ttt_linear_bwd.  No counterpart in the reference. */
   int32_t kernel_hint;         /* 0 (TTT_HINT_AUTO): the library chooses the kernel from the shape.  Otherwise a
                                   tuning / testing request, read by the entry point the desc is passed to:
                                   low byte = wavefronts per (batch, head) unit for the TTT-Linear kernels
@@ -79,6 +89,7 @@ typedef struct ttt_desc {
 } ttt_desc;
 #define TTT_CKPT_F32 0
 #define TTT_CKPT_PACKED 1
+#define TTT_CKPT_FACTORS 2
 #define TTT_HINT_AUTO 0
 #define TTT_HINT_WAVES_MASK 0xff
 #define TTT_HINT_LDS_TILES 0x100

@@ -51,9 +51,10 @@ def test_shape_validation(P):
     assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_interval=0))) == P.TTT_ERR_SHAPE
     assert L.ttt_linear_supported(C.byref(desc(P, io_dtype=7))) == P.TTT_ERR_UNSUPPORTED
     assert L.ttt_linear_supported(None) == P.TTT_ERR_NULL
-    # checkpoint formats: 0 (f32 row-major) and 1 (packed) exist
+    # checkpoint formats: 0 (f32 row-major), 1 (packed) and 2 (update factors) exist
     assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_format=1))) == P.TTT_OK
-    assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_format=2))) == P.TTT_ERR_SHAPE
+    assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_format=2))) == P.TTT_OK
+    assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_format=3))) == P.TTT_ERR_SHAPE
     assert b"checkpoint_format" in L.ttt_last_error()
 
 
@@ -78,6 +79,13 @@ def test_backward_support_query_and_kernel_hints(P):
     assert ok(checkpoint_format=1, checkpoint_interval=2) == P.TTT_ERR_UNSUPPORTED
     # packed checkpoints exist for the register-resident kernels only
     assert ok(checkpoint_format=1, kernel_hint=P.TTT_HINT_LDS_TILES) == P.TTT_ERR_UNSUPPORTED
+    # update factors: bf16 I/O, a checkpoint per mini-batch, head_dim <= 96, the register-resident kernels
+    fac = lambda **kw: ok(checkpoint_format=2, **{"io_dtype": P.TTT_BF16, **kw})
+    assert fac() == P.TTT_OK and fac(head_dim=96) == P.TTT_OK and fac(seq=16) == P.TTT_OK
+    for bad in (dict(io_dtype=P.TTT_F32), dict(head_dim=128), dict(checkpoint_interval=2),
+                dict(kernel_hint=P.TTT_HINT_LDS_TILES)):
+        assert fac(**bad) == P.TTT_ERR_UNSUPPORTED, bad
+        assert b"update-factor checkpoints" in L.ttt_last_error()
     assert ok(kernel_hint=P.TTT_HINT_LDS_TILES) == P.TTT_OK
     assert ok(kernel_hint=4) == P.TTT_OK and ok(kernel_hint=1, io_dtype=P.TTT_BF16) == P.TTT_OK
     # a hint that names no kernel for the desc is ignored (no LDS-tile backward at head_dim 96)

@@ -234,10 +234,12 @@ def test_linear_fwd_rows_far_from_zero_mean(P, d, hint, dtype, kind):
 @pytest.mark.parametrize("dtype,d,hint", [(torch.float32, 64, 4), (torch.bfloat16, 64, 4), (torch.bfloat16, 64, 1),
                                           (torch.bfloat16, 128, 0), (torch.float32, 64, 0x100)],
                          ids=["f32-mw", "bf16-mw", "bf16-rr", "bf16-d128", "f32-lds"])
-@pytest.mark.parametrize("packed", [False, True], ids=["ckpt-f32", "ckpt-packed"])
+@pytest.mark.parametrize("packed", [0, 1, 2], ids=["ckpt-f32", "ckpt-packed", "ckpt-factors"])
 def test_linear_bwd_rows_far_from_zero_mean(P, dtype, d, hint, kind, packed):
     if packed and hint == 0x100:
         pytest.skip("packed checkpoints are for the register-resident kernels")
+    if packed == 2 and (dtype != torch.bfloat16 or d > 96 or hint != 4):
+        pytest.skip("update factors: bf16 I/O, head_dim <= 96, feature-split backward")
     B, H, K, N = 1, 2, 16, (1 if kind == "const" else 4)
     print(f"case linear bwd offset rows {kind} d{d} hint {hint:#x} {dtype} packed={packed}", flush=True)
     c = offset_case(P, 50 + d, B, H, N * K, d, K, dtype, kind)

@@ -143,8 +143,19 @@ def test_config1_shape_linear_fwd_bwd_bf16_full(P):
     assert torch.equal(outp, out)
     for k in ("grad_xq", "grad_xk", "grad_xv", "grad_weight", "grad_bias", "grad_ttt_lr_eta"):
         assert_close(gp[k], g[k].double(), 1e-2, "packed " + k, min_frac=0.99)
+    # update factors instead of states (what bench.py measures at this shape): the backward walks the state back
+    # over all 128 mini-batches; gradients as close to the packed run as that is to the first.  The forward that
+    # saves factors is a compilation of its own: the same source, but the compiler is free to fuse a multiply and an
+    # add in one and not in the other, so its output may differ from the other formats' in the last bit of a few
+    # elements (seen: 1 element in 50 million by one bf16 step), not bit for bit.
+    outf, gf = fwd_bwd(dv, packed=2)
+    assert (outf != out).float().mean().item() < 1e-5
+    assert_close(outf, out.double(), 2.0 ** -7, "factors out")
+    for k in ("grad_xq", "grad_xk", "grad_xv", "grad_weight", "grad_bias", "grad_ttt_lr_eta"):
+        assert_close(gf[k], gp[k].double(), 1e-2, "factors " + k, min_frac=0.99)
     for k, v in g.items():
         assert torch.isfinite(v.float()).all(), k
+        assert torch.isfinite(gf[k].float()).all(), "factors " + k
     # one batch entry alone: per-unit gradients are bit-identical
     one = {k: (v[5:6].contiguous() if k in ("xq", "xk", "xv", "lr", "d_out") else v) for k, v in dv.items()}
     o1, g1 = fwd_bwd(one)

@@ -206,6 +206,52 @@ def test_bwd_packed_checkpoints_change_nothing(P, B, H, d, K, N, waves, dtype):
     compare(res[1][3], oracle_bwd(c, dO.cpu(), K), TOL[dtype])
 
 
+@pytest.mark.parametrize("B,H,d,K,N", [(2, 2, 32, 8, 3), (2, 3, 64, 16, 8), (1, 2, 64, 5, 3), (1, 2, 96, 16, 3),
+                                       (1, 2, 64, 16, 1), (1, 3, 64, 16, 2), (1, 2, 64, 16, 40)])
+@pytest.mark.parametrize("eta_last", ["positive", "zero"])
+def test_bwd_from_update_factors(P, B, H, d, K, N, eta_last):
+    """checkpoint_format 2 (bf16 I/O): the forward saves the final state and the [16 x d] factor of every state
+    update instead of the states; the backward walks the state back from the end with the operands the forward
+    multiplied.  The forward's outputs do not depend on the format beyond the last bit (the forward that saves
+    factors is a compilation of its own, free to fuse a multiply and an add where the other does not).  The
+    recovered states differ from the saved ones by f32 roundings, which move a bf16 operand here and there, as the two state formats differ among themselves:
+    the gradients agree with those from packed states to 5e-3 and with the oracle to the bf16 bar.  One mini-batch
+    (N = 1) is saved packed by the library; token_eta[K-1] = 0 means the forward never changed the state and the
+    walk back must not either."""
+    dtype = torch.bfloat16
+    print(f"case bwd factor ckpt B{B} H{H} d{d} K{K} N{N} eta_last {eta_last}", flush=True)
+    c = P.synthetic.reference_test_inputs(700 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
+    if eta_last == "zero":
+        c["token_eta"] = c["token_eta"].clone()
+        c["token_eta"][K - 1] = 0.0
+    dv = to_dev(c)
+    g = torch.Generator().manual_seed(12)
+    dO = torch.randn(B, H, N * K, d, generator=g).to(dtype).to("cuda:0")
+    res = []
+    for fmt in (1, 2):
+        out, W, b, Wc, bc = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"],
+                                                     dv["lr"], dv["gamma"], dv["beta"], K, 1e-6, 1,
+                                                     want_checkpoints=True, packed_checkpoints=fmt)
+        gr = P.ttt_linear_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                                       dv["gamma"], dv["beta"], Wc, bc, dO, K, 1e-6, 1, packed_checkpoints=fmt)
+        torch.cuda.synchronize()
+        res.append((out, W, b, gr))
+    assert_close(res[1][0], res[0][0].double(), 2.0 ** -7, "out")
+    assert_close(res[1][1], res[0][1].double(), 1e-5, "W")
+    assert_close(res[1][2], res[0][2].double(), 1e-5, "b")
+    for k in res[0][3]:
+        assert_close(res[1][3][k], res[0][3][k].double(), 5e-3, k, min_frac=0.99)
+    compare(res[1][3], oracle_bwd(c, dO.cpu(), K), TOL[dtype])
+
+
+def test_update_factors_rejected_where_unsupported(P):
+    c = P.synthetic.reference_test_inputs(2, 1, 1, 64, 32, 16)
+    dv = to_dev(c)
+    with pytest.raises(Exception, match="update-factor checkpoints"):
+        P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                                 dv["gamma"], dv["beta"], 16, 1e-6, 1, want_checkpoints=True, packed_checkpoints=2)
+
+
 def test_packed_checkpoints_rejected_where_unsupported(P):
     c = P.synthetic.reference_test_inputs(2, 1, 1, 64, 32, 16)
     dv = to_dev(c)

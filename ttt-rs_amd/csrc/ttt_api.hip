@@ -49,12 +49,31 @@ int check_common(const ttt_desc* d) {
   if (d->io_dtype != TTT_F32 && d->io_dtype != TTT_BF16)
     return fail(TTT_ERR_UNSUPPORTED, "io_dtype %d is neither TTT_F32 nor TTT_BF16", d->io_dtype);
   if (!(d->eps > 0.f)) return fail(TTT_ERR_SHAPE, "eps must be positive");
-  if (d->checkpoint_format != TTT_CKPT_F32 && d->checkpoint_format != TTT_CKPT_PACKED)
-    return fail(TTT_ERR_SHAPE, "checkpoint_format %d is neither TTT_CKPT_F32 nor TTT_CKPT_PACKED", d->checkpoint_format);
+  if (d->checkpoint_format != TTT_CKPT_F32 && d->checkpoint_format != TTT_CKPT_PACKED &&
+      d->checkpoint_format != TTT_CKPT_FACTORS)
+    return fail(TTT_ERR_SHAPE, "checkpoint_format %d is none of TTT_CKPT_F32, TTT_CKPT_PACKED, TTT_CKPT_FACTORS",
+                d->checkpoint_format);
   if (d->seq_stride != 0 && d->seq_stride < d->seq)
     return fail(TTT_ERR_SHAPE, "seq_stride (%d) must be 0 or >= seq (%d)", d->seq_stride, d->seq);
   if ((int64_t)d->batch * d->heads > 0x7fffffffLL)
     return fail(TTT_ERR_SHAPE, "batch*heads exceeds the grid limit");
+  return TTT_OK;
+}
+
+// The checkpoint format a desc stands for after the one substitution the library makes: update factors share the W
+// checkpoint buffer with the final state, which takes two or more mini-batches' worth of it, so a sequence of a
+// single mini-batch is saved packed.  Forward and backward both decide through this function.
+int ckpt_format_of(const ttt_desc* d) {
+  if (d->checkpoint_format == TTT_CKPT_FACTORS && d->seq / d->mini_batch < 2) return TTT_CKPT_PACKED;
+  return d->checkpoint_format;
+}
+// What TTT_CKPT_FACTORS needs of a desc (0 = fine); the same for the forward that writes and the backward that reads.
+int check_factors(const ttt_desc* d) {
+  if (d->io_dtype != TTT_BF16 || d->checkpoint_interval != 1 || d->head_dim > 96 ||
+      (d->kernel_hint & TTT_HINT_LDS_TILES) != 0)
+    return fail(TTT_ERR_UNSUPPORTED,
+                "update-factor checkpoints need bf16 I/O, checkpoint_interval 1, head_dim <= 96 and the "
+                "register-resident kernels");
   return TTT_OK;
 }
 
@@ -86,13 +105,34 @@ int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream
   // holds the whole state and all rows in one wave, has registers for one mini-batch ahead only)
   constexpr int PF = (NW == 1 && sizeof(typename ttt::Io<T>::elem) == 4) ? 1 : 2;
   const dim3 grid((unsigned)(a.B * a.H), ny), block(64 * NW);
+  // the variants that save update factors exist for bf16 I/O only (prepare_linear_fwd lets no other desc ask)
+  constexpr bool can_fac = sizeof(typename ttt::Io<T>::elem) == 2;
+  const bool fac = can_fac && a.ckpt_packed == ttt::kCkptFactors;
   if constexpr (NW == 1) {
+    if constexpr (can_fac) {
+      if (fac) {
+        if (a.K == 16)
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, true, true>), grid, block, 0, s, P);
+        else
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, false, true>), grid, block, 0, s, P);
+        return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+      }
+    }
     if (a.K == 16)
       hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, true>), grid, block, 0, s, P);
     else
       hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, false>), grid, block, 0, s, P);
   } else {
     constexpr int NWS = NW > 1 ? NW : 2;  // the skewed kernel needs at least two waves
+    if constexpr (can_fac) {
+      if (fac) {
+        if (a.K == 16)
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true, true>), grid, block, 0, s, P);
+        else
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, false, true>), grid, block, 0, s, P);
+        return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+      }
+    }
     if (a.K == 16)
       hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true>), grid, block, 0, s, P);
     else
@@ -139,6 +179,15 @@ int launch_linear_fwd_wide(const ttt::LinearFwdArgs* probs, unsigned ny, hipStre
   constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
   constexpr int PF = f32 ? 1 : 2;  // f32 fragments are twice as large: prefetch one mini-batch ahead
   const dim3 grid((unsigned)(a.B * a.H), ny), block(64 * NW);
+  if constexpr (!f32 && D == 96) {
+    if (a.ckpt_packed == ttt::kCkptFactors) {
+      if (a.K == 16)
+        hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, true, true>), grid, block, 0, s, P);
+      else
+        hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, false, true>), grid, block, 0, s, P);
+      return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+    }
+  }
   if (a.K == 16)
     hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, true>), grid, block, 0, s, P);
   else
@@ -260,10 +309,10 @@ int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
 }
 
 // one checkpoint per mini-batch, NW waves per (batch, head): feature axis split, exchanges through LDS
-template <class T, int D, int NW, bool PK = false>
+template <class T, int D, int NW, bool PK = false, bool FM = false>
 int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK>;
-  constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem), PK>::BYTES;
+  constexpr auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK, FM>;
+  constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem), PK, FM>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), bytes, s, a);
@@ -295,7 +344,12 @@ int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
   if (rc != TTT_OK) return rc;
   const int D = d->head_dim;
   const bool f32 = d->io_dtype == TTT_F32;
-  const bool packed = d->checkpoint_format == TTT_CKPT_PACKED;
+  if (d->checkpoint_format == TTT_CKPT_FACTORS) {
+    rc = check_factors(d);
+    if (rc != TTT_OK) return rc;
+  }
+  const bool packed = ckpt_format_of(d) == TTT_CKPT_PACKED;
+  const bool factors = ckpt_format_of(d) == TTT_CKPT_FACTORS;
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && D <= 64;
   if (packed && (d->checkpoint_interval != 1 || want_lds))
     return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
@@ -304,6 +358,7 @@ int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
       return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
     int waves = d->kernel_hint & TTT_HINT_WAVES_MASK;
     if (waves == 0) waves = (f32 || D > 64 || (long)d->batch * d->heads <= 512) ? 4 : 1;
+    if (factors) waves = 4;  // the walk back of the state exists in the feature-split kernel only
     ch->kind = LinearBwdChoice::REG;
     ch->waves = waves;
     return TTT_OK;
@@ -509,11 +564,17 @@ int prepare_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const 
   a.ckpt_interval = d->checkpoint_interval;
   a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
   a.state_per_batch = d->state_per_batch ? 1 : 0;
-  a.ckpt_packed = (W_ckpt != nullptr && d->checkpoint_format == TTT_CKPT_PACKED) ? 1 : 0;
+  if (W_ckpt != nullptr && d->checkpoint_format == TTT_CKPT_FACTORS) {
+    rc = check_factors(d);
+    if (rc != TTT_OK) return rc;
+  }
+  a.ckpt_packed = W_ckpt == nullptr ? 0
+                  : ckpt_format_of(d) == TTT_CKPT_PACKED ? 1
+                  : ckpt_format_of(d) == TTT_CKPT_FACTORS ? ttt::kCkptFactors : 0;
   a.eps = d->eps;
   // the LDS-tile forward exists for head_dim 96/128 only; elsewhere the hint names no kernel and is ignored
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
-  if (a.ckpt_packed && (d->checkpoint_interval != 1 || want_lds))
+  if (a.ckpt_packed == 1 && (d->checkpoint_interval != 1 || want_lds))
     return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
   return TTT_OK;
 }
@@ -595,7 +656,7 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   a.n_stages = d->seq / d->mini_batch;
   a.ckpt_interval = d->checkpoint_interval;
   a.n_ckpt = (int)ttt_linear_num_checkpoints(d);
-  a.ckpt_packed = d->checkpoint_format == TTT_CKPT_PACKED;
+  a.ckpt_packed = ckpt_format_of(d) == TTT_CKPT_PACKED ? 1 : ckpt_format_of(d) == TTT_CKPT_FACTORS ? ttt::kCkptFactors : 0;
   a.eps = d->eps;
   const int D = d->head_dim;
   if (ch.kind != LinearBwdChoice::LDS &&
@@ -619,6 +680,11 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   if (ch.kind == LinearBwdChoice::LDS) {
     if (f32) return D == 64 ? launch_linear_bwd<ttt::F32, 64>(a, grid, s) : launch_linear_bwd<ttt::F32, 32>(a, grid, s);
     return D == 64 ? launch_linear_bwd<ttt::BF16, 64>(a, grid, s) : launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
+  }
+  if (a.ckpt_packed == ttt::kCkptFactors) {
+    if (D == 32) return launch_linear_bwd_mw<ttt::BF16, 32, 2, true, true>(a, grid, s);
+    if (D == 64) return launch_linear_bwd_mw<ttt::BF16, 64, 4, true, true>(a, grid, s);
+    return launch_linear_bwd_mw<ttt::BF16, 96, 3, true, true>(a, grid, s);
   }
   if (f32 && a.ckpt_packed) {
     if (D == 32) return launch_linear_bwd_mw<ttt::F32, 32, 2, true>(a, grid, s);

@@ -28,7 +28,10 @@
 namespace ttt {
 
 // PK: the W checkpoint arrives packed (bf16 fragments in accumulator order, see store_ckpt_packed)
-template <int D, int NW, int ES, bool PK = false>
+// FM: no states were saved but the update factors and the final state (see store_factor): the f32 state lives in
+//     the registers of the waves (each its column tiles, as in the forward), is walked back by one mini-batch per
+//     pass, and its packed image is written where a packed checkpoint would have been copied to
+template <int D, int NW, int ES, bool PK = false, bool FM = false>
 struct LinBwdMwLds {
   static constexpr int NT = D / 16, TPW = NT / NW;
   static constexpr int XS = (ES == 2) ? NT / 2 : NT;  // 1 KiB slots per activation tensor
@@ -43,19 +46,22 @@ struct LinBwdMwLds {
   static constexpr int PT = SUM + 3 * 8 * 16 * NW * 4;  // 4 kinds x [NW][64] f32x4: partial [16 x 16] blocks
   static constexpr int FR = PT + 4 * NW * 1024;       // 7 kinds x [NT][64] fragments
   static constexpr int M0 = FR + 7 * NT * FT;         // D row means of the initial W, then mean(b): the centred state
-  static constexpr int BYTES = M0 + (D + 4) * 4;
+  static constexpr int GDS = M0 + (D + 4) * 4;         // FM: NT half slots: the factor fragments of tile J
+  static constexpr int BYTES = GDS + (FM ? NT * 512 : 0);
+  static_assert(!FM || (PK && ES == 2), "factors: bf16 I/O, packed image of the state");
+  static_assert(GDS % 16 == 0, "copy targets are 16-byte aligned");
   static_assert(NT % NW == 0 && WSLOTS % NW == 0, "feature tiles must divide among the waves");
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
 
-template <class T, int D, int NW, bool PK = false>
+template <class T, int D, int NW, bool PK = false, bool FM = false>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;
   constexpr int ES = sizeof(elem);
   constexpr bool BF = ES == 2;
-  using L = LinBwdMwLds<D, NW, ES, PK>;
+  using L = LinBwdMwLds<D, NW, ES, PK, FM>;
   constexpr int NT = D / 16, TPW = NT / NW, NQ = NT / 2, XS = L::XS;
   constexpr float inv_d = 1.0f / D;
   enum { KD = 0, QD, GF, ZF, ZD, Z1F, Z1D };
@@ -132,7 +138,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         M0p[i] = sum * inv_d;
       }
     }
-    if (threadIdx.x == 0) {
+    if (!FM && threadIdx.x == 0) {
       float sum = 0.f;
       for (int f = 0; f < D; ++f) sum += a.b_ckpt[c0 * D + f];
       M0p[D] = sum * inv_d;
@@ -149,22 +155,35 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
 
   // ---- copies of one mini-batch, dealt round-robin to the waves
   const unsigned stg = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  // FM: the unit's share of the W checkpoint buffer holds the final state and, behind it, one factor per mini-batch
+  const unsigned char* const fac0 =
+      reinterpret_cast<const unsigned char*>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D)) + D * D * 4;
   auto fetch = [&](int stage) {
     if (stage < 0) return;
-    const size_t ci = bh * (size_t)a.n_ckpt + stage;
-    const float* Wg = a.W_ckpt + ci * D * D;
+    if constexpr (FM) {
+      // the factor of the mini-batch: tile J is 512 bytes, copied by half a wave
+      const unsigned char* fp = fac0 + (size_t)stage * (32 * D);
 #pragma unroll
-    for (int it = 0; it < L::WSLOTS / NW; ++it) {
-      const int n = w + NW * it, I = n / NT, J = n - I * NT;
-      if (PK)  // whole 1 KiB rows
-        lds_dma16(Wg, (unsigned)(n * 1024 + lane * 16), stg + L::W + n * 1024);
-      else
-        lds_dma16(Wg, (unsigned)(feat(I, c) * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::W + n * 1024);
-    }
-    if (w == 1 % NW) {
-      const float* bg = a.b_ckpt + ci * D;
+      for (int it = 0; it < TPW; ++it) {
+        const int J = w + NW * it;
+        if (lane < 32) lds_dma16(fp, (unsigned)(J * 512 + lane * 16), stg + L::GDS + J * 512);
+      }
+    } else {
+      const size_t ci = bh * (size_t)a.n_ckpt + stage;
+      const float* Wg = a.W_ckpt + ci * D * D;
 #pragma unroll
-      for (int J = 0; J < NT; ++J) lds_dma16(bg, (unsigned)(32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::Bv + J * 1024);
+      for (int it = 0; it < L::WSLOTS / NW; ++it) {
+        const int n = w + NW * it, I = n / NT, J = n - I * NT;
+        if (PK)  // whole 1 KiB rows
+          lds_dma16(Wg, (unsigned)(n * 1024 + lane * 16), stg + L::W + n * 1024);
+        else
+          lds_dma16(Wg, (unsigned)(feat(I, c) * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::W + n * 1024);
+      }
+      if (w == 1 % NW) {
+        const float* bg = a.b_ckpt + ci * D;
+#pragma unroll
+        for (int J = 0; J < NT; ++J) lds_dma16(bg, (unsigned)(32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, stg + L::Bv + J * 1024);
+      }
     }
     const size_t tok0 = (bh * (size_t)a.seq_stride + (size_t)stage * K) * D;
 #pragma unroll
@@ -249,11 +268,72 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     }
   };
 
+  // FM: the state after the last mini-batch (centred, as the forward carried it) is where the walk back starts
+  f32x4 bTm[TPW], Wm[FM ? NT : 1][TPW];  // bias of the own features; W[all row tiles][own column tiles]
+  const bool upd = te_last != 0.f;  // the forward leaves the state alone when token_eta[K-1] is zero
+  if constexpr (FM) {
+    const unsigned char* Wl = reinterpret_cast<const unsigned char*>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D));
+    const float* bl = a.b_ckpt + bh * (size_t)a.n_ckpt * D;
+#pragma unroll
+    for (int I = 0; I < NT; ++I)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj)
+        Wm[I][jj] = *reinterpret_cast<const f32x4*>(Wl + (I * NT + w * TPW + jj) * 1024 + lane * 16);
+#pragma unroll
+    for (int ii = 0; ii < TPW; ++ii) bTm[ii] = *reinterpret_cast<const f32x4*>(bl + own_offset<TPW>(w, ii, g));
+  }
   fetch(a.n_stages - 1);
+
+  // FM: the state entering the mini-batch whose copies are staged: W_t = W_{t+1} - XK_t^T G''_t and
+  // b_t = b_{t+1} - colsum G''_t, with the operands the forward multiplied (XK as staged, G'' as saved).  This wave's
+  // column tiles of the f32 state are updated in its registers and their packed image is written where the products
+  // of the next pass read it.  Runs in the tail of the pass before (the staged rows have all been moved to registers, the
+  // packed image of the current state is no longer read), so it is off the chain of dependent exchanges.
+  auto walk_back = [&]() {
+    if constexpr (FM) {
+      const unsigned char* sl = smem + lane * 16;
+      frag kda[NT];
+#pragma unroll
+      for (int s = 0; s < XS; ++s) {
+        const u32x4 rk = *reinterpret_cast<const u32x4*>(sl + L::X + (1 * XS + s) * 1024);
+        kda[2 * s] = tokens_k(__builtin_bit_cast(frag, u32x2{rk[0], rk[1]}));
+        kda[2 * s + 1] = tokens_k(__builtin_bit_cast(frag, u32x2{rk[2], rk[3]}));
+      }
+      frag nG[TPW];
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        u32x2 raw = *reinterpret_cast<const u32x2*>(smem + L::GDS + (w * TPW + jj) * 512 + lane * 8);
+        raw[0] = upd ? raw[0] ^ 0x80008000u : 0u;
+        raw[1] = upd ? raw[1] ^ 0x80008000u : 0u;
+        nG[jj] = __builtin_bit_cast(frag, raw);
+        IO::mma(bTm[jj], nG[jj], ones);
+      }
+#pragma unroll
+      for (int I = 0; I < NT; ++I)
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          IO::mma(Wm[I][jj], kda[I], nG[jj]);
+          *reinterpret_cast<frag*>(smem + lane * 16 + pk_off(I, w * TPW + jj)) = IO::to_frag(Wm[I][jj]);
+        }
+    }
+  };
+  if constexpr (FM) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+    walk_back();
+  }
 
   for (int st = a.n_stages - 1; st >= 0; --st) {
     // ---- the mini-batch's copies have landed (every wave waits for its own, then all meet)
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // Memory operations complete in the order they were issued, stores included (they count until the cache has
+    // acknowledged them).  Behind the copies of this mini-batch (issued early in the previous pass of the loop) every
+    // wave has issued at least three stores (its d_xq, d_xv and d_xk rows); waiting for everything would wait for
+    // those as well, a store latency per mini-batch, so all but the three youngest operations are waited for.  The
+    // first pass has no stores behind its copies.
+    if (st == a.n_stages - 1)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
     lds_barrier();
     const unsigned char* sl = smem + lane * 16;
     frag q[NT], k[NT], qo[TPW], ko[TPW], vo[TPW], oo[TPW];  // full rows of xq, xk; own features of all four
@@ -304,7 +384,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
 #pragma unroll
     for (int ii = 0; ii < TPW; ++ii) {
       const int Io = w * TPW + ii;
-      bT[ii] = *reinterpret_cast<const f32x4*>(sl + L::Bv + Io * 1024) - bbar;
+      if constexpr (FM)
+        bT[ii] = bTm[ii];
+      else
+        bT[ii] = *reinterpret_cast<const f32x4*>(sl + L::Bv + Io * 1024) - bbar;
 #pragma unroll
       for (int J = 0; J < NT; ++J) {
         if constexpr (PK)  // stored as (m = j, k = i): transposed on the matrix pipe
@@ -574,7 +657,16 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       if (tok_ok) store_own(a.d_xv, tokoff, ndy);
     }
     // ---- X4: dZ1 fragments
+    // FM: the copies of the next mini-batch (issued behind X1; two stores, d_xq and d_xv, are younger) have to be
+    // visible to every wave behind this barrier: the walk back at the end of the pass reads them
+    if constexpr (FM) {
+      static_assert(TPW <= 2, "one store per tensor and wave");
+      asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    }
     lds_barrier();
+    // (behind the first mini-batch of the sequence nothing new is staged: the walk then works on stale rows, its
+    // result is never read, and the loop keeps one shape)
+    if constexpr (FM) walk_back();
     {
       frag Z1fa[NT];
 #pragma unroll
@@ -601,6 +693,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       if (c == K - 1) dte += tail;
       if (g == 0 && tok_ok) atomicAdd(a.d_token_eta + (size_t)st * K + c, dte);
     }
+
     // ---- state gradient: dW += XQ^T dZb + XK^T dZ1 (column slice and transposed row slice), db
 #pragma unroll
     for (int I = 0; I < NT; ++I) {

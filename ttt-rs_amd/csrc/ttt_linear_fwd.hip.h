@@ -6,6 +6,8 @@
 
 namespace ttt {
 
+constexpr int kCkptFactors = 2;  // value of ckpt_packed for TTT_CKPT_FACTORS
+
 struct LinearFwdArgs {
   const void* xq;
   const void* xk;
@@ -22,7 +24,8 @@ struct LinearFwdArgs {
   float* W_ckpt;
   float* b_ckpt;
   int B, H, seq, seq_stride, K, n_stages, ckpt_interval, n_ckpt, state_per_batch;
-  int ckpt_packed;  // W checkpoints as bf16 operand fragments (see store_ckpt_packed)
+  int ckpt_packed;  // 1: W checkpoints as bf16 operand fragments (see store_ckpt_packed); kCkptFactors: update
+                    // factors and the final state instead of states (see store_factor)
   float eps;
 };
 

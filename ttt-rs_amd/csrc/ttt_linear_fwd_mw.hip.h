@@ -102,7 +102,7 @@ struct CkptCursor {
   int left;      // mini-batches until the next checkpoint (0: due now)
   bool packed;
   __device__ __forceinline__ CkptCursor(const LinearFwdArgs& a, size_t bh) {
-    const bool on = a.W_ckpt != nullptr;
+    const bool on = a.W_ckpt != nullptr && a.ckpt_packed != kCkptFactors;
     W = on ? a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D) : nullptr;
     b = on ? a.b_ckpt + bh * (size_t)a.n_ckpt * D : nullptr;
     every = on ? a.ckpt_interval : 1;
@@ -120,6 +120,43 @@ struct CkptCursor {
     if (W != nullptr) --left;
   }
 };
+
+// ---- Update factors instead of states (ckpt_packed == kCkptFactors; bf16 I/O, two or more mini-batches) ---------
+// The state changes by W += XK^T G'' and b += colsum G'' per mini-batch, with G'' rounded to the operand type and
+// XK an input: the [16 x d] factor G'' (2 KiB at d = 64) says as much as the [d x d] state entering the mini-batch
+// (8 KiB packed), given the state at the END of the sequence.  The backward then walks the states back:
+// W_t = W_{t+1} - XK_t^T G''_t with the very operands the forward multiplied, so it recovers W_t up to the rounding
+// of one f32 addition per element and mini-batch.
+// Layout of a unit's share of the W checkpoint buffer (n_ckpt * d * d floats, as for the other formats):
+//   bytes [0, 4 d^2)                       the centred state after the last mini-batch, f32, tile (I, J) = 1 KiB
+//                                          row I * (d/16) + J, 16 bytes per lane (accumulator order)
+//   bytes [4 d^2 + t * 32 d, + 32 d)       factor of mini-batch t: tile J = 512 bytes, 8 per lane: the fragment
+//                                          Gd of the wave that owns feature tile J (tokens along k)
+// and of the b checkpoint buffer: the centred bias after the last mini-batch (d floats).
+template <int D>
+__device__ __forceinline__ unsigned char* factor_base(float* W_ckpt, int n_ckpt, size_t bh) {
+  return reinterpret_cast<unsigned char*>(W_ckpt + bh * (size_t)n_ckpt * (D * D)) + D * D * 4;
+}
+template <int TPW>
+__device__ __forceinline__ void store_factor(unsigned char* slot, const bf16x4 (&Gd)[TPW], int w, int lane) {
+#pragma unroll
+  for (int jj = 0; jj < TPW; ++jj)
+    *reinterpret_cast<u32x2*>(slot + ((w * TPW + jj) * 64 + lane) * 8) = __builtin_bit_cast(u32x2, Gd[jj]);
+}
+template <int D, int TPW>
+__device__ __forceinline__ void store_state_tiles(float* Wd, float* bd, const f32x4 (&Wc)[D / 16][TPW],
+                                                  const f32x4 (&bT)[TPW], int w, int lane) {
+  constexpr int NT = D / 16;
+  unsigned char* base = reinterpret_cast<unsigned char*>(Wd) + lane * 16;
+#pragma unroll
+  for (int I = 0; I < NT; ++I)
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) *reinterpret_cast<f32x4*>(base + (I * NT + w * TPW + jj) * 1024) = Wc[I][jj];
+  if ((lane & 15) == 0) {
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) *reinterpret_cast<f32x4*>(bd + own_offset<TPW>(w, jj, lane >> 4)) = bT[jj];
+  }
+}
 
 // ---- State centring -------------------------------------------------------------------------------------------
 // LayerNorm does not see a shift common to all d features of a row, and the inner loop looks at the state only
@@ -325,7 +362,7 @@ __device__ __forceinline__ float xg_reduce(float v) {
   return xg_sum(v);
 }
 
-template <class T, int D, int NW, int PF, bool FULL>
+template <class T, int D, int NW, int PF, bool FULL, bool FAC = false>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<LinearFwdArgs> problems) {
   const LinearFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
@@ -395,6 +432,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
   for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], ub, K_, n_stages_, u, c, g, w);
   CkptCursor<D> ck(a, bh);
   const float b_mean = __builtin_amdgcn_readfirstlane(m0s[D]);  // mean of the initial bias (split off by centre_state)
+  static_assert(!FAC || BF, "update factors are saved with bf16 I/O only");
+  unsigned char* fac = FAC ? factor_base<D>(a.W_ckpt, a.n_ckpt, bh) : nullptr;
 
   for (int st0 = 0; st0 < a.n_stages; st0 += R) {
 #pragma unroll
@@ -498,6 +537,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
         IO::mma(t, IO::to_frag(G[jj]), ident);
         Gd[jj] = IO::to_frag(t);
       }
+      if constexpr (FAC) {
+        store_factor<TPW>(fac, Gd, w, lane);
+        fac += 32 * D;
+      }
       {
         f32x4 m;
 #pragma unroll
@@ -571,6 +614,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_mw_kernel(Problems<Lin
   }
 
   store_state_final<D, TPW>(a.W_out + bh * D * D, a.b_out + bh * D, a.W0 + sb * D * D, a.b0 + sb * D, Wc, bT, m0s, w, c, g);
+  if constexpr (FAC)
+    store_state_tiles<D, TPW>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D), a.b_ckpt + bh * (size_t)a.n_ckpt * D, Wc, bT, w, lane);
 }
 
 }  // namespace ttt

@@ -17,7 +17,7 @@
 
 namespace ttt {
 
-template <class T, int D, int NW, int PF, bool FULL>
+template <class T, int D, int NW, int PF, bool FULL, bool FAC = false>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
   const LinearFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
@@ -167,6 +167,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
   float ps0 = 0.f, ps1 = 0.f;
   CkptCursor<D> ck(a, bh);
   const float b_mean = __builtin_amdgcn_readfirstlane(m0s[D]);  // mean of the initial bias (split off by centre_state)
+  static_assert(!FAC || BF, "update factors are saved with bf16 I/O only");
+  unsigned char* fac = FAC ? factor_base<D>(a.W_ckpt, a.n_ckpt, bh) : nullptr;
   auto pass = [&](auto checked_tag, int st0) {
     constexpr bool CHECKED = decltype(checked_tag)::value;
 #pragma unroll
@@ -270,6 +272,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
         f32x4 t = {0.f, 0.f, 0.f, 0.f};
         IO::mma(t, IO::to_frag(G[jj]), ident);
         Gd[jj] = IO::to_frag(t);
+      }
+      if constexpr (FAC) {
+        store_factor<TPW>(fac, Gd, w, lane);
+        fac += 32 * D;
       }
       {
         f32x4 m;
@@ -404,6 +410,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
           IO::mma(t, IO::to_frag(G[jj]), ident);
           Gd[jj] = IO::to_frag(t);
         }
+        if constexpr (FAC) {
+          store_factor<TPW>(fac, Gd, w, lane);
+          fac += 32 * D;
+        }
         {
           f32x4 m;
 #pragma unroll
@@ -440,6 +450,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
     emit_output(S[6], S[7], a.n_stages - 1, zbp, qop);
   }
   store_state_final<D, TPW>(a.W_out + bh * D * D, a.b_out + bh * D, a.W0 + sb * D * D, a.b0 + sb * D, Wc, bT, m0s, w, c, g);
+  if constexpr (FAC)
+    store_state_tiles<D, TPW>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D), a.b_ckpt + bh * (size_t)a.n_ckpt * D, Wc, bT, w, lane);
 }
 
 }  // namespace ttt

@@ -39,9 +39,11 @@ struct TTTConfig {
   float base_lr = 1.0f;
   float epsilon = 1e-6f;
   int checkpoint_interval = 1;
-  /// Checkpoints as operand fragments in kernel order (ttt_desc.checkpoint_format = TTT_CKPT_PACKED):
-  /// interval 1 only, same gradients, less traffic.  No counterpart in the reference's config.
-  bool packed_checkpoints = false;
+  /// ttt_desc.checkpoint_format: TTT_CKPT_F32 (what the reference saves), TTT_CKPT_PACKED (states as operand
+  /// fragments in kernel order: interval 1 only, same gradients, less traffic) or TTT_CKPT_FACTORS (bf16 I/O,
+  /// interval 1, head_dim <= 96: the update factors and the final state, least traffic).  No counterpart in
+  /// the reference's config.
+  int checkpoint_format = TTT_CKPT_F32;
   /// ttt_desc.kernel_hint (TTT_HINT_AUTO: the library chooses the kernels).
   int kernel_hint = TTT_HINT_AUTO;
 };
@@ -133,7 +135,7 @@ class FusedTileMulti {
     d.io_dtype = dtype;
     d.state_per_batch = state_per_batch ? 1 : 0;
     d.seq_stride = 0;
-    d.checkpoint_format = config_.ttt.packed_checkpoints ? TTT_CKPT_PACKED : TTT_CKPT_F32;
+    d.checkpoint_format = config_.ttt.checkpoint_format;
     d.kernel_hint = config_.ttt.kernel_hint;
     return d;
   }

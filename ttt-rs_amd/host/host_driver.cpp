@@ -23,7 +23,7 @@ const char* ttt_host_last_error(void) { return g_msg; }
 // TTT-Linear: forward over `seq` tokens (any length), state buffers {w,b}[2] of [B,H,d,d] / [B,H,d];
 // on return *cur says which of the two pairs holds the final state.  ck_w/ck_b may be null.
 int ttt_host_linear_forward(int B, int H, int d, int K, int seq, int dtype, float eps, int ckpt_interval,
-                            int packed, const float* W0, const float* b0, const float* gamma, const float* beta,
+                            int ckpt_format, const float* W0, const float* b0, const float* gamma, const float* beta,
                             const void* xq, const void* xk, const void* xv, const float* token_eta, const void* lr,
                             void* out, float* w_a, float* b_a, float* w_b, float* b_b, float* ck_w, float* ck_b,
                             int* cur, void* stream) {
@@ -34,7 +34,7 @@ int ttt_host_linear_forward(int B, int H, int d, int K, int seq, int dtype, floa
     cfg.ttt.mini_batch_size = K;
     cfg.ttt.epsilon = eps;
     cfg.ttt.checkpoint_interval = ckpt_interval;
-    cfg.ttt.packed_checkpoints = packed != 0;
+    cfg.ttt.checkpoint_format = ckpt_format;
     ttt::FusedTileMulti model(cfg, W0, b0, gamma, beta);
     ttt::TTTInputsInner in;
     in.qkv = ttt::Qkv{xq, xk, xv};
@@ -54,7 +54,7 @@ int ttt_host_linear_forward(int B, int H, int d, int K, int seq, int dtype, floa
 }
 
 int ttt_host_linear_backward(int B, int H, int d, int K, int seq, int dtype, float eps, int ckpt_interval,
-                             int packed, const float* W0, const float* b0, const float* gamma,
+                             int ckpt_format, const float* W0, const float* b0, const float* gamma,
                              const float* beta, const void* xq, const void* xk, const void* xv,
                              const float* token_eta, const void* lr, const float* ck_w, const float* ck_b,
                              const void* d_out, void* d_xq, void* d_xk, void* d_xv, float* d_W, float* d_b,
@@ -66,7 +66,7 @@ int ttt_host_linear_backward(int B, int H, int d, int K, int seq, int dtype, flo
     cfg.ttt.mini_batch_size = K;
     cfg.ttt.epsilon = eps;
     cfg.ttt.checkpoint_interval = ckpt_interval;
-    cfg.ttt.packed_checkpoints = packed != 0;
+    cfg.ttt.checkpoint_format = ckpt_format;
     ttt::FusedTileMulti model(cfg, W0, b0, gamma, beta);
     ttt::TTTInputsInner in;
     in.qkv = ttt::Qkv{xq, xk, xv};

@@ -132,8 +132,10 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
     Counterpart of fused_ttt_tile_forward_multi (rust/fused/src/linear_fused_tile/api.rs:52-83):
     weight [B,H,d,d] or [H,d,d], bias [B,H,d] or [H,d], token_eta [>=K] (first K entries used).
     Returns (output, weight_out, bias_out[, weight_ckpt, bias_ckpt]).
-    packed_checkpoints (bf16 I/O, interval 1): W checkpoints as bf16 operand fragments in kernel order, to be
-    handed to ttt_linear_backward_raw with the same flag; the tensor keeps its f32 [B,H,n,d,d] allocation.
+    packed_checkpoints is ttt_desc.checkpoint_format: False/0 f32 matrices; True/1 (interval 1) W checkpoints as
+    operand fragments in kernel order; 2 (bf16 I/O, interval 1, d <= 96) the update factors and the final state
+    instead of states.  The result is to be handed to ttt_linear_backward_raw with the same value; the tensors keep
+    their f32 [B,H,n,d,d] / [B,H,n,d] allocations whatever the format.
     """
     B, H, seq, d = xq.shape
     io = xq.dtype
