@@ -1,0 +1,134 @@
+"""GPU: the entry points can be recorded into a HIP graph and replayed.
+
+The library enqueues kernels on the caller's stream and nothing else: outputs that are accumulated with atomics are
+cleared by fill kernels, not by memset nodes (memset nodes recorded into a graph have given wrong results on
+replays after the first), and per-kernel set-up (the request for more than 64 KiB of LDS) happens on the first
+eager call of a kernel, which a caller makes before capturing anyway.  Every test records one call sequence,
+replays it several times with eager work and synchronisations of the program in between, and compares every
+replay with the eager result of the same inputs: bit for bit where nothing is accumulated with atomics, to 1e-5
+where it is (d_token_eta, d_gamma, d_beta: the order of the atomic additions is free).
+"""
+import importlib
+
+import pytest
+import torch
+
+from helpers import assert_close, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+ATOMIC = ("grad_token_eta", "grad_ln_weight", "grad_ln_bias")
+
+
+def replay_and_compare(record, eager, refresh, names_atomic=()):
+    """record(): the calls to capture, returning a dict of output tensors; eager(): the same calls outside a graph;
+    refresh(i): overwrite the (static) input tensors in place with the i-th set of values."""
+    refresh(0)
+    eager()  # first eager call: per-kernel set-up happens here, not under capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            held = record()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for i in (1, 2, 0, 3):
+        refresh(i)
+        want = {k: v.clone() for k, v in eager().items()}
+        torch.cuda.synchronize()
+        for v in held.values():  # what the replay must overwrite
+            v.fill_(float("nan")) if v.is_floating_point() else v.zero_()
+        scratch = torch.randn(1 << 16, device="cuda:0").sum()  # the program's own eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(scratch)
+        for k, v in want.items():
+            if k in names_atomic:
+                assert_close(held[k], v.double(), 1e-5, f"replay {i} {k}", min_frac=0.99)
+            else:
+                assert torch.equal(held[k], v), f"replay {i}: {k} differs from the eager call"
+
+
+@pytest.mark.parametrize("dtype,fmt", [(torch.float32, 0), (torch.bfloat16, 1), (torch.bfloat16, 2)],
+                         ids=["f32", "bf16-packed", "bf16-factors"])
+def test_linear_forward_backward_replays(P, dtype, fmt):
+    B, H, d, K, N = 2, 3, 64, 16, 6
+    print(f"case graph capture linear fwd+bwd {dtype} format {fmt}", flush=True)
+    sets = [to_dev(P.synthetic.reference_test_inputs(900 + i, B, H, N * K, d, K, io_dtype=dtype)) for i in range(4)]
+    gen = torch.Generator().manual_seed(5)
+    douts = [torch.randn(B, H, N * K, d, generator=gen).to(dtype).to("cuda:0") for _ in range(4)]
+    x = {k: v.clone() for k, v in sets[0].items()}
+    dO = douts[0].clone()
+
+    def refresh(i):
+        for k in x:
+            x[k].copy_(sets[i][k])
+        dO.copy_(douts[i])
+
+    def calls():
+        out, W, b, Wc, bc = P.ttt_linear_forward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"],
+                                                     x["gamma"], x["beta"], K, 1e-6, 1, want_checkpoints=True,
+                                                     packed_checkpoints=fmt)
+        g = P.ttt_linear_backward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"], x["gamma"],
+                                      x["beta"], Wc, bc, dO, K, 1e-6, 1, packed_checkpoints=fmt)
+        return dict(out=out, W=W, b=b, **g)
+
+    replay_and_compare(calls, calls, refresh, ATOMIC)
+
+
+@pytest.mark.parametrize("d", [64, 128], ids=["d64-one-cu", "d128-two-cus"])
+def test_mlp_forward_replays(P, d):
+    B, H, K, N = 1, 2, 16, 4
+    print(f"case graph capture mlp fwd d{d}", flush=True)
+    sets = [to_dev(P.synthetic.baseline_inputs(940 + i, B, H, N * K, d, K, io_dtype=torch.bfloat16, mlp=True))
+            for i in range(4)]
+    x = {k: v.clone() for k, v in sets[0].items()}
+
+    def refresh(i):
+        for k in x:
+            x[k].copy_(sets[i][k])
+
+    def calls():
+        r = P.ttt_mlp_forward_raw(x["xq"], x["xk"], x["xv"], x["W1"], x["b1"], x["W2"], x["b2"], x["token_eta"], x["lr"],
+                                  x["gamma"], x["beta"], K)
+        return dict(zip(("out", "W1", "b1", "W2", "b2"), r))
+
+    replay_and_compare(calls, calls, refresh)
+
+
+@pytest.mark.parametrize("streams", [1, 2], ids=["one-stream", "two-streams"])
+def test_stack_wavefront_replays(P, streams):
+    """ttt_stack_fwd as a wavefront over sequence windows.  With a second stream the call forks from the stream it is
+    given and joins it again before it returns (events), which a capture records as parallel branches."""
+    from test_stack_gpu import make_layers
+    B, H, d, K, seq, chunk = 2, 2, 64, 16, 128, 32
+    kinds = [False, True, False, True]
+    print(f"case graph capture stack, {streams} stream(s)", flush=True)
+    sets = [[{k: v.to("cuda:0") for k, v in L.items()}
+             for L in make_layers(P, B, H, seq, d, K, torch.bfloat16, kinds, seed0=300 + 10 * i)] for i in range(4)]
+    x = [{k: v.clone() for k, v in L.items()} for L in sets[0]]
+    aux = torch.cuda.Stream("cuda:0") if streams == 2 else None
+
+    def refresh(i):
+        for L, S in zip(x, sets[i]):
+            for k in L:
+                L[k].copy_(S[k])
+
+    def calls():
+        out, states = P.ttt_stack_forward_raw(x, x[0]["token_eta"], K, chunk_tokens=chunk, aux_stream=aux)
+        res = dict(out=out)
+        for li, st in enumerate(states):
+            for si, t in enumerate(st):
+                res[f"state{li}_{si}"] = t
+        return res
+
+    replay_and_compare(calls, calls, refresh)
