@@ -422,10 +422,18 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         IO::mma2(zb[jj], wa0, wa1, q[2 * qq], q[2 * qq + 1]);
       }
     }
-    {
-      f32x4 at = zero4, at2 = zero4;
-      mma_own(at, ko, qo);   // [s = 4g+r][t = c]
-      mma_own(at2, qo, ko);  // [t = 4g+r][s = c]
+    // bf16: every wave forms the whole attention block itself (it holds the full rows of XQ and XK anyway, and the
+    // matrix pipe has room): two k = 32 instructions per orientation instead of one partial block per wave that
+    // crosses LDS (a write, NW reads and NW - 1 vector additions per orientation).  f32 products are bound by the
+    // matrix pipe, there the waves share the work; so they do at d = 128, where the register file is full.
+    constexpr bool FULL_AT = BF && D <= 96;
+    f32x4 at = zero4, at2 = zero4;
+    if constexpr (FULL_AT) {
+      mma_all(at, k, q);   // [s = 4g+r][t = c]
+      mma_all(at2, q, k);  // [t = 4g+r][s = c]
+    } else {
+      mma_own(at, ko, qo);
+      mma_own(at2, qo, ko);
       pt(P_AT, w) = at;
       pt(P_AT2, w) = at2;
     }
@@ -477,7 +485,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     // ---- eta, tril(A), M = eta (1 + A) in both orientations
     f32x4 eta, onepA, eta2, onepA2, nM, M2;
     {
-      const f32x4 At = ptsum(P_AT), At2 = ptsum(P_AT2);
+      const f32x4 At = FULL_AT ? at : ptsum(P_AT), At2 = FULL_AT ? at2 : ptsum(P_AT2);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const bool low = 4 * g + r <= c;
