@@ -44,8 +44,8 @@ struct LinBwdMwLds {
   static constexpr int LR = X + 4 * XS * 1024;        // 16 dwords: lr of token c (bf16 zero-extended, or f32)
   static constexpr int SUM = LR + 256;                // 3 exchanges x [8 sums][16 tokens][NW]
   static constexpr int PT = SUM + 3 * 8 * 16 * NW * 4;  // 4 kinds x [NW][64] f32x4: partial [16 x 16] blocks
-  static constexpr int FR = PT + 4 * NW * 1024;       // 7 kinds x [NT][64] fragments
-  static constexpr int M0 = FR + 7 * NT * FT;         // D row means of the initial W, then mean(b): the centred state
+  static constexpr int FR = PT + 4 * NW * 1024;       // 9 kinds x [NT][64] fragments
+  static constexpr int M0 = FR + 9 * NT * FT;         // D row means of the initial W, then mean(b): the centred state
   static constexpr int GDS = M0 + (D + 4) * 4;         // FM: NT half slots: the factor fragments of tile J
   static constexpr int BYTES = GDS + (FM ? NT * 512 : 0);
   static_assert(!FM || (PK && ES == 2), "factors: bf16 I/O, packed image of the state");
@@ -64,8 +64,12 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
   using L = LinBwdMwLds<D, NW, ES, PK, FM>;
   constexpr int NT = D / 16, TPW = NT / NW, NQ = NT / 2, XS = L::XS;
   constexpr float inv_d = 1.0f / D;
-  enum { KD = 0, QD, GF, ZF, ZD, Z1F, Z1D };
+  enum { KD = 0, QD, GF, ZF, ZD, Z1F, Z1D, GL, ZL };
   enum { P_AT = 0, P_AT2, P_P, P_P2 };
+  // bf16, d <= 96: the [16 x 16] blocks that contract over all d features (attention, P = dZbar G^T) are formed
+  // whole by every wave on the matrix pipe, from fragments that cross LDS anyway, instead of per-wave partial
+  // blocks that are written, read NW times and added up on the VALU
+  constexpr bool FULL_AT = BF && D <= 96;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
   const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
@@ -287,7 +291,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
   // FM: the state entering the mini-batch whose copies are staged: W_t = W_{t+1} - XK_t^T G''_t and
   // b_t = b_{t+1} - colsum G''_t, with the operands the forward multiplied (XK as staged, G'' as saved).  This wave's
   // column tiles of the f32 state are updated in its registers and their packed image is written where the products
-  // of the next pass read it.  Runs in the tail of the pass before (the staged rows have all been moved to registers, the
+  // of the next pass read it.  Runs at the end of the pass before (the staged rows have all been moved to registers, the
   // packed image of the current state is no longer read), so it is off the chain of dependent exchanges.
   auto walk_back = [&]() {
     if constexpr (FM) {
@@ -426,7 +430,6 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     // matrix pipe has room): two k = 32 instructions per orientation instead of one partial block per wave that
     // crosses LDS (a write, NW reads and NW - 1 vector additions per orientation).  f32 products are bound by the
     // matrix pipe, there the waves share the work; so they do at d = 128, where the register file is full.
-    constexpr bool FULL_AT = BF && D <= 96;
     f32x4 at = zero4, at2 = zero4;
     if constexpr (FULL_AT) {
       mma_all(at, k, q);   // [s = 4g+r][t = c]
@@ -543,19 +546,25 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
           // P feeds the gradients of eta (small differences of large sums): bf16 head + tail of both factors
           Gl[jj] = IO::to_frag(G[jj] - IO::to_f32(Gf[jj]));
           Zl[jj] = IO::to_frag(dzb - IO::to_f32(Zf[jj]));
+          if constexpr (FULL_AT) {
+            fr(GL, w * TPW + jj) = Gl[jj];
+            fr(ZL, w * TPW + jj) = Zl[jj];
+          }
         }
       }
-      // ---- partial P = dZb G^T in both orientations
-      mma_own(P, Gf, Zf);   // [s][t]
-      mma_own(P2, Zf, Gf);  // [t][s]
-      if (BF) {
-        mma_own(P, Gl, Zf);
-        mma_own(P, Gf, Zl);
-        mma_own(P2, Zl, Gf);
-        mma_own(P2, Zf, Gl);
+      // ---- partial P = dZb G^T in both orientations (FULL_AT: formed whole behind the next exchange)
+      if constexpr (!FULL_AT) {
+        mma_own(P, Gf, Zf);   // [s][t]
+        mma_own(P2, Zf, Gf);  // [t][s]
+        if (BF) {
+          mma_own(P, Gl, Zf);
+          mma_own(P, Gf, Zl);
+          mma_own(P2, Zl, Gf);
+          mma_own(P2, Zf, Gl);
+        }
+        pt(P_P, w) = P;
+        pt(P_P2, w) = P2;
       }
-      pt(P_P, w) = P;
-      pt(P_P2, w) = P2;
     }
     // ---- DGM = M^T dZb (own features) ; X3: the partial P blocks and dZb / G fragments travel with the six
     //      sums of the second-order LayerNorm, none of which needs P
@@ -600,17 +609,35 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
         IO::mma2(TMP[ii], IO::to_frag(DT[2 * qq][ii]), IO::to_frag(DT[2 * qq + 1][ii]), Gfa[2 * qq], Gfa[2 * qq + 1]);
     }
     xcol(2, S4);
+    frag Zfa[NT];
+#pragma unroll
+    for (int J = 0; J < NT; ++J) Zfa[J] = fr(ZF, J);
     f32x4 dA, dEta, dA2, dEta2;
     {
-      const f32x4 P = ptsum(P_P), P2 = ptsum(P_P2);
+      f32x4 P, P2;
+      if constexpr (FULL_AT) {
+        frag Gla[NT], Zla[NT];
+#pragma unroll
+        for (int J = 0; J < NT; ++J) {
+          Gla[J] = fr(GL, J);
+          Zla[J] = fr(ZL, J);
+        }
+        P = P2 = zero4;
+        mma_all(P, Gfa, Zfa);   // [s][t]
+        mma_all(P2, Zfa, Gfa);  // [t][s]
+        mma_all(P, Gla, Zfa);
+        mma_all(P2, Zla, Gfa);
+        mma_all(P, Gfa, Zla);
+        mma_all(P2, Zfa, Gla);
+      } else {
+        P = ptsum(P_P);
+        P2 = ptsum(P_P2);
+      }
       dA = -P * eta;
       dEta = -P * onepA;
       dA2 = -P2 * eta2;
       dEta2 = -P2 * onepA2;
     }
-    frag Zfa[NT];
-#pragma unroll
-    for (int J = 0; J < NT; ++J) Zfa[J] = fr(ZF, J);
     // ---- dXQ = dO + dZb W^T + dA XK   (own features)
     {
       const frag dAf = IO::to_frag(dA);
@@ -672,9 +699,6 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
     }
     lds_barrier();
-    // (behind the first mini-batch of the sequence nothing new is staged: the walk then works on stale rows, its
-    // result is never read, and the loop keeps one shape)
-    if constexpr (FM) walk_back();
     {
       frag Z1fa[NT];
 #pragma unroll
@@ -714,6 +738,11 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     }
 #pragma unroll
     for (int jj = 0; jj < TPW; ++jj) IO::mma2(dbT[jj], Zd[jj], Z1d[jj], ones, ones);
+    // FM: the state entering the next mini-batch of the scan.  Placed last: its short dependent chain (transposes,
+    // products, conversions, LDS writes) then runs behind the state-gradient products instead of in front of the
+    // dXK products and stores (measured 479 -> 463 us).  Behind the first mini-batch of the sequence nothing new is
+    // staged: the walk then works on stale rows, its result is never read, and the loop keeps one shape.
+    if constexpr (FM) walk_back();
   }
 
   // ---- results carried over the whole scan
