@@ -311,8 +311,18 @@ int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
 // one checkpoint per mini-batch, NW waves per (batch, head): feature axis split, exchanges through LDS
 template <class T, int D, int NW, bool PK = false, bool FM = false>
 int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK, FM>;
   constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem), PK, FM>::BYTES;
+  // bf16 I/O with opaque checkpoints (the training path): a variant for whole mini-batches of 16 tokens
+  if constexpr (PK && sizeof(typename ttt::Io<T>::elem) == 2) {
+    if (a.K == 16) {
+      constexpr auto kern16 = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK, FM, true>;
+      int rc = opt_in_lds<kern16>(bytes);
+      if (rc != TTT_OK) return rc;
+      hipLaunchKernelGGL(kern16, dim3(grid), dim3(64 * NW), bytes, s, a);
+      return hip_status(hipGetLastError(), "ttt_linear_bwd (multi-wave register-resident kernel) launch");
+    }
+  }
+  constexpr auto kern = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK, FM>;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), bytes, s, a);

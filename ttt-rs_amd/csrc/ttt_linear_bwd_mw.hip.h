@@ -54,7 +54,9 @@ struct LinBwdMwLds {
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
 
-template <class T, int D, int NW, bool PK = false, bool FM = false>
+// FULL: mini_batch == 16, every lane's token exists: the stores and copies of a mini-batch need no lane mask (and no
+// branch around them, which would also end the block the scheduler can reorder within)
+template <class T, int D, int NW, bool PK = false, bool FM = false, bool FULL = false>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using frag = typename IO::frag;
@@ -194,7 +196,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     for (int ten = 0; ten < 4; ++ten) {
       if (ten % NW != w) continue;
       const elem* src = static_cast<const elem*>(ten == 0 ? a.xq : ten == 1 ? a.xk : ten == 2 ? a.xv : a.d_out) + tok0;
-      if (c < K) {
+      if (FULL || c < K) {
 #pragma unroll
         for (int s = 0; s < XS; ++s) {
           // bf16: 8 features of tiles 2s, 2s+1; f32: the 4 features of tile s
@@ -379,9 +381,9 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       const uint32_t* lrw = reinterpret_cast<const uint32_t*>(smem + L::LR);
       const u32x4 w4 = *reinterpret_cast<const u32x4*>(lrw + 4 * g);
       auto cv = [&](uint32_t x) { return BF ? __uint_as_float(x << 16) : __uint_as_float(x); };
-      lr_c = (c < K) ? cv(lrw[c]) : 0.f;
+      lr_c = (FULL || c < K) ? cv(lrw[c]) : 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) lr_s[r] = (4 * g + r < K) ? cv(w4[r]) : 0.f;
+      for (int r = 0; r < 4; ++r) lr_s[r] = (FULL || 4 * g + r < K) ? cv(w4[r]) : 0.f;
     }
     f32x4 bT[TPW];
     frag Wn[TPW][NT], kdo[TPW], qdo[TPW];
@@ -568,7 +570,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     }
     // ---- DGM = M^T dZb (own features) ; X3: the partial P blocks and dZb / G fragments travel with the six
     //      sums of the second-order LayerNorm, none of which needs P
-    const bool tok_ok = c < K;
+    const bool tok_ok = FULL || c < K;
     const size_t tokoff = (bh * (size_t)a.seq_stride + (size_t)st * K + c) * D;
     f32x4 dK[TPW], DGM[TPW], TMP[TPW];
     {
