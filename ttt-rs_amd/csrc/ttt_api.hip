@@ -312,8 +312,8 @@ int launch_linear_bwd_rr(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
 template <class T, int D, int NW, bool PK = false, bool FM = false>
 int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
   constexpr size_t bytes = ttt::LinBwdMwLds<D, NW, sizeof(typename ttt::Io<T>::elem), PK, FM>::BYTES;
-  // bf16 I/O with opaque checkpoints (the training path): a variant for whole mini-batches of 16 tokens
-  if constexpr (PK && sizeof(typename ttt::Io<T>::elem) == 2) {
+  // opaque checkpoints (the training path): a variant for whole mini-batches of 16 tokens
+  if constexpr (PK) {
     if (a.K == 16) {
       constexpr auto kern16 = ttt::ttt_linear_bwd_mw_kernel<T, D, NW, PK, FM, true>;
       int rc = opt_in_lds<kern16>(bytes);
