@@ -56,8 +56,12 @@ struct LinBwdMwLds {
 
 // FULL: mini_batch == 16, every lane's token exists: the stores and copies of a mini-batch need no lane mask (and no
 // branch around them, which would also end the block the scheduler can reorder within)
+// Up to d = 64 with one feature tile per wave the kernel is held to 256 registers: two workgroups then share a compute
+// unit (two waves per SIMD), which is what 257 registers would silently halve (f32 I/O with f32 row-major checkpoints
+// excepted: it needs 265 and would spill).
 template <class T, int D, int NW, bool PK = false, bool FM = false, bool FULL = false>
-__global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArgs a) {
+__global__ void __launch_bounds__(64 * NW, (D <= 64 && D / 16 == NW && (PK || sizeof(typename Io<T>::elem) == 2)) ? 2 : 1)
+    ttt_linear_bwd_mw_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;
@@ -709,25 +713,30 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
       for (int ii = 0; ii < TPW; ++ii) mma_all(dK[ii], Wn[ii], Z1fa);
       if (tok_ok) store_own(a.d_xk, tokoff, dK);
     }
-    // ---- d lr (first wave), d token_eta (last wave): work of a single wave is skew at the next barrier
-    if (w == 0) {
-      float e2 = 0.f;
+    // ---- d lr (first wave), d token_eta (last wave): work of a single wave is skew at the next barrier.  Where it
+    // goes is a matter of measurement: in front of the state-gradient products when the walk back follows them
+    // (451 against 454 us at B = 32, 335 against 350 at B = 16), behind them otherwise (packed states 450 -> 438 us,
+    // f32 741 -> 726 us)
+    auto single_wave_outputs = [&]() {
+      if (w == 0) {
+        float e2 = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) e2 += dEta2[r] * te_s[r];
-      const float dlr = xg_sum(e2) + te_last * dl;
-      if (g == 0 && tok_ok)
-        IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + c, dlr);
-    }
-    if (w == NW - 1) {
-      float e1 = 0.f;
+        for (int r = 0; r < 4; ++r) e2 += dEta2[r] * te_s[r];
+        const float dlr = xg_sum(e2) + te_last * dl;
+        if (g == 0 && tok_ok)
+          IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + c, dlr);
+      }
+      if (w == NW - 1) {
+        float e1 = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) e1 += dEta[r] * lr_s[r];
-      float dte = xg_sum(e1);
-      const float tail = row16_sum_dpp(dl * lr_c);
-      if (c == K - 1) dte += tail;
-      if (g == 0 && tok_ok) atomicAdd(a.d_token_eta + (size_t)st * K + c, dte);
-    }
-
+        for (int r = 0; r < 4; ++r) e1 += dEta[r] * lr_s[r];
+        float dte = xg_sum(e1);
+        const float tail = row16_sum_dpp(dl * lr_c);
+        if (c == K - 1) dte += tail;
+        if (g == 0 && tok_ok) atomicAdd(a.d_token_eta + (size_t)st * K + c, dte);
+      }
+    };
+    if constexpr (FM) single_wave_outputs();
     // ---- state gradient: dW += XQ^T dZb + XK^T dZ1 (column slice and transposed row slice), db
 #pragma unroll
     for (int I = 0; I < NT; ++I) {
@@ -740,6 +749,7 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_bwd_mw_kernel(LinearBwdArg
     }
 #pragma unroll
     for (int jj = 0; jj < TPW; ++jj) IO::mma2(dbT[jj], Zd[jj], Z1d[jj], ones, ones);
+    if constexpr (!FM) single_wave_outputs();
     // FM: the state entering the next mini-batch of the scan.  Placed last: its short dependent chain (transposes,
     // products, conversions, LDS writes) then runs behind the state-gradient products instead of in front of the
     // dXK products and stores (measured 479 -> 463 us).  Behind the first mini-batch of the sequence nothing new is
