@@ -28,6 +28,13 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
   constexpr float inv_d = 1.0f / D;
   static_assert(NW > 1, "the skewed kernel is for two or more waves per unit");
   __shared__ float ex[2][8 * 16 * NW];
+  // f32 products with one feature tile per wave are bound by the f32 matrix instructions: the waves then share what
+  // each would otherwise compute for itself.  Every wave transposes its own XK tile and forms the attention block over
+  // its own 16 features; both cross LDS with the row sums (same barrier, same double buffering) and are read back
+  // behind it: 8 matrix instructions per wave and mini-batch instead of 32.
+  constexpr bool SHARE = !BF && TPW == 1;
+  __shared__ f32x4 kdx[SHARE ? 2 : 1][SHARE ? NT : 1][64];
+  __shared__ f32x4 atx[SHARE ? 2 : 1][SHARE ? NW : 1][64];
 
   const int lane = threadIdx.x & 63, w = (threadIdx.x >> 6) % NW;
   const int c = lane & 15, g = lane >> 4;
@@ -181,11 +188,17 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
       // ---- XK with tokens along k for the state update: depends on nothing computed here, so it
       // is issued first and fills the gaps of the dependent chain below
       frag kd[NT];
-#pragma unroll
-      for (int I = 0; I < NT; ++I) {
+      if constexpr (SHARE) {
         f32x4 t = {0.f, 0.f, 0.f, 0.f};
-        IO::mma(t, cur.k[I], ident_upd);  // t[r] = XK[s = 4g+r][feat(I,c)]
-        kd[I] = IO::to_frag(t);
+        IO::mma(t, cur.ko[0], ident_upd);  // the own tile; the others come back from LDS behind the barrier
+        kdx[st & 1][w][lane] = t;
+      } else {
+#pragma unroll
+        for (int I = 0; I < NT; ++I) {
+          f32x4 t = {0.f, 0.f, 0.f, 0.f};
+          IO::mma(t, cur.k[I], ident_upd);  // t[r] = XK[s = 4g+r][feat(I,c)]
+          kd[I] = IO::to_frag(t);
+        }
       }
       // ---- Z1^T, Zbar^T (this wave's feature rows) and the attention block
       f32x4 z1[TPW], zb[TPW], At = {0.f, 0.f, 0.f, 0.f};
@@ -202,7 +215,11 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
           IO::mma2(z1[jj], w0, w1, cur.k[2 * q], cur.k[2 * q + 1]);
           IO::mma2(zb[jj], w0, w1, cur.q[2 * q], cur.q[2 * q + 1]);
         }
-        IO::mma2(At, cur.k[2 * q], cur.k[2 * q + 1], cur.q[2 * q], cur.q[2 * q + 1]);
+        if constexpr (!SHARE) IO::mma2(At, cur.k[2 * q], cur.k[2 * q + 1], cur.q[2 * q], cur.q[2 * q + 1]);
+      }
+      if constexpr (SHARE) {
+        IO::mma(At, cur.ko[0], cur.qo[0]);  // over the own 16 features
+        atx[st & 1][w][lane] = At;
       }
       // ---- row sums: six raw moments of Z1 (this mini-batch), two of the pending Zbar
       f32x4 bq[TPW];
@@ -251,6 +268,13 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
       for (int jj = 0; jj < TPW; ++jj) {
         zbo[jj] = zbp[jj];
         qoo[jj] = qop[jj];
+      }
+      if constexpr (SHARE) {
+#pragma unroll
+        for (int I = 0; I < NT; ++I) kd[I] = IO::to_frag(kdx[st & 1][I][lane]);
+        At = atx[st & 1][0][lane];
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) At += atx[st & 1][ww][lane];
       }
 
       // ---- recurrence: G'' , causal correction, state update
