@@ -501,9 +501,11 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   copy_or_zero(d_b1, d_b1_out, U * M, s);
   copy_or_zero(d_W2, d_W2_out, U * M * D, s);
   copy_or_zero(d_b2, d_b2_out, U * D, s);
-  copy_or_zero(d_token_eta, nullptr, (size_t)d->seq, s);
-  copy_or_zero(d_gamma, nullptr, (size_t)d->heads * D, s);
-  copy_or_zero(d_beta, nullptr, (size_t)d->heads * D, s);
+  {
+    const size_t hd = (size_t)d->heads * D, nmax = (size_t)d->seq > hd ? (size_t)d->seq : hd;
+    hipLaunchKernelGGL(ttt::ttt_fill_zero3_kernel, dim3((unsigned)((nmax + 255) / 256)), dim3(256), 0, s, d_token_eta,
+                       (size_t)d->seq, d_gamma, hd, d_beta, hd);
+  }
   rc = hip_status(hipGetLastError(), "ttt_mlp_bwd fills");
   if (rc != TTT_OK) return rc;
 
@@ -678,12 +680,11 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   // accumulated outputs start from zero; a fill kernel (not a memset node) so the sequence
   // can be captured into a graph
   const size_t hd = (size_t)d->heads * d->head_dim;
-  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((d->seq + 255) / 256)), dim3(256), 0, s,
-                     d_token_eta, (size_t)d->seq);
-  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((hd + 255) / 256)), dim3(256), 0, s,
-                     d_gamma, hd);
-  hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((hd + 255) / 256)), dim3(256), 0, s,
-                     d_beta, hd);
+  {
+    const size_t nmax = (size_t)d->seq > hd ? (size_t)d->seq : hd;
+    hipLaunchKernelGGL(ttt::ttt_fill_zero3_kernel, dim3((unsigned)((nmax + 255) / 256)), dim3(256), 0, s, d_token_eta,
+                       (size_t)d->seq, d_gamma, hd, d_beta, hd);
+  }
   const unsigned grid = (unsigned)(a.B * a.H);
   const bool f32 = d->io_dtype == TTT_F32;
   const int waves = ch.waves;

@@ -455,6 +455,14 @@ __global__ void ttt_fill_zero_kernel(float* p, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0.f;
 }
+// three small buffers in one launch (the accumulated outputs of a backward: every launch costs a few microseconds
+// on the stream whatever it does)
+__global__ void ttt_fill_zero3_kernel(float* p0, size_t n0, float* p1, size_t n1, float* p2, size_t n2) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n0) p0[i] = 0.f;
+  if (i < n1) p1[i] = 0.f;
+  if (i < n2) p2[i] = 0.f;
+}
 
 // tanh-approximated GELU and its derivative (reference rust/thundercube/src/unary_ops.rs:136-173)
 __device__ __forceinline__ void gelu_tanh_pair(float x, float& y, float& dy) {
