@@ -207,7 +207,8 @@ def test_bwd_packed_checkpoints_change_nothing(P, B, H, d, K, N, waves, dtype):
 
 
 @pytest.mark.parametrize("B,H,d,K,N", [(2, 2, 32, 8, 3), (2, 3, 64, 16, 8), (1, 2, 64, 5, 3), (1, 2, 96, 16, 3),
-                                       (1, 2, 64, 16, 1), (1, 3, 64, 16, 2), (1, 2, 64, 16, 40)])
+                                       (1, 2, 64, 16, 1), (1, 3, 64, 16, 2), (1, 2, 64, 16, 40), (1, 2, 96, 16, 24),
+                                       (2, 1, 32, 16, 48), (1, 2, 96, 7, 5)])
 @pytest.mark.parametrize("eta_last", ["positive", "zero"])
 def test_bwd_from_update_factors(P, B, H, d, K, N, eta_last):
     """checkpoint_format 2 (bf16 I/O): the forward saves the final state and the [16 x d] factor of every state
