@@ -217,14 +217,18 @@ def run_workload(name, a, pkg, torch):
                                           mlp=kind in ("mlp_fwd", "mlp_fwd_bwd"))
         dv = {k: v.to(dev) for k, v in c.items()}
         if kind in ("linear_fwd", "linear_fwd_bwd"):
-            # a checkpoint per mini-batch: what is saved for the backward is the library's cheapest form for the shape
-            # ("auto"): bf16 I/O up to 512 units and head_dim 96, the update factors and the final state (a quarter of
-            # the packed bytes; the feature-split backward walks the states back); otherwise the states as operand
-            # fragments in kernel order ("packed").  --checkpoint-format f32 keeps the reference's f32 matrices.
+            # a checkpoint per mini-batch: what is saved for the backward is the form the library names as the cheapest
+            # for the shape ("auto", ttt_linear_best_checkpoint_format): bf16 I/O up to 512 units and head_dim 96, the
+            # update factors and the final state (a quarter of the packed bytes; the feature-split backward walks the
+            # states back); otherwise the states as operand fragments in kernel order ("packed").
+            # --checkpoint-format f32 keeps the reference's f32 matrices.
             ckfmt = 0
             if kind == "linear_fwd_bwd" and ci == 1:
-                fits = dtype == torch.bfloat16 and d <= 96 and B * H <= 512 and seq // K >= 2
-                ckfmt = {"f32": 0, "packed": 1, "factors": 2, "auto": 2 if fits else 1}[a.checkpoint_format]
+                import ctypes as C
+                probe = pkg.TttDesc(B, H, seq, d, K, 1e-6, ci, pkg.TTT_BF16 if dtype == torch.bfloat16 else pkg.TTT_F32,
+                                    0, 0, 0, 0)
+                best = pkg.lib().ttt_linear_best_checkpoint_format(C.byref(probe))
+                ckfmt = {"f32": 0, "packed": 1, "factors": 2, "auto": best}[a.checkpoint_format]
             calls = LinearCalls(pkg, dv, B, H, seq, d, K, dtype, ci, ckfmt, kind == "linear_fwd_bwd")
             if kind == "linear_fwd":
                 parts = [("ttt_linear_fwd", calls.fwd)]

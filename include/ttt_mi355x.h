@@ -113,6 +113,12 @@ int64_t ttt_linear_num_checkpoints(const ttt_desc* desc);
  * ttt_linear_bwd would return.  A training caller asks this before the forward, as the reference asks
  * FusedTttConfig::is_supported (rust/fused/src/lib.rs:313-322) before it builds the layer. */
 int ttt_linear_bwd_supported(const ttt_desc* desc);
+/* The checkpoint_format that makes ttt_linear_fwd + ttt_linear_bwd fastest for this desc (its own checkpoint_format
+ * field is not read) when nothing but ttt_linear_bwd reads the checkpoints: TTT_CKPT_FACTORS for bf16 I/O,
+ * checkpoint_interval 1, head_dim <= 96, two or more mini-batches and up to 512 (batch, head) units; else
+ * TTT_CKPT_PACKED for checkpoint_interval 1; else TTT_CKPT_F32.  Negative if the desc is invalid.  No counterpart
+ * in the reference (its checkpoints have one format). */
+int ttt_linear_best_checkpoint_format(const ttt_desc* desc);
 
 /*
  * TTT-Linear multi-stage forward.  Replaces

@@ -58,6 +58,25 @@ def test_shape_validation(P):
     assert b"checkpoint_format" in L.ttt_last_error()
 
 
+def test_best_checkpoint_format(P):
+    L = P.lib()
+    best = lambda **kw: L.ttt_linear_best_checkpoint_format(C.byref(desc(P, **kw)))
+    assert best(io_dtype=P.TTT_BF16) == 2                            # update factors
+    assert best(io_dtype=P.TTT_BF16, head_dim=96) == 2
+    assert best(io_dtype=P.TTT_BF16, checkpoint_format=0) == 2       # the desc's own format field is not read
+    assert best(io_dtype=P.TTT_BF16, head_dim=128) == 1              # packed states
+    assert best(io_dtype=P.TTT_BF16, seq=16) == 1                    # one mini-batch
+    assert best(io_dtype=P.TTT_BF16, batch=64, heads=12) == 1        # more than 512 units: single-wave backward
+    assert best(io_dtype=P.TTT_F32) == 1
+    assert best(checkpoint_interval=2) == 0 and best(io_dtype=P.TTT_BF16, checkpoint_interval=4) == 0
+    assert best(seq=33) < 0
+    # what it names is accepted by the backward
+    for kw in (dict(io_dtype=P.TTT_BF16), dict(io_dtype=P.TTT_F32), dict(io_dtype=P.TTT_BF16, head_dim=128),
+               dict(checkpoint_interval=2)):
+        fmt = best(**kw)
+        assert L.ttt_linear_bwd_supported(C.byref(desc(P, checkpoint_format=fmt, **kw))) == P.TTT_OK
+
+
 def test_num_checkpoints(P):
     L = P.lib()
     assert L.ttt_linear_num_checkpoints(C.byref(desc(P, seq=16 * 9, checkpoint_interval=4))) == 3

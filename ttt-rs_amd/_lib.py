@@ -15,6 +15,7 @@ TTT_HINT_TEST_LOST_PARTNER = 0x200
 
 EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_bwd_supported",
+    "ttt_linear_best_checkpoint_format",
     "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
     "ttt_mlp_fwd_lost_workgroups", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue",
@@ -61,6 +62,8 @@ def lib() -> C.CDLL:
         L.ttt_last_error.restype = C.c_char_p
         L.ttt_linear_supported.argtypes = [dp]
         L.ttt_linear_bwd_supported.argtypes = [dp]
+        L.ttt_linear_best_checkpoint_format.argtypes = [dp]
+        L.ttt_linear_best_checkpoint_format.restype = C.c_int
         L.ttt_linear_num_checkpoints.argtypes = [dp]
         L.ttt_linear_num_checkpoints.restype = C.c_int64
         L.ttt_linear_fwd.argtypes = [dp] + [vp] * 15

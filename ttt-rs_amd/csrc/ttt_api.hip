@@ -638,6 +638,16 @@ int ttt_linear_bwd_supported(const ttt_desc* d) {
   return choose_linear_bwd(d, &ch);
 }
 
+int ttt_linear_best_checkpoint_format(const ttt_desc* d) {
+  if (check_common(d) != TTT_OK) return -1;
+  if (d->checkpoint_interval != 1) return TTT_CKPT_F32;
+  // measured at head_dim 64 (125M shape): factors win up to 512 units, where the feature-split backward runs anyway;
+  // beyond, the single-wave backward from packed states and the feature-split one from factors are even
+  const bool factors = d->io_dtype == TTT_BF16 && d->head_dim <= 96 && d->seq / d->mini_batch >= 2 &&
+                       (int64_t)d->batch * d->heads <= 512;
+  return factors ? TTT_CKPT_FACTORS : TTT_CKPT_PACKED;
+}
+
 int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
                    const float* W0, const float* b0, const float* token_eta, const void* lr,
                    const float* gamma, const float* beta, const float* W_ckpt,
