@@ -264,7 +264,8 @@ int launch_mlp_fwd_cl2(const ttt::MlpFwdArgs* probs, int n, hipStream_t s) {
   if (rc != TTT_OK) return rc;
   const size_t units = (size_t)probs[0].B * probs[0].H, nz = units * 128 * 512;
   for (int p = 0; p < n; ++p)
-    hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, s, probs[p].W2, nz);
+    if (!probs[p].exchange_cleared)
+      hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, s, probs[p].W2, nz);
   const size_t per_launch = (size_t)(cus / 16 > 0 ? cus / 16 : 1) * 8;  // groups of 16 workgroups = 8 units
   const size_t wg_per_problem = ((units + 7) / 8) * 16;
   int together = (int)((size_t)cus / wg_per_problem);  // whole problems that fit the device at once
@@ -473,7 +474,7 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
   fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
   fa.W1 = ws + w.W1; fa.b1 = ws + w.b1; fa.W2 = ws + w.W2; fa.b2 = ws + w.b2;
-  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s; fa.unit_base = 0; fa.spin_limit = 1 << 21;
+  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s; fa.unit_base = 0; fa.spin_limit = 1 << 21; fa.exchange_cleared = 0;
   fa.B = d->batch; fa.H = d->heads; fa.seq = d->seq; fa.K = d->mini_batch;
   fa.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   fa.n_stages = d->seq / d->mini_batch;
@@ -763,7 +764,7 @@ int prepare_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const voi
   a.xq = xq; a.xk = xk; a.xv = xv; a.W1_0 = W1_0; a.b1_0 = b1_0; a.W2_0 = W2_0; a.b2_0 = b2_0;
   a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
   a.W1 = W1_out; a.b1 = b1_out; a.W2 = W2_out; a.b2 = b2_out;
-  a.G1_save = nullptr; a.G2_save = nullptr; a.unit_base = 0;
+  a.G1_save = nullptr; a.G2_save = nullptr; a.unit_base = 0; a.exchange_cleared = 0;
   a.spin_limit = (d->kernel_hint & TTT_HINT_TEST_LOST_PARTNER) ? 0 : (1 << 21);
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
   a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
@@ -969,6 +970,7 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
   };
   std::vector<ttt::LinearFwdArgs> lin;
   std::vector<ttt::MlpFwdArgs> mlp;
+  std::vector<int> mlp_first;  // the first windows of the TTT-MLP layers (indices into mlp)
   std::vector<Group> groups;
   for (int l = 0; l < n_layers; ++l) {
     const ttt_stack_layer& L = layers[l];
@@ -1045,6 +1047,7 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
           ttt::MlpFwdArgs a;
           rc = prepare_mlp_fwd(&ld, q, k, v, W1i, b1i, W2i, b2i, token_eta, lr, L.gamma, L.beta, ow, to[0], to[1], to[2], to[3], &a);
           if (rc != TTT_OK) return rc;
+          if (j == 0) mlp_first.push_back((int)mlp.size());
           mlp.push_back(a);
         }
         ++g.count;
@@ -1072,6 +1075,17 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
     hipEvent_t fork;
     if ((rc = mark(main_s, &fork)) != TTT_OK) return cleanup(rc);
     if ((rc = wait(lane_s[1], fork)) != TTT_OK) return cleanup(rc);
+  }
+  // The two-CU TTT-MLP kernel exchanges through the window's W2 output buffer, which has to be zero when it starts.
+  // Nothing reads or writes that buffer before a layer's FIRST window, so those are cleared here, while the stream
+  // of the TTT-MLP launches has nothing else to do, instead of in front of the kernel, where the fill competes with
+  // the other stream's traffic on the path to the first TTT-MLP launch (88 us in the trace instead of 7).
+  if (d->io_dtype != TTT_F32 && d->head_dim == 128 && (d->kernel_hint & TTT_HINT_LDS_TILES) == 0) {
+    const size_t nz = U * 128 * 512;
+    for (int i : mlp_first) {
+      hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, lane_s[1], mlp[i].W2, nz);
+      mlp[i].exchange_cleared = 1;
+    }
   }
   auto input_sums = [&](const std::vector<ttt::LayerInputsArgs>& v, hipStream_t s) {
     for (size_t i = 0; i < v.size(); i += ttt::kMaxProblems) {

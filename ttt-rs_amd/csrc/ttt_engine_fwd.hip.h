@@ -207,6 +207,7 @@ struct MlpFwdArgs {
   float eps;
   int unit_base;  // two-CU kernel only: first (batch, head) unit of this launch (the units are launched in batches)
   int spin_limit;  // two-CU kernel only: polls before a wait for the partner gives up (0: give up at once; testing)
+  int exchange_cleared;  // two-CU kernel only, read by the host: the exchange area (W2) has been zeroed by the caller
 };
 
 template <int D>
