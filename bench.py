@@ -91,6 +91,44 @@ def cpu_baseline(c, K, kind, budget_s=12.0):
                       f"{B} (tokens/s is batch-normalised), mean of 3 runs, {t:.3f} s per run"}
 
 
+def cpu_baseline_stack(layers_cpu, K, io_dtype, torch, B):
+    """The long-context stack on the host cores: the C/OpenMP ports of the TTT-Linear and TTT-MLP forward chained
+    layer by layer as the workload defines it (layer input = previous output + that layer's projections, sums rounded
+    to the I/O type), on batch entry 0 of the same inputs (units are independent, tokens/s is batch-normalised)."""
+    import numpy as np
+    from oracle import c_oracle
+    cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "9999")))
+    L1 = [{k: (v[:1] if k in ("xq", "xk", "xv", "lr") else v) for k, v in L.items()} for L in layers_cpu]
+    seq = layers_cpu[0]["xq"].shape[2]
+    f = lambda t: t.float().numpy()
+
+    def run():
+        x = None
+        for L in L1:
+            q, k, v = (L["xq"], L["xk"], L["xv"]) if x is None else \
+                tuple((x + L[n].float()).to(io_dtype) for n in ("xq", "xk", "xv"))
+            if "W2" in L:
+                o = c_oracle.mlp_fwd(f(L["W1"]), f(L["b1"]), f(L["W2"]), f(L["b2"]), f(q), f(k), f(v), f(L["token_eta"]),
+                                     f(L["lr"]), f(L["gamma"]), f(L["beta"]), K=K, dtype=np.float32, nthreads=cores)[0]
+            else:
+                o = c_oracle.linear_fwd(f(L["W0"]), f(L["b0"]), f(q), f(k), f(v), f(L["token_eta"]), f(L["lr"]),
+                                        f(L["gamma"]), f(L["beta"]), K=K, dtype=np.float32, nthreads=cores)[0]
+            x = torch.from_numpy(o).to(io_dtype).float()
+        return x
+
+    run()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    t = sum(times) / len(times)
+    return {"value": seq / t, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"C/OpenMP f32 ports of the reference CPU path (TTT-Linear and TTT-MLP forward) chained through the "
+                      f"{len(L1)} layers, same inputs, batch 1 of {B} (tokens/s is batch-normalised), mean of 3 runs after "
+                      f"one warm-up, {t:.3f} s per run"}
+
+
 class LinearCalls:
     """The TTT-Linear entry points on preallocated buffers: what a step of the benchmark issues is the C-ABI call
     and nothing else (no allocation, no copies), so the device time between the events around a call is the time of
@@ -174,10 +212,14 @@ def run_workload(name, a, pkg, torch):
 
     if kind == "stack":
         # 8 layers (6 TTT-Linear then 2 TTT-MLP); layer input = previous output + fresh projections
-        layers = []
+        layers, layers_cpu = [], []
         for li in range(8):
             cl = pkg.synthetic.baseline_inputs(40 + li, B, H, seq, d, K, io_dtype=dtype, mlp=li >= 6)
             layers.append({k: v.to(dev) for k, v in cl.items()})
+            if not a.no_cpu_baseline:   # batch entry 0 is all the CPU leg reads
+                layers_cpu.append({k: (v[:1].clone() if k in ("xq", "xk", "xv", "lr") else v) for k, v in cl.items()
+                                   if k != "lr_logits"})
+            del cl
 
         stack = [dict(L, pq=L["xq"], pk=L["xk"], pv=L["xv"]) for L in layers]
         # wavefront over sequence windows: layer l + 1 works on a window as soon as layer l has left it, windows
@@ -191,7 +233,7 @@ def run_workload(name, a, pkg, torch):
         def step():
             # one call: per layer and window the input sums (x read once for xq, xk, xv) and the inner loop
             return (pkg.ttt_stack_forward_raw(stack, layers[0]["token_eta"], K, workspace=ws, chunk_tokens=chunk,
-                                              aux_stream=aux)[0],)
+                                              aux_stream=aux, check_lost=False)[0],)
     elif kind in ("inner_inputs", "layer_epilogue"):
         g = torch.Generator().manual_seed(1234 + w["cfg"])
         rn = lambda *sh: torch.randn(*sh, generator=g).to(dtype).to(dev)
@@ -256,6 +298,8 @@ def run_workload(name, a, pkg, torch):
                                              dv["d_out"], K)
                 return (fw[0], g["d_xq"])
 
+    # status word of the two-CU TTT-MLP kernel (head_dim 128): it must not move while this workload runs
+    lost0 = pkg.mlp_fwd_lost_workgroups()
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
@@ -270,6 +314,8 @@ def run_workload(name, a, pkg, torch):
     # call of a step that consists of several
     dev_s = time_parts([("step", step)], a.steps, torch)["step"]
     part_s = time_parts(parts, a.steps, torch) if parts else None
+    lost = pkg.mlp_fwd_lost_workgroups() - lost0
+    assert lost == 0, f"{lost} workgroups of the two-CU TTT-MLP kernel waited for their partner in vain"
 
     pass_name = {"linear_fwd": "fwd", "linear_fwd_bwd": "fwd+bwd", "mlp_fwd": "fwd", "mlp_fwd_bwd": "fwd+bwd",
                  "stack": "fwd", "inner_inputs": "inner-loop inputs", "layer_epilogue": "layer epilogue"}[kind]
@@ -374,12 +420,17 @@ def run_workload(name, a, pkg, torch):
         out["config"]["stack_streams"] = 2 if (a.stack_chunk and a.stack_streams > 1) else 1
     if not a.no_cpu_baseline and c is not None:
         out["cpu_baseline"] = cpu_baseline(c, K, kind)
+    elif not a.no_cpu_baseline and kind == "stack":
+        out["cpu_baseline"] = cpu_baseline_stack(layers_cpu, K, dtype, torch, B)
     return out
 
 
 # the headline metric names the forward AND the forward+backward at the 125M shape: the default run measures the
-# forward (BASELINE config 1) as the line's own value and these two forward+backward workloads as `extra` entries
-DEFAULT_EXTRA = ("linear_fwd_bwd_125m_bf16_b32", "linear_fwd_bwd_125m_f32_b8")
+# forward (BASELINE config 1) as the line's own value and, as `extra` entries, the two forward+backward workloads
+# (bf16 at the config-1 shape, f32 = BASELINE config 2), the TTT-MLP forward (config 3) with its forward+backward,
+# and the 8-layer long-context stack (config 4)
+DEFAULT_EXTRA = ("linear_fwd_bwd_125m_bf16_b32", "linear_fwd_bwd_125m_f32_b8", "mlp_fwd_d96_bf16",
+                 "mlp_fwd_bwd_d96_bf16", "stack8_d128_seq8192_bf16")
 
 
 def main():

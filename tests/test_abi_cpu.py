@@ -70,9 +70,15 @@ def test_best_checkpoint_format(P):
     assert best(io_dtype=P.TTT_F32) == 1
     assert best(checkpoint_interval=2) == 0 and best(io_dtype=P.TTT_BF16, checkpoint_interval=4) == 0
     assert best(seq=33) < 0
+    # the hint is part of the question: the LDS-tile backward reads f32 matrices only
+    assert best(io_dtype=P.TTT_BF16, kernel_hint=P.TTT_HINT_LDS_TILES) == 0
+    assert best(io_dtype=P.TTT_F32, kernel_hint=P.TTT_HINT_LDS_TILES) == 0
+    # no backward kernel at all (f32 I/O at head_dim 128, an unsupported head_dim): the backward's status, no format
+    assert best(io_dtype=P.TTT_F32, head_dim=128) == P.TTT_ERR_UNSUPPORTED
+    assert best(head_dim=48) == P.TTT_ERR_UNSUPPORTED
     # what it names is accepted by the backward
     for kw in (dict(io_dtype=P.TTT_BF16), dict(io_dtype=P.TTT_F32), dict(io_dtype=P.TTT_BF16, head_dim=128),
-               dict(checkpoint_interval=2)):
+               dict(checkpoint_interval=2), dict(io_dtype=P.TTT_BF16, kernel_hint=P.TTT_HINT_LDS_TILES)):
         fmt = best(**kw)
         assert L.ttt_linear_bwd_supported(C.byref(desc(P, checkpoint_format=fmt, **kw))) == P.TTT_OK
 

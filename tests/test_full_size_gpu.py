@@ -134,8 +134,10 @@ def test_config1_shape_linear_fwd_bwd_bf16_full(P):
                                       x["gamma"], x["beta"], Wc, bc, x["d_out"], K, 1e-6, 1,
                                       packed_checkpoints=packed, kernel_hint=bwd_hint)
         torch.cuda.synchronize()
+        last_state[:] = [W, b]
         return out, g
 
+    last_state = []
     out, g = fwd_bwd(dv)
     # packed checkpoints (what bench.py measures): same outputs bit for bit, gradients far inside the tolerance
     # (the f32 row-major checkpoint reproduces the centred state to an ulp, which can move a bf16 operand by 2^-8)
@@ -175,6 +177,23 @@ def test_config1_shape_linear_fwd_bwd_bf16_full(P):
              ("grad_token_eta", "d_token_eta", 0.0), ("grad_ln_weight", "d_gamma", 0.0), ("grad_ln_bias", "d_beta", 0.0)]
     for gn, rn, frac in names:
         assert_close(g1[gn], r[rn], TOL[torch.bfloat16], gn, min_frac=frac)
+    # the path bench.py times at this shape -- the forward that saves update factors and the backward that walks
+    # the state back over all 128 mini-batches -- against the oracle directly, same bands: output, final state and
+    # all nine gradients of that batch entry
+    of, gfo = fwd_bwd(one, packed=2)
+    Wf, bf = last_state
+    ro, rW, rb = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                                    n["gamma"], n["beta"], K=K)
+    assert_close(of, ro, TOL[torch.bfloat16], "factors out vs oracle")
+    assert_close(Wf, rW, TOL[torch.bfloat16], "factors W_out vs oracle")
+    assert_close(bf, rb, TOL[torch.bfloat16], "factors b_out vs oracle")
+    for gn, rn, frac in names:
+        assert_close(gfo[gn], r[rn], TOL[torch.bfloat16], "factors " + gn, min_frac=frac)
+    # and the packed-state run of the same entry
+    op, gpo = fwd_bwd(one, packed=True)
+    assert_close(op, ro, TOL[torch.bfloat16], "packed out vs oracle")
+    for gn, rn, frac in names:
+        assert_close(gpo[gn], r[rn], TOL[torch.bfloat16], "packed " + gn, min_frac=frac)
 
 
 def test_config3_mlp_fwd_bf16_full(P):

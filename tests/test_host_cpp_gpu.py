@@ -173,3 +173,26 @@ def test_cpp_mlp_forward_remainder_and_backward_equal_python_mirror(P, drv):
         assert torch.equal(got[k], ref[k]), k
     for k in ("d_token_eta", "d_gamma", "d_beta"):
         assert_close(got[k], ref[k].double().cpu().numpy(), 1e-5, k)
+
+
+def test_cpp_lost_workgroup_guard(P, drv):
+    """LostWorkgroupGuard around a TTT-MLP forward at head_dim 128 (two workgroups per unit): silent on a healthy
+    run, an error when the waits are made to give up at once (TTT_HINT_TEST_LOST_PARTNER)."""
+    print("case host C++ lost-workgroup guard", flush=True)
+    B, H, d, K, N = 1, 2, 128, 16, 2
+    dv = to_dev(mlp_case(P, 93, B, H, N * K, d, K, torch.bfloat16, "ref"))
+    args = (dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"],
+            dv["beta"], K)
+    drv.ttt_host_lost_guard_new.restype = C.c_void_p
+    drv.ttt_host_lost_guard_verify_and_free.argtypes = [C.c_void_p]
+    torch.cuda.synchronize()
+    g = drv.ttt_host_lost_guard_new()
+    assert g
+    P.ttt_mlp_forward_raw(*args)
+    torch.cuda.synchronize()
+    assert drv.ttt_host_lost_guard_verify_and_free(g) == P.TTT_OK
+    g = drv.ttt_host_lost_guard_new()
+    P.ttt_mlp_forward_raw(*args, kernel_hint=P.TTT_HINT_TEST_LOST_PARTNER)
+    torch.cuda.synchronize()
+    assert drv.ttt_host_lost_guard_verify_and_free(g) == P.TTT_ERR_HIP
+    assert b"partner" in drv.ttt_host_last_error()

@@ -56,9 +56,9 @@ def oracle_layer(L, x, bs, hs, K, dtype):
                               par(L["beta"]), K=K)
 
 
-def run_stack_layerwise(P, dl, K, n):
+def run_stack_layerwise(P, dl, K, n, chunk_tokens=0, aux_stream=None):
     """The first n layers through ttt_stack_fwd: output and states of layer n-1."""
-    out, states = P.ttt_stack_forward_raw(dl[:n], dl[0]["token_eta"], K)
+    out, states = P.ttt_stack_forward_raw(dl[:n], dl[0]["token_eta"], K, chunk_tokens=chunk_tokens, aux_stream=aux_stream)
     torch.cuda.synchronize()
     return out, states[n - 1]
 
@@ -94,18 +94,22 @@ def test_small_stack_matches_oracle_layer_by_layer(P, dtype):
     assert torch.equal(x, out)
 
 
-def test_config4_stack_chain_full_size(P):
+@pytest.mark.parametrize("chunk,two_streams", [(0, False), (2048, True)], ids=["one-launch-per-layer", "wavefront-2048-two-streams"])
+def test_config4_stack_chain_full_size(P, chunk, two_streams):
+    """Both plans -- one launch per layer, and the wavefront bench.py times (windows of 2048 tokens, TTT-MLP launches
+    on a second stream) -- against the float64 oracle carried through all eight layers on two units."""
     B, H, d, K, seq = 4, 16, 128, 16, 8192
     kinds = [False] * 6 + [True] * 2
     dtype = torch.bfloat16
-    print("case stack config 4 (8 layers, B4 H16 d128 seq8192 bf16)", flush=True)
+    print(f"case stack config 4 (8 layers, B4 H16 d128 seq8192 bf16), chunk {chunk}, second stream {two_streams}", flush=True)
     layers = make_layers(P, B, H, seq, d, K, dtype, kinds)
     dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    aux = torch.cuda.Stream("cuda:0") if two_streams else None
     bs, hs = [1], [3, 12]          # two units
     x_gpu, x_free = None, None
     tol = TOL[dtype]
     for n in range(1, 9):
-        out, st = run_stack_layerwise(P, dl, K, n)
+        out, st = run_stack_layerwise(P, dl, K, n, chunk, aux)
         assert torch.isfinite(out.float()).all()
         sub = out[bs][:, hs]
         # (1) this layer alone, on the input the GPU produced
@@ -209,6 +213,27 @@ def test_stack_wavefront_rejects_bad_plans(P):
         with pytest.raises(P.TttError):
             P.ttt_stack_forward_raw(dl, dl[0]["token_eta"], K, chunk_tokens=bad, aux_stream=aux)
     torch.cuda.synchronize()
+
+
+def test_stack_reports_lost_workgroups(P):
+    """A stack with a TTT-MLP layer at head_dim 128 (two workgroups per unit): the mirror reads the kernel's status
+    word around the call.  With the waits made to give up at once the call would return NaN outputs and TTT_OK; the
+    word moves, which the test reads itself (the mirror does not raise for the testing hint), and a healthy call
+    afterwards leaves it where it was."""
+    B, H, d, K, seq = 1, 2, 128, 16, 64
+    print("case stack lost workgroups", flush=True)
+    layers = make_layers(P, B, H, seq, d, K, torch.bfloat16, [False, True], seed0=97)
+    dl = [{k: v.to("cuda:0") for k, v in L.items()} for L in layers]
+    torch.cuda.synchronize()
+    before = P.mlp_fwd_lost_workgroups()
+    out, _ = P.ttt_stack_forward_raw(dl, dl[0]["token_eta"], K, kernel_hint=P.TTT_HINT_TEST_LOST_PARTNER)
+    torch.cuda.synchronize()
+    assert torch.isnan(out.float()).all()
+    assert P.mlp_fwd_lost_workgroups() == before + 2 * B * H
+    out, _ = P.ttt_stack_forward_raw(dl, dl[0]["token_eta"], K)   # check_lost defaults to on here
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert P.mlp_fwd_lost_workgroups() == before + 2 * B * H
 
 
 def test_config4_stack_wavefront_full_size(P):

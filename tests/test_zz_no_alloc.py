@@ -1,7 +1,7 @@
 """GPU test of ttt_mlp_bwd_static, the entry point that allocates nothing: its workspace is a buffer
 inside the library's device image.  Through the C ABI, against ttt_mlp_bwd (caller-owned workspace) on
-the same inputs: two calls in a row, the second with a smaller input, so the second call runs on whatever
-the first left in the shared buffer.
+the same inputs: three calls in a row, the second with a smaller input and the third with the first shape again,
+so each later call runs on whatever the earlier ones left in the shared buffer, shrinking and growing.
 
 Outputs written by plain stores must agree bit for bit (same kernels, same order of operations); the three
 outputs accumulated with floating-point atomics over (batch, head) units (d_token_eta, d_gamma, d_beta)
@@ -44,10 +44,15 @@ def both(P, B, H, d, K, N, dtype, seed, state_grads):
     into = {k: torch.full_like(v, float("nan")) for k, v in ref.items()}
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    # free device memory as the driver sees it: an allocation made behind torch's back (hipMalloc, a memory pool,
+    # a runtime object that takes device memory) would lower it
+    free_before = torch.cuda.mem_get_info()[0]
     got = P.ttt_mlp_backward_raw(*args, d_state_out=dst, static_scratch=True, into=into)
     after = torch.cuda.memory_stats()["allocation.all.allocated"]
     torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
     assert after == before, "the static-scratch call allocated device memory through torch"
+    assert free_after == free_before, f"free device memory changed by {free_before - free_after} bytes over the static-scratch call"
     return got, ref
 
 
@@ -63,6 +68,10 @@ def test_static_scratch_matches_workspace_call_twice(P):
     got, ref = both(P, 2, 2, 64, 16, 4, torch.float32, 901, True)
     check(got, ref)
     got, ref = both(P, 1, 2, 32, 8, 2, torch.bfloat16, 902, False)
+    check(got, ref)
+    # and back to the first shape: the buffer now holds the smaller call's leftovers inside the larger call's extent
+    print("case no-alloc: B2 H2 d64 K16 N4 f32 again", flush=True)
+    got, ref = both(P, 2, 2, 64, 16, 4, torch.float32, 903, True)
     check(got, ref)
 
 

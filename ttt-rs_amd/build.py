@@ -25,13 +25,38 @@ HIPCC_FLAGS = [
 
 
 def build_library(verbose: bool = False, extra_flags=()) -> str:
+    """Compiles the library, then scans the gfx950 assembly the compiler produced on the way (isa_check.py: a
+    matrix-instruction hazard the compiler does not guard and the hardware does not interlock).  The library is
+    installed only if the scan is clean."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-o", LIB_PATH, *SOURCES]
+    tmp = os.path.join(HERE, "build", "lib")   # intermediate files of the compilation land beside the output
+    shutil.rmtree(tmp, ignore_errors=True)
+    os.makedirs(tmp)
+    out = os.path.join(tmp, os.path.basename(LIB_PATH))
+    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-save-temps=obj", "-o", out, *SOURCES]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
         raise RuntimeError("hipcc failed building " + LIB_PATH)
+    sys.path.insert(0, HERE)
+    try:
+        import isa_check
+    finally:
+        sys.path.pop(0)
+    asm = [os.path.join(tmp, f) for f in os.listdir(tmp) if f.endswith("gfx950.s")]
+    if not asm:
+        raise RuntimeError("no gfx950 assembly found beside " + out + ": the hazard scan cannot run")
+    for path in asm:
+        bad = isa_check.check_file(path)
+        if bad:
+            for func, no, a, b, ws in bad[:20]:
+                sys.stderr.write(f"{os.path.basename(path)}:{no}: in {func}: {ws} wait state(s) between\n    {a}\n    {b}\n")
+            raise RuntimeError(f"{len(bad)} in-place accumulations onto a matrix instruction of another shape sit closer "
+                               "than the hardware needs (see isa_check.py); library not installed")
+    shutil.copyfile(out, LIB_PATH)
+    shutil.copymode(out, LIB_PATH)
+    shutil.rmtree(os.path.join(HERE, "build"), ignore_errors=True)
     if verbose:
         # the host pass does not know the gfx950 feature flag and says so; drop that noise
         for line in (res.stdout + res.stderr).splitlines():

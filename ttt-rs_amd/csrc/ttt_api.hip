@@ -22,6 +22,7 @@
 #include "ttt_mlp_bwd.hip.h"
 #include "ttt_mlp_fwd_cl2.hip.h"
 #include "ttt_mlp_fwd_rr.hip.h"
+#include "ttt_selftest.hip.h"
 
 // Scratch of ttt_mlp_bwd_static (file scope, outside any namespace so that HIP_SYMBOL names it plainly).
 static __device__ __align__(256) unsigned char ttt_mlp_bwd_scratch_mem[TTT_MLP_BWD_STATIC_MAX_BYTES];
@@ -640,13 +641,21 @@ int ttt_linear_bwd_supported(const ttt_desc* d) {
 }
 
 int ttt_linear_best_checkpoint_format(const ttt_desc* d) {
-  if (check_common(d) != TTT_OK) return -1;
-  if (d->checkpoint_interval != 1) return TTT_CKPT_F32;
+  int rc = ttt_linear_supported(d);
+  if (rc != TTT_OK) return rc;
   // measured at head_dim 64 (125M shape): factors win up to 512 units, where the feature-split backward runs anyway;
   // beyond, the single-wave backward from packed states and the feature-split one from factors are even
-  const bool factors = d->io_dtype == TTT_BF16 && d->head_dim <= 96 && d->seq / d->mini_batch >= 2 &&
-                       (int64_t)d->batch * d->heads <= 512;
-  return factors ? TTT_CKPT_FACTORS : TTT_CKPT_PACKED;
+  const bool factors_pay = d->seq / d->mini_batch >= 2 && (int64_t)d->batch * d->heads <= 512;
+  // the first candidate, cheapest first, for which the backward has a kernel under this desc's interval and hint
+  const int order[3] = {TTT_CKPT_FACTORS, TTT_CKPT_PACKED, TTT_CKPT_F32};
+  for (int i = factors_pay ? 0 : 1; i < 3; ++i) {
+    ttt_desc trial = *d;
+    trial.checkpoint_format = order[i];
+    LinearBwdChoice ch;
+    rc = choose_linear_bwd(&trial, &ch);
+    if (rc == TTT_OK) return order[i];
+  }
+  return rc;  // no format has a backward kernel: the status ttt_linear_bwd would return for the f32 format
 }
 
 int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
@@ -1060,7 +1069,20 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
   // events (two lanes only): created here and destroyed before returning; the runtime keeps a recorded event
   // alive until the work it marks has finished
   std::vector<hipEvent_t> ev;
+  bool forked = false;  // the second stream has been made to wait for `stream` and has not been joined back yet
   auto cleanup = [&](int r) {
+    if (forked) {
+      // an error between fork and join: `stream` still has to wait for whatever the second stream was given, or a
+      // caller that is capturing `stream` into a graph is left with a branch that never rejoins (an invalid
+      // capture), and any caller with work on the second stream that nothing orders.  Best effort: the call is
+      // failing already and reports its first error.
+      hipEvent_t e = nullptr;
+      if (hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess) {
+        ev.push_back(e);
+        if (hipEventRecord(e, lane_s[1]) == hipSuccess) (void)hipStreamWaitEvent(main_s, e, 0);
+      }
+      forked = false;
+    }
     for (hipEvent_t e : ev) (void)hipEventDestroy(e);
     return r;
   };
@@ -1075,6 +1097,7 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
     hipEvent_t fork;
     if ((rc = mark(main_s, &fork)) != TTT_OK) return cleanup(rc);
     if ((rc = wait(lane_s[1], fork)) != TTT_OK) return cleanup(rc);
+    forked = true;
   }
   // The two-CU TTT-MLP kernel exchanges through the window's W2 output buffer, which has to be zero when it starts.
   // Nothing reads or writes that buffer before a layer's FIRST window, so those are cleared here, while the stream
@@ -1133,8 +1156,17 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
     hipEvent_t join;
     if ((rc = mark(lane_s[1], &join)) != TTT_OK) return cleanup(rc);
     if ((rc = wait(main_s, join)) != TTT_OK) return cleanup(rc);
+    forked = false;
   }
   return cleanup(TTT_OK);
+}
+
+int ttt_selftest_mfma_mixed(int order, int gap, float* out, void* stream) {
+  if (!out) return fail(TTT_ERR_NULL, "ttt_selftest_mfma_mixed: out is NULL");
+  if ((order != 0 && order != 1) || (gap != 0 && gap != 4 && gap != 5))
+    return fail(TTT_ERR_SHAPE, "ttt_selftest_mfma_mixed: order must be 0 or 1 and gap 0, 4 or 5 (got %d, %d)", order, gap);
+  hipLaunchKernelGGL(ttt::ttt_selftest_mfma_mixed_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), order, gap, out);
+  return hip_status(hipGetLastError(), "ttt_selftest_mfma_mixed launch");
 }
 
 int ttt_inner_inputs(const ttt_desc* d, const void* xq, const void* xk, const void* xv,

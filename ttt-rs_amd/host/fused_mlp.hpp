@@ -154,4 +154,33 @@ class FusedMlp {
   const float* ln_bias_;
 };
 
+/// The status word of the two-CU TTT-MLP forward (head_dim 128, bf16 I/O; see ttt_mlp_fwd in the C header): a
+/// workgroup that waited for its partner in vain cannot fail the call that enqueued it, so a caller that runs such
+/// layers -- directly or inside ttt_stack_fwd -- brackets its work with this guard: construct it before enqueueing,
+/// call verify() once the stream's work has finished (both read the word with a blocking copy from the device).
+class LostWorkgroupGuard {
+ public:
+  LostWorkgroupGuard() { check(ttt_mlp_fwd_lost_workgroups(&before_)); }
+  /// Throws if the word moved since construction: the outputs of the affected units are NaN.
+  void verify() const {
+    std::int64_t now = 0;
+    check(ttt_mlp_fwd_lost_workgroups(&now));
+    if (now != before_)
+      throw Error(TTT_ERR_HIP, std::to_string(now - before_) +
+                                   " workgroups of the two-CU TTT-MLP kernel waited for their partner in vain");
+  }
+
+ private:
+  std::int64_t before_ = 0;
+};
+
+/// ttt_stack_fwd (inner models applied layer by layer, optionally as a cross-layer wavefront over windows of
+/// chunk_tokens tokens with the TTT-MLP launches on aux_stream) with the arguments of the C entry point.  Enqueues
+/// only; a caller whose stack holds TTT-MLP layers at head_dim 128 keeps a LostWorkgroupGuard around the call and
+/// verifies it after synchronising.
+inline void stack_forward(const ttt_desc& desc, int n_layers, const ttt_stack_layer* layers, const float* token_eta,
+                          void* out, void* workspace, int chunk_tokens, void* aux_stream, void* stream) {
+  check(ttt_stack_fwd(&desc, n_layers, layers, token_eta, out, workspace, chunk_tokens, aux_stream, stream));
+}
+
 }  // namespace ttt

@@ -127,4 +127,38 @@ int ttt_host_mlp_forward_backward(int B, int H, int d, int K, int seq, int dtype
   }
 }
 
+// LostWorkgroupGuard (fused_mlp.hpp) for a test process: new -> its work -> synchronise -> verify -> free.
+// These two calls read the device's status word with a blocking copy.
+void* ttt_host_lost_guard_new(void) {
+  try {
+    return new ttt::LostWorkgroupGuard();
+  } catch (const ttt::Error& e) {
+    report(e);
+    return nullptr;
+  }
+}
+
+int ttt_host_lost_guard_verify_and_free(void* guard) {
+  ttt::LostWorkgroupGuard* g = static_cast<ttt::LostWorkgroupGuard*>(guard);
+  int rc = TTT_OK;
+  try {
+    g->verify();
+  } catch (const ttt::Error& e) {
+    rc = report(e);
+  }
+  delete g;
+  return rc;
+}
+
+// ttt::stack_forward with the arguments of ttt_stack_fwd.
+int ttt_host_stack_forward(const ttt_desc* desc, int n_layers, const ttt_stack_layer* layers, const float* token_eta,
+                           void* out, void* workspace, int chunk_tokens, void* aux_stream, void* stream) {
+  try {
+    ttt::stack_forward(*desc, n_layers, layers, token_eta, out, workspace, chunk_tokens, aux_stream, stream);
+    return TTT_OK;
+  } catch (const ttt::Error& e) {
+    return report(e);
+  }
+}
+
 }  // extern "C"

@@ -515,9 +515,18 @@ def ttt_stack_workspace_bytes(B: int, H: int, seq: int, d: int, mini_batch: int,
     return n
 
 
+def mlp_fwd_lost_workgroups() -> int:
+    """ttt_mlp_fwd_lost_workgroups of the current device: how many workgroups of the two-CU TTT-MLP forward
+    (head_dim 128, bf16 I/O) gave up waiting for their partner since the library was loaded.  A blocking copy from
+    the device; meaningful once the work in question has finished."""
+    n = C.c_int64(0)
+    check(lib().ttt_mlp_fwd_lost_workgroups(C.byref(n)))
+    return n.value
+
+
 def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6, kernel_hint: int = 0,
                           workspace: Optional[torch.Tensor] = None, chunk_tokens: int = 0,
-                          aux_stream: Optional[torch.cuda.Stream] = None):
+                          aux_stream: Optional[torch.cuda.Stream] = None, check_lost: Optional[bool] = None):
     """One call of ttt_stack_fwd on the current stream: inner models applied layer by layer, layer l on
     xq = x + pq, xk = x + pk, xv = x + pv with x the previous layer's output (0 for the first layer).
     chunk_tokens > 0 runs the layers as a wavefront over sequence windows of that many tokens (layer l + 1 works on
@@ -525,7 +534,12 @@ def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6,
     torch.cuda.Stream, lets the TTT-MLP launches run beside the TTT-Linear ones.
     layers: list of dicts with pq, pk, pv [B,H,seq,d], lr [B,H,seq], gamma, beta [H,d] and either W0, b0
     (TTT-Linear) or W1, b1, W2, b2 (TTT-MLP), parameters [H,..].  Returns (out, states) with states[l] the final
-    state tensors of layer l (per batch element)."""
+    state tensors of layer l (per batch element).
+    check_lost: a stack with a TTT-MLP layer at head_dim 128 and bf16 I/O runs the two-CU kernel, whose failure
+    (a workgroup that waited for its partner in vain) shows only in the data (NaN) and in the device's status word.
+    With check_lost the call waits for the device, reads that word before and after and raises if it moved.
+    Default (None): checked unless the current stream is being captured into a graph; callers that must not
+    synchronise (timed loops) pass False and compare mlp_fwd_lost_workgroups() around their own region."""
     B, H, seq, d = layers[0]["pq"].shape
     io = layers[0]["pq"].dtype
     dev = layers[0]["pq"].device
@@ -574,10 +588,24 @@ def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6,
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "workspace too small")
     out = torch.empty((B, H, seq, d), dtype=io, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    two_cu = d == 128 and io == torch.bfloat16 and any("W2" in L for L in layers) and \
+        not (kernel_hint & _lib.TTT_HINT_LDS_TILES)
+    if check_lost is None:
+        check_lost = two_cu and not torch.cuda.is_current_stream_capturing()
     with torch.cuda.device(dev):
+        lost_before = 0
+        if check_lost and two_cu:
+            torch.cuda.synchronize(dev)
+            lost_before = mlp_fwd_lost_workgroups()
         check(lib().ttt_stack_fwd(C.byref(desc), len(layers), arr, _ptr(te), _ptr(out), _ptr(workspace),
                                   chunk_tokens, C.c_void_p(aux_stream.cuda_stream) if aux_stream is not None else None,
                                   stream))
+        if check_lost and two_cu:
+            torch.cuda.synchronize(dev)
+            lost = mlp_fwd_lost_workgroups() - lost_before
+            if lost and not (kernel_hint & _lib.TTT_HINT_TEST_LOST_PARTNER):
+                raise _lib.TttError(_lib.TTT_ERR_HIP, f"ttt_stack_fwd: {lost} workgroups of the two-CU TTT-MLP kernel "
+                                    "waited for their partner in vain; the outputs of their units are NaN")
     # aux_stream reads and writes tensors that torch's allocator ties to the current stream only; the call joins
     # it into the current stream before it returns, so later work on that stream is ordered after it
     return out, states
