@@ -93,10 +93,18 @@ typedef struct ttt_desc {
 #define TTT_HINT_AUTO 0
 #define TTT_HINT_WAVES_MASK 0xff
 #define TTT_HINT_LDS_TILES 0x100
+/* ttt_mlp_fwd, bf16 I/O at head_dim 96: spread every (batch, head) unit over a pair of CUs, as head_dim 128 always is
+ * (see ttt_mlp_fwd), when the units number at most half the device's CUs.  Not the default: measured on MI355X the
+ * pair gains 2 - 3 % at 128 units.  Ignored where only one of the two kernels exists. */
+#define TTT_HINT_TWO_CU 0x400
 /* Testing only: the two workgroups that share a (batch, head) unit in ttt_mlp_fwd at head_dim 128 (bf16 I/O) give
  * up waiting for each other at once, as if the partner had never become resident.  Exercises the failure path
  * described at ttt_mlp_fwd: every output of the affected units is NaN.  All kernels still run to their end. */
 #define TTT_HINT_TEST_LOST_PARTNER 0x200
+/* Testing only: the same two workgroups treat each other as running on different XCDs whatever they find at start,
+ * i.e. take the path of a pair that was not placed on one XCD: every word they exchange is stored at device scope
+ * instead of staying in the XCD's L2.  Slower; results identical. */
+#define TTT_HINT_TEST_OTHER_XCD 0x800
 
 /* Library / build identification. */
 const char* ttt_version(void);
@@ -177,12 +185,15 @@ int ttt_linear_bwd(const ttt_desc* desc, const void* xq, const void* xk, const v
  *
  * head_dim 128 with bf16 I/O: a unit's state (512 KiB) is the whole register file of a CU, so a PAIR of
  * workgroups on two CUs of one XCD shares each unit and exchanges partial results once per mini-batch through
- * global memory, in the L2 cache those two CUs share.  During the call W2_out is also that exchange area (the
+ * global memory, in the L2 cache those two CUs share (the two workgroups tell each other at start which XCD they run
+ * on; a pair that was not placed on one XCD exchanges through device-scope stores instead: slower, same results).
+ * head_dim 96 with bf16 I/O runs on one CU per unit, or on a pair like head_dim 128 when TTT_HINT_TWO_CU asks for it;
+ * everything said here of head_dim 128 then holds for it too.  During the call W2_out is also that exchange area (the
  * library zero-fills it first; its contents are meaningless until the call's work has finished); it must be
  * ordinary device memory (hipMalloc), not fine-grained or host memory.  The library launches at most as many workgroups at a time as
  * the device has CUs, so on a GPU that is not shared both halves of every pair are resident together.  If a
  * workgroup nevertheless waits for its partner in vain (2^21 polls, seconds: CUs held by other processes or
- * streams, or a pair that was not placed on one XCD), the
+ * streams), the
  * call cannot report it -- it returned TTT_OK when the work was enqueued -- so the failure is made impossible to
  * miss in the data instead: EVERY output of that unit (its rows of out, W1_out, b1_out, W2_out, b2_out) is NaN.
  * A caller that shares the GPU checks one output element per unit, reads the status word below, or passes

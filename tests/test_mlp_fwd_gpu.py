@@ -54,6 +54,32 @@ def test_mlp_fwd_matches_oracle(P, B, H, d, K, N, style, dtype):
                      min_frac=0.99 if loose else 0.999)
 
 
+@pytest.mark.parametrize("B,H,K,N", [(2, 2, 16, 4), (1, 1, 7, 2), (1, 3, 16, 9)])
+def test_mlp_fwd_d96_one_cu_and_two_cu_kernels(P, B, H, K, N):
+    """head_dim 96, bf16 I/O: the one-CU register-resident kernel (default) and, with TTT_HINT_TWO_CU, the kernel
+    that spreads a unit over a pair of CUs as head_dim 128 always does.  Both against the oracle, and close to each
+    other."""
+    print(f"case mlp d96 one/two CU B{B} H{H} K{K} N{N}", flush=True)
+    d = 96
+    c = mlp_case(P, 410 + K + N, B, H, N * K, d, K, torch.bfloat16, "ref")
+    dv = to_dev(c)
+    args = (dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"],
+            dv["beta"], K)
+    two = P.ttt_mlp_forward_raw(*args, kernel_hint=P.TTT_HINT_TWO_CU)
+    two_again = P.ttt_mlp_forward_raw(*args, kernel_hint=P.TTT_HINT_TWO_CU)
+    one = P.ttt_mlp_forward_raw(*args)
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ref = orc.mlp_forward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"],
+                          n["lr"], n["gamma"], n["beta"], K=K)
+    for name, g2, g1, ga, r in zip(("out", "W1", "b1", "W2", "b2"), two, one, two_again, ref):
+        assert torch.equal(g2, ga), f"{name}: the two-CU kernel is not deterministic"
+        assert_close(g2, r, TOL[torch.bfloat16], "two-CU " + name, min_frac=0.99 if name in ("b1", "b2") else 0.999)
+        assert_close(g1, r, TOL[torch.bfloat16], "one-CU " + name, min_frac=0.99 if name in ("b1", "b2") else 0.999)
+    # different kernels (the order in which the halves of the hidden axis are summed differs): not the same bits
+    assert (two[0].float() - one[0].float()).abs().max().item() <= 2.0 ** -5
+
+
 def test_mlp_fwd_bf16_lds_kernel_keeps_f32_products(P):
     """kernel_hint TTT_HINT_LDS_TILES selects the LDS-tile kernel for bf16 I/O too: f32 products, so the
     state meets the f32 bar."""
@@ -144,6 +170,27 @@ def test_mlp_fwd_d128_lost_partner_is_loud(P):
     for t in ok:
         assert torch.isfinite(t.float()).all()
     assert lost_workgroups() == before + 2 * B * H
+
+
+@pytest.mark.parametrize("d", [96, 128])
+def test_mlp_fwd_two_cu_pair_on_two_xcds_takes_device_scope_stores(P, d):
+    """The two workgroups of a pair tell each other at start which XCD they run on; a pair on two XCDs exchanges through
+    device-scope stores instead of words that stay in one XCD's L2.  TTT_HINT_TEST_OTHER_XCD makes every pair take that
+    path: same kernel, same order of operations, so the same bits as the default path, and nothing lost."""
+    print(f"case mlp two-CU other-XCD path d{d}", flush=True)
+    B, H, K, N = 1, 3, 16, 5
+    dv = to_dev(mlp_case(P, 95 + d, B, H, N * K, d, K, torch.bfloat16, "ref"))
+    args = (dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"],
+            dv["beta"], K)
+    torch.cuda.synchronize()
+    before = P.mlp_fwd_lost_workgroups()
+    ref = P.ttt_mlp_forward_raw(*args, kernel_hint=P.TTT_HINT_TWO_CU)
+    got = P.ttt_mlp_forward_raw(*args, kernel_hint=P.TTT_HINT_TWO_CU | P.TTT_HINT_TEST_OTHER_XCD)
+    torch.cuda.synchronize()
+    for name, x, y in zip(("out", "W1", "b1", "W2", "b2"), got, ref):
+        assert torch.isfinite(x.float()).all(), name
+        assert torch.equal(x, y), f"{name}: device-scope exchange differs from the L2-resident one"
+    assert P.mlp_fwd_lost_workgroups() == before
 
 
 def test_mlp_fwd_d128_more_units_than_one_launch(P):

@@ -12,6 +12,8 @@ TTT_OK, TTT_ERR_SHAPE, TTT_ERR_UNSUPPORTED, TTT_ERR_HIP, TTT_ERR_NULL = 0, -1, -
 TTT_F32, TTT_BF16 = 0, 1
 TTT_HINT_AUTO, TTT_HINT_LDS_TILES = 0, 0x100  # kernel_hint: low byte = waves per unit (1, 2, 4)
 TTT_HINT_TEST_LOST_PARTNER = 0x200
+TTT_HINT_TWO_CU = 0x400
+TTT_HINT_TEST_OTHER_XCD = 0x800
 
 EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_bwd_supported",

@@ -247,23 +247,30 @@ int launch_mlp_fwd_rr(const ttt::MlpFwdArgs* probs, unsigned ny, hipStream_t s) 
   return hip_status(hipGetLastError(), "ttt_mlp_fwd (register-resident kernel) launch");
 }
 
-// head_dim 128, bf16 I/O: a pair of workgroups per (batch, head); the exchange flags live in W2_out,
-// which is zeroed first (a fill kernel, not a memset node).
+// bf16 I/O, head_dim 128 (and 96 when there are few units): a pair of workgroups per (batch, head); the exchange flags
+// live in W2_out, which is zeroed first (a fill kernel, not a memset node).
 // The two workgroups of a pair wait for each other, so both must be resident: a workgroup fills a CU (LDS,
 // registers), hence no launch may hold more workgroups than the device has CUs.  The units are independent, so
 // more units than that go in several launches on the stream.  Several problems travel together while they fit
 // that limit, otherwise one after the other.
+int device_cus(int* cus) {
+  int dev = 0;
+  int rc = hip_status(hipGetDevice(&dev), "hipGetDevice");
+  if (rc != TTT_OK) return rc;
+  return hip_status(hipDeviceGetAttribute(cus, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute(CU count)");
+}
+
+template <int D>
 int launch_mlp_fwd_cl2(const ttt::MlpFwdArgs* probs, int n, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_mlp_fwd_cl2_kernel<ttt::BF16, 128>;
-  constexpr size_t bytes = ttt::MlpCl2Lds<128, 2>::BYTES;
+  constexpr auto kern = ttt::ttt_mlp_fwd_cl2_kernel<ttt::BF16, D>;
+  constexpr size_t bytes = ttt::MlpCl2Lds<D, 2>::BYTES;
+  constexpr unsigned threads = 64 * (D / 16);
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  int dev = 0, cus = 0;
-  rc = hip_status(hipGetDevice(&dev), "hipGetDevice");
+  int cus = 0;
+  rc = device_cus(&cus);
   if (rc != TTT_OK) return rc;
-  rc = hip_status(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev), "hipDeviceGetAttribute(CU count)");
-  if (rc != TTT_OK) return rc;
-  const size_t units = (size_t)probs[0].B * probs[0].H, nz = units * 128 * 512;
+  const size_t units = (size_t)probs[0].B * probs[0].H, nz = units * D * (4 * D);
   for (int p = 0; p < n; ++p)
     if (!probs[p].exchange_cleared)
       hipLaunchKernelGGL(ttt::ttt_fill_zero_kernel, dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, s, probs[p].W2, nz);
@@ -274,7 +281,7 @@ int launch_mlp_fwd_cl2(const ttt::MlpFwdArgs* probs, int n, hipStream_t s) {
   for (int p = 0; p < n;) {
     if (together >= 2 && n - p >= 2) {
       const int cnt = n - p < together ? n - p : together;
-      hipLaunchKernelGGL(kern, dim3((unsigned)wg_per_problem, (unsigned)cnt), dim3(512), bytes, s, pack_of(probs + p, (unsigned)cnt));
+      hipLaunchKernelGGL(kern, dim3((unsigned)wg_per_problem, (unsigned)cnt), dim3(threads), bytes, s, pack_of(probs + p, (unsigned)cnt));
       p += cnt;
       continue;
     }
@@ -282,11 +289,31 @@ int launch_mlp_fwd_cl2(const ttt::MlpFwdArgs* probs, int n, hipStream_t s) {
     for (size_t base = 0; base < units; base += per_launch) {
       const size_t cnt = units - base < per_launch ? units - base : per_launch;
       a.unit_base = (int)base;
-      hipLaunchKernelGGL(kern, dim3((unsigned)(((cnt + 7) / 8) * 16)), dim3(512), bytes, s, pack_of(&a, 1));
+      hipLaunchKernelGGL(kern, dim3((unsigned)(((cnt + 7) / 8) * 16)), dim3(threads), bytes, s, pack_of(&a, 1));
     }
     ++p;
   }
   return hip_status(hipGetLastError(), "ttt_mlp_fwd (two-CU kernel) launch");
+}
+
+// Whether ttt_mlp_fwd runs the two-CU kernel for this desc and this many problems of its shape in one dispatch:
+// bf16 I/O without TTT_HINT_LDS_TILES; head_dim 128 always (the state does not fit one CU); head_dim 96 on request
+// (TTT_HINT_TWO_CU), for a single problem with at most half as many units as the device has CUs.  Measured at
+// B = 8, H = 16, seq 2048 (128 units on 256 CUs): 0.83 - 0.85 ms on pairs against 0.86 ms on single CUs -- the
+// exchange through global memory costs what halving each CU's share of the hidden axis saves -- so it is not the default.
+int uses_two_cu_mlp(const ttt_desc* d, int n_problems, bool* yes) {
+  *yes = false;
+  if (d->io_dtype == TTT_F32 || (d->kernel_hint & TTT_HINT_LDS_TILES) != 0) return TTT_OK;
+  if (d->head_dim == 128) {
+    *yes = true;
+    return TTT_OK;
+  }
+  if (d->head_dim != 96 || n_problems != 1 || (d->kernel_hint & TTT_HINT_TWO_CU) == 0) return TTT_OK;
+  int cus = 0;
+  const int rc = device_cus(&cus);
+  if (rc != TTT_OK) return rc;
+  *yes = 2 * (int64_t)d->batch * d->heads <= cus;
+  return TTT_OK;
 }
 
 template <class T, int D>
@@ -475,7 +502,7 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
   fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
   fa.W1 = ws + w.W1; fa.b1 = ws + w.b1; fa.W2 = ws + w.W2; fa.b2 = ws + w.b2;
-  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s; fa.unit_base = 0; fa.spin_limit = 1 << 21; fa.exchange_cleared = 0;
+  fa.G1_save = ws + w.G1s; fa.G2_save = ws + w.G2s; fa.unit_base = 0; fa.spin_limit = 1 << 21; fa.exchange_cleared = 0; fa.assume_other_xcd = 0;
   fa.B = d->batch; fa.H = d->heads; fa.seq = d->seq; fa.K = d->mini_batch;
   fa.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   fa.n_stages = d->seq / d->mini_batch;
@@ -775,6 +802,7 @@ int prepare_mlp_fwd(const ttt_desc* d, const void* xq, const void* xk, const voi
   a.W1 = W1_out; a.b1 = b1_out; a.W2 = W2_out; a.b2 = b2_out;
   a.G1_save = nullptr; a.G2_save = nullptr; a.unit_base = 0; a.exchange_cleared = 0;
   a.spin_limit = (d->kernel_hint & TTT_HINT_TEST_LOST_PARTNER) ? 0 : (1 << 21);
+  a.assume_other_xcd = (d->kernel_hint & TTT_HINT_TEST_OTHER_XCD) ? 1 : 0;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
   a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.n_stages = d->seq / d->mini_batch;
@@ -802,13 +830,15 @@ int dispatch_mlp_fwd_pack(const ttt_desc* d, const ttt::MlpFwdArgs* a, unsigned 
 }
 
 int dispatch_mlp_fwd(const ttt_desc* d, const ttt::MlpFwdArgs* probs, int n, hipStream_t s) {
-  // bf16 I/O, d <= 96: the state fits the register file of one CU; d = 128: of two.  TTT_HINT_LDS_TILES forces
-  // the LDS-tile kernel (f32 products, state in global memory) that the other cases use.
-  const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0;
-  if (d->io_dtype != TTT_F32 && d->head_dim == 128 && !want_lds) return launch_mlp_fwd_cl2(probs, n, s);
+  // bf16 I/O, d <= 96: the state fits the register file of one CU; d = 128: of two (see uses_two_cu_mlp).
+  // TTT_HINT_LDS_TILES forces the LDS-tile kernel (f32 products, state in global memory) that the other cases use.
+  bool two_cu = false;
+  int rc = uses_two_cu_mlp(d, n, &two_cu);
+  if (rc != TTT_OK) return rc;
+  if (two_cu) return d->head_dim == 128 ? launch_mlp_fwd_cl2<128>(probs, n, s) : launch_mlp_fwd_cl2<96>(probs, n, s);
   for (int p = 0; p < n; p += ttt::kMaxProblems) {
     const int cnt = n - p < ttt::kMaxProblems ? n - p : ttt::kMaxProblems;
-    const int rc = dispatch_mlp_fwd_pack(d, probs + p, (unsigned)cnt, s);
+    rc = dispatch_mlp_fwd_pack(d, probs + p, (unsigned)cnt, s);
     if (rc != TTT_OK) return rc;
   }
   return TTT_OK;

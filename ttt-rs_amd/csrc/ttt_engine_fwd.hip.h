@@ -208,6 +208,7 @@ struct MlpFwdArgs {
   int unit_base;  // two-CU kernel only: first (batch, head) unit of this launch (the units are launched in batches)
   int spin_limit;  // two-CU kernel only: polls before a wait for the partner gives up (0: give up at once; testing)
   int exchange_cleared;  // two-CU kernel only, read by the host: the exchange area (W2) has been zeroed by the caller
+  int assume_other_xcd;  // two-CU kernel only: treat the partner as sitting on another XCD whatever it reports (testing)
 };
 
 template <int D>

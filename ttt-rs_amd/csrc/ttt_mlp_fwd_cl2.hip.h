@@ -1,12 +1,15 @@
-// TTT-MLP multi-stage forward for head_dim 128 on gfx950: the register-resident kernel of
+// TTT-MLP multi-stage forward for head_dim 128 (and 96) on gfx950: the register-resident kernel of
 // ttt_mlp_fwd_rr.hip.h spread over a PAIR of workgroups (two CUs) per (batch, head).
 //
 // Arithmetic: reference rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50.
 //
 // At d = 128 the f32 state (W1 [128,512], W2 [512,128]: 512 KiB) equals the whole register file of
 // one CU, so the hidden axis is cut in two: workgroup `cu` of a pair owns hidden units
-// [256 cu, 256 cu + 256), i.e. W1[:, half], W2[half, :], b1[half] (128 VGPRs of state per lane), and
-// runs the register-resident scheme on its half.  What crosses the pair, once per mini-batch:
+// [2d cu, 2d cu + 2d), i.e. W1[:, half], W2[half, :], b1[half] (128 VGPRs of state per lane), and
+// runs the register-resident scheme on its half.  A workgroup has d/16 waves: one per d-feature tile
+// (reducer and output roles) and two hidden tiles each.  At d = 96 (six waves, 96 VGPRs of state) the
+// state fits one CU and the pair is an option for launches with at most half as many units as CUs.
+// What crosses the pair, once per mini-batch:
 //   X1  (recurrence)  each CU's locally reduced Z2^T tiles [d x 16]: both CUs add the two halves
 //       (always in the order cu 0 + cu 1, so both hold bit-identical Z2, G2, b2);
 //   X2  (output path) CU 1's locally reduced Zbar2^T tiles and A2 tile go to CU 0, which finishes
@@ -21,8 +24,10 @@
 // final store is ordered after its last read by program order, and the partner never writes there
 // again after its last mini-batch.  The host zeroes W2_out (tag 0 = nothing sent) before the launch.
 // Pairs are blocks (i, i + 8): with workgroups dealt round-robin to the eight XCDs both land on the
-// same XCD (shared L2); nothing depends on it.  Every wait is bounded, so a missing partner ends in
-// wrong numbers, never in a hang.
+// same XCD (shared L2), and the exchange then never leaves that L2 (workgroup-scope stores, see send_tagged).
+// That placement is checked, not assumed: at start the two workgroups tell each other which XCD they run on
+// (device-scope words), and a pair that sits on two XCDs stores at device scope for the whole launch -- slower,
+// same results.  Every wait is bounded, so a missing partner ends in NaN outputs, never in a hang.
 #pragma once
 #include "ttt_mlp_fwd_rr.hip.h"
 
@@ -30,7 +35,7 @@ namespace ttt {
 
 template <int D, int ES>
 struct MlpCl2Lds {
-  static constexpr int NW = 8, NT = D / 16, FH = 2 * D;  // FH: hidden units of one CU
+  static constexpr int NW = D / 16, NT = D / 16, FH = 2 * D;  // FH: hidden units of one CU; one wave per d-feature tile
   static constexpr int TILE = 16 * D * ES;
   static constexpr int IN1 = 3 * TILE;
   static constexpr int IN = 0;                  // [2 buffers][3][16][d]
@@ -47,12 +52,14 @@ struct MlpCl2Lds {
   static constexpr int LOST = EXO + 2 * 2 * 16 * 16;  // one word: a wait for the partner ran out
   static constexpr int BYTES = LOST + 16;
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
-  static_assert(NT == NW && D % 64 == 0 && ES == 2, "one reducer and one output tile per wave, bf16 I/O");
+  static_assert(NT == NW && NW <= 8 && D % 32 == 0 && ES == 2, "one reducer and one output tile per wave, bf16 I/O");
+  static_assert(FH % (16 * NW) == 0, "whole hidden tiles per wave");
   static_assert(TILE % 1024 == 0 && P1 % 16 == 0, "input tiles are staged in 1 KiB wave blocks");
   // exchange area inside this CU's rows of W2_out (bytes): two parities of X1 tiles, X2 tiles, A2 tile,
   // each tile as 64 lanes x 4 tagged 64-bit words
   static constexpr int XTILE = 2048, XSLOT = (2 * NT + 1) * XTILE;
-  static_assert(2 * XSLOT <= FH * D * 4, "exchange area exceeds this CU's rows of W2_out");
+  static constexpr int XHELLO = 2 * XSLOT;  // one tagged word behind the tiles: the partner's XCD
+  static_assert(XHELLO + 16 <= FH * D * 4, "exchange area exceeds this CU's rows of W2_out");
 };
 
 // One [16 x 16] f32 tile (this lane's four values) as four (value, tag) words.
@@ -60,13 +67,20 @@ struct MlpCl2Lds {
 // The stores therefore carry workgroup scope: they leave the CU (its L1 writes through) and stay in that L2, where
 // the partner's device-scope loads, which bypass its own L1, find them.  Device-scope stores would also be written
 // through to memory, every one of them: measured at 2.8 GB of writes per launch of 128 units x 2048 tokens, which
-// made the kernel 40 % slower on a full GPU than on a quarter of it.  Should a pair ever land on two XCDs, its
-// words never arrive, the waits run out and the unit's outputs are NaN (see recv_tagged): loud, not wrong.
-__device__ __forceinline__ void send_tagged(unsigned long long* slot, f32x4 v, unsigned tag) {
+// made the kernel 40 % slower on a full GPU than on a quarter of it.  `same_xcd` is what the two workgroups found
+// out about each other at start (see the kernel): a pair on two XCDs stores at device scope.
+__device__ __forceinline__ void send_tagged(unsigned long long* slot, f32x4 v, unsigned tag, bool same_xcd) {
+  if (same_xcd) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r)
-    __hip_atomic_store(slot + r, ((unsigned long long)tag << 32) | __float_as_uint(v[r]), __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_WORKGROUP);
+    for (int r = 0; r < 4; ++r)
+      __hip_atomic_store(slot + r, ((unsigned long long)tag << 32) | __float_as_uint(v[r]), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_WORKGROUP);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      __hip_atomic_store(slot + r, ((unsigned long long)tag << 32) | __float_as_uint(v[r]), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 // Receives N tiles at once: polls until the four words of every slot carry that slot's tag, all
 // loads of a round in flight together (one memory round trip per round, not one per tile).  The wait
@@ -119,14 +133,14 @@ __device__ unsigned int g_mlp_fwd_lost_workgroups = 0u;
 #define RELANE() asm volatile("" : "+v"(lane))
 
 template <class T, int D>
-__global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArgs> problems) {
+__global__ void __launch_bounds__(64 * (D / 16)) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArgs> problems) {
   const MlpFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;
   constexpr int ES = sizeof(elem);
   using L = MlpCl2Lds<D, ES>;
-  constexpr int NW = 8, NT = D / 16, F = 4 * D, FH = L::FH, HT = FH / 16 / NW;
+  constexpr int NW = L::NW, NT = D / 16, F = 4 * D, FH = L::FH, HT = FH / 16 / NW, NTHR = 64 * NW;
   constexpr float inv_d = 1.0f / D;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -159,6 +173,16 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArg
   // exchange areas: what this CU receives lies in its own rows of W2_out, what it sends in the partner's
   unsigned char* const xin = reinterpret_cast<unsigned char*>(a.W2 + (bh * F + hoff) * (size_t)D);
   unsigned char* const xout = reinterpret_cast<unsigned char*>(a.W2 + (bh * F + (FH - hoff)) * (size_t)D);
+
+  // ---- which XCD does the partner run on?  One device-scope word each way (tag 0xffffffff: no mini-batch uses it),
+  // sent before the state is loaded and read after, so the round trip costs nothing.  The answer decides the scope
+  // of every later store to the partner.
+  unsigned my_xcc;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(my_xcc));
+  my_xcc &= 15u;
+  if (tid == 0)
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(xout + L::XHELLO), (0xffffffffull << 32) | my_xcc, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 
   const float te_last = a.token_eta[K - 1];
   const bool upd = te_last != 0.f;
@@ -199,11 +223,11 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArg
   }
   b2T -= mean_of(a.b2_0 + sb * D, D, inv_d);
   for (int f = 0; f < D; ++f) sum_a += a.gamma[h * D + f] * a.gamma[h * D + f];
-  for (int i = tid; i < D; i += 512) {
+  for (int i = tid; i < D; i += NTHR) {
     GAM[i] = a.gamma[h * D + i];
     BET[i] = a.beta[h * D + i];
   }
-  for (int i = tid; i < FH; i += 512) B1s[i] = a.b1_0[sb * F + hoff + i];
+  for (int i = tid; i < FH; i += NTHR) B1s[i] = a.b1_0[sb * F + hoff + i];
 
   // ---- staging of the xq / xk / xv rows: global -> LDS, two buffers.  The fetch of mini-batch st+1 is
   // issued after the first barrier of mini-batch st (every wave has then finished reading the buffer it
@@ -240,10 +264,23 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArg
     return reinterpret_cast<const elem*>(smem + L::IN + buf * L::IN1 + ten * L::TILE) + c * D;
   };
 
-  for (int i = tid; i < (L::P1 - L::IN) / 4; i += 512) reinterpret_cast<float*>(smem)[i] = 0.f;
-  for (int i = tid; i < 8 * 2 * 16 * 4; i += 512) EX[i] = 0.f;
+  for (int i = tid; i < (L::P1 - L::IN) / 4; i += NTHR) reinterpret_cast<float*>(smem)[i] = 0.f;
+  for (int i = tid; i < 8 * 2 * 16 * 4; i += NTHR) EX[i] = 0.f;
   if (tid < 2 * 2 * 16 * 4) EXO[tid] = 0.f;
+  int& partner_xcc = *reinterpret_cast<int*>(smem + L::LOST + 4);  // -1: the partner never said
+  if (tid == 0) {
+    const unsigned long long* hello = reinterpret_cast<const unsigned long long*>(xin + L::XHELLO);
+    unsigned long long wd = 0;
+    int it = 0;
+    while ((unsigned)((wd = __hip_atomic_load(hello, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) != 0xffffffffu) {
+      if (++it >= a.spin_limit) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+    partner_xcc = (unsigned)(wd >> 32) == 0xffffffffu ? (int)(wd & 15u) : -1;
+  }
   __syncthreads();
+  // a partner that never said where it runs is treated like one on another XCD; the first wait for it will run out
+  const bool same_xcd = !a.assume_other_xcd && __builtin_amdgcn_readfirstlane(partner_xcc) == (int)my_xcc;
   fetch(0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -262,7 +299,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArg
   // tile slot `idx` of parity `par`: X1 tiles 0..NT-1, X2 tiles NT..2NT-1, the A2 tile 2NT
   bool alive = a.spin_limit > 0;
   auto send_tile = [&](int par_, int idx, f32x4 v, unsigned tag) {
-    send_tagged(reinterpret_cast<unsigned long long*>(xout + par_ * L::XSLOT + idx * L::XTILE) + 4 * lane, v, tag);
+    send_tagged(reinterpret_cast<unsigned long long*>(xout + par_ * L::XSLOT + idx * L::XTILE) + 4 * lane, v, tag, same_xcd);
   };
   auto slot_in = [&](int par_, int idx) -> const unsigned long long* {
     return reinterpret_cast<const unsigned long long*>(xin + par_ * L::XSLOT + idx * L::XTILE) + 4 * lane;
@@ -624,7 +661,7 @@ __global__ void __launch_bounds__(512) ttt_mlp_fwd_cl2_kernel(Problems<MlpFwdArg
       if (tid == 0) atomicAdd(&g_mlp_fwd_lost_workgroups, 1u);
       elem* po = static_cast<elem*>(a.out) + bh * (size_t)a.seq_stride * D;
       const size_t n = (size_t)a.n_stages * K * D;
-      for (size_t i = tid; i < n; i += 512) IO::store1(po + i, poison);
+      for (size_t i = tid; i < n; i += NTHR) IO::store1(po + i, poison);
     }
   }
 }

@@ -588,8 +588,8 @@ def ttt_stack_forward_raw(layers, token_eta, mini_batch: int, eps: float = 1e-6,
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "workspace too small")
     out = torch.empty((B, H, seq, d), dtype=io, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    two_cu = d == 128 and io == torch.bfloat16 and any("W2" in L for L in layers) and \
-        not (kernel_hint & _lib.TTT_HINT_LDS_TILES)
+    two_cu = (d == 128 or (d == 96 and kernel_hint & _lib.TTT_HINT_TWO_CU)) and io == torch.bfloat16 and \
+        any("W2" in L for L in layers) and not (kernel_hint & _lib.TTT_HINT_LDS_TILES)
     if check_lost is None:
         check_lost = two_cu and not torch.cuda.is_current_stream_capturing()
     with torch.cuda.device(dev):
