@@ -268,6 +268,21 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && D / 16 == NW && (PK || si
       for (int jj = 0; jj < TPW; ++jj) IO::mma(acc, A[jj], B[jj]);
     }
   };
+  // The counted waits of the scan.  Memory operations of a wave retire in the order they were issued, stores
+  // included, so "s_waitcnt vmcnt(n)" with n = the number of operations a wave is KNOWN to have issued behind its
+  // global->LDS copies waits for the copies and not for those younger operations.  Counted are the row stores of the
+  // three activation gradients, one store_own per tensor, wave and pass, issued by every wave on every path: the
+  // guard in front of each is a lane mask (c < K), never a wave-uniform branch, so a mini-batch shorter than 16 tokens
+  // still issues it, and store_own is at least one instruction for TPW <= 2 (an f32 store of two tiles is two: more
+  // operations than counted only make the wait longer).  Operations that only some waves issue (d_lr by the first
+  // wave, the d_token_eta atomics by the last) are not counted.  Fewer operations than counted would let the loop
+  // read staged rows before they have landed, so whoever moves a store_own across one of the two waits, or makes one
+  // conditional at wave level, changes these numbers with it.
+  //   loop top: d_xq, d_xv and d_xk of the pass before lie behind the copies (issued before the first of them)
+  //   X4 barrier (FM only; the walk back reads the staged rows): d_xq and d_xv lie behind the copies
+  static_assert(TPW <= 2, "store_own must stay one store instruction (bf16) per tensor and wave");
+  constexpr int kStoresBehindCopiesAtLoopTop = 3;
+  constexpr int kStoresBehindCopiesAtX4 = 2;
   auto store_own = [&](void* base, size_t tokoff, const f32x4 (&x)[TPW]) {
     elem* p = static_cast<elem*>(base) + tokoff;
     if (TPW == 1) {
@@ -343,7 +358,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && D / 16 == NW && (PK || si
     if (st == a.n_stages - 1)
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     else
-      asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStoresBehindCopiesAtLoopTop) : "memory");
     lds_barrier();
     const unsigned char* sl = smem + lane * 16;
     frag q[NT], k[NT], qo[TPW], ko[TPW], vo[TPW], oo[TPW];  // full rows of xq, xk; own features of all four
@@ -700,10 +715,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && D / 16 == NW && (PK || si
     // ---- X4: dZ1 fragments
     // FM: the copies of the next mini-batch (issued behind X1; two stores, d_xq and d_xv, are younger) have to be
     // visible to every wave behind this barrier: the walk back at the end of the pass reads them
-    if constexpr (FM) {
-      static_assert(TPW <= 2, "one store per tensor and wave");
-      asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-    }
+    if constexpr (FM) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStoresBehindCopiesAtX4) : "memory");
     lds_barrier();
     {
       frag Z1fa[NT];
