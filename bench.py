@@ -37,6 +37,9 @@ WORKLOADS = {
     # the elementwise passes either side of the inner loop at the 125M shape (hidden 768)
     "inner_inputs_125m_bf16": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="inner_inputs"),
     "layer_epilogue_125m_bf16": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="layer_epilogue"),
+    # the forward on the projections as the GEMMs leave them: head split, RoPE, lr gate and token_eta formed inside the
+    # inner kernel's tile loads (one kernel in place of ttt_inner_inputs followed by ttt_linear_fwd)
+    "linear_fwd_fused_inputs_125m_bf16": dict(cfg=1, B=32, H=12, d=64, seq=2048, K=16, io="bf16", kind="linear_fwd_fused"),
     "stack8_d128_seq8192_bf16": dict(cfg=4, B=4, H=16, d=128, seq=8192, K=16, io="bf16", kind="stack"),
 }
 
@@ -127,6 +130,43 @@ def cpu_baseline_stack(layers_cpu, K, io_dtype, torch, B):
             "sample": f"C/OpenMP f32 ports of the reference CPU path (TTT-Linear and TTT-MLP forward) chained through the "
                       f"{len(L1)} layers, same inputs, batch 1 of {B} (tokens/s is batch-normalised), mean of 3 runs after "
                       f"one warm-up, {t:.3f} s per run"}
+
+
+def cpu_baseline_fused(fused_cpu, K, base_lr, budget_s=12.0):
+    """The forward from the projections on the host cores: the numpy restatement of the producers (head split, RoPE,
+    lr gate, token_eta: oracle.inner_loop_inputs, float32) followed by the C/OpenMP port of the TTT-Linear forward, on
+    a bounded batch slice of the same inputs."""
+    import numpy as np
+    from oracle import c_oracle, ttt_oracle as orc
+    cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "9999")))
+    raw = {k: v.float().numpy() for k, v in fused_cpu["raw"].items()}
+    par = {k: v.float().numpy() for k, v in fused_cpu["par"].items()}
+    B, seq, H, d = raw["xq"].shape
+    cos, sin = orc.rope_cos_sin(seq, 0, K, d)
+    tidx = (1.0 / np.arange(1, K + 1)).astype(np.float32)
+
+    def run(nb):
+        q, k, v, lr, te = orc.inner_loop_inputs(raw["xq"][:nb], raw["xk"][:nb], raw["xv"][:nb], raw["lg"][:nb],
+                                                np.zeros(H, np.float32), base_lr, tidx, np.zeros(K, np.float32), K,
+                                                cos, sin, dtype=np.float32)
+        c = np.ascontiguousarray
+        c_oracle.linear_fwd(par["W0"], par["b0"], c(q), c(k), c(v), te[:K].astype(np.float32), c(lr), par["gamma"],
+                            par["beta"], K=K, dtype=np.float32, nthreads=cores)
+
+    t0 = time.perf_counter()
+    run(1)
+    t_one = time.perf_counter() - t0
+    Bs = max(1, min(B, int(budget_s / 4 / max(t_one, 1e-4))))
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run(Bs)
+        times.append(time.perf_counter() - t0)
+    t = sum(times) / len(times)
+    return {"value": Bs * seq / t, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"numpy f32 restatement of the producers (one thread) + C/OpenMP f32 port of the TTT-Linear forward "
+                      f"({cores} threads), same inputs, batch {Bs} of {B} (tokens/s is batch-normalised), mean of 3 runs "
+                      f"after one probe, {t:.3f} s per run"}
 
 
 class LinearCalls:
@@ -234,6 +274,44 @@ def run_workload(name, a, pkg, torch):
             # one call: per layer and window the input sums (x read once for xq, xk, xv) and the inner loop
             return (pkg.ttt_stack_forward_raw(stack, layers[0]["token_eta"], K, workspace=ws, chunk_tokens=chunk,
                                               aux_stream=aux, check_lost=False)[0],)
+    elif kind == "linear_fwd_fused":
+        import ctypes as C
+        g = torch.Generator().manual_seed(1234 + w["cfg"])
+        raw = {k: torch.randn(*sh, generator=g).to(dtype) for k, sh in
+               (("xq", (B, seq, H, d)), ("xk", (B, seq, H, d)), ("xv", (B, seq, H, d)), ("lg", (B, seq, H)))}
+        par = pkg.synthetic.baseline_inputs(w["cfg"], 1, H, K, d, K, io_dtype=dtype)   # W0, b0, gamma, beta of the shape
+        fused_cpu = dict(raw=raw, par=par)
+        rd = {k: v.to(dev) for k, v in raw.items()}
+        pd = {k: par[k].to(dev) for k in ("W0", "b0", "gamma", "beta")}
+        bias = torch.zeros(H, device=dev)
+        tidx = (1.0 / torch.arange(1, K + 1, dtype=torch.float32)).to(dev)
+        ltidx = torch.zeros(K, device=dev)
+        rope = pkg.rope_cos_sin(K, 0, None, d, dev)
+        f32 = dict(dtype=torch.float32, device=dev)
+        fo = dict(out=torch.empty((B, H, seq, d), dtype=dtype, device=dev), W=torch.empty((B, H, d, d), **f32),
+                  b=torch.empty((B, H, d), **f32))
+        desc = pkg.TttDesc(B, H, seq, d, K, 1e-6, 1, pkg.TTT_BF16, 0, 0, 0, 0)
+        ptr = lambda t: C.c_void_p(t.data_ptr())
+        stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+        def fused_call():
+            pkg._lib.check(pkg.lib().ttt_linear_fwd_fused_inputs(
+                C.byref(desc), ptr(rd["xq"]), ptr(rd["xk"]), ptr(rd["xv"]), ptr(rd["lg"]), ptr(bias), C.c_float(1.0),
+                ptr(tidx), ptr(ltidx), ptr(rope[0]), ptr(rope[1]), 0, K, ptr(pd["W0"]), ptr(pd["b0"]), ptr(pd["gamma"]),
+                ptr(pd["beta"]), ptr(fo["out"]), ptr(fo["W"]), ptr(fo["b"]), None, None, None, None, None, None, None,
+                stream))
+
+        def two_pass():
+            i = pkg.inner_loop_inputs_raw(rd["xq"], rd["xk"], rd["xv"], rd["lg"], bias, 1.0, tidx, ltidx, K, rope=rope,
+                                          pos_wrap=K)
+            return pkg.ttt_linear_forward_raw(i.qkv.xq, i.qkv.xk, i.qkv.xv, pd["W0"], pd["b0"], i.token_eta,
+                                              i.ttt_lr_eta, pd["gamma"], pd["beta"], K)
+
+        parts = [("ttt_linear_fwd_fused_inputs", fused_call), ("ttt_inner_inputs + ttt_linear_fwd", two_pass)]
+
+        def step():
+            fused_call()
+            return (fo["out"], fo["W"])
     elif kind in ("inner_inputs", "layer_epilogue"):
         g = torch.Generator().manual_seed(1234 + w["cfg"])
         rn = lambda *sh: torch.randn(*sh, generator=g).to(dtype).to(dev)
@@ -318,7 +396,8 @@ def run_workload(name, a, pkg, torch):
     assert lost == 0, f"{lost} workgroups of the two-CU TTT-MLP kernel waited for their partner in vain"
 
     pass_name = {"linear_fwd": "fwd", "linear_fwd_bwd": "fwd+bwd", "mlp_fwd": "fwd", "mlp_fwd_bwd": "fwd+bwd",
-                 "stack": "fwd", "inner_inputs": "inner-loop inputs", "layer_epilogue": "layer epilogue"}[kind]
+                 "stack": "fwd", "inner_inputs": "inner-loop inputs", "layer_epilogue": "layer epilogue",
+                 "linear_fwd_fused": "fwd from the projections"}[kind]
     out = {
         "metric": f"inner-loop tokens/sec ({pass_name}) at 125M shape" if d == 64 else
                   f"inner-loop tokens/sec ({pass_name})",
@@ -346,6 +425,21 @@ def run_workload(name, a, pkg, torch):
                            "frac": alg / k_s / 1e9 / HBM_PEAK_GBS, **counters,
                            "kernel": "ttt_linear_fwd_sk_kernel", "kernel_avg_us": k_s * 1e6,
                            "step_avg_us": dev_s * 1e6, "algorithmic_bytes": alg}
+    elif kind == "linear_fwd_fused":
+        # the projections and the logits in, out written once: the bytes of the inner loop itself; the two-pass path
+        # moves 6 d s + 2 s more per token-head (the [B,H,seq,d] copies written and read back)
+        alg = linear_fwd_bytes(B, H, seq, d, s)
+        k_s, two_s = part_s["ttt_linear_fwd_fused_inputs"], part_s["ttt_inner_inputs + ttt_linear_fwd"]
+        out["dtype"] = "bf16"
+        out["config"]["inner_model"] = "TTT-Linear"
+        out["roofline"] = {"bound": "hbm", "achieved": alg / k_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": alg / k_s / 1e9 / HBM_PEAK_GBS, **counters,
+                           "kernel": "ttt_linear_fwd_fi_kernel", "kernel_avg_us": k_s * 1e6,
+                           "step_avg_us": dev_s * 1e6, "algorithmic_bytes": alg,
+                           "other_kernels": [{"kernel": "ttt_inner_inputs_kernel + ttt_linear_fwd_sk_kernel (the two "
+                                                        "passes this kernel replaces, same inputs, same run)",
+                                              "kernel_avg_us": two_s * 1e6,
+                                              "algorithmic_bytes": alg + th * (6 * d * s + 2 * s)}]}
     elif kind in ("inner_inputs", "layer_epilogue"):
         # inner_inputs: xq, xk, xv read and written once, logits in, lr out; epilogue: inner_out and gate in, out written
         alg = th * (6 * d * s + 2 * s) if kind == "inner_inputs" else th * 3 * d * s
@@ -422,15 +516,17 @@ def run_workload(name, a, pkg, torch):
         out["cpu_baseline"] = cpu_baseline(c, K, kind)
     elif not a.no_cpu_baseline and kind == "stack":
         out["cpu_baseline"] = cpu_baseline_stack(layers_cpu, K, dtype, torch, B)
+    elif not a.no_cpu_baseline and kind == "linear_fwd_fused":
+        out["cpu_baseline"] = cpu_baseline_fused(fused_cpu, K, 1.0)
     return out
 
 
 # the headline metric names the forward AND the forward+backward at the 125M shape: the default run measures the
 # forward (BASELINE config 1) as the line's own value and, as `extra` entries, the two forward+backward workloads
 # (bf16 at the config-1 shape, f32 = BASELINE config 2), the TTT-MLP forward (config 3) with its forward+backward,
-# and the 8-layer long-context stack (config 4)
+# the 8-layer long-context stack (config 4), and the forward of config 1 on the projections (producers fused in)
 DEFAULT_EXTRA = ("linear_fwd_bwd_125m_bf16_b32", "linear_fwd_bwd_125m_f32_b8", "mlp_fwd_d96_bf16",
-                 "mlp_fwd_bwd_d96_bf16", "stack8_d128_seq8192_bf16")
+                 "mlp_fwd_bwd_d96_bf16", "stack8_d128_seq8192_bf16", "linear_fwd_fused_inputs_125m_bf16")
 
 
 def main():

@@ -349,6 +349,35 @@ int ttt_layer_epilogue(const ttt_desc* desc, const void* inner_out, const float*
                        const float* post_norm_bias, float eps, const void* gate, void* out, void* stream);
 
 /*
+ * ttt_inner_inputs and ttt_linear_fwd in one kernel: the TTT-Linear forward on the projections as they leave the
+ * GEMMs.  Replaces TTT::get_inner_loop_inputs after the projections (rust/layer/src/ttt.rs:147-194 get_qkv, :205-227
+ * get_lr, :247-268) followed by FusedKernelBackend<TttTileMultiKernel>::forward (rust/kernels/src/kernel.rs:62-69):
+ * the head split is a row stride of the kernel's loads, the rotary embedding of xq and xk and the lr gate are applied
+ * to the tiles in registers (each feature by the one wave that owns it), token_eta is formed from its two addends;
+ * the [B,H,seq,d] copies of xq, xk, xv that ttt_inner_inputs writes and ttt_linear_fwd reads are never made.
+ *   xq,xk,xv [B,seq,H,d] io; lr_logits [B,seq,H] io; lr_bias [H]; token_idx, learnable_token_idx [mini_batch];
+ *   rope_cos, rope_sin [npos, d/2] f32 or both NULL; pos_offset, pos_wrap as for ttt_inner_inputs, with pos_wrap
+ *   either a divisor of mini_batch (positions repeat with the mini-batch: the reference's default, ttt.rs:186-189)
+ *   or 0 (positions over the sequence, RopeGlobal).
+ *   W0 .. b_ckpt as for ttt_linear_fwd (out [B,H,seq,d] io).
+ *   xq_out, xk_out, xv_out [B,H,seq,d] io, lr_out [B,H,seq] io, token_eta_out [seq] f32: the operands as the
+ *   kernel used them, i.e. exactly what ttt_inner_inputs would have written; ttt_linear_bwd takes them as its saved
+ *   inputs.  Each may be NULL (not stored: inference).
+ * Exists for bf16 I/O, head_dim 32 and 64, checkpoint formats TTT_CKPT_F32 and TTT_CKPT_PACKED, seq_stride 0;
+ * ttt_linear_fwd_fused_inputs_supported says so beforehand (TTT_OK or the status the call would return; has_rope:
+ * whether tables will be passed).  Results equal ttt_inner_inputs followed by ttt_linear_fwd on the same values
+ * (same rounding of the rotated operands and of lr to the I/O type).
+ */
+int ttt_linear_fwd_fused_inputs_supported(const ttt_desc* desc, int pos_wrap, int has_rope);
+int ttt_linear_fwd_fused_inputs(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                                const void* lr_logits, const float* lr_bias, float base_lr, const float* token_idx,
+                                const float* learnable_token_idx, const float* rope_cos, const float* rope_sin,
+                                int pos_offset, int pos_wrap, const float* W0, const float* b0, const float* gamma,
+                                const float* beta, void* out, float* W_out, float* b_out, float* W_ckpt, float* b_ckpt,
+                                void* xq_out, void* xk_out, void* xv_out, void* lr_out, float* token_eta_out,
+                                void* stream);
+
+/*
  * Self-test of a hardware fact the bf16 kernels rely on; no counterpart in the reference.  One wavefront computes
  * D = A1*B1 with one bf16 matrix instruction and accumulates A2*B2 onto it, in place, with an instruction of the
  * other shape (order 0: 16x16x32 then 16x16x16; order 1: the reverse), `gap` wait states apart (0, 4 or 5), on

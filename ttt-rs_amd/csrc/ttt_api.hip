@@ -662,6 +662,75 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   return dispatch_linear_fwd(d, &a, 1, static_cast<hipStream_t>(stream));
 }
 
+int ttt_linear_fwd_fused_inputs_supported(const ttt_desc* d, int pos_wrap, int has_rope) {
+  int rc = ttt_linear_supported(d);
+  if (rc != TTT_OK) return rc;
+  if (d->io_dtype != TTT_BF16 || (d->head_dim != 64 && d->head_dim != 32))
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_fwd_fused_inputs: bf16 I/O and head_dim 32 or 64 (got %s, %d)",
+                d->io_dtype == TTT_BF16 ? "bf16" : "f32", d->head_dim);
+  if (d->seq_stride != 0 && d->seq_stride != d->seq)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_fwd_fused_inputs: seq_stride must be 0");
+  if (d->checkpoint_format == TTT_CKPT_FACTORS)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_fwd_fused_inputs: checkpoint formats f32 and packed only");
+  if ((d->kernel_hint & TTT_HINT_LDS_TILES) != 0)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_fwd_fused_inputs: the register-resident kernel only");
+  if (has_rope && pos_wrap < 0) return fail(TTT_ERR_SHAPE, "pos_wrap must be >= 0");
+  if (has_rope && pos_wrap > 0 && d->mini_batch % pos_wrap != 0)
+    return fail(TTT_ERR_UNSUPPORTED,
+                "ttt_linear_fwd_fused_inputs: pos_wrap %d must divide mini_batch %d (positions that repeat with the "
+                "mini-batch) or be 0 (positions over the sequence)", pos_wrap, d->mini_batch);
+  return TTT_OK;
+}
+
+int ttt_linear_fwd_fused_inputs(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                                const void* lr_logits, const float* lr_bias, float base_lr, const float* token_idx,
+                                const float* learnable_token_idx, const float* rope_cos, const float* rope_sin,
+                                int pos_offset, int pos_wrap, const float* W0, const float* b0, const float* gamma,
+                                const float* beta, void* out, float* W_out, float* b_out, float* W_ckpt, float* b_ckpt,
+                                void* xq_out, void* xk_out, void* xv_out, void* lr_out, float* token_eta_out,
+                                void* stream) {
+  if ((rope_cos == nullptr) != (rope_sin == nullptr))
+    return fail(TTT_ERR_NULL, "rope_cos and rope_sin must both be given or both be NULL");
+  int rc = ttt_linear_fwd_fused_inputs_supported(d, pos_wrap, rope_cos != nullptr);
+  if (rc != TTT_OK) return rc;
+  if (!lr_logits || !lr_bias || !token_idx || !learnable_token_idx)
+    return fail(TTT_ERR_NULL, "ttt_linear_fwd_fused_inputs: a required pointer is NULL");
+  if (pos_offset < 0) return fail(TTT_ERR_SHAPE, "pos_offset must be >= 0");
+  if (!aligned16(xq_out) || !aligned16(xk_out) || !aligned16(xv_out))
+    return fail(TTT_ERR_SHAPE, "xq_out/xk_out/xv_out must be 16-byte aligned");
+  if ((rope_cos != nullptr && (reinterpret_cast<uintptr_t>(rope_cos) & 7u) != 0) ||
+      (rope_sin != nullptr && (reinterpret_cast<uintptr_t>(rope_sin) & 7u) != 0))
+    return fail(TTT_ERR_SHAPE, "rope_cos/rope_sin must be 8-byte aligned");
+  ttt::LinearFwdArgs a;
+  // the operand fields of the argument block are not read in this mode; the raw tensors stand in for the checks
+  rc = prepare_linear_fwd(d, xq, xk, xv, W0, b0, token_idx, lr_logits, gamma, beta, out, W_out, b_out, W_ckpt, b_ckpt, &a);
+  if (rc != TTT_OK) return rc;
+  a.xq = a.xk = a.xv = a.lr = nullptr;
+  a.token_eta = nullptr;
+  a.seq_stride = d->seq;
+  ttt::FusedInputsArgs fi;
+  fi.xq = xq; fi.xk = xk; fi.xv = xv; fi.lr_logits = lr_logits; fi.lr_bias = lr_bias;
+  fi.token_idx = token_idx; fi.learnable_token_idx = learnable_token_idx; fi.cos = rope_cos; fi.sin = rope_sin;
+  fi.xq_out = xq_out; fi.xk_out = xk_out; fi.xv_out = xv_out; fi.lr_out = lr_out; fi.token_eta_out = token_eta_out;
+  fi.lr_scale = base_lr / (float)d->head_dim;
+  fi.pos_offset = pos_offset; fi.pos_wrap = pos_wrap;
+  const bool per_token = rope_cos != nullptr && pos_wrap == 0;  // positions run over the sequence
+  const bool full = d->mini_batch == 16;
+  const dim3 grid((unsigned)(a.B * a.H)), block(128);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define TTT_FI_LAUNCH(D_, FULL_, RAW_) \
+  hipLaunchKernelGGL((ttt::ttt_linear_fwd_fi_kernel<ttt::BF16, D_, 2, 2, FULL_, false, RAW_>), grid, block, 0, s, a, fi)
+  if (d->head_dim == 64) {
+    if (per_token) { if (full) TTT_FI_LAUNCH(64, true, 2); else TTT_FI_LAUNCH(64, false, 2); }
+    else { if (full) TTT_FI_LAUNCH(64, true, 1); else TTT_FI_LAUNCH(64, false, 1); }
+  } else {
+    if (per_token) { if (full) TTT_FI_LAUNCH(32, true, 2); else TTT_FI_LAUNCH(32, false, 2); }
+    else { if (full) TTT_FI_LAUNCH(32, true, 1); else TTT_FI_LAUNCH(32, false, 1); }
+  }
+#undef TTT_FI_LAUNCH
+  return hip_status(hipGetLastError(), "ttt_linear_fwd_fused_inputs launch");
+}
+
 int ttt_linear_bwd_supported(const ttt_desc* d) {
   LinearBwdChoice ch;
   return choose_linear_bwd(d, &ch);

@@ -189,6 +189,8 @@ struct Io<F32> {
   }
   __device__ static __forceinline__ float load1(const elem* p) { return *p; }
   __device__ static __forceinline__ void store1(elem* p, float v) { *p = v; }
+  // what load1 reads back after store1(v)
+  __device__ static __forceinline__ float rounded(float v) { return v; }
 };
 
 // ---- bf16 storage, bf16 MFMA with f32 accumulation
@@ -233,6 +235,9 @@ struct Io<BF16> {
   __device__ static __forceinline__ void store1(elem* p, float v) {
     *p = __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
   }
+  __device__ static __forceinline__ float rounded(float v) {
+    return __builtin_bit_cast(float, static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<__bf16>(v))) << 16);
+  }
 };
 
 // Identity fragment: as B operand, B[k = 4g+r, n = c] = (c == 4g+r).  acc = mma(0, X, I) turns
@@ -249,6 +254,16 @@ template <class T>
 __device__ __forceinline__ typename Io<T>::frag splat_frag(float x) {
   return Io<T>::to_frag(f32x4{x, x, x, x});
 }
+
+// Rotary embedding of four consecutive features: the adjacent pairs (x0, x1) and (x2, x3) are rotated by the angles
+// whose cosines and sines are cs, sn.  One routine with explicit fused multiply-adds for every kernel that rotates:
+// the pass that prepares the inner loop's inputs and the forward that forms them itself must give the same bits.
+__device__ __forceinline__ f32x4 rope_rotate4(f32x4 x, f32x2 cs, f32x2 sn) {
+  return f32x4{__builtin_fmaf(x[0], cs[0], -(x[1] * sn[0])), __builtin_fmaf(x[1], cs[0], x[0] * sn[0]),
+               __builtin_fmaf(x[2], cs[1], -(x[3] * sn[1])), __builtin_fmaf(x[3], cs[1], x[2] * sn[1])};
+}
+// ttt_lr_eta of a token: scale * sigmoid(z), scale = base_lr / head_dim (reference rust/layer/src/ttt.rs:205-227)
+__device__ __forceinline__ float lr_gate(float z, float scale) { return scale / (1.f + __expf(-z)); }
 
 // A launch may carry several independent problems of one shape, gridDim.y of them (windows of different layers of
 // a stack that are ready at the same time: one layer's 64 units alone leave three quarters of the CUs idle).  The

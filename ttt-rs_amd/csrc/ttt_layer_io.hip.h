@@ -68,18 +68,14 @@ __global__ void __launch_bounds__(256) ttt_inner_inputs_kernel(InnerInputsArgs a
   }
   auto rotate = [&](const void* in, void* out) {
     IO::load8(static_cast<const elem*>(in) + src, true, lo, hi);
-    const f32x4 x0 = IO::to_f32(lo), x1 = IO::to_f32(hi);
-    const f32x4 y0 = {x0[0] * cs[0] - x0[1] * sn[0], x0[1] * cs[0] + x0[0] * sn[0],
-                      x0[2] * cs[1] - x0[3] * sn[1], x0[3] * cs[1] + x0[2] * sn[1]};
-    const f32x4 y1 = {x1[0] * cs[2] - x1[1] * sn[2], x1[1] * cs[2] + x1[0] * sn[2],
-                      x1[2] * cs[3] - x1[3] * sn[3], x1[3] * cs[3] + x1[2] * sn[3]};
-    IO::store8(static_cast<elem*>(out) + dst, y0, y1);
+    IO::store8(static_cast<elem*>(out) + dst, rope_rotate4(IO::to_f32(lo), f32x2{cs[0], cs[1]}, f32x2{sn[0], sn[1]}),
+               rope_rotate4(IO::to_f32(hi), f32x2{cs[2], cs[3]}, f32x2{sn[2], sn[3]}));
   };
   rotate(a.xq, a.xq_out);
   rotate(a.xk, a.xk_out);
   if (ch == 0) {
     const float z = IO::load1(static_cast<const elem*>(a.lr_logits) + r) + a.lr_bias[h];
-    IO::store1(static_cast<elem*>(a.lr_out) + (b * a.H + h) * (size_t)a.seq + t, a.lr_scale / (1.f + __expf(-z)));
+    IO::store1(static_cast<elem*>(a.lr_out) + (b * a.H + h) * (size_t)a.seq + t, lr_gate(z, a.lr_scale));
   }
 }
 

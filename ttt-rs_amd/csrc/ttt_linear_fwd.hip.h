@@ -29,4 +29,26 @@ struct LinearFwdArgs {
   float eps;
 };
 
+// What the forward needs beside LinearFwdArgs when it forms its operands from the projections itself
+// (ttt_linear_fwd_fi_kernel): the inputs and parameters of ttt_inner_inputs.  In that mode the fields xq, xk, xv, lr
+// and token_eta of LinearFwdArgs are not read.
+struct FusedInputsArgs {
+  const void* xq;  // [B,seq,H,d] io, as the projections leave them
+  const void* xk;
+  const void* xv;
+  const void* lr_logits;             // [B,seq,H] io
+  const float* lr_bias;              // [H]
+  const float* token_idx;            // [K]
+  const float* learnable_token_idx;  // [K]
+  const float* cos;                  // [npos, d/2] or null: no rotary embedding
+  const float* sin;
+  void* xq_out;  // [B,H,seq,d] io: the operands as the kernel used them (what ttt_linear_bwd needs); each may be null
+  void* xk_out;
+  void* xv_out;
+  void* lr_out;          // [B,H,seq] io or null
+  float* token_eta_out;  // [seq] or null
+  float lr_scale;        // base_lr / d
+  int pos_offset, pos_wrap;  // position of token t: (pos_offset + t) [% pos_wrap if > 0]
+};
+
 }  // namespace ttt

@@ -17,9 +17,21 @@
 
 namespace ttt {
 
-template <class T, int D, int NW, int PF, bool FULL, bool FAC = false>
-__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
-  const LinearFwdArgs& a = problems.p[blockIdx.y];
+// RAW = 0: the operands are given (xq, xk, xv [B,H,seq,d], lr, token_eta of LinearFwdArgs).
+// RAW > 0: the kernel forms them from the projections (FusedInputsArgs: head split by addressing, rotary embedding
+// of xq and xk, lr gate, token_eta), i.e. it does the work of ttt_inner_inputs_kernel inside its tile loads:
+//   * a wave loads only the features it owns of the raw xq, xk, xv rows (strided [B,seq,H,d] rows), three
+//     mini-batches ahead, rotates its xq and xk features in the shadow of the state update two mini-batches ahead
+//     of their use, and puts them into LDS; behind the next barrier (the one the recurrence has anyway) every wave
+//     reads the full rotated rows back.  The rotation is therefore done once per unit, not once per wave, and no
+//     barrier is added;
+//   * RAW = 1: the position of a token repeats with the mini-batch (pos_wrap divides K: the reference's default),
+//     cosines and sines stay in registers; RAW = 2: positions run over the sequence (pos_wrap = 0), cosines and sines
+//     are loaded with the rows;
+//   * the operands as used (rotated xq, xk; xv; lr) are written out in [B,H,seq,d] order when the caller asks for them
+//     (ttt_linear_bwd needs them): the wave that owns a feature stores it.
+template <class T, int D, int NW, int PF, bool FULL, bool FAC, int RAW>
+__device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const FusedInputsArgs* fip) {
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;
@@ -44,10 +56,14 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
   const UnitBase<T, D> ub(a, bh);
 
   // same scale folding as the unskewed kernel: G'' = -sc lr G, M'' = (token_eta[t]/sc)(1 + A)
-  const float te_last = a.token_eta[K - 1];
+  auto tok_eta = [&](int i) {
+    if constexpr (RAW != 0) return fmaxf(fip->token_idx[i] + fip->learnable_token_idx[i], 0.f);
+    else return a.token_eta[i];
+  };
+  const float te_last = tok_eta(K - 1);
   const bool upd = te_last != 0.f;
   const float sc = upd ? te_last : 1.f;
-  const float rho_c = (c < K) ? a.token_eta[c] / sc : 0.f;
+  const float rho_c = (c < K) ? tok_eta(c) / sc : 0.f;
   const frag ident = identity_frag<T>(c, g);
   const frag nident = identity_frag<T>(c, g, -1.f);
   const frag ones = splat_frag<T>(1.f);
@@ -163,8 +179,159 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
 
   constexpr int R = PF + 1;
   StageInMw<T, NT, TPW> buf[R];
+  // ---- RAW: the raw rows of the own features, three mini-batches ahead (ring index = mini-batch % R, as for buf)
+  struct RawIn {
+    frag q[TPW], k[TPW], v[TPW];
+    float z;                    // lr logit of the lane's token
+    f32x2 cs[TPW], sn[TPW];     // RAW = 2 only
+  };
+  RawIn raw[RAW != 0 ? R : 1];
+  f32x2 cs_fix[TPW], sn_fix[TPW];  // RAW = 1: cosines and sines of the lane's token position and own feature pairs
+  u32x4* xrot = nullptr;           // rotated rows in LDS: [2 buffers][xq, xk][feature pair][lane]
+  float lr_bias_h = 0.f;
+  if constexpr (RAW != 0) {
+    static_assert(BF && NT <= 4 && PF == 2, "the forward that forms its own operands: bf16 I/O, head_dim <= 64");
+    __shared__ u32x4 xrot_s[2][2][NT / 2][64];
+    xrot = &xrot_s[0][0][0][0];
+    lr_bias_h = fip->lr_bias[h];
 #pragma unroll
-  for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], ub, K, n_stages_, u, c, g, w);
+    for (int jj = 0; jj < TPW; ++jj) {
+      cs_fix[jj] = f32x2{1.f, 1.f};
+      sn_fix[jj] = f32x2{0.f, 0.f};
+    }
+    if (RAW == 1 && fip->cos != nullptr) {
+      const int pos = (fip->pos_offset + c) % fip->pos_wrap;
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const size_t o = (size_t)pos * (D / 2) + own_offset<TPW>(w, jj, g) / 2;
+        cs_fix[jj] = *reinterpret_cast<const f32x2*>(fip->cos + o);
+        sn_fix[jj] = *reinterpret_cast<const f32x2*>(fip->sin + o);
+      }
+    }
+    if (fip->token_eta_out != nullptr && bh == 0)
+      for (int i = threadIdx.x; i < a.seq; i += 64 * NW) fip->token_eta_out[i] = tok_eta(i % K);
+  }
+  // raw rows of unit (b, h): token t of the unit is row (b * seq + t) * H + h of the [B,seq,H,d] tensors
+  const size_t bidx = bh / a.H;
+  const unsigned raw_row = (unsigned)a.H * (unsigned)(D * sizeof(elem));  // bytes from one token to the next
+  auto load_raw = [&](RawIn& r, int stage) {
+    if constexpr (RAW != 0) {
+      if (FULL) stage = min(stage, n_stages_ - 1);
+      const bool ok = FULL || ((c < K) && (stage < n_stages_));
+      const unsigned t = (unsigned)stage * (unsigned)K + (unsigned)c;
+      const size_t row0 = (bidx * (size_t)a.seq * a.H + h) * (D * sizeof(elem));
+      const unsigned char* bq = static_cast<const unsigned char*>(fip->xq) + row0;
+      const unsigned char* bk = static_cast<const unsigned char*>(fip->xk) + row0;
+      const unsigned char* bv = static_cast<const unsigned char*>(fip->xv) + row0;
+      const unsigned off = t * raw_row;
+      if (TPW == 1) {
+        const unsigned o1 = off + own_offset<TPW>(w, 0, g) * (unsigned)sizeof(elem);
+        r.q[0] = ok ? load4<T>(reinterpret_cast<const elem*>(bq + o1)) : IO::zero();
+        r.k[0] = ok ? load4<T>(reinterpret_cast<const elem*>(bk + o1)) : IO::zero();
+        r.v[0] = ok ? load4<T>(reinterpret_cast<const elem*>(bv + o1)) : IO::zero();
+      } else {
+#pragma unroll
+        for (int qq = 0; qq < TPW / 2; ++qq) {
+          const unsigned o2 = off + own_offset<TPW>(w, 2 * qq, g) * (unsigned)sizeof(elem);
+          IO::load8(reinterpret_cast<const elem*>(bq + o2), ok, r.q[2 * qq], r.q[2 * qq + 1]);
+          IO::load8(reinterpret_cast<const elem*>(bk + o2), ok, r.k[2 * qq], r.k[2 * qq + 1]);
+          IO::load8(reinterpret_cast<const elem*>(bv + o2), ok, r.v[2 * qq], r.v[2 * qq + 1]);
+        }
+      }
+      const elem* zl = static_cast<const elem*>(fip->lr_logits) + (bidx * (size_t)a.seq * a.H + h);
+      r.z = ok ? IO::load1(zl + (size_t)t * a.H) : 0.f;
+      if constexpr (RAW == 2) {
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          const size_t o = (size_t)(fip->pos_offset + (int)t) * (D / 2) + own_offset<TPW>(w, jj, g) / 2;
+          r.cs[jj] = fip->cos != nullptr ? *reinterpret_cast<const f32x2*>(fip->cos + o) : f32x2{1.f, 1.f};
+          r.sn[jj] = fip->sin != nullptr ? *reinterpret_cast<const f32x2*>(fip->sin + o) : f32x2{0.f, 0.f};
+        }
+      }
+    }
+  };
+  // own features of a mini-batch: rotate, keep (own-feature operands of dst), share through LDS buffer `pb`, store
+  auto rotate_share = [&](const RawIn& r, StageInMw<T, NT, TPW>& dst, int stage, int pb) {
+    if constexpr (RAW != 0) {
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const f32x2 cs = RAW == 2 ? r.cs[jj] : cs_fix[jj], sn = RAW == 2 ? r.sn[jj] : sn_fix[jj];
+        dst.qo[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.q[jj]), cs, sn));
+        dst.ko[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.k[jj]), cs, sn));
+        dst.vo[jj] = r.v[jj];
+      }
+      // the gate in the precision the operand has when it is a tensor of its own
+      // (a token past the end of a short mini-batch has no learning rate: it must not reach the state update)
+      const bool tok = FULL || c < K;
+      dst.lr = tok ? IO::rounded(lr_gate(r.z + lr_bias_h, fip->lr_scale)) : 0.f;
+      u32x4* xb = xrot + (size_t)pb * 2 * (NT / 2) * 64;
+      if (TPW == 1) {
+        const int J = w;
+        unsigned char* pq_ = reinterpret_cast<unsigned char*>(xb + (0 * (NT / 2) + (J >> 1)) * 64 + lane) + 8 * (J & 1);
+        unsigned char* pk_ = reinterpret_cast<unsigned char*>(xb + (1 * (NT / 2) + (J >> 1)) * 64 + lane) + 8 * (J & 1);
+        *reinterpret_cast<u32x2*>(pq_) = __builtin_bit_cast(u32x2, dst.qo[0]);
+        *reinterpret_cast<u32x2*>(pk_) = __builtin_bit_cast(u32x2, dst.ko[0]);
+      } else {
+#pragma unroll
+        for (int qq = 0; qq < TPW / 2; ++qq) {
+          const int q = w * (TPW / 2) + qq;
+          const u32x2 a0 = __builtin_bit_cast(u32x2, dst.qo[2 * qq]), a1 = __builtin_bit_cast(u32x2, dst.qo[2 * qq + 1]);
+          const u32x2 b0 = __builtin_bit_cast(u32x2, dst.ko[2 * qq]), b1 = __builtin_bit_cast(u32x2, dst.ko[2 * qq + 1]);
+          xb[(0 * (NT / 2) + q) * 64 + lane] = u32x4{a0[0], a0[1], a1[0], a1[1]};
+          xb[(1 * (NT / 2) + q) * 64 + lane] = u32x4{b0[0], b0[1], b1[0], b1[1]};
+        }
+      }
+      if (stage < n_stages_ && tok) {
+        const unsigned off = UnitBase<T, D>::row_off(stage, K, c);
+        const size_t u0 = bh * (size_t)a.seq * (D * sizeof(elem));
+        auto put = [&](void* base, const frag (&x)[TPW]) {
+          if (base == nullptr) return;
+          unsigned char* pb_ = static_cast<unsigned char*>(base) + u0 + off;
+          if (TPW == 1) {
+            *reinterpret_cast<u32x2*>(pb_ + own_offset<TPW>(w, 0, g) * sizeof(elem)) = __builtin_bit_cast(u32x2, x[0]);
+          } else {
+#pragma unroll
+            for (int qq = 0; qq < TPW / 2; ++qq) {
+              const u32x2 a0 = __builtin_bit_cast(u32x2, x[2 * qq]), a1 = __builtin_bit_cast(u32x2, x[2 * qq + 1]);
+              *reinterpret_cast<u32x4*>(pb_ + own_offset<TPW>(w, 2 * qq, g) * sizeof(elem)) = u32x4{a0[0], a0[1], a1[0], a1[1]};
+            }
+          }
+        };
+        put(fip->xq_out, dst.qo);
+        put(fip->xk_out, dst.ko);
+        put(fip->xv_out, dst.vo);
+        if (fip->lr_out != nullptr && w == 0 && g == 0)
+          IO::store1(static_cast<elem*>(fip->lr_out) + bh * (size_t)a.seq + (size_t)stage * K + c, dst.lr);
+      }
+    }
+  };
+  // the full rotated rows of a mini-batch, from LDS buffer `pb` (behind a barrier that follows rotate_share)
+  auto gather_rows = [&](StageInMw<T, NT, TPW>& dst, int pb) {
+    if constexpr (RAW != 0) {
+      const u32x4* xb = xrot + (size_t)pb * 2 * (NT / 2) * 64;
+#pragma unroll
+      for (int q = 0; q < NT / 2; ++q) {
+        const u32x4 vq = xb[(0 * (NT / 2) + q) * 64 + lane], vk = xb[(1 * (NT / 2) + q) * 64 + lane];
+        dst.q[2 * q] = __builtin_bit_cast(frag, u32x2{vq[0], vq[1]});
+        dst.q[2 * q + 1] = __builtin_bit_cast(frag, u32x2{vq[2], vq[3]});
+        dst.k[2 * q] = __builtin_bit_cast(frag, u32x2{vk[0], vk[1]});
+        dst.k[2 * q + 1] = __builtin_bit_cast(frag, u32x2{vk[2], vk[3]});
+      }
+    }
+  };
+  if constexpr (RAW != 0) {
+    // mini-batch 0 complete, mini-batch 1 rotated and on its way through LDS (read behind the first barrier of the
+    // loop), the raw rows of mini-batch 2 in flight
+#pragma unroll
+    for (int u = 0; u < R; ++u) load_raw(raw[u], u);
+    rotate_share(raw[0], buf[0], 0, 0);
+    lds_barrier();
+    gather_rows(buf[0], 0);
+    rotate_share(raw[1], buf[1], 1, 1);
+  } else {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) load_stage_mw<T, D, NW, FULL>(buf[u], ub, K, n_stages_, u, c, g, w);
+  }
 
   // One pass over R mini-batches (the ring of prefetch registers is indexed at compile time).  CHECKED:
   // the first and the last pass, which test for "no pending output yet" and "past the end"; the passes in
@@ -181,7 +348,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int st = st0 + u;
-      load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], ub, K, n_stages_, st + PF, c, g, w);
+      if constexpr (RAW != 0)
+        load_raw(raw[u], st + R);  // its previous content, mini-batch st, was rotated two mini-batches ago
+      else
+        load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], ub, K, n_stages_, st + PF, c, g, w);
       if (CHECKED && st >= a.n_stages) continue;
       const StageInMw<T, NT, TPW>& cur = buf[u];
 
@@ -262,6 +432,8 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
       // for it, and here it runs while this exchange is in flight (LDS write, barrier, LDS read)
       if (!CHECKED || st > 1) emit_output(so0, so1, st - 2, zbo, qoo);
       exchange8_collect(S, st & 1);
+      // RAW: the rows of the next mini-batch, rotated by their owners before this barrier
+      if constexpr (RAW != 0) gather_rows(buf[(u + 1) % R], (st + 1) & 1);
       so0 = S[6];
       so1 = S[7];
 #pragma unroll
@@ -323,6 +495,10 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
         qop[jj] = cur.qo[jj];
       }
       pend_sums(zbp, ps0, ps1);
+      // RAW: the own features of the mini-batch after the next, loaded during the previous pass of the loop; read
+      // back by every wave behind the next barrier.  LDS buffer st & 1 was last read behind the barrier of the
+      // previous mini-batch, which every wave has left.
+      if constexpr (RAW != 0) rotate_share(raw[(u + 2) % R], buf[(u + 2) % R], st + 2, st & 1);
     }
   };
   if constexpr (NT <= 4) {
@@ -476,6 +652,18 @@ __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<Lin
   store_state_final<D, TPW>(a.W_out + bh * D * D, a.b_out + bh * D, a.W0 + sb * D * D, a.b0 + sb * D, Wc, bT, m0s, w, c, g);
   if constexpr (FAC)
     store_state_tiles<D, TPW>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D), a.b_ckpt + bh * (size_t)a.n_ckpt * D, Wc, bT, w, lane);
+}
+
+template <class T, int D, int NW, int PF, bool FULL, bool FAC = false>
+__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
+  linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, 0>(problems.p[blockIdx.y], nullptr);
+}
+
+// The same forward on the projections as they leave the GEMMs: see RAW above.
+template <class T, int D, int NW, int PF, bool FULL, bool FAC, int RAW>
+__global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_fi_kernel(LinearFwdArgs a, FusedInputsArgs fi) {
+  static_assert(RAW == 1 || RAW == 2, "RAW selects how positions are looked up");
+  linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, RAW>(a, &fi);
 }
 
 }  // namespace ttt

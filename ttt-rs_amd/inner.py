@@ -669,6 +669,70 @@ def inner_loop_inputs_raw(xq, xk, xv, lr_logits, lr_bias, base_lr: float, token_
     return TTTInputsInner(Qkv(q, k, v), te, lr)
 
 
+def ttt_linear_forward_fused_inputs_raw(xq, xk, xv, lr_logits, lr_bias, base_lr: float, token_idx,
+                                        learnable_token_idx, weight, bias, ln_weight, ln_bias, mini_batch: int,
+                                        rope=None, pos_offset: int = 0, pos_wrap: int = 0, eps: float = 1e-6,
+                                        checkpoint_interval: int = 1, want_checkpoints: bool = False,
+                                        packed_checkpoints: int = 0, save_inputs: bool = False):
+    """One call of ttt_linear_fwd_fused_inputs: inner_loop_inputs_raw and ttt_linear_forward_raw in one kernel
+    (rust/layer/src/ttt.rs:147-268 followed by rust/kernels/src/kernel.rs:62-69).  xq,xk,xv [B,seq,H,d];
+    lr_logits [B,seq,H]; rope = (cos, sin) tables [npos, d/2] f32 or None; weight/bias/ln_* as for
+    ttt_linear_forward_raw.  Returns (output, weight_out, bias_out[, weight_ckpt, bias_ckpt][, TTTInputsInner]):
+    the last item, with save_inputs, holds the operands as the kernel used them (what the backward needs)."""
+    B, seq, H, d = xq.shape
+    io = xq.dtype
+    xq = _need(xq, (B, seq, H, d), io, "xq")
+    xk = _need(xk, (B, seq, H, d), io, "xk")
+    xv = _need(xv, (B, seq, H, d), io, "xv")
+    lg = _need(lr_logits, (B, seq, H), io, "lr_logits")
+    lb = _need(lr_bias.reshape(-1), (H,), torch.float32, "lr_bias")
+    ti = _need(token_idx, (mini_batch,), torch.float32, "token_idx")
+    lti = _need(learnable_token_idx, (mini_batch,), torch.float32, "learnable_token_idx")
+    per_batch = weight.dim() == 4
+    W0 = _need(weight, (B, H, d, d) if per_batch else (H, d, d), torch.float32, "weight")
+    b0 = _need(bias, (B, H, d) if per_batch else (H, d), torch.float32, "bias")
+    gam = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+    bet = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+    null = C.c_void_p(None)
+    cos = sin = None
+    if rope is not None:
+        cos = _need(rope[0], (rope[0].shape[0], d // 2), torch.float32, "rope cos")
+        sin = _need(rope[1], (rope[0].shape[0], d // 2), torch.float32, "rope sin")
+        last = (pos_offset + seq - 1) if pos_wrap == 0 else min(pos_wrap - 1, pos_offset + seq - 1)
+        if last >= cos.shape[0]:
+            raise _lib.TttError(_lib.TTT_ERR_SHAPE, "rope table shorter than the positions used")
+    dev = xq.device
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, checkpoint_interval, _io_dtype(xq), 1 if per_batch else 0, 0,
+                   int(packed_checkpoints), 0)
+    check(lib().ttt_linear_fwd_fused_inputs_supported(C.byref(desc), pos_wrap, 0 if rope is None else 1))
+    out = torch.empty((B, H, seq, d), dtype=io, device=dev)
+    W_out = torch.empty((B, H, d, d), dtype=torch.float32, device=dev)
+    b_out = torch.empty((B, H, d), dtype=torch.float32, device=dev)
+    Wc = bc = None
+    if want_checkpoints:
+        n = int(lib().ttt_linear_num_checkpoints(C.byref(desc)))
+        Wc = torch.empty((B, H, n, d, d), dtype=torch.float32, device=dev)
+        bc = torch.empty((B, H, n, d), dtype=torch.float32, device=dev)
+    q = k = v = lr = te = None
+    if save_inputs:
+        q, k, v = (torch.empty((B, H, seq, d), dtype=io, device=dev) for _ in range(3))
+        lr = torch.empty((B, H, seq), dtype=io, device=dev)
+        te = torch.empty(seq, dtype=torch.float32, device=dev)
+    opt = lambda t: null if t is None else _ptr(t)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_linear_fwd_fused_inputs(
+            C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(lg), _ptr(lb), C.c_float(base_lr), _ptr(ti), _ptr(lti),
+            opt(cos), opt(sin), pos_offset, pos_wrap, _ptr(W0), _ptr(b0), _ptr(gam), _ptr(bet), _ptr(out), _ptr(W_out),
+            _ptr(b_out), opt(Wc), opt(bc), opt(q), opt(k), opt(v), opt(lr), opt(te), stream))
+    res = [out, W_out, b_out]
+    if want_checkpoints:
+        res += [Wc, bc]
+    if save_inputs:
+        res.append(TTTInputsInner(Qkv(q, k, v), te, lr))
+    return tuple(res)
+
+
 def layer_epilogue_raw(inner_out, post_norm_weight, post_norm_bias, gate=None, eps: float = 1e-6):
     """One call of ttt_layer_epilogue: head merge + post_norm LayerNorm (+ tanh-GELU gate) of
     TTT::forward (rust/layer/src/ttt.rs:285-297).  inner_out [B,H,seq,d] -> [B,seq,H*d]."""
