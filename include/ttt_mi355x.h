@@ -97,6 +97,12 @@ typedef struct ttt_desc {
  * (see ttt_mlp_fwd), when the units number at most half the device's CUs.  Not the default: measured on MI355X the
  * pair gains 2 - 3 % at 128 units.  Ignored where only one of the two kernels exists. */
 #define TTT_HINT_TWO_CU 0x400
+/* ttt_linear_fwd, bf16 I/O at head_dim 64 with two waves per unit: TTT_HINT_OWN_LOADS = every wave loads only the
+ * features it owns of xq, xk, xv and the full rows reach the waves through LDS (half the vector loads; the library's
+ * choice above 256 units, where two workgroups share a CU); TTT_HINT_ALL_LOADS = every wave loads every row (the
+ * library's choice up to 256 units).  Same results bit for bit.  Ignored where only one of the two exists. */
+#define TTT_HINT_OWN_LOADS 0x1000
+#define TTT_HINT_ALL_LOADS 0x2000
 /* Testing only: the two workgroups that share a (batch, head) unit in ttt_mlp_fwd at head_dim 128 (bf16 I/O) give
  * up waiting for each other at once, as if the partner had never become resident.  Exercises the failure path
  * described at ttt_mlp_fwd: every output of the affected units is NaN.  All kernels still run to their end. */
@@ -379,12 +385,13 @@ int ttt_linear_fwd_fused_inputs(const ttt_desc* desc, const void* xq, const void
 
 /*
  * Self-test of a hardware fact the bf16 kernels rely on; no counterpart in the reference.  One wavefront computes
- * D = A1*B1 with one bf16 matrix instruction and accumulates A2*B2 onto it, in place, with an instruction of the
- * other shape (order 0: 16x16x32 then 16x16x16; order 1: the reverse), `gap` wait states apart (0, 4 or 5), on
- * fixed small-integer operands: A_p[i][k] = (7 i + 3 k + 5 p) mod 7 - 3 and B_p[k][j] = (5 j + 11 k + 3 p) mod 7 - 3
- * for product p (0 first, 1 second; k < 32 or 16 by shape).  out: 256 floats, D row-major [16][16].  With five wait
- * states the result is exact; closer pairs are what the library's build refuses in compiler-generated code
- * (MI355X returns wrong sums for them).  Enqueues one tiny kernel on `stream`.
+ * D = A1*B1 with one bf16 matrix instruction and D2 = A2*B2 + D with an instruction of the other shape (order 0:
+ * 16x16x32 then 16x16x16 with D2 written over D; order 1: the reverse; orders 2, 3: the same two with D2 in other
+ * registers), `gap` wait states apart (0, 4 or 5), on fixed small-integer operands:
+ * A_p[i][k] = (7 i + 3 k + 5 p) mod 7 - 3 and B_p[k][j] = (5 j + 11 k + 3 p) mod 7 - 3 for product p (0 first, 1 second;
+ * k < 32 or 16 by shape).  out: 256 floats, D2 row-major [16][16].  With five wait states the result is exact; closer
+ * pairs are what the library's build refuses in compiler-generated code (MI355X returns wrong sums for them).
+ * Enqueues one tiny kernel on `stream`.
  */
 int ttt_selftest_mfma_mixed(int order, int gap, float* out, void* stream);
 

@@ -1,7 +1,7 @@
 """The build's assembly scan (ttt-rs_amd/isa_check.py) and the hardware fact behind it.
 
-CPU: the scanner flags an in-place accumulation onto a matrix instruction of another shape that follows too closely,
-and nothing else.  GPU: the library's self-test entry point runs such pairs at chosen distances; at the distance
+CPU: the scanner flags a matrix instruction that takes its accumulator from one of another shape too closely behind
+it (in place or into other registers, in text order or across a branch), and nothing else.  GPU: the library's self-test entry point runs such pairs at chosen distances; at the distance
 the scanner demands the result is exact, and what the hardware does with closer pairs is printed for the record
 (MI355X returns wrong sums; nothing is asserted about them, a later part may forward them correctly)."""
 import ctypes as C
@@ -47,18 +47,38 @@ def test_scanner_accepts_what_the_hardware_forwards():
     # the same shape back to back, in place
     assert flagged([K32.format(c="0"), K32.format(c="v[0:3]")]) == []
     assert flagged([K16.format(d="v[0:3]", c="0"), K16.format(d="v[0:3]", c="v[0:3]")]) == []
-    # another shape, but the result goes to other registers than it accumulates from (interlocked by the hardware)
-    assert flagged([K32.format(c="0"), K16.format(d="v[12:15]", c="v[0:3]")]) == []
+    # another shape reading the first's result as an A or B operand (interlocked by the hardware)
+    assert flagged([K32.format(c="0"), "\tv_mfma_f32_16x16x16_bf16 v[12:15], v[0:1], v[2:3], 0"]) == []
     # another shape accumulating onto registers the first did not write
     assert flagged([K32.format(c="0"), K16.format(d="v[12:15]", c="v[12:15]")]) == []
     # the self-test kernel places such pairs on purpose
     assert list(isa_check.scan(["ttt_selftest_kernel:", K32.format(c="0"), K16.format(d="v[0:3]", c="v[0:3]")])) == []
 
 
+def test_scanner_flags_a_mixed_pair_that_writes_elsewhere():
+    """The accumulator input is what matters, not where the result goes: found in a forward kernel whose bias update
+    (k = 16) the compiler had placed right in front of the next mini-batch's k = 32 product that starts from the bias."""
+    assert len(flagged([K32.format(c="0"), K16.format(d="v[12:15]", c="v[0:3]")])) == 1
+    assert len(flagged([K16.format(d="v[52:55]", c="v[52:55]"),
+                        "\tv_mfma_f32_16x16x32_bf16 v[100:103], v[132:135], a[4:7], v[52:55]"])) == 1
+    # partial overlap of the register ranges counts
+    assert len(flagged([K32.format(c="0"), K16.format(d="v[12:15]", c="v[2:5]")])) == 1
+    assert flagged([K32.format(c="0"), "\ts_nop 4", K16.format(d="v[12:15]", c="v[0:3]")]) == []
+
+
+def test_scanner_follows_branches():
+    loop = [".LBB0_1:", K32.format(c="v[12:15]"), "\tv_add_f32_e32 v40, v41, v42",
+            K16.format(d="v[12:15]", c="v[12:15]"), "\ts_cbranch_scc1 .LBB0_1", "\ts_endpgm"]
+    assert len(flagged(loop)) == 1          # the pair meets only across the back edge
+    assert flagged([loop[0], "\ts_nop 4"] + loop[1:]) == []
+    fwd = [K32.format(c="0"), "\ts_branch .LBB0_2", "\ts_nop 7", ".LBB0_2:", K16.format(d="v[0:3]", c="v[0:3]")]
+    assert len(flagged(fwd)) == 1           # the s_nop is jumped over
+
+
 def expected(order):
     a = lambda p, i, k: float((i * 7 + k * 3 + p * 5) % 7 - 3)
     b = lambda p, k, j: float((j * 5 + k * 11 + p * 3) % 7 - 3)
-    ks = (32, 16) if order == 0 else (16, 32)
+    ks = (32, 16) if order % 2 == 0 else (16, 32)
     D = np.zeros((16, 16))
     for p, kk in enumerate(ks):
         A = np.array([[a(p, i, k) for k in range(kk)] for i in range(16)])
@@ -73,7 +93,7 @@ def test_mixed_shapes_five_wait_states_apart_are_exact():
     P = importlib.import_module("ttt-rs_amd")
     out = torch.empty(256, device="cuda:0")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    for order in (0, 1):
+    for order in (0, 1, 2, 3):  # 0, 1: the second instruction writes over its accumulator; 2, 3: into other registers
         want = expected(order)
         for gap in (5, 4, 0):
             print(f"case mfma mixed shapes order {order} gap {gap}", flush=True)
@@ -85,4 +105,4 @@ def test_mixed_shapes_five_wait_states_apart_are_exact():
             print(f"  order {order}, {gap} wait states: {'exact' if exact else 'WRONG (max abs error %.3g)' % np.nanmax(np.abs(got - want))}", flush=True)
             if gap == 5:
                 assert exact, f"order {order}: five wait states between the two shapes no longer suffice"
-    assert P.lib().ttt_selftest_mfma_mixed(2, 5, C.c_void_p(out.data_ptr()), stream) == P.TTT_ERR_SHAPE
+    assert P.lib().ttt_selftest_mfma_mixed(4, 5, C.c_void_p(out.data_ptr()), stream) == P.TTT_ERR_SHAPE

@@ -143,3 +143,38 @@ def test_mlp_bwd_repeat_calls(P, d, K, dtype):
             assert torch.equal(r[k], runs[0][k]), (k, dtype)
         for k in ("d_token_eta", "d_gamma", "d_beta"):
             assert_close(r[k], runs[0][k].double().cpu().numpy(), 1e-5, k)
+
+
+@pytest.mark.parametrize("fmt", [None, 0, 1, 2], ids=["no-ckpt", "f32-ckpt", "packed", "factors"])
+@pytest.mark.parametrize("B,H,K,N", [(2, 3, 16, 5), (1, 2, 7, 4), (1, 1, 16, 1), (2, 2, 16, 2), (3, 2, 5, 7)])
+def test_linear_fwd_own_loads_variant_gives_the_same_bits(P, B, H, K, N, fmt):
+    """bf16, head_dim 64, two waves per unit: the variant in which a wave loads only the features it owns and the
+    full rows cross LDS (the library's choice above 256 units; TTT_HINT_OWN_LOADS asks for it at any size) against
+    the variant in which every wave loads every row (TTT_HINT_ALL_LOADS): the same arithmetic on the same values."""
+    if fmt == 2 and N < 2:
+        pytest.skip("one mini-batch is saved packed")
+    d = 64
+    print(f"case fwd own loads B{B} H{H} K{K} N{N} fmt{fmt}", flush=True)
+    c = P.synthetic.reference_test_inputs(1200 + K + N, B, H, N * K, d, K, io_dtype=torch.bfloat16)
+    dv = to_dev(c)
+    runs = []
+    for hint in (P.TTT_HINT_ALL_LOADS, P.TTT_HINT_OWN_LOADS, P.TTT_HINT_OWN_LOADS):
+        r = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                                     dv["gamma"], dv["beta"], K, 1e-6, 1, want_checkpoints=fmt is not None,
+                                     packed_checkpoints=fmt or 0, kernel_hint=hint)
+        torch.cuda.synchronize()
+        runs.append(tuple(r) if fmt in (None, 0) else tuple(r[:3]))
+    same_bits(runs, f"forward own/all loads K{K} N{N} fmt{fmt}")
+    if fmt in (1, 2):  # what the backward makes of the saved state must agree as well
+        dO = torch.randn(B, H, N * K, d, generator=torch.Generator().manual_seed(31)).to(torch.bfloat16).to("cuda:0")
+        gs = []
+        for hint in (P.TTT_HINT_ALL_LOADS, P.TTT_HINT_OWN_LOADS):
+            fw = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                                          dv["gamma"], dv["beta"], K, 1e-6, 1, want_checkpoints=True,
+                                          packed_checkpoints=fmt, kernel_hint=hint)
+            gs.append(P.ttt_linear_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"],
+                                                dv["lr"], dv["gamma"], dv["beta"], fw[3], fw[4], dO, K, 1e-6, 1,
+                                                packed_checkpoints=fmt))
+        torch.cuda.synchronize()
+        for k in PLAIN_LINEAR:
+            assert torch.equal(gs[0][k], gs[1][k]), k

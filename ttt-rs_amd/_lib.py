@@ -13,6 +13,8 @@ TTT_F32, TTT_BF16 = 0, 1
 TTT_HINT_AUTO, TTT_HINT_LDS_TILES = 0, 0x100  # kernel_hint: low byte = waves per unit (1, 2, 4)
 TTT_HINT_TEST_LOST_PARTNER = 0x200
 TTT_HINT_TWO_CU = 0x400
+TTT_HINT_OWN_LOADS = 0x1000
+TTT_HINT_ALL_LOADS = 0x2000
 TTT_HINT_TEST_OTHER_XCD = 0x800
 
 EXPORTS = (

@@ -99,7 +99,7 @@ ttt::Problems<A> pack_of(const A* probs, unsigned n) {
 // (skewed workgroup kernel).  Many units: one wave per unit (no exchange at all).
 // desc.kernel_hint (low byte) = 1 | 2 | 4 overrides the number of waves per unit (tuning / tests).
 template <class T, int D, int NW>
-int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s) {
+int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s, bool own_loads = false) {
   const ttt::LinearFwdArgs& a = probs[0];
   const auto P = pack_of(probs, ny);
   // mini-batches prefetched ahead, in registers (f32 fragments are twice as large: the one-wave f32 kernel, which
@@ -125,6 +125,24 @@ int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream
       hipLaunchKernelGGL((ttt::ttt_linear_fwd_mw_kernel<T, D, 1, PF, false>), grid, block, 0, s, P);
   } else {
     constexpr int NWS = NW > 1 ? NW : 2;  // the skewed kernel needs at least two waves
+    // bf16, head_dim 64, two waves per unit: the variant in which a wave loads only the features it owns and the
+    // full rows cross LDS (same bits).  Measured on MI355X (seq 2048): 24 units 117 us against 114 us, 252 units
+    // 120 against 120, 384 units 129 - 139 against 137 - 146: it pays once two workgroups share a CU's load path.
+    if constexpr (can_fac && NWS == 2 && D == 64) {
+      if (own_loads) {
+        if (fac) {
+          if (a.K == 16)
+            hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true, true, true>), grid, block, 0, s, P);
+          else
+            hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, false, true, true>), grid, block, 0, s, P);
+        } else if (a.K == 16) {
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true, false, true>), grid, block, 0, s, P);
+        } else {
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, false, false, true>), grid, block, 0, s, P);
+        }
+        return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+      }
+    }
     if constexpr (can_fac) {
       if (fac) {
         if (a.K == 16)
@@ -143,7 +161,8 @@ int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream
 }
 
 template <class T, int D>
-int launch_linear_fwd(const ttt::LinearFwdArgs* probs, int waves_hint, unsigned ny, hipStream_t s) {
+int launch_linear_fwd(const ttt::LinearFwdArgs* probs, int hint, unsigned ny, hipStream_t s) {
+  const int waves_hint = hint & TTT_HINT_WAVES_MASK;
   const ttt::LinearFwdArgs& a = probs[0];
   constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
   // bf16 I/O: one or two waves per unit.  A four-wave bf16 variant (one feature tile per wave) is not offered: it
@@ -164,7 +183,9 @@ int launch_linear_fwd(const ttt::LinearFwdArgs* probs, int waves_hint, unsigned 
   if constexpr (max_nw >= 4) {
     if (nw >= 4) return launch_linear_fwd_nw<T, D, 4>(probs, ny, s);
   }
-  if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(probs, ny, s);
+  // a launch that puts two workgroups on a CU, or a caller that asks for it
+  const bool own_loads = units > 256 ? (hint & TTT_HINT_ALL_LOADS) == 0 : (hint & TTT_HINT_OWN_LOADS) != 0;
+  if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(probs, ny, s, own_loads);
   return launch_linear_fwd_nw<T, D, 1>(probs, ny, s);
 }
 
@@ -621,12 +642,11 @@ int prepare_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const 
 }
 
 int dispatch_linear_fwd_pack(const ttt_desc* d, const ttt::LinearFwdArgs* a, unsigned ny, hipStream_t s) {
-  const int waves_hint = d->kernel_hint & TTT_HINT_WAVES_MASK;
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
   const bool f32 = d->io_dtype == TTT_F32;
   switch (d->head_dim) {
-    case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, waves_hint, ny, s) : launch_linear_fwd<ttt::BF16, 32>(a, waves_hint, ny, s);
-    case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, waves_hint, ny, s) : launch_linear_fwd<ttt::BF16, 64>(a, waves_hint, ny, s);
+    case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, d->kernel_hint, ny, s) : launch_linear_fwd<ttt::BF16, 32>(a, d->kernel_hint, ny, s);
+    case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, d->kernel_hint, ny, s) : launch_linear_fwd<ttt::BF16, 64>(a, d->kernel_hint, ny, s);
     default: break;
   }
   if (want_lds) {
@@ -1262,8 +1282,8 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
 
 int ttt_selftest_mfma_mixed(int order, int gap, float* out, void* stream) {
   if (!out) return fail(TTT_ERR_NULL, "ttt_selftest_mfma_mixed: out is NULL");
-  if ((order != 0 && order != 1) || (gap != 0 && gap != 4 && gap != 5))
-    return fail(TTT_ERR_SHAPE, "ttt_selftest_mfma_mixed: order must be 0 or 1 and gap 0, 4 or 5 (got %d, %d)", order, gap);
+  if (order < 0 || order > 3 || (gap != 0 && gap != 4 && gap != 5))
+    return fail(TTT_ERR_SHAPE, "ttt_selftest_mfma_mixed: order must be 0 .. 3 and gap 0, 4 or 5 (got %d, %d)", order, gap);
   hipLaunchKernelGGL(ttt::ttt_selftest_mfma_mixed_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), order, gap, out);
   return hip_status(hipGetLastError(), "ttt_selftest_mfma_mixed launch");
 }

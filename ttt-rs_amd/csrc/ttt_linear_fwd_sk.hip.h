@@ -30,6 +30,8 @@ namespace ttt {
 //     are loaded with the rows;
 //   * the operands as used (rotated xq, xk; xv; lr) are written out in [B,H,seq,d] order when the caller asks for them
 //     (ttt_linear_bwd needs them): the wave that owns a feature stores it.
+// RAW = 3: the operands are given, and fetched the same way: every wave loads only the features it owns and the
+// full xq, xk rows reach the waves through LDS (half the vector loads of RAW = 0, where every wave loads every row).
 template <class T, int D, int NW, int PF, bool FULL, bool FAC, int RAW>
 __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const FusedInputsArgs* fip) {
   using IO = Io<T>;
@@ -56,8 +58,9 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   const UnitBase<T, D> ub(a, bh);
 
   // same scale folding as the unskewed kernel: G'' = -sc lr G, M'' = (token_eta[t]/sc)(1 + A)
+  constexpr bool FORM = RAW == 1 || RAW == 2;  // the operands are formed here from the projections
   auto tok_eta = [&](int i) {
-    if constexpr (RAW != 0) return fmaxf(fip->token_idx[i] + fip->learnable_token_idx[i], 0.f);
+    if constexpr (FORM) return fmaxf(fip->token_idx[i] + fip->learnable_token_idx[i], 0.f);
     else return a.token_eta[i];
   };
   const float te_last = tok_eta(K - 1);
@@ -172,6 +175,27 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
     }
   };
 
+  // b += colsum G''.  The bias is the accumulator input of the next mini-batch's Z1 and Zbar products, which are
+  // k = 32 matrix instructions with bf16 I/O, and the scheduler is free to place them right behind this k = 16 update:
+  // a matrix instruction that takes its accumulator from one of ANOTHER shape less than five wait states earlier
+  // reads a stale value (the hardware interlocks only equal shapes; measured, see ttt_selftest.hip.h).  The wait
+  // states are therefore put behind the update by hand, tied to the bias registers so that no reader of the bias can
+  // be scheduled in front of them: nothing measurable at any size.  (Issuing the update as a k = 32 instruction with
+  // a zero half, the other way to make the shapes equal, cost 10 % of the kernel's time at every size.)  In most
+  // instantiations the scheduler leaves the W update's matrix instructions between the pair anyway; the one that had
+  // them adjacent gave outputs 1 % off from the sixth mini-batch on.  The build's assembly scan (isa_check.py) refuses
+  // any code in which such a pair is closer than five wait states.
+  auto bias_update = [&](f32x4 (&b)[TPW], const frag (&gd)[TPW], frag ones_or_zero) {
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj) IO::mma(b[jj], gd[jj], ones_or_zero);
+    if constexpr (BF) {
+      if constexpr (TPW == 1) asm volatile("s_nop 4" : "+v"(b[0]));
+      else if constexpr (TPW == 2) asm volatile("s_nop 4" : "+v"(b[0]), "+v"(b[1]));
+      else
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) asm volatile("s_nop 4" : "+v"(b[jj]));
+    }
+  };
   // token_eta[K-1] == 0 means "no state update": instead of a branch inside the loop the two operands
   // that carry tokens into the update (XK^T, the ones column of the bias update) are made zero
   const frag ident_upd = upd ? ident : IO::zero();
@@ -190,15 +214,17 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   u32x4* xrot = nullptr;           // rotated rows in LDS: [2 buffers][xq, xk][feature pair][lane]
   float lr_bias_h = 0.f;
   if constexpr (RAW != 0) {
-    static_assert(BF && NT <= 4 && PF == 2, "the forward that forms its own operands: bf16 I/O, head_dim <= 64");
+    static_assert(BF && NT <= 4 && PF == 2, "rows shared through LDS: bf16 I/O, head_dim <= 64");
     __shared__ u32x4 xrot_s[2][2][NT / 2][64];
     xrot = &xrot_s[0][0][0][0];
-    lr_bias_h = fip->lr_bias[h];
 #pragma unroll
     for (int jj = 0; jj < TPW; ++jj) {
       cs_fix[jj] = f32x2{1.f, 1.f};
       sn_fix[jj] = f32x2{0.f, 0.f};
     }
+  }
+  if constexpr (FORM) {
+    lr_bias_h = fip->lr_bias[h];
     if (RAW == 1 && fip->cos != nullptr) {
       const int pos = (fip->pos_offset + c) % fip->pos_wrap;
 #pragma unroll
@@ -219,11 +245,20 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
       if (FULL) stage = min(stage, n_stages_ - 1);
       const bool ok = FULL || ((c < K) && (stage < n_stages_));
       const unsigned t = (unsigned)stage * (unsigned)K + (unsigned)c;
-      const size_t row0 = (bidx * (size_t)a.seq * a.H + h) * (D * sizeof(elem));
-      const unsigned char* bq = static_cast<const unsigned char*>(fip->xq) + row0;
-      const unsigned char* bk = static_cast<const unsigned char*>(fip->xk) + row0;
-      const unsigned char* bv = static_cast<const unsigned char*>(fip->xv) + row0;
-      const unsigned off = t * raw_row;
+      const unsigned char *bq, *bk, *bv;
+      unsigned off;
+      if constexpr (FORM) {
+        const size_t row0 = (bidx * (size_t)a.seq * a.H + h) * (D * sizeof(elem));
+        bq = static_cast<const unsigned char*>(fip->xq) + row0;
+        bk = static_cast<const unsigned char*>(fip->xk) + row0;
+        bv = static_cast<const unsigned char*>(fip->xv) + row0;
+        off = t * raw_row;
+      } else {
+        bq = ub.xq;
+        bk = ub.xk;
+        bv = ub.xv;
+        off = UnitBase<T, D>::row_off(stage, K, c);
+      }
       if (TPW == 1) {
         const unsigned o1 = off + own_offset<TPW>(w, 0, g) * (unsigned)sizeof(elem);
         r.q[0] = ok ? load4<T>(reinterpret_cast<const elem*>(bq + o1)) : IO::zero();
@@ -238,8 +273,12 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
           IO::load8(reinterpret_cast<const elem*>(bv + o2), ok, r.v[2 * qq], r.v[2 * qq + 1]);
         }
       }
-      const elem* zl = static_cast<const elem*>(fip->lr_logits) + (bidx * (size_t)a.seq * a.H + h);
-      r.z = ok ? IO::load1(zl + (size_t)t * a.H) : 0.f;
+      if constexpr (FORM) {
+        const elem* zl = static_cast<const elem*>(fip->lr_logits) + (bidx * (size_t)a.seq * a.H + h);
+        r.z = ok ? IO::load1(zl + (size_t)t * a.H) : 0.f;
+      } else {
+        r.z = ok ? IO::load1(reinterpret_cast<const elem*>(ub.lr + t * (unsigned)sizeof(elem))) : 0.f;  // lr itself
+      }
       if constexpr (RAW == 2) {
 #pragma unroll
         for (int jj = 0; jj < TPW; ++jj) {
@@ -253,17 +292,23 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   // own features of a mini-batch: rotate, keep (own-feature operands of dst), share through LDS buffer `pb`, store
   auto rotate_share = [&](const RawIn& r, StageInMw<T, NT, TPW>& dst, int stage, int pb) {
     if constexpr (RAW != 0) {
+      const bool tok = FULL || c < K;
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) {
-        const f32x2 cs = RAW == 2 ? r.cs[jj] : cs_fix[jj], sn = RAW == 2 ? r.sn[jj] : sn_fix[jj];
-        dst.qo[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.q[jj]), cs, sn));
-        dst.ko[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.k[jj]), cs, sn));
+        if constexpr (FORM) {
+          const f32x2 cs = RAW == 2 ? r.cs[jj] : cs_fix[jj], sn = RAW == 2 ? r.sn[jj] : sn_fix[jj];
+          dst.qo[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.q[jj]), cs, sn));
+          dst.ko[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.k[jj]), cs, sn));
+        } else {
+          dst.qo[jj] = r.q[jj];
+          dst.ko[jj] = r.k[jj];
+        }
         dst.vo[jj] = r.v[jj];
       }
       // the gate in the precision the operand has when it is a tensor of its own
       // (a token past the end of a short mini-batch has no learning rate: it must not reach the state update)
-      const bool tok = FULL || c < K;
-      dst.lr = tok ? IO::rounded(lr_gate(r.z + lr_bias_h, fip->lr_scale)) : 0.f;
+      if constexpr (FORM) dst.lr = tok ? IO::rounded(lr_gate(r.z + lr_bias_h, fip->lr_scale)) : 0.f;
+      else dst.lr = r.z;
       u32x4* xb = xrot + (size_t)pb * 2 * (NT / 2) * 64;
       if (TPW == 1) {
         const int J = w;
@@ -281,7 +326,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
           xb[(1 * (NT / 2) + q) * 64 + lane] = u32x4{b0[0], b0[1], b1[0], b1[1]};
         }
       }
-      if (stage < n_stages_ && tok) {
+      if (FORM && stage < n_stages_ && tok) {
         const unsigned off = UnitBase<T, D>::row_off(stage, K, c);
         const size_t u0 = bh * (size_t)a.seq * (D * sizeof(elem));
         auto put = [&](void* base, const frag (&x)[TPW]) {
@@ -485,8 +530,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
       for (int I = 0; I < NT; ++I)
 #pragma unroll
         for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
-#pragma unroll
-      for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones_upd);
+      bias_update(bT, Gd, ones_upd);
       // this mini-batch's Zbar and xq become the pending output; its in-lane sums are formed here, in the
       // shadow of the state update, not between the next Z1 and its exchange
 #pragma unroll
@@ -627,8 +671,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
           for (int I = 0; I < NT; ++I)
 #pragma unroll
             for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
-#pragma unroll
-          for (int jj = 0; jj < TPW; ++jj) IO::mma(bT[jj], Gd[jj], ones);
+          bias_update(bT, Gd, ones);
         }
         // this mini-batch's Zbar and xq become the pending output
 #pragma unroll
@@ -654,9 +697,10 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
     store_state_tiles<D, TPW>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D), a.b_ckpt + bh * (size_t)a.n_ckpt * D, Wc, bT, w, lane);
 }
 
-template <class T, int D, int NW, int PF, bool FULL, bool FAC = false>
+// OWN: every wave loads only the features it owns, full rows through LDS (RAW = 3)
+template <class T, int D, int NW, int PF, bool FULL, bool FAC = false, bool OWN = false>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
-  linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, 0>(problems.p[blockIdx.y], nullptr);
+  linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, OWN ? 3 : 0>(problems.p[blockIdx.y], nullptr);
 }
 
 // The same forward on the projections as they leave the GEMMs: see RAW above.
