@@ -93,6 +93,13 @@ ttt::Problems<A> pack_of(const A* probs, unsigned n) {
   return P;
 }
 
+// whether any problem of a launch asks the kernel to form its operands as x + projections (LinearFwdArgs::xin)
+bool any_input_sums(const ttt::LinearFwdArgs* probs, unsigned ny) {
+  for (unsigned i = 0; i < ny; ++i)
+    if (probs[i].xin != nullptr) return true;
+  return false;
+}
+
 // ---- TTT-Linear forward, head_dim 32/64: kernel choice --------------------------------------
 // A (batch, head) unit is a strictly sequential chain of mini-batches, so the launch is latency
 // bound until there are more units than SIMDs.  Few units: split each unit over several waves
@@ -101,6 +108,7 @@ ttt::Problems<A> pack_of(const A* probs, unsigned n) {
 template <class T, int D, int NW>
 int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s, bool own_loads = false) {
   const ttt::LinearFwdArgs& a = probs[0];
+  const bool sums = any_input_sums(probs, ny);
   const auto P = pack_of(probs, ny);
   // mini-batches prefetched ahead, in registers (f32 fragments are twice as large: the one-wave f32 kernel, which
   // holds the whole state and all rows in one wave, has registers for one mini-batch ahead only)
@@ -129,6 +137,13 @@ int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream
     // full rows cross LDS (same bits).  Measured on MI355X (seq 2048): 24 units 117 us against 114 us, 252 units
     // 120 against 120, 384 units 129 - 139 against 137 - 146: it pays once two workgroups share a CU's load path.
     if constexpr (can_fac && NWS == 2 && D == 64) {
+      if (sums) {  // operands formed as x + projections (a layer of a stack); no checkpoints in that mode
+        if (a.K == 16)
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, true, false, 2>), grid, block, 0, s, P);
+        else
+          hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NWS, PF, false, false, 2>), grid, block, 0, s, P);
+        return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+      }
       if (own_loads) {
         if (fac) {
           if (a.K == 16)
@@ -180,6 +195,9 @@ int launch_linear_fwd(const ttt::LinearFwdArgs* probs, int hint, unsigned ny, hi
       nw = units <= 512 ? 2 : 1;
   }
   if (nw > max_nw) nw = max_nw;
+  if constexpr (!f32 && D == 64) {
+    if (any_input_sums(probs, ny)) nw = 2;  // the kernel that forms x + projections is the two-wave one
+  }
   if constexpr (max_nw >= 4) {
     if (nw >= 4) return launch_linear_fwd_nw<T, D, 4>(probs, ny, s);
   }
@@ -201,6 +219,15 @@ int launch_linear_fwd_wide(const ttt::LinearFwdArgs* probs, unsigned ny, hipStre
   constexpr bool f32 = sizeof(typename ttt::Io<T>::elem) == 4;
   constexpr int PF = f32 ? 1 : 2;  // f32 fragments are twice as large: prefetch one mini-batch ahead
   const dim3 grid((unsigned)(a.B * a.H), ny), block(64 * NW);
+  if constexpr (!f32 && D == 128) {
+    if (any_input_sums(probs, ny)) {
+      if (a.K == 16)
+        hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, true, false, 2>), grid, block, 0, s, P);
+      else
+        hipLaunchKernelGGL((ttt::ttt_linear_fwd_sk_kernel<T, D, NW, PF, false, false, 2>), grid, block, 0, s, P);
+      return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+    }
+  }
   if constexpr (!f32 && D == 96) {
     if (a.ckpt_packed == ttt::kCkptFactors) {
       if (a.K == 16)
@@ -619,7 +646,7 @@ int prepare_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const 
   ttt::LinearFwdArgs& a = *pa;
   a.xq = xq; a.xk = xk; a.xv = xv; a.W0 = W0; a.b0 = b0; a.token_eta = token_eta; a.lr = lr;
   a.gamma = gamma; a.beta = beta; a.out = out; a.W_out = W_out; a.b_out = b_out;
-  a.W_ckpt = W_ckpt; a.b_ckpt = b_ckpt;
+  a.W_ckpt = W_ckpt; a.b_ckpt = b_ckpt; a.xin = nullptr;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
   a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.n_stages = d->seq / d->mini_batch;
@@ -1106,6 +1133,10 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
     if (!aligned16(L.pq) || !aligned16(L.pk) || !aligned16(L.pv))
       return fail(TTT_ERR_SHAPE, "ttt_stack_fwd: layer %d: pq/pk/pv must be 16-byte aligned", l);
   }
+  // bf16 I/O at head_dim 64 and 128: the TTT-Linear kernels form x + pq, x + pk, x + pv in their own loads (in place:
+  // x is what the layer below left in `out`), so those windows need no launch and no workspace for their input sums
+  const bool fuse_linear_sums = d->io_dtype == TTT_BF16 && (d->head_dim == 64 || d->head_dim == 128) &&
+                                (d->kernel_hint & (TTT_HINT_LDS_TILES | TTT_HINT_WAVES_MASK)) == 0;
   for (int t = 0; t < C + n_layers - 1; ++t) {
     for (int kind = 0; kind < 2; ++kind) {
       Group g{t, kind, kind == TTT_LAYER_LINEAR ? (int)lin.size() : (int)mlp.size(), 0, false, {}, {}};
@@ -1119,7 +1150,12 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
         const unsigned char *q = static_cast<const unsigned char*>(L.pq) + woff, *k = static_cast<const unsigned char*>(L.pk) + woff,
                             *v = static_cast<const unsigned char*>(L.pv) + woff;
         unsigned char* ow = static_cast<unsigned char*>(out) + woff;  // `out` is the hand-over tensor too
-        if (l > 0) {
+        const void* x_in = nullptr;
+        if (l > 0 && !is_mlp && fuse_linear_sums) {
+          // the TTT-Linear kernel forms x + projections itself, reading x from `out` in place
+          x_in = ow;
+          if (layers[l - 1].kind != kind) g.waits_other = true;
+        } else if (l > 0) {
           // window j of the sums tensors is free: its previous user (l-1, j) is done before this window starts
           ttt::LayerInputsArgs a;
           a.x = ow; a.pq = q; a.pk = k; a.pv = v;
@@ -1170,6 +1206,7 @@ int ttt_stack_fwd(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* la
           ttt::LinearFwdArgs a;
           rc = prepare_linear_fwd(&ld, q, k, v, W1i, b1i, token_eta, lr, L.gamma, L.beta, ow, to[0], to[1], nullptr, nullptr, &a);
           if (rc != TTT_OK) return rc;
+          a.xin = x_in;
           lin.push_back(a);
         } else {
           ttt::MlpFwdArgs a;

@@ -12,6 +12,8 @@ struct LinearFwdArgs {
   const void* xq;
   const void* xk;
   const void* xv;
+  const void* xin;  // null, or x [B,H,seq,d] io: the operands are x + xq, x + xk, x + xv (sums rounded to the I/O
+                    // type), formed by the kernel; may be the same memory as `out` (a layer of a stack working in place)
   const float* W0;
   const float* b0;
   const float* token_eta;

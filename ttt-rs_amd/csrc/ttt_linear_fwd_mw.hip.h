@@ -291,10 +291,11 @@ __device__ __forceinline__ void store_state_final(float* Wd, float* bd, const fl
 template <class T, int D>
 struct UnitBase {
   using elem = typename Io<T>::elem;
-  const unsigned char *xq, *xk, *xv, *lr;
+  const unsigned char *xq, *xk, *xv, *lr, *xin;
   unsigned char* out;
   __device__ __forceinline__ UnitBase(const LinearFwdArgs& a, size_t bh) {
     const size_t row0 = bh * (size_t)a.seq_stride;
+    xin = static_cast<const unsigned char*>(a.xin) + row0 * (D * sizeof(elem));
     xq = static_cast<const unsigned char*>(a.xq) + row0 * (D * sizeof(elem));
     xk = static_cast<const unsigned char*>(a.xk) + row0 * (D * sizeof(elem));
     xv = static_cast<const unsigned char*>(a.xv) + row0 * (D * sizeof(elem));

@@ -32,6 +32,10 @@ namespace ttt {
 //     (ttt_linear_bwd needs them): the wave that owns a feature stores it.
 // RAW = 3: the operands are given, and fetched the same way: every wave loads only the features it owns and the
 // full xq, xk rows reach the waves through LDS (half the vector loads of RAW = 0, where every wave loads every row).
+// RAW = 4: as RAW = 3 with the operands formed as x + xq, x + xk, x + xv (LinearFwdArgs::xin: a layer of a stack whose
+// input is the output of the layer below plus its own projections); x may be the memory `out` is written to: a wave
+// reads a row's own features three mini-batches before it writes that row's own features, and no other wave
+// touches them.
 template <class T, int D, int NW, int PF, bool FULL, bool FAC, int RAW>
 __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const FusedInputsArgs* fip) {
   using IO = Io<T>;
@@ -206,6 +210,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   // ---- RAW: the raw rows of the own features, three mini-batches ahead (ring index = mini-batch % R, as for buf)
   struct RawIn {
     frag q[TPW], k[TPW], v[TPW];
+    frag x[TPW];                // RAW = 4 only
     float z;                    // lr logit of the lane's token
     f32x2 cs[TPW], sn[TPW];     // RAW = 2 only
   };
@@ -214,7 +219,8 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   u32x4* xrot = nullptr;           // rotated rows in LDS: [2 buffers][xq, xk][feature pair][lane]
   float lr_bias_h = 0.f;
   if constexpr (RAW != 0) {
-    static_assert(BF && NT <= 4 && PF == 2, "rows shared through LDS: bf16 I/O, head_dim <= 64");
+    static_assert(BF && PF == 2, "rows shared through LDS: bf16 I/O");
+    static_assert(!FORM || NT <= 4, "operands formed from the projections: head_dim <= 64");
     __shared__ u32x4 xrot_s[2][2][NT / 2][64];
     xrot = &xrot_s[0][0][0][0];
 #pragma unroll
@@ -237,6 +243,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
     if (fip->token_eta_out != nullptr && bh == 0)
       for (int i = threadIdx.x; i < a.seq; i += 64 * NW) fip->token_eta_out[i] = tok_eta(i % K);
   }
+  const bool has_x = a.xin != nullptr;  // RAW = 4: a problem without x takes the operands as they are (x = 0)
   // raw rows of unit (b, h): token t of the unit is row (b * seq + t) * H + h of the [B,seq,H,d] tensors
   const size_t bidx = bh / a.H;
   const unsigned raw_row = (unsigned)a.H * (unsigned)(D * sizeof(elem));  // bytes from one token to the next
@@ -264,6 +271,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
         r.q[0] = ok ? load4<T>(reinterpret_cast<const elem*>(bq + o1)) : IO::zero();
         r.k[0] = ok ? load4<T>(reinterpret_cast<const elem*>(bk + o1)) : IO::zero();
         r.v[0] = ok ? load4<T>(reinterpret_cast<const elem*>(bv + o1)) : IO::zero();
+        if constexpr (RAW == 4) r.x[0] = (ok && has_x) ? load4<T>(reinterpret_cast<const elem*>(ub.xin + o1)) : IO::zero();
       } else {
 #pragma unroll
         for (int qq = 0; qq < TPW / 2; ++qq) {
@@ -271,6 +279,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
           IO::load8(reinterpret_cast<const elem*>(bq + o2), ok, r.q[2 * qq], r.q[2 * qq + 1]);
           IO::load8(reinterpret_cast<const elem*>(bk + o2), ok, r.k[2 * qq], r.k[2 * qq + 1]);
           IO::load8(reinterpret_cast<const elem*>(bv + o2), ok, r.v[2 * qq], r.v[2 * qq + 1]);
+          if constexpr (RAW == 4) IO::load8(reinterpret_cast<const elem*>(ub.xin + o2), ok && has_x, r.x[2 * qq], r.x[2 * qq + 1]);
         }
       }
       if constexpr (FORM) {
@@ -299,11 +308,17 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
           const f32x2 cs = RAW == 2 ? r.cs[jj] : cs_fix[jj], sn = RAW == 2 ? r.sn[jj] : sn_fix[jj];
           dst.qo[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.q[jj]), cs, sn));
           dst.ko[jj] = IO::to_frag(rope_rotate4(IO::to_f32(r.k[jj]), cs, sn));
+          dst.vo[jj] = r.v[jj];
+        } else if constexpr (RAW == 4) {
+          const f32x4 x = IO::to_f32(r.x[jj]);
+          dst.qo[jj] = IO::to_frag(x + IO::to_f32(r.q[jj]));
+          dst.ko[jj] = IO::to_frag(x + IO::to_f32(r.k[jj]));
+          dst.vo[jj] = IO::to_frag(x + IO::to_f32(r.v[jj]));
         } else {
           dst.qo[jj] = r.q[jj];
           dst.ko[jj] = r.k[jj];
+          dst.vo[jj] = r.v[jj];
         }
-        dst.vo[jj] = r.v[jj];
       }
       // the gate in the precision the operand has when it is a tensor of its own
       // (a token past the end of a short mini-batch has no learning rate: it must not reach the state update)
@@ -557,7 +572,10 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         const int st = st0 + u;
-        load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], ub, K, n_stages_, st + PF, c, g, w);
+        if constexpr (RAW != 0)
+          load_raw(raw[u], st + R);
+        else
+          load_stage_mw<T, D, NW, FULL>(buf[(u + PF) % R], ub, K, n_stages_, st + PF, c, g, w);
         if (st >= a.n_stages) continue;
         const StageInMw<T, NT, TPW>& cur = buf[u];
 
@@ -626,6 +644,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
         exchange8_publish(S, st & 1);
         if (st > 1) emit_output(so0, so1, st - 2, zbo, qoo);  // inside the exchange window, as above
         exchange8_collect(S, st & 1);
+        if constexpr (RAW != 0) gather_rows(buf[(u + 1) % R], (st + 1) & 1);
         so0 = S[6];
         so1 = S[7];
 #pragma unroll
@@ -679,6 +698,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
           zbp[jj] = zb[jj];
           qop[jj] = cur.qo[jj];
         }
+        if constexpr (RAW != 0) rotate_share(raw[(u + 2) % R], buf[(u + 2) % R], st + 2, st & 1);
       }
     }
 
@@ -697,10 +717,11 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
     store_state_tiles<D, TPW>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D), a.b_ckpt + bh * (size_t)a.n_ckpt * D, Wc, bT, w, lane);
 }
 
-// OWN: every wave loads only the features it owns, full rows through LDS (RAW = 3)
-template <class T, int D, int NW, int PF, bool FULL, bool FAC = false, bool OWN = false>
+// OWN = 1: every wave loads only the features it owns, full rows through LDS (RAW = 3); OWN = 2: the same with the
+// operands formed as x + xq, x + xk, x + xv (RAW = 4)
+template <class T, int D, int NW, int PF, bool FULL, bool FAC = false, int OWN = 0>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
-  linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, OWN ? 3 : 0>(problems.p[blockIdx.y], nullptr);
+  linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, OWN == 0 ? 0 : OWN + 2>(problems.p[blockIdx.y], nullptr);
 }
 
 // The same forward on the projections as they leave the GEMMs: see RAW above.
