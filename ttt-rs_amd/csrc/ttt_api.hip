@@ -444,8 +444,16 @@ int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
     if (f32 && D == 128)
       return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
     int waves = d->kernel_hint & TTT_HINT_WAVES_MASK;
-    if (waves == 0) waves = (f32 || D > 64 || (long)d->batch * d->heads <= 512) ? 4 : 1;
-    if (factors) waves = 4;  // the walk back of the state exists in the feature-split kernel only
+    const long units = (long)d->batch * d->heads;
+    // bf16 at head_dim 64 between 257 and 512 units, f32 row-major checkpoints: two waves per unit.  Four waves per
+    // unit put eight waves on the four SIMDs of every CU that hosts two workgroups; with two, every wave keeps a SIMD
+    // to itself (measured at 384 units: 544 us against 606 us; at 192 units 513 against 392).  With packed states or
+    // update factors the four-wave kernel stays ahead at 384 units as well (456 against 468 us, 440 against 473 us),
+    // so there two waves are a matter of the hint.
+    const bool two = !f32 && D == 64 && units > 256 && units <= 512 && !packed && !factors;
+    if (waves == 0) waves = two ? 2 : (f32 || D > 64 || units <= 512) ? 4 : 1;
+    // the walk back of the state exists in the feature-split kernel only
+    if (factors && (waves < 2 || (waves == 2 && D != 64))) waves = 4;
     ch->kind = LinearBwdChoice::REG;
     ch->waves = waves;
     return TTT_OK;
@@ -857,7 +865,9 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   }
   if (a.ckpt_packed == ttt::kCkptFactors) {
     if (D == 32) return launch_linear_bwd_mw<ttt::BF16, 32, 2, true, true>(a, grid, s);
-    if (D == 64) return launch_linear_bwd_mw<ttt::BF16, 64, 4, true, true>(a, grid, s);
+    if (D == 64)
+      return waves == 2 ? launch_linear_bwd_mw<ttt::BF16, 64, 2, true, true>(a, grid, s)
+                        : launch_linear_bwd_mw<ttt::BF16, 64, 4, true, true>(a, grid, s);
     return launch_linear_bwd_mw<ttt::BF16, 96, 3, true, true>(a, grid, s);
   }
   if (f32 && a.ckpt_packed) {
@@ -873,7 +883,10 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   }
   if (a.ckpt_packed) {
     if (D == 32) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 32, 2, true>(a, grid, s) : launch_linear_bwd_rr<32, true>(a, grid, s);
-    if (D == 64) return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 64, 4, true>(a, grid, s) : launch_linear_bwd_rr<64, true>(a, grid, s);
+    if (D == 64) {
+      if (waves == 2) return launch_linear_bwd_mw<ttt::BF16, 64, 2, true>(a, grid, s);
+      return waves > 1 ? launch_linear_bwd_mw<ttt::BF16, 64, 4, true>(a, grid, s) : launch_linear_bwd_rr<64, true>(a, grid, s);
+    }
     if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3, true>(a, grid, s);
     return launch_linear_bwd_mw<ttt::BF16, 128, 4, true>(a, grid, s);
   }
