@@ -384,6 +384,26 @@ int ttt_linear_fwd_fused_inputs(const ttt_desc* desc, const void* xq, const void
                                 void* stream);
 
 /*
+ * TTT-Linear with an Adam inner optimiser, multi-stage forward.  The fused counterpart of TTTLinearAdam::forward
+ * (rust/core/src/linear_adam.rs:183-236 looped as rust/core/src/inner.rs:25-50; the reference has no fused kernel for
+ * it): the mini-batch of ttt_linear_fwd with the state update W -= XK^T (eta_last G), b -= colsum(eta_last G)
+ * replaced by one Adam step on those gradients (adam_update, linear_adam.rs:76-128):
+ *   m = beta1 m + (1 - beta1) g;  v = beta2 v + (1 - beta2) g^2;  t = step0 + mini-batches so far + 1;
+ *   theta -= adam_lr (m / (1 - beta1^t)) / (sqrt(v / (1 - beta2^t)) + adam_eps).
+ * xq .. beta, out, W_out, b_out as for ttt_linear_fwd (no checkpoints: forward only).  Moments are f32 in the layout of
+ * the state, per batch element: Wm0, Wv0 [B,H,d,d], bm0, bv0 [B,H,d] enter (all four NULL: zero moments and step0 = 0,
+ * TTTLinearAdam::init_state, linear_adam.rs:164-177), Wm_out .. bv_out leave; the step counter after the call is
+ * step0 + seq / mini_batch.  State, moments and arithmetic are f32 for both I/O types (the reference keeps the first
+ * moment in the backend's float type).  head_dim 32 and 64; ttt_linear_adam_supported says so beforehand.
+ */
+int ttt_linear_adam_supported(const ttt_desc* desc);
+int ttt_linear_adam_fwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv, const float* W0,
+                        const float* b0, const float* Wm0, const float* bm0, const float* Wv0, const float* bv0,
+                        int step0, float beta1, float beta2, float adam_eps, float adam_lr, const float* token_eta,
+                        const void* lr, const float* gamma, const float* beta, void* out, float* W_out, float* b_out,
+                        float* Wm_out, float* bm_out, float* Wv_out, float* bv_out, void* stream);
+
+/*
  * Self-test of a hardware fact the bf16 kernels rely on; no counterpart in the reference.  One wavefront computes
  * D = A1*B1 with one bf16 matrix instruction and D2 = A2*B2 + D with an instruction of the other shape (order 0:
  * 16x16x32 then 16x16x16 with D2 written over D; order 1: the reverse; orders 2, 3: the same two with D2 in other

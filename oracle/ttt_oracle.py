@@ -19,6 +19,8 @@ reference checkout):
                       backward/stage.rs:42-1006, layer_norm.rs:428-709
   mlp_mini_batch      rust/core/src/mlp.rs:127-208
   mlp_forward         rust/core/src/inner.rs:25-50
+  linear_adam_mini_batch, linear_adam_forward
+                      rust/core/src/linear_adam.rs:76-128 (adam_update), :183-236 (forward_mini_batch)
 
 How each function is pinned (tests/test_oracle_*.py):
   ln_fwd            == torch.nn.functional.layer_norm (library routine)
@@ -35,6 +37,9 @@ How each function is pinned (tests/test_oracle_*.py):
   mlp_mini_batch    == primal per-token GD on both layers, written in the test
   mlp_backward      == torch autograd (float64, double backward) through a torch restatement of the dual
                        form whose forward is checked against mlp_forward, plus linearity
+  linear_adam_*     == the gradients of linear_mini_batch fed to torch.optim.Adam (library routine) step by step;
+                       first step from zero moments moves every element by lr*g/(|g|+eps) (closed form);
+                       output of a mini-batch == linear_mini_batch's (the output does not see the update)
   lr_logit_grad     == central finite differences of linear_forward through the gate
   rope_apply        == complex rotation of adjacent pairs; inner_loop_inputs, layer_epilogue == their pieces
                        (torch sigmoid / layer_norm / gelu) assembled independently in the test
@@ -175,6 +180,62 @@ def linear_forward(W0, b0, xq, xk, xv, token_eta, lr, gamma, beta, K=16, eps=1e-
     if checkpoint_interval:
         return out, W, b, np.stack(Wc, 2), np.stack(bc, 2)
     return out, W, b
+
+
+# --------------------------------------------------------------------------- TTT-Linear with an Adam inner optimiser
+def linear_adam_mini_batch(state, xq, xk, xv, token_eta, lr, gamma, beta, eps=1e-6, beta1=0.9, beta2=0.999,
+                           adam_eps=1e-8, adam_lr=1e-3):
+    """linear_adam.rs:183-236: the mini-batch of TTT-Linear with the state update replaced by one Adam step on the
+    same eta-weighted gradients (adam_update, linear_adam.rs:76-128).  state = dict(W, b, Wm, bm, Wv, bv, step);
+    returns (out, new state).  The output is computed from the state entering the mini-batch, as in linear.rs."""
+    W, b = state["W"], state["b"]
+    k = xq.shape[2]
+    tri = np.tril(np.ones((k, k), dtype=W.dtype))
+    z1 = xk @ W + b[:, :, None, :]                                  # :196
+    g = ln_l2_grad(z1, xv - xk, _hb(gamma), _hb(beta), eps)         # :198-202
+    eta = _eta(token_eta, lr)                                       # :204-208
+    attn = (xq @ _T(xk)) * tri                                      # :210
+    b_bar = b[:, :, None, :] - eta @ g                              # :212-213
+    z_bar = xq @ W - (eta * attn) @ g + b_bar                       # :215-217
+    last = eta[:, :, -1, :]                                         # :219-220
+    gW = _T(last[..., None] * xk) @ g                               # :222-224
+    gb = (last[..., None] * g).sum(2)                               # :226-228
+    step = state["step"] + 1                                        # :91
+    Wm = state["Wm"] * beta1 + gW * (1.0 - beta1)                   # :102-103
+    bm = state["bm"] * beta1 + gb * (1.0 - beta1)
+    Wv = state["Wv"] * beta2 + gW ** 2 * (1.0 - beta2)              # :106-111
+    bv = state["bv"] * beta2 + gb ** 2 * (1.0 - beta2)
+    c1, c2 = 1.0 - beta1 ** step, 1.0 - beta2 ** step               # :113-114
+    W_new = W - (Wm / c1) / (np.sqrt(Wv / c2) + adam_eps) * adam_lr  # :116-126
+    b_new = b - (bm / c1) / (np.sqrt(bv / c2) + adam_eps) * adam_lr
+    out = xq + ln_fwd(z_bar, _hb(gamma), _hb(beta), eps)            # :232-234
+    return out, dict(W=W_new, b=b_new, Wm=Wm, bm=bm, Wv=Wv, bv=bv, step=step)
+
+
+def linear_adam_forward(W0, b0, xq, xk, xv, token_eta, lr, gamma, beta, K=16, eps=1e-6, beta1=0.9, beta2=0.999,
+                        adam_eps=1e-8, adam_lr=1e-3, state0=None, dtype=np.float64):
+    """inner.rs:25-50 over linear_adam_mini_batch; the state starts with zero moments and step 0
+    (init_state, linear_adam.rs:164-177) unless state0 = dict(Wm, bm, Wv, bv, step) continues an earlier call.
+    Returns (out, final state dict)."""
+    xq, xk, xv, lr = (np.asarray(a, dtype=dtype) for a in (xq, xk, xv, lr))
+    gamma, beta = np.asarray(gamma, dtype=dtype), np.asarray(beta, dtype=dtype)
+    token_eta = np.asarray(token_eta, dtype=dtype)
+    B, H, seq, d = xq.shape
+    W, b = np.asarray(W0, dtype=dtype), np.asarray(b0, dtype=dtype)
+    if W.ndim == 3:
+        W = np.broadcast_to(W[None], (B, H, d, d)).copy()
+        b = np.broadcast_to(b[None], (B, H, d)).copy()
+    st = dict(W=W, b=b, Wm=np.zeros_like(W), bm=np.zeros_like(b), Wv=np.zeros_like(W), bv=np.zeros_like(b), step=0)
+    if state0 is not None:
+        st.update({k: (np.asarray(v, dtype=dtype) if k != "step" else int(v)) for k, v in state0.items()})
+    out = np.zeros_like(xq)
+    for s0 in range(0, seq, K):
+        s1 = min(s0 + K, seq)
+        te = token_eta[s0:s1] if token_eta.shape[0] == seq and seq != K else token_eta[: s1 - s0]
+        o, st = linear_adam_mini_batch(st, xq[:, :, s0:s1], xk[:, :, s0:s1], xv[:, :, s0:s1], te, lr[:, :, s0:s1],
+                                       gamma, beta, eps, beta1, beta2, adam_eps, adam_lr)
+        out[:, :, s0:s1] = o
+    return out, st
 
 
 def _ln_l2_parts(z1, target, gamma, beta, eps):

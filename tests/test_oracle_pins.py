@@ -460,3 +460,57 @@ def test_lr_logit_grad_is_the_derivative_through_the_gate():
         zm[idx] -= h
         fd = (loss(zp) - loss(zm)) / (2 * h)
         assert abs(fd - dz[idx]) <= 1e-6 * max(1.0, abs(fd)), (idx, fd, dz[idx])
+
+
+# ------------------------------------------------------------------ TTT-Linear with the Adam inner optimiser
+def test_linear_adam_is_torch_adam_on_the_sgd_gradients():
+    """linear_adam.rs replaces the state update of TTT-Linear by an Adam step on the same eta-weighted gradients.
+    The gradients are taken from linear_mini_batch (pinned to primal gradient descent above) as W - W_sgd, the
+    optimiser is torch.optim.Adam (library routine), stepped mini-batch by mini-batch; the output of a mini-batch
+    does not see its own update, so it equals linear_mini_batch's output at the same state."""
+    B, H, seq, d, K = 2, 2, 24, 8, 4
+    c = make_linear_case(41, B, H, seq, d, K)
+    hp = dict(beta1=0.8, beta2=0.95, adam_eps=1e-6, adam_lr=3e-2)
+    out, st = orc.linear_adam_forward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"], c["gamma"],
+                                      c["beta"], K=K, **hp)
+    W = torch.tensor(np.broadcast_to(c["W0"][None], (B, H, d, d)).copy(), requires_grad=True)
+    b = torch.tensor(np.broadcast_to(c["b0"][None], (B, H, d)).copy(), requires_grad=True)
+    opt = torch.optim.Adam([W, b], lr=hp["adam_lr"], betas=(hp["beta1"], hp["beta2"]), eps=hp["adam_eps"])
+    for t in range(seq // K):
+        sl = slice(t * K, (t + 1) * K)
+        Wn, bn = W.detach().numpy().copy(), b.detach().numpy().copy()
+        o, Ws, bs = orc.linear_mini_batch(Wn, bn, c["xq"][:, :, sl], c["xk"][:, :, sl], c["xv"][:, :, sl], c["te"],
+                                          c["lr"][:, :, sl], c["gamma"], c["beta"])
+        np.testing.assert_allclose(out[:, :, sl], o, rtol=1e-10, atol=1e-12)
+        W.grad, b.grad = torch.tensor(Wn - Ws), torch.tensor(bn - bs)
+        opt.step()
+    np.testing.assert_allclose(st["W"], W.detach().numpy(), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(st["b"], b.detach().numpy(), rtol=1e-9, atol=1e-11)
+    assert st["step"] == seq // K
+
+
+def test_linear_adam_first_step_moves_every_element_by_lr_sign():
+    """From zero moments the bias corrections cancel: m_hat = g, v_hat = g^2, so the first step is
+    lr * g / (|g| + eps) whatever beta1 and beta2 are."""
+    B, H, d, K = 1, 2, 8, 4
+    c = make_linear_case(43, B, H, K, d, K)
+    _, Ws, bs = orc.linear_forward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"], c["gamma"],
+                                   c["beta"], K=K)
+    gW = np.broadcast_to(c["W0"][None], Ws.shape) - Ws
+    _, st = orc.linear_adam_forward(c["W0"], c["b0"], c["xq"], c["xk"], c["xv"], c["te"], c["lr"], c["gamma"],
+                                    c["beta"], K=K, beta1=0.7, beta2=0.9, adam_eps=1e-9, adam_lr=0.05)
+    np.testing.assert_allclose(np.broadcast_to(c["W0"][None], Ws.shape) - st["W"], 0.05 * gW / (np.abs(gW) + 1e-9),
+                               rtol=1e-9, atol=1e-12)
+
+
+def test_linear_adam_continues_from_a_saved_state():
+    B, H, seq, d, K = 1, 2, 16, 8, 4
+    c = make_linear_case(45, B, H, seq, d, K)
+    args = lambda a, b_: (c["xq"][:, :, a:b_], c["xk"][:, :, a:b_], c["xv"][:, :, a:b_], c["te"], c["lr"][:, :, a:b_],
+                          c["gamma"], c["beta"])
+    out, st = orc.linear_adam_forward(c["W0"], c["b0"], *args(0, seq), K=K)
+    o1, s1 = orc.linear_adam_forward(c["W0"], c["b0"], *args(0, 8), K=K)
+    o2, s2 = orc.linear_adam_forward(s1["W"], s1["b"], *args(8, seq), K=K,
+                                     state0={k: s1[k] for k in ("Wm", "bm", "Wv", "bv", "step")})
+    np.testing.assert_array_equal(np.concatenate([o1, o2], 2), out)
+    np.testing.assert_array_equal(s2["W"], st["W"])

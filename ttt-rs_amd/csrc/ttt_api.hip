@@ -717,6 +717,59 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   return dispatch_linear_fwd(d, &a, 1, static_cast<hipStream_t>(stream));
 }
 
+int ttt_linear_adam_supported(const ttt_desc* d) {
+  int rc = ttt_linear_supported(d);
+  if (rc != TTT_OK) return rc;
+  if (d->head_dim != 32 && d->head_dim != 64)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_adam_fwd: head_dim 32 or 64 (got %d)", d->head_dim);
+  if ((d->kernel_hint & TTT_HINT_LDS_TILES) != 0)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_adam_fwd: the register-resident kernel only");
+  return TTT_OK;
+}
+
+int ttt_linear_adam_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv, const float* W0,
+                        const float* b0, const float* Wm0, const float* bm0, const float* Wv0, const float* bv0,
+                        int step0, float beta1, float beta2, float adam_eps, float adam_lr, const float* token_eta,
+                        const void* lr, const float* gamma, const float* beta, void* out, float* W_out, float* b_out,
+                        float* Wm_out, float* bm_out, float* Wv_out, float* bv_out, void* stream) {
+  int rc = ttt_linear_adam_supported(d);
+  if (rc != TTT_OK) return rc;
+  const int n_in = (Wm0 != nullptr) + (bm0 != nullptr) + (Wv0 != nullptr) + (bv0 != nullptr);
+  if (n_in != 0 && n_in != 4)
+    return fail(TTT_ERR_NULL, "ttt_linear_adam_fwd: the four moments entering the call are given together or not at all");
+  if (!Wm_out || !bm_out || !Wv_out || !bv_out)
+    return fail(TTT_ERR_NULL, "ttt_linear_adam_fwd: a required pointer is NULL");
+  if (step0 < 0 || (n_in == 0 && step0 != 0))
+    return fail(TTT_ERR_SHAPE, "ttt_linear_adam_fwd: step0 must be >= 0, and 0 when no moments are given");
+  if (!(beta1 >= 0.f && beta1 < 1.f) || !(beta2 >= 0.f && beta2 < 1.f) || !(adam_eps >= 0.f))
+    return fail(TTT_ERR_SHAPE, "ttt_linear_adam_fwd: beta1, beta2 in [0, 1) and adam_eps >= 0");
+  if (!aligned16(bm_out) || !aligned16(bv_out))
+    return fail(TTT_ERR_SHAPE, "ttt_linear_adam_fwd: bm_out/bv_out must be 16-byte aligned");
+  ttt::LinearFwdArgs a;
+  rc = prepare_linear_fwd(d, xq, xk, xv, W0, b0, token_eta, lr, gamma, beta, out, W_out, b_out, nullptr, nullptr, &a);
+  if (rc != TTT_OK) return rc;
+  ttt::AdamArgs ad;
+  ad.Wm0 = Wm0; ad.bm0 = bm0; ad.Wv0 = Wv0; ad.bv0 = bv0;
+  ad.Wm_out = Wm_out; ad.bm_out = bm_out; ad.Wv_out = Wv_out; ad.bv_out = bv_out;
+  ad.beta1 = beta1; ad.beta2 = beta2; ad.eps = adam_eps; ad.lr = adam_lr; ad.step0 = step0;
+  const dim3 grid((unsigned)(a.B * a.H)), block(128);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool full = d->mini_batch == 16, f32 = d->io_dtype == TTT_F32;
+  // head_dim 64 holds state and both moments in 96 registers per wave: the rows are prefetched one mini-batch ahead
+  // there (two ahead would spill hundreds of registers), two ahead at head_dim 32
+#define TTT_ADAM_LAUNCH(T_, D_, FULL_) \
+  hipLaunchKernelGGL((ttt::ttt_linear_adam_fwd_kernel<T_, D_, 2, (D_ == 64 ? 1 : 2), FULL_>), grid, block, 0, s, a, ad)
+  if (d->head_dim == 64) {
+    if (f32) { if (full) TTT_ADAM_LAUNCH(ttt::F32, 64, true); else TTT_ADAM_LAUNCH(ttt::F32, 64, false); }
+    else { if (full) TTT_ADAM_LAUNCH(ttt::BF16, 64, true); else TTT_ADAM_LAUNCH(ttt::BF16, 64, false); }
+  } else {
+    if (f32) { if (full) TTT_ADAM_LAUNCH(ttt::F32, 32, true); else TTT_ADAM_LAUNCH(ttt::F32, 32, false); }
+    else { if (full) TTT_ADAM_LAUNCH(ttt::BF16, 32, true); else TTT_ADAM_LAUNCH(ttt::BF16, 32, false); }
+  }
+#undef TTT_ADAM_LAUNCH
+  return hip_status(hipGetLastError(), "ttt_linear_adam_fwd launch");
+}
+
 int ttt_linear_fwd_fused_inputs_supported(const ttt_desc* d, int pos_wrap, int has_rope) {
   int rc = ttt_linear_supported(d);
   if (rc != TTT_OK) return rc;

@@ -53,4 +53,19 @@ struct FusedInputsArgs {
   int pos_offset, pos_wrap;  // position of token t: (pos_offset + t) [% pos_wrap if > 0]
 };
 
+// TTT-Linear with an Adam inner optimiser (reference rust/core/src/linear_adam.rs): the moments of the state and the
+// optimiser's constants.  Moments are per (batch, head) unit, f32, in the layout of the state.
+struct AdamArgs {
+  const float* Wm0;  // [B,H,d,d] first moment entering the call; the four inputs are null together: zero moments
+  const float* bm0;  // [B,H,d]
+  const float* Wv0;  // second moment
+  const float* bv0;
+  float* Wm_out;
+  float* bm_out;
+  float* Wv_out;
+  float* bv_out;
+  float beta1, beta2, eps, lr;
+  int step0;  // Adam steps taken before this call (the reference's state.step)
+};
+
 }  // namespace ttt

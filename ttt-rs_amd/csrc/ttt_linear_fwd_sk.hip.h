@@ -36,8 +36,15 @@ namespace ttt {
 // input is the output of the layer below plus its own projections); x may be the memory `out` is written to: a wave
 // reads a row's own features three mini-batches before it writes that row's own features, and no other wave
 // touches them.
-template <class T, int D, int NW, int PF, bool FULL, bool FAC, int RAW>
-__device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const FusedInputsArgs* fip) {
+// ADAM: the state update W -= XK^T (eta_last G) is replaced by one Adam step on that gradient per mini-batch
+// (reference rust/core/src/linear_adam.rs:76-128): the gradient tile is formed by the same matrix instructions into a
+// zero accumulator, the moments live in registers beside the state (three times the state's registers), bias
+// corrections come from running powers of beta1, beta2.  Everything else -- products, LayerNorm, output -- is the
+// plain kernel's; the output of a mini-batch does not see its own update in either.
+template <class T, int D, int NW, int PF, bool FULL, bool FAC, int RAW, bool ADAM = false>
+__device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const FusedInputsArgs* fip,
+                                                   const AdamArgs* adam = nullptr) {
+  static_assert(!ADAM || (D <= 64 && !FAC && RAW == 0), "Adam inner optimiser: head_dim <= 64, no checkpoints");
   using IO = Io<T>;
   using frag = typename IO::frag;
   using elem = typename IO::elem;
@@ -103,6 +110,49 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   static_assert(NW * D <= 2 * 8 * 16 * NW, "the exchange buffer doubles as scratch of centre_state");
   centre_state<D, NW, TPW>(Wc, bT, a.b0 + sb * D, m0s, &ex[0][0], w, c, g);
 
+  // ADAM: first and second moments of this wave's W tiles and bias rows, and the running powers beta^step
+  f32x4 Wm[ADAM ? NT : 1][TPW], Wv[ADAM ? NT : 1][TPW], bm[TPW], bv[TPW];
+  float pw1 = 1.f, pw2 = 1.f;
+  if constexpr (ADAM) {
+    const bool have = adam->Wm0 != nullptr;
+#pragma unroll
+    for (int I = 0; I < NT; ++I)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const size_t at = bh * D * D + feat(I, 4 * g + r) * D + feat(w * TPW + jj, c);
+          Wm[I][jj][r] = have ? adam->Wm0[at] : 0.f;
+          Wv[I][jj][r] = have ? adam->Wv0[at] : 0.f;
+        }
+#pragma unroll
+    for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const size_t at = bh * D + own_offset<TPW>(w, jj, g) + r;
+        bm[jj][r] = have ? adam->bm0[at] : 0.f;
+        bv[jj][r] = have ? adam->bv0[at] : 0.f;
+      }
+    for (int i = 0; i < adam->step0; ++i) {
+      pw1 *= adam->beta1;
+      pw2 *= adam->beta2;
+    }
+  }
+  // one Adam step on a tile: gneg = -gradient (what the plain kernel would add to the state)
+  float ad_a1 = 0.f, ad_ic2 = 0.f;  // lr / (1 - beta1^t), 1 / (1 - beta2^t) of the current step
+  auto adam_tile = [&](f32x4& x, f32x4& m, f32x4& v, f32x4 gneg) {
+    if constexpr (ADAM) {
+      const float b1 = adam->beta1, b2 = adam->beta2;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float gr = -gneg[r];
+        m[r] = __builtin_fmaf(b1, m[r], (1.f - b1) * gr);
+        v[r] = __builtin_fmaf(b2, v[r], (1.f - b2) * (gr * gr));
+        const float den = __builtin_sqrtf(v[r] * ad_ic2) + adam->eps;
+        x[r] = __builtin_fmaf(-(ad_a1 * m[r]), __builtin_amdgcn_rcpf(den), x[r]);
+      }
+    }
+  };
   // pending output of the previous mini-batch (its LayerNorm sums travel in the next exchange) and of the
   // one before (sums known: it is finished while the next exchange is in flight)
   f32x4 zbp[TPW], zbo[TPW];
@@ -541,11 +591,32 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
 #pragma unroll
         for (int jj = 0; jj < TPW; ++jj) IO::mma(zb[jj], Gd[jj], Mf);
       }
+      if constexpr (ADAM) {
+        pw1 *= adam->beta1;
+        pw2 *= adam->beta2;
+        ad_a1 = adam->lr / (1.f - pw1);
+        ad_ic2 = 1.f / (1.f - pw2);
 #pragma unroll
-      for (int I = 0; I < NT; ++I)
+        for (int I = 0; I < NT; ++I)
 #pragma unroll
-        for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
-      bias_update(bT, Gd, ones_upd);
+          for (int jj = 0; jj < TPW; ++jj) {
+            f32x4 gneg = {0.f, 0.f, 0.f, 0.f};
+            IO::mma(gneg, kd[I], Gd[jj]);
+            adam_tile(Wc[I][jj], Wm[I][jj], Wv[I][jj], gneg);
+          }
+#pragma unroll
+        for (int jj = 0; jj < TPW; ++jj) {
+          f32x4 gneg = {0.f, 0.f, 0.f, 0.f};
+          IO::mma(gneg, Gd[jj], ones_upd);
+          adam_tile(bT[jj], bm[jj], bv[jj], gneg);
+        }
+      } else {
+#pragma unroll
+        for (int I = 0; I < NT; ++I)
+#pragma unroll
+          for (int jj = 0; jj < TPW; ++jj) IO::mma(Wc[I][jj], kd[I], Gd[jj]);
+        bias_update(bT, Gd, ones_upd);
+      }
       // this mini-batch's Zbar and xq become the pending output; its in-lane sums are formed here, in the
       // shadow of the state update, not between the next Z1 and its exchange
 #pragma unroll
@@ -713,6 +784,26 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
     emit_output(S[6], S[7], a.n_stages - 1, zbp, qop);
   }
   store_state_final<D, TPW>(a.W_out + bh * D * D, a.b_out + bh * D, a.W0 + sb * D * D, a.b0 + sb * D, Wc, bT, m0s, w, c, g);
+  if constexpr (ADAM) {
+#pragma unroll
+    for (int I = 0; I < NT; ++I)
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const size_t at = bh * D * D + feat(I, 4 * g + r) * D + feat(w * TPW + jj, c);
+          adam->Wm_out[at] = Wm[I][jj][r];
+          adam->Wv_out[at] = Wv[I][jj][r];
+        }
+    if (c == 0) {
+#pragma unroll
+      for (int jj = 0; jj < TPW; ++jj) {
+        const size_t at = bh * D + own_offset<TPW>(w, jj, g);
+        *reinterpret_cast<f32x4*>(adam->bm_out + at) = bm[jj];
+        *reinterpret_cast<f32x4*>(adam->bv_out + at) = bv[jj];
+      }
+    }
+  }
   if constexpr (FAC)
     store_state_tiles<D, TPW>(a.W_ckpt + bh * (size_t)a.n_ckpt * (D * D), a.b_ckpt + bh * (size_t)a.n_ckpt * D, Wc, bT, w, lane);
 }
@@ -722,6 +813,12 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
 template <class T, int D, int NW, int PF, bool FULL, bool FAC = false, int OWN = 0>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
   linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, OWN == 0 ? 0 : OWN + 2>(problems.p[blockIdx.y], nullptr);
+}
+
+// TTT-Linear with the Adam inner optimiser: see ADAM above.
+template <class T, int D, int NW, int PF, bool FULL>
+__global__ void __launch_bounds__(64 * NW) ttt_linear_adam_fwd_kernel(LinearFwdArgs a, AdamArgs ad) {
+  linear_fwd_sk_body<T, D, NW, PF, FULL, false, 0, true>(a, nullptr, &ad);
 }
 
 // The same forward on the projections as they leave the GEMMs: see RAW above.

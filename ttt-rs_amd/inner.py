@@ -183,6 +183,47 @@ def ttt_linear_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_w
     return out, w_out, b_out
 
 
+def ttt_linear_adam_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias, mini_batch: int,
+                                beta1: float = 0.9, beta2: float = 0.999, adam_eps: float = 1e-8, adam_lr: float = 1e-3,
+                                moments=None, step: int = 0, eps: float = 1e-6):
+    """One call of ttt_linear_adam_fwd on the current stream: TTTLinearAdam::forward
+    (rust/core/src/linear_adam.rs:183-236 looped as rust/core/src/inner.rs:25-50).  Arguments as
+    ttt_linear_forward_raw; moments = (weight_m, bias_m, weight_v, bias_v) per batch element to continue an earlier call
+    at `step`, or None for a fresh state.  Returns (output, weight, bias, (weight_m, bias_m, weight_v, bias_v), step)."""
+    B, H, seq, d = xq.shape
+    io = xq.dtype
+    xq = _need(xq, (B, H, seq, d), io, "xq")
+    xk = _need(xk, (B, H, seq, d), io, "xk")
+    xv = _need(xv, (B, H, seq, d), io, "xv")
+    per_batch = weight.dim() == 4
+    W0 = _need(weight, (B, H, d, d) if per_batch else (H, d, d), torch.float32, "weight")
+    b0 = _need(bias, (B, H, d) if per_batch else (H, d), torch.float32, "bias")
+    te = _need(token_eta[:mini_batch], (mini_batch,), torch.float32, "token_eta")
+    lr = _need(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta")
+    gam = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+    bet = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+    dev = xq.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    null = C.c_void_p(None)
+    m_in = [null] * 4
+    if moments is not None:
+        shapes = ((B, H, d, d), (B, H, d), (B, H, d, d), (B, H, d))
+        m_in = [_ptr(_need(t, sh, torch.float32, "moment")) for t, sh in zip(moments, shapes)]
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), 1 if per_batch else 0, 0, 0, 0)
+    check(lib().ttt_linear_adam_supported(C.byref(desc)))
+    out = torch.empty((B, H, seq, d), dtype=io, device=dev)
+    W, b = torch.empty((B, H, d, d), **f32), torch.empty((B, H, d), **f32)
+    mo = (torch.empty((B, H, d, d), **f32), torch.empty((B, H, d), **f32), torch.empty((B, H, d, d), **f32),
+          torch.empty((B, H, d), **f32))
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_linear_adam_fwd(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(W0), _ptr(b0), *m_in, int(step),
+                                        C.c_float(beta1), C.c_float(beta2), C.c_float(adam_eps), C.c_float(adam_lr),
+                                        _ptr(te), _ptr(lr), _ptr(gam), _ptr(bet), _ptr(out), _ptr(W), _ptr(b),
+                                        *[_ptr(t) for t in mo], stream))
+    return out, W, b, mo, step + seq // mini_batch
+
+
 def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
                             weight_ckpt, bias_ckpt, grad_output, mini_batch: int, eps: float = 1e-6,
                             checkpoint_interval: int = 1, grad_weight_out=None, grad_bias_out=None, packed_checkpoints: bool = False,
