@@ -100,3 +100,26 @@ def test_linear_adam_repeat_calls_are_identical_and_bad_arguments_are_refused(P)
     with pytest.raises(P.TttError) as e:
         run(P, to_dev(c96), 16, **HP)
     assert e.value.code == P.TTT_ERR_UNSUPPORTED
+
+
+def test_linear_adam_inner_model_with_remainder(P):
+    """FusedLinearAdam.forward over a sequence that is not a multiple of the mini-batch: the remainder is one short
+    mini-batch (inner.rs:40-47) that continues from the moments and the step count of the full ones."""
+    B, H, d, K, seq = 2, 2, 64, 16, 16 * 3 + 5
+    c = P.synthetic.reference_test_inputs(1600, B, H, seq, d, K, io_dtype=torch.float32)
+    dv = to_dev(c)
+    model = P.FusedLinearAdam(P.ModelConfig(H, d, P.TTTConfig(mini_batch_size=K)), P.TTTLinearAdamConfig(lr=5e-3),
+                              dv["W0"], dv["b0"], dv["gamma"], dv["beta"])
+    assert model.name() == "TTTLinearAdam"
+    state = model.init_state(B)
+    te_seq = c["token_eta"].repeat(seq // K + 1)[:seq]   # token_eta [seq], sliced per mini-batch (inner.rs:123-130)
+    out = model.forward(state, P.TTTInputsInner(P.Qkv(dv["xq"], dv["xk"], dv["xv"]), te_seq.to("cuda:0"), dv["lr"]))
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ro, st = orc.linear_adam_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], te_seq.double().numpy(), n["lr"],
+                                     n["gamma"], n["beta"], K=K, adam_lr=5e-3)
+    assert state.step == st["step"] == 4
+    assert_close(out, ro, 1e-4, "out")
+    W0 = np.broadcast_to(n["W0"][None], st["W"].shape)
+    assert_close(state.weight.double().cpu().numpy() - W0, st["W"] - W0, 1e-3, "W movement", min_frac=0.99)
+    assert_close(state.weight_v, st["Wv"], 1e-4, "Wv")

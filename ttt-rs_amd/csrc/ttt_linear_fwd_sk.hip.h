@@ -148,7 +148,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
         const float gr = -gneg[r];
         m[r] = __builtin_fmaf(b1, m[r], (1.f - b1) * gr);
         v[r] = __builtin_fmaf(b2, v[r], (1.f - b2) * (gr * gr));
-        const float den = __builtin_sqrtf(v[r] * ad_ic2) + adam->eps;
+        const float den = __builtin_amdgcn_sqrtf(v[r] * ad_ic2) + adam->eps;  // 1 ulp; v is far above the denormals
         x[r] = __builtin_fmaf(-(ad_a1 * m[r]), __builtin_amdgcn_rcpf(den), x[r]);
       }
     }

@@ -543,6 +543,83 @@ class FusedTileMulti:
         return self._launch(state, inputs.slice_seq(r), len(r))
 
 
+@dataclass
+class TTTLinearAdamState:
+    """linear_adam.rs:28-44: state, first and second moments (per batch element, f32) and the step counter."""
+    weight: torch.Tensor
+    bias: torch.Tensor
+    weight_m: torch.Tensor
+    bias_m: torch.Tensor
+    weight_v: torch.Tensor
+    bias_v: torch.Tensor
+    step: int = 0
+
+
+@dataclass
+class TTTLinearAdamConfig:
+    """linear_adam.rs:46-62."""
+    beta1: float = 0.9
+    beta2: float = 0.999
+    epsilon: float = 1e-8
+    lr: float = 1e-3
+
+
+class FusedLinearAdam:
+    """TTTLinearAdam (rust/core/src/linear_adam.rs) on the fused kernel: the parameters of TTTLinear, an Adam step
+    on the eta-weighted gradients per mini-batch instead of the plain update."""
+
+    def __init__(self, config: ModelConfig, adam: TTTLinearAdamConfig, weight_init, bias_init, ln_weight, ln_bias):
+        H, d = config.num_heads, config.head_dim
+        self.config, self.adam = config, adam
+        self.weight_init = _need(weight_init, (H, d, d), torch.float32, "weight_init")
+        self.bias_init = _need(bias_init, (H, d), torch.float32, "bias_init")
+        self.ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+        self.ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+
+    @staticmethod
+    def name() -> str:
+        return "TTTLinearAdam"  # linear_adam.rs:134-136
+
+    def get_config(self) -> ModelConfig:
+        return self.config
+
+    def init_state(self, batch_size: int) -> TTTLinearAdamState:
+        """linear_adam.rs:164-177: parameters repeated over the batch, zero moments, step 0."""
+        w = self.weight_init.unsqueeze(0).repeat(batch_size, 1, 1, 1)
+        b = self.bias_init.unsqueeze(0).repeat(batch_size, 1, 1)
+        return TTTLinearAdamState(w, b, torch.zeros_like(w), torch.zeros_like(b), torch.zeros_like(w),
+                                  torch.zeros_like(b), 0)
+
+    def _launch(self, state: TTTLinearAdamState, inputs: TTTInputsInner, mini_batch: int):
+        a = self.adam
+        out, w, b, mo, step = ttt_linear_adam_forward_raw(
+            inputs.qkv.xq, inputs.qkv.xk, inputs.qkv.xv, state.weight, state.bias, inputs.token_eta,
+            inputs.ttt_lr_eta, self.ln_weight, self.ln_bias, mini_batch, a.beta1, a.beta2, a.epsilon, a.lr,
+            moments=(state.weight_m, state.bias_m, state.weight_v, state.bias_v), step=state.step,
+            eps=self.config.ttt.epsilon)
+        state.weight, state.bias = w, b
+        state.weight_m, state.bias_m, state.weight_v, state.bias_v = mo
+        state.step = step
+        return out
+
+    def forward(self, state: TTTLinearAdamState, inputs: TTTInputsInner) -> torch.Tensor:
+        """inner.rs:25-50: all full mini-batches in one launch, a trailing remainder as one short mini-batch."""
+        K = self.config.ttt.mini_batch_size
+        seq = inputs.qkv.xq.shape[2]
+        full = (seq // K) * K
+        outs = []
+        if full > 0:
+            outs.append(self._launch(state, inputs.slice_seq(range(0, full)), K))
+        if full < seq:
+            outs.append(self._launch(state, inputs.slice_seq(range(full, seq)), seq - full))
+        return outs[0] if len(outs) == 1 else torch.cat(outs, 2)
+
+    def forward_mini_batch(self, state: TTTLinearAdamState, inputs: TTTInputsInner, r: range) -> torch.Tensor:
+        if len(r) > self.config.ttt.mini_batch_size or len(r) == 0:
+            raise _lib.TttError(_lib.TTT_ERR_SHAPE, "range longer than mini_batch_size")
+        return self._launch(state, inputs.slice_seq(r), len(r))
+
+
 def ttt_stack_workspace_bytes(B: int, H: int, seq: int, d: int, mini_batch: int, io: torch.dtype, mlp_flags,
                               chunk_tokens: int = 0) -> int:
     """ttt_stack_fwd_workspace_bytes for a stack whose layer l is TTT-MLP where mlp_flags[l] is true."""
