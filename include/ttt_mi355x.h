@@ -384,6 +384,22 @@ int ttt_linear_fwd_fused_inputs(const ttt_desc* desc, const void* xq, const void
                                 void* stream);
 
 /*
+ * TTT-MLP with n_hidden = 2, 3 or 4 hidden layers of width 4 d (d -> 4d -> ... -> 4d -> d, tanh-GELU between),
+ * multi-stage forward: the fused counterpart of TTTMLP2 / TTTMLP3 / TTTMLP4::forward (rust/core/src/mlp2.rs:152-243,
+ * mlp3.rs:162-279, mlp4.rs:186-324 looped as rust/core/src/inner.rs:25-50; the reference has no fused kernel for them).
+ * W0, b0: host arrays of n_hidden + 1 device pointers, weight layer i = [H,in_i,out_i] or [B,H,in_i,out_i] and
+ * [H,out_i] or [B,H,out_i] (state_per_batch selects; in_0 = out_last = d, every other side 4 d); W_out, b_out: the
+ * same shapes per batch element, also the live state during the call (W_out[i] must not alias W0[i]).
+ * Products are f32 for both I/O types.  head_dim 32 with 2 - 4 hidden layers, head_dim 64 with 2 (what fits the
+ * LDS of a CU); ttt_mlpn_supported says so beforehand.  One hidden layer is ttt_mlp_fwd.
+ */
+int ttt_mlpn_supported(const ttt_desc* desc, int n_hidden);
+int ttt_mlpn_fwd(const ttt_desc* desc, int n_hidden, const void* xq, const void* xk, const void* xv,
+                 const float* const* W0, const float* const* b0, const float* token_eta, const void* lr,
+                 const float* gamma, const float* beta, void* out, float* const* W_out, float* const* b_out,
+                 void* stream);
+
+/*
  * TTT-Linear with an Adam inner optimiser, multi-stage forward.  The fused counterpart of TTTLinearAdam::forward
  * (rust/core/src/linear_adam.rs:183-236 looped as rust/core/src/inner.rs:25-50; the reference has no fused kernel for
  * it): the mini-batch of ttt_linear_fwd with the state update W -= XK^T (eta_last G), b -= colsum(eta_last G)

@@ -19,6 +19,8 @@ reference checkout):
                       backward/stage.rs:42-1006, layer_norm.rs:428-709
   mlp_mini_batch      rust/core/src/mlp.rs:127-208
   mlp_forward         rust/core/src/inner.rs:25-50
+  mlpn_mini_batch, mlpn_forward
+                      rust/core/src/mlp2.rs:152-243, mlp3.rs:162-279, mlp4.rs:186-324 (2, 3, 4 hidden layers)
   linear_adam_mini_batch, linear_adam_forward
                       rust/core/src/linear_adam.rs:76-128 (adam_update), :183-236 (forward_mini_batch)
 
@@ -37,6 +39,8 @@ How each function is pinned (tests/test_oracle_*.py):
   mlp_mini_batch    == primal per-token GD on both layers, written in the test
   mlp_backward      == torch autograd (float64, double backward) through a torch restatement of the dual
                        form whose forward is checked against mlp_forward, plus linearity
+  mlpn_*            == mlp_mini_batch for one hidden layer; primal per-token GD on all layers (autograd through the
+                       network, written in the test) for two and three
   linear_adam_*     == the gradients of linear_mini_batch fed to torch.optim.Adam (library routine) step by step;
                        first step from zero moments moves every element by lr*g/(|g|+eps) (closed form);
                        output of a mini-batch == linear_mini_batch's (the output does not see the update)
@@ -180,6 +184,56 @@ def linear_forward(W0, b0, xq, xk, xv, token_eta, lr, gamma, beta, K=16, eps=1e-
     if checkpoint_interval:
         return out, W, b, np.stack(Wc, 2), np.stack(bc, 2)
     return out, W, b
+
+
+# --------------------------------------------------------------------------- TTT-MLP with several hidden layers
+def mlpn_mini_batch(Ws, bs, xq, xk, xv, token_eta, lr, gamma, beta, eps=1e-6):
+    """mlp2.rs:152-243 (two hidden layers), mlp3.rs:162-279 (three), mlp4.rs:186-324 (four); with one hidden layer it is
+    mlp.rs:127-208.  Ws[i] [B,H,in_i,out_i], bs[i] [B,H,out_i] for the n+1 weight layers d -> 4d -> ... -> 4d -> d.
+    Returns (out, new Ws, new bs)."""
+    n = len(Ws) - 1                                                 # hidden layers
+    k = xq.shape[2]
+    tri = np.tril(np.ones((k, k), dtype=xq.dtype))
+    x, z = [xk], []                                                 # x[i]: input of weight layer i
+    for i in range(n):                                              # mlp2.rs:162-168
+        z.append(x[i] @ Ws[i] + bs[i][:, :, None, :])
+        x.append(gelu_tanh(z[i]))
+    z.append(x[n] @ Ws[n] + bs[n][:, :, None, :])                   # :170
+    g = [None] * (n + 1)
+    g[n] = ln_l2_grad(z[n], xv - xk, _hb(gamma), _hb(beta), eps)    # :172-176
+    for i in range(n - 1, -1, -1):                                  # :178-182
+        g[i] = (g[i + 1] @ _T(Ws[i + 1])) * gelu_tanh_bwd(z[i])
+    eta = _eta(token_eta, lr)                                       # :184-187
+    xb = xq
+    for i in range(n + 1):                                          # :189-211
+        attn = (xb @ _T(x[i])) * tri
+        zb = xb @ Ws[i] - (eta * attn) @ g[i] + (bs[i][:, :, None, :] - eta @ g[i])
+        xb = gelu_tanh(zb) if i < n else zb
+    last = eta[:, :, -1, :]                                         # :213-214
+    Wn = [Ws[i] - _T(last[..., None] * x[i]) @ g[i] for i in range(n + 1)]   # :216-238
+    bn = [bs[i] - (last[..., None] * g[i]).sum(2) for i in range(n + 1)]
+    return xq + ln_fwd(xb, _hb(gamma), _hb(beta), eps), Wn, bn      # :240-242
+
+
+def mlpn_forward(Ws0, bs0, xq, xk, xv, token_eta, lr, gamma, beta, K=16, eps=1e-6, dtype=np.float64):
+    """inner.rs:25-50 over mlpn_mini_batch.  Ws0[i] [H,in,out] (or [B,H,in,out]); returns (out, Ws, bs)."""
+    xq, xk, xv, lr = (np.asarray(a, dtype=dtype) for a in (xq, xk, xv, lr))
+    gamma, beta = np.asarray(gamma, dtype=dtype), np.asarray(beta, dtype=dtype)
+    token_eta = np.asarray(token_eta, dtype=dtype)
+    B, H, seq, d = xq.shape
+    Ws = [np.asarray(a, dtype=dtype) for a in Ws0]
+    bs = [np.asarray(a, dtype=dtype) for a in bs0]
+    if Ws[0].ndim == 3:
+        Ws = [np.broadcast_to(a[None], (B,) + a.shape).copy() for a in Ws]
+        bs = [np.broadcast_to(a[None], (B,) + a.shape).copy() for a in bs]
+    out = np.zeros_like(xq)
+    for s0 in range(0, seq, K):
+        s1 = min(s0 + K, seq)
+        te = token_eta[s0:s1] if token_eta.shape[0] == seq and seq != K else token_eta[: s1 - s0]
+        o, Ws, bs = mlpn_mini_batch(Ws, bs, xq[:, :, s0:s1], xk[:, :, s0:s1], xv[:, :, s0:s1], te, lr[:, :, s0:s1],
+                                    gamma, beta, eps)
+        out[:, :, s0:s1] = o
+    return out, Ws, bs
 
 
 # --------------------------------------------------------------------------- TTT-Linear with an Adam inner optimiser

@@ -514,3 +514,74 @@ def test_linear_adam_continues_from_a_saved_state():
                                      state0={k: s1[k] for k in ("Wm", "bm", "Wv", "bv", "step")})
     np.testing.assert_array_equal(np.concatenate([o1, o2], 2), out)
     np.testing.assert_array_equal(s2["W"], st["W"])
+
+
+# ------------------------------------------------------------------ TTT-MLP with several hidden layers (MLP2/3/4)
+def primal_mlpn(Ws, bs, xq, xk, xv, te, lr, gamma, beta, K, eps=1e-6):
+    """Per-token GD on every layer of a d -> 4d -> ... -> 4d -> d network; the parameter gradients come from autograd
+    through the network itself, so nothing of the dual form (mlp2.rs) is retyped here."""
+    B, H, seq, d = xq.shape
+    n = len(Ws)
+
+    def net(x, P):
+        for i in range(n):
+            x = torch.einsum("bhi,bhio->bho", x, P[2 * i]) + P[2 * i + 1]
+            if i < n - 1:
+                x = F.gelu(x, approximate="tanh")
+        return torch.stack([F.layer_norm(x[:, h], (d,), gamma[h], beta[h], eps=eps) for h in range(H)], 1)
+
+    P = [t for pair in zip(Ws, bs) for t in pair]
+    outs = []
+    for s0 in range(0, seq, K):
+        k = min(K, seq - s0)
+        xq_, xk_, xv_, lr_ = (a[:, :, s0:s0 + k] for a in (xq, xk, xv, lr))
+        Pl = [p.detach().requires_grad_(True) for p in P]
+        g = []
+        for j in range(k):
+            loss = 0.5 * ((net(xk_[:, :, j], Pl) - (xv_[:, :, j] - xk_[:, :, j])) ** 2).sum()
+            g.append(torch.autograd.grad(loss, Pl))
+        rows = []
+        for i in range(k):
+            cur = list(P)
+            for j in range(i + 1):
+                e = te[i] * lr_[:, :, j]
+                cur = [p - e.reshape(e.shape + (1,) * (p.dim() - 2)) * g[j][a] for a, p in enumerate(cur)]
+            rows.append(xq_[:, :, i] + net(xq_[:, :, i], cur))
+        outs.append(torch.stack(rows, 2))
+        P = cur
+    return torch.cat(outs, 2), P[0::2], P[1::2]
+
+
+def make_mlpn(rng, H, d, n_hidden):
+    m = 4 * d
+    dims = [d] + [m] * n_hidden + [d]
+    Ws = [rnd(rng, H, dims[i], dims[i + 1], scale=0.3 if i == 0 else 0.15) for i in range(n_hidden + 1)]
+    bs = [rnd(rng, H, dims[i + 1], scale=0.1) for i in range(n_hidden + 1)]
+    return Ws, bs
+
+
+@pytest.mark.parametrize("n_hidden,B,H,seq,d,K", [(2, 2, 2, 8, 4, 4), (3, 1, 2, 7, 4, 4), (4, 1, 1, 4, 4, 4)])
+def test_mlpn_dual_form_equals_primal_gd(n_hidden, B, H, seq, d, K):
+    rng = np.random.default_rng(60 + n_hidden)
+    c = make_linear_case(61 + n_hidden, B, H, seq, d, K)
+    Ws, bs = make_mlpn(rng, H, d, n_hidden)
+    t = {k: torch.tensor(v) for k, v in c.items()}
+    ex = lambda a: torch.tensor(a)[None].expand((B,) + a.shape)
+    ro, rW, rb = primal_mlpn([ex(w) for w in Ws], [ex(b) for b in bs], t["xq"], t["xk"], t["xv"], t["te"], t["lr"],
+                             t["gamma"], t["beta"], K)
+    out, W, b = orc.mlpn_forward(Ws, bs, c["xq"], c["xk"], c["xv"], c["te"], c["lr"], c["gamma"], c["beta"], K=K)
+    np.testing.assert_allclose(out, ro.numpy(), rtol=1e-8, atol=1e-10)
+    for i in range(n_hidden + 1):
+        np.testing.assert_allclose(W[i], rW[i].numpy(), rtol=1e-8, atol=1e-10)
+        np.testing.assert_allclose(b[i], rb[i].numpy(), rtol=1e-8, atol=1e-10)
+
+
+def test_mlpn_with_one_hidden_layer_is_the_mlp():
+    rng = np.random.default_rng(70)
+    B, H, seq, d, K = 2, 2, 12, 8, 4
+    c = make_linear_case(71, B, H, seq, d, K)
+    Ws, bs = make_mlpn(rng, H, d, 1)
+    a = orc.mlp_forward(Ws[0], bs[0], Ws[1], bs[1], c["xq"], c["xk"], c["xv"], c["te"], c["lr"], c["gamma"], c["beta"], K=K)
+    out, W, b = orc.mlpn_forward(Ws, bs, c["xq"], c["xk"], c["xv"], c["te"], c["lr"], c["gamma"], c["beta"], K=K)
+    for x, y in zip(a, (out, W[0], b[0], W[1], b[1])):
+        np.testing.assert_allclose(y, x, rtol=1e-12, atol=1e-13)

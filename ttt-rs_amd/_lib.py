@@ -22,7 +22,7 @@ EXPORTS = (
     "ttt_linear_best_checkpoint_format",
     "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
-    "ttt_mlp_fwd_lost_workgroups", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue", "ttt_linear_fwd_fused_inputs_supported", "ttt_linear_fwd_fused_inputs", "ttt_linear_adam_supported", "ttt_linear_adam_fwd", "ttt_selftest_mfma_mixed",
+    "ttt_mlp_fwd_lost_workgroups", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue", "ttt_linear_fwd_fused_inputs_supported", "ttt_linear_fwd_fused_inputs", "ttt_linear_adam_supported", "ttt_linear_adam_fwd", "ttt_mlpn_supported", "ttt_mlpn_fwd", "ttt_selftest_mfma_mixed",
 )
 
 
@@ -84,6 +84,8 @@ def lib() -> C.CDLL:
         L.ttt_stack_fwd.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), vp, vp, vp, C.c_int32, vp, vp]
         L.ttt_inner_inputs.argtypes = [dp] + [vp] * 5 + [C.c_float] + [vp] * 4 + [C.c_int, C.c_int] + [vp] * 6
         L.ttt_layer_epilogue.argtypes = [dp] + [vp] * 3 + [C.c_float] + [vp] * 3
+        L.ttt_mlpn_supported.argtypes = [dp, C.c_int]
+        L.ttt_mlpn_fwd.argtypes = [dp, C.c_int] + [vp] * 13
         L.ttt_linear_adam_supported.argtypes = [dp]
         L.ttt_linear_adam_fwd.argtypes = [dp] + [vp] * 9 + [C.c_int] + [C.c_float] * 4 + [vp] * 12
         L.ttt_linear_fwd_fused_inputs_supported.argtypes = [dp, C.c_int, C.c_int]

@@ -22,6 +22,7 @@
 #include "ttt_mlp_bwd.hip.h"
 #include "ttt_mlp_fwd_cl2.hip.h"
 #include "ttt_mlp_fwd_rr.hip.h"
+#include "ttt_mlpn_fwd.hip.h"
 #include "ttt_selftest.hip.h"
 
 // Scratch of ttt_mlp_bwd_static (file scope, outside any namespace so that HIP_SYMBOL names it plainly).
@@ -705,6 +706,18 @@ int dispatch_linear_fwd(const ttt_desc* d, const ttt::LinearFwdArgs* probs, int 
 }
 }  // namespace
 
+namespace {
+template <class T, int D, int NL>
+int launch_mlpn(const ttt::MlpNFwdArgs& a, hipStream_t s) {
+  constexpr auto kern = ttt::ttt_mlpn_fwd_kernel<T, D, NL>;
+  constexpr size_t bytes = ttt::MlpNLds<D, NL>::BYTES;
+  int rc = opt_in_lds<kern>(bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
+  return hip_status(hipGetLastError(), "ttt_mlpn_fwd launch");
+}
+}  // namespace
+
 extern "C" {
 
 int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
@@ -715,6 +728,54 @@ int ttt_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const void
   int rc = prepare_linear_fwd(d, xq, xk, xv, W0, b0, token_eta, lr, gamma, beta, out, W_out, b_out, W_ckpt, b_ckpt, &a);
   if (rc != TTT_OK) return rc;
   return dispatch_linear_fwd(d, &a, 1, static_cast<hipStream_t>(stream));
+}
+
+int ttt_mlpn_supported(const ttt_desc* d, int n_hidden) {
+  int rc = check_common(d);
+  if (rc != TTT_OK) return rc;
+  if (d->mini_batch > 16) return fail(TTT_ERR_UNSUPPORTED, "mini_batch %d > 16 has no kernel", d->mini_batch);
+  if (d->seq_stride != 0 && d->seq_stride != d->seq)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_mlpn_fwd: seq_stride must be 0");
+  const bool ok = (d->head_dim == 32 && n_hidden >= 2 && n_hidden <= 4) || (d->head_dim == 64 && n_hidden == 2);
+  if (!ok)
+    return fail(TTT_ERR_UNSUPPORTED,
+                "ttt_mlpn_fwd: head_dim 32 with 2, 3 or 4 hidden layers, head_dim 64 with 2 (got head_dim %d, %d hidden "
+                "layers; one hidden layer is ttt_mlp_fwd)", d->head_dim, n_hidden);
+  return TTT_OK;
+}
+
+int ttt_mlpn_fwd(const ttt_desc* d, int n_hidden, const void* xq, const void* xk, const void* xv,
+                 const float* const* W0, const float* const* b0, const float* token_eta, const void* lr,
+                 const float* gamma, const float* beta, void* out, float* const* W_out, float* const* b_out,
+                 void* stream) {
+  int rc = ttt_mlpn_supported(d, n_hidden);
+  if (rc != TTT_OK) return rc;
+  if (!xq || !xk || !xv || !W0 || !b0 || !token_eta || !lr || !gamma || !beta || !out || !W_out || !b_out)
+    return fail(TTT_ERR_NULL, "ttt_mlpn_fwd: a required pointer is NULL");
+  ttt::MlpNFwdArgs a;
+  for (int i = 0; i < ttt::kMlpNMaxLayers; ++i) {
+    a.W0[i] = a.b0[i] = nullptr;
+    a.W[i] = a.b[i] = nullptr;
+  }
+  for (int i = 0; i <= n_hidden; ++i) {
+    if (!W0[i] || !b0[i] || !W_out[i] || !b_out[i])
+      return fail(TTT_ERR_NULL, "ttt_mlpn_fwd: layer %d: a required pointer is NULL", i);
+    if (W_out[i] == W0[i])
+      return fail(TTT_ERR_SHAPE, "ttt_mlpn_fwd: W_out[%d] is the live state and must not alias W0[%d]", i, i);
+    a.W0[i] = W0[i]; a.b0[i] = b0[i]; a.W[i] = W_out[i]; a.b[i] = b_out[i];
+  }
+  a.xq = xq; a.xk = xk; a.xv = xv; a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
+  a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch; a.n_stages = d->seq / d->mini_batch;
+  a.state_per_batch = d->state_per_batch ? 1 : 0;
+  a.eps = d->eps;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool f32 = d->io_dtype == TTT_F32;
+  if (d->head_dim == 64) return f32 ? launch_mlpn<ttt::F32, 64, 2>(a, s) : launch_mlpn<ttt::BF16, 64, 2>(a, s);
+  switch (n_hidden) {
+    case 2: return f32 ? launch_mlpn<ttt::F32, 32, 2>(a, s) : launch_mlpn<ttt::BF16, 32, 2>(a, s);
+    case 3: return f32 ? launch_mlpn<ttt::F32, 32, 3>(a, s) : launch_mlpn<ttt::BF16, 32, 3>(a, s);
+    default: return f32 ? launch_mlpn<ttt::F32, 32, 4>(a, s) : launch_mlpn<ttt::BF16, 32, 4>(a, s);
+  }
 }
 
 int ttt_linear_adam_supported(const ttt_desc* d) {

@@ -319,6 +319,41 @@ def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_we
     return (out, *o)
 
 
+def ttt_mlpn_forward_raw(xq, xk, xv, weights, biases, token_eta, ttt_lr_eta, ln_weight, ln_bias, mini_batch: int,
+                         eps: float = 1e-6):
+    """One call of ttt_mlpn_fwd on the current stream: TTTMLP2/3/4::forward (rust/core/src/mlp2.rs, mlp3.rs, mlp4.rs
+    looped as rust/core/src/inner.rs:25-50).  weights / biases: lists of the n_hidden + 1 layers, [H,in,out] / [H,out] or
+    with a leading batch dimension.  Returns (output, weights_out, biases_out), state per batch element."""
+    B, H, seq, d = xq.shape
+    io = xq.dtype
+    n_hidden = len(weights) - 1
+    m = 4 * d
+    dims = [d] + [m] * n_hidden + [d]
+    xq = _need(xq, (B, H, seq, d), io, "xq")
+    xk = _need(xk, (B, H, seq, d), io, "xk")
+    xv = _need(xv, (B, H, seq, d), io, "xv")
+    per_batch = weights[0].dim() == 4
+    lead = (B, H) if per_batch else (H,)
+    Ws = [_need(w, lead + (dims[i], dims[i + 1]), torch.float32, f"weights[{i}]") for i, w in enumerate(weights)]
+    bs = [_need(b, lead + (dims[i + 1],), torch.float32, f"biases[{i}]") for i, b in enumerate(biases)]
+    te = _need(token_eta[:mini_batch], (mini_batch,), torch.float32, "token_eta")
+    lr = _need(ttt_lr_eta, (B, H, seq), io, "ttt_lr_eta")
+    gam = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+    bet = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+    dev = xq.device
+    desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), 1 if per_batch else 0, 0, 0, 0)
+    check(lib().ttt_mlpn_supported(C.byref(desc), n_hidden))
+    out = torch.empty((B, H, seq, d), dtype=io, device=dev)
+    Wo = [torch.empty((B, H, dims[i], dims[i + 1]), dtype=torch.float32, device=dev) for i in range(n_hidden + 1)]
+    bo = [torch.empty((B, H, dims[i + 1]), dtype=torch.float32, device=dev) for i in range(n_hidden + 1)]
+    arr = lambda ts: (C.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    with torch.cuda.device(dev):
+        check(lib().ttt_mlpn_fwd(C.byref(desc), n_hidden, _ptr(xq), _ptr(xk), _ptr(xv), arr(Ws), arr(bs), _ptr(te),
+                                 _ptr(lr), _ptr(gam), _ptr(bet), _ptr(out), arr(Wo), arr(bo), stream))
+    return out, Wo, bo
+
+
 def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias, d_out,
                          mini_batch: int, eps: float = 1e-6, d_state_out=None, static_scratch: bool = False,
                          into=None):
