@@ -132,3 +132,44 @@ def test_stack_wavefront_replays(P, streams):
         return res
 
     replay_and_compare(calls, calls, refresh)
+
+
+def test_other_forwards_replay(P):
+    """The forward on the projections, the Adam forward and the forward of a TTT-MLP with two hidden layers, recorded
+    together in one graph: each enqueues one kernel and nothing else."""
+    print("case graph capture fused inputs + adam + mlp2", flush=True)
+    B, H, d, K, N = 2, 2, 32, 16, 4
+    seq = N * K
+    dt = torch.bfloat16
+    gen = torch.Generator().manual_seed(21)
+    sets = [to_dev(P.synthetic.reference_test_inputs(950 + i, B, H, seq, d, K, io_dtype=dt)) for i in range(4)]
+    raws = [dict(q=torch.randn(B, seq, H, d, generator=gen).to(dt).to("cuda:0"),
+                 k=torch.randn(B, seq, H, d, generator=gen).to(dt).to("cuda:0"),
+                 v=torch.randn(B, seq, H, d, generator=gen).to(dt).to("cuda:0"),
+                 lg=torch.randn(B, seq, H, generator=gen).to(dt).to("cuda:0")) for _ in range(4)]
+    dims = [d, 4 * d, 4 * d, d]
+    Ws = [(torch.randn(H, dims[i], dims[i + 1], generator=gen) * 0.02).to("cuda:0") for i in range(3)]
+    bs = [(torch.randn(H, dims[i + 1], generator=gen) * 0.02).to("cuda:0") for i in range(3)]
+    bias = torch.zeros(H, device="cuda:0")
+    tidx = (1.0 / torch.arange(1, K + 1, dtype=torch.float32)).to("cuda:0")
+    ltidx = torch.zeros(K, device="cuda:0")
+    rope = P.rope_cos_sin(K, 0, None, d, "cuda:0")
+    x = {k: v.clone() for k, v in sets[0].items()}
+    r = {k: v.clone() for k, v in raws[0].items()}
+
+    def refresh(i):
+        for k in x:
+            x[k].copy_(sets[i][k])
+        for k in r:
+            r[k].copy_(raws[i][k])
+
+    def calls():
+        f = P.ttt_linear_forward_fused_inputs_raw(r["q"], r["k"], r["v"], r["lg"], bias, 0.8, tidx, ltidx, x["W0"], x["b0"],
+                                                  x["gamma"], x["beta"], K, rope=rope, pos_offset=0, pos_wrap=K)
+        a = P.ttt_linear_adam_forward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"], x["gamma"],
+                                          x["beta"], K)
+        m = P.ttt_mlpn_forward_raw(x["xq"], x["xk"], x["xv"], Ws, bs, x["token_eta"], x["lr"], x["gamma"], x["beta"], K)
+        return {"fused out": f[0], "fused W": f[1], "adam out": a[0], "adam W": a[1], "adam Wv": a[3][2],
+                "mlp2 out": m[0], "mlp2 W2": m[1][1], "mlp2 b3": m[2][2]}
+
+    replay_and_compare(calls, calls, refresh)
