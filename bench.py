@@ -505,10 +505,14 @@ def run_workload(name, a, pkg, torch):
         # (56 + 14*8 + 7*8) d^2 flop per token-head, K-sized terms aside.  The backward's own forward sweep (the
         # register-resident forward once more for bf16 I/O up to head_dim 96) is overhead, not algorithmic work.
         flops = th * (224 * d * d)
-        out["dtype"] = "f32"
+        # bf16 I/O up to head_dim 96: every product of the scan takes bf16 operands (f32 accumulation, f32 state and
+        # gradient accumulators in memory); otherwise true-f32 products
+        bf = io == "bf16" and d <= 96
+        peak = BF16_MFMA_PEAK_TF if bf else F32_MFMA_PEAK_TF
+        out["dtype"] = "bf16" if bf else "f32"
         out["config"]["inner_model"] = "TTT-MLP"
-        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": F32_MFMA_PEAK_TF,
-                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / F32_MFMA_PEAK_TF, **counters,
+        out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": peak,
+                           "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / peak, **counters,
                            "kernel": "ttt_mlp_fwd_rr_kernel (forward, and again as the backward's sweep) + ttt_mlp_bwd_kernel (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     else:

@@ -103,6 +103,11 @@ typedef struct ttt_desc {
  * library's choice up to 256 units).  Same results bit for bit.  Ignored where only one of the two exists. */
 #define TTT_HINT_OWN_LOADS 0x1000
 #define TTT_HINT_ALL_LOADS 0x2000
+/* ttt_mlp_bwd / ttt_mlp_bwd_static, bf16 I/O up to head_dim 96: the reverse scan normally rounds the operands of its
+ * products to bf16, as the forward of the step did (f32 accumulation, f32 state and gradient accumulators);
+ * TTT_HINT_F32_PRODUCTS keeps every product of the scan in f32 (about twice the time).  Ignored elsewhere: f32 I/O and
+ * head_dim 128 always compute in f32. */
+#define TTT_HINT_F32_PRODUCTS 0x4000
 /* Testing only: the two workgroups that share a (batch, head) unit in ttt_mlp_fwd at head_dim 128 (bf16 I/O) give
  * up waiting for each other at once, as if the partner had never become resident.  Exercises the failure path
  * described at ttt_mlp_fwd: every output of the affected units is NaN.  All kernels still run to their end. */

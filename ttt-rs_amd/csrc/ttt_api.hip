@@ -407,9 +407,9 @@ int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
   return hip_status(hipGetLastError(), "ttt_linear_bwd (multi-wave register-resident kernel) launch");
 }
 
-template <class T, int D>
+template <class T, int D, bool BF = false>
 int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_mlp_bwd_kernel<T, D>;
+  constexpr auto kern = ttt::ttt_mlp_bwd_kernel<T, D, BF>;
   constexpr size_t bytes = ttt::MlpBwdLds<D>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
@@ -603,6 +603,13 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   a.d_lr = d_lr; a.d_token_eta = d_token_eta; a.d_gamma = d_gamma; a.d_beta = d_beta;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
   a.seq_stride = fa.seq_stride; a.n_stages = fa.n_stages; a.eps = d->eps;
+  // behind the register-resident sweep the scan takes bf16 operands too (the states it walks back through were
+  // formed from bf16 operands); TTT_HINT_F32_PRODUCTS keeps the scan's products in f32
+  if (rr_sweep && !(d->kernel_hint & TTT_HINT_F32_PRODUCTS)) switch (d->head_dim) {
+      case 32: return launch_mlp_bwd<ttt::BF16, 32, true>(a, s);
+      case 64: return launch_mlp_bwd<ttt::BF16, 64, true>(a, s);
+      default: return launch_mlp_bwd<ttt::BF16, 96, true>(a, s);
+    }
   switch (d->head_dim) {
     case 32: return f32 ? launch_mlp_bwd<ttt::F32, 32>(a, s) : launch_mlp_bwd<ttt::BF16, 32>(a, s);
     case 64: return f32 ? launch_mlp_bwd<ttt::F32, 64>(a, s) : launch_mlp_bwd<ttt::BF16, 64>(a, s);

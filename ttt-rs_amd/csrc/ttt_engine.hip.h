@@ -32,7 +32,19 @@ __device__ __forceinline__ f32x4 rows_to_operand(const f32x4& v, int lane) {
   return o;
 }
 
-// C[16*Mt x 16*Nt] (row-major, stride ldc)  op=  A * B over k in [k0, k0+Kd), Kd a multiple of 4.
+// One 16-deep step of a product: lane (c, g) holds four k slots of A (row c) and of B (column c).  BF: the operands
+// are rounded to bf16 and take one v_mfma_f32_16x16x16_bf16 (a quarter of the issue slots of the f32 form at an
+// eighth of the matrix-pipe time); otherwise four true-f32 v_mfma_f32_16x16x4_f32.  The accumulator is f32 either way.
+// A kernel uses ONE of the two forms throughout, so no matrix instruction ever follows one of another opcode.
+template <bool BF>
+__device__ __forceinline__ void mma16(f32x4& acc, const f32x4& a, const f32x4& b) {
+  if constexpr (BF)
+    Io<BF16>::mma(acc, Io<BF16>::to_frag(a), Io<BF16>::to_frag(b));
+  else
+    Io<F32>::mma(acc, a, b);
+}
+
+// C[16*Mt x 16*Nt] (row-major, stride ldc)  op=  A * B over k in [k0, k0+Kd), Kd a multiple of 4 (of 16 with BF).
 // A(m,k) = A[m*a_rs + k*a_cs], B(k,n) = B[k*b_rs + n*b_cs].
 // MODE 0: C = AB   1: C += AB   2: C -= AB   3: C *= AB (elementwise)
 //
@@ -42,10 +54,12 @@ __device__ __forceinline__ f32x4 rows_to_operand(const f32x4& v, int lane) {
 // before the first MFMA of the group issues, so the loads of a group overlap its MFMAs.
 // BG: B is in global memory and contiguous along k (a transposed weight matrix): loaded four lanes to a row and
 // exchanged between lanes before use (load_rows_raw / rows_to_operand).
-template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false>
-__device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_rs, int a_cs,
-                                       const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
-                                       int wave, int lane, int first = 0, int k0 = 0) {
+// BF: bf16 operands (mma16); the k-steps outside the contiguous-A path are then taken four at a time.
+template <bool BF, int MODE, int NW, int NB, int KU0, bool BG>
+__device__ __forceinline__ void mm_lds_t(float* C, int ldc, const float* A, int a_rs, int a_cs,
+                                         const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
+                                         int wave, int lane, int first, int k0) {
+  constexpr int KU = BF ? ((KU0 + 3) / 4) * 4 : KU0;
   const int c = lane & 15, g = lane >> 4;
   const int nblk = (Nt + NB - 1) / NB;
   const int njobs = Mt * nblk;
@@ -88,11 +102,21 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
       }
     };
     auto fma_group = [&](const float (&av)[KU], const float (&bv)[KU][NB]) {
+      if constexpr (BF) {
 #pragma unroll
-      for (int u = 0; u < KU; ++u)
+        for (int u = 0; u < KU; u += 4) {
+          const auto af = Io<BF16>::to_frag(f32x4{av[u], av[u + 1], av[u + 2], av[u + 3]});
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
-          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u][j], acc[j], 0, 0, 0);
+          for (int j = 0; j < NB; ++j)
+            Io<BF16>::mma(acc[j], af, Io<BF16>::to_frag(f32x4{bv[u][j], bv[u + 1][j], bv[u + 2][j], bv[u + 3][j]}));
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < KU; ++u)
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u][j], acc[j], 0, 0, 0);
+      }
     };
     constexpr int KG = 4 * KU;
     // Operand A contiguous along k (rows 16-byte aligned): the k values of a 16-deep step are re-assigned so
@@ -123,10 +147,16 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
         return v;
       };
       auto step = [&](const f32x4& av, const f32x4 (&bv)[NB]) {
+        if constexpr (BF) {
+          const auto af = Io<BF16>::to_frag(av);
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+          for (int j = 0; j < NB; ++j) Io<BF16>::mma(acc[j], af, Io<BF16>::to_frag(bv[j]));
+        } else {
 #pragma unroll
-          for (int j = 0; j < NB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[r], bv[j][r], acc[j], 0, 0, 0);
+          for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int j = 0; j < NB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[r], bv[j][r], acc[j], 0, 0, 0);
+        }
       };
       // PF 16-deep steps of operands are in flight at any time (a ring of PF register buffers, refilled
       // right after use): the operands come from global memory, and with one step in flight a product
@@ -202,13 +232,33 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
       if (gi < ngroups) fma_group(avA, bvA);
       k = ngroups * KG;
     }
+    if constexpr (BF) {
 #pragma nounroll
-    for (; k < Kd; k += 4) {
-      const float av = A[aoff + k * a_cs];
+      for (; k < Kd; k += 16) {
+        f32x4 av, bv[NB];
 #pragma unroll
-      for (int j = 0; j < NB; ++j) {
-        const float bv = (tn0 + j < Nt) ? B[boff + k * b_rs + j * bcol] : 0.f;
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[j], 0, 0, 0);
+        for (int u = 0; u < 4; ++u) {
+          av[u] = A[aoff + (k + 4 * u) * a_cs];
+#pragma unroll
+          for (int j = 0; j < NB; ++j) {
+            const bool live = Nt % NB == 0 || tn0 + j < Nt;
+            const float v = B[boff + (k + 4 * u) * b_rs + (live ? j : 0) * bcol];
+            bv[j][u] = live ? v : 0.f;
+          }
+        }
+        const auto af = Io<BF16>::to_frag(av);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) Io<BF16>::mma(acc[j], af, Io<BF16>::to_frag(bv[j]));
+      }
+    } else {
+#pragma nounroll
+      for (; k < Kd; k += 4) {
+        const float av = A[aoff + k * a_cs];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          const float bv = (tn0 + j < Nt) ? B[boff + k * b_rs + j * bcol] : 0.f;
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[j], 0, 0, 0);
+        }
       }
     }
 #pragma unroll
@@ -224,6 +274,13 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
       }
     }
   }
+}
+
+template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false>
+__device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_rs, int a_cs,
+                                       const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
+                                       int wave, int lane, int first = 0, int k0 = 0) {
+  mm_lds_t<false, MODE, NW, NB, KU, BG>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, Kd, wave, lane, first, k0);
 }
 
 // Rank-K update of a matrix in global memory, K = 4 * KS small (16, 32, 48):
@@ -257,11 +314,13 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
 // sets then live in per-lane scratch memory and are addressed with the loop-carried parity), i.e. the failure was
 // in code generated for that form, which is why it is not used.  The head_dim-128 instance (256 VGPRs, a handful of
 // registers spilled outside the loops) is held by a test that runs it three times and asks for identical bits.
-template <int MODE, int NW, int NB, int KS, bool FZ = false>
-__device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
-                                        int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
-                                        const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
+// BF: bf16 operands, four k-steps per matrix instruction (mma16).
+template <bool BF, int MODE, int NW, int NB, int KS, bool FZ>
+__device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
+                                          int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
+                                          const float* X, int x_rs, float* Z, int ldz) {
   static_assert(MODE == 1 || MODE == 2, "read-modify-write modes only");
+  static_assert(!BF || KS % 4 == 0, "bf16 operands: whole 16-deep steps");
   const int c = lane & 15, g = lane >> 4;
   const int nblk = Nt / NB, njobs = Mt * nblk;
   f32x4 zacc[NB];
@@ -306,21 +365,40 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
 #pragma unroll
       for (int u = 0; u < KS; ++u) s.av[u] = -s.av[u];
     }
+    if constexpr (BF) {
 #pragma unroll
-    for (int u = 0; u < KS; ++u)
+      for (int u = 0; u < KS; u += 4) {
+        const auto af = Io<BF16>::to_frag(f32x4{s.av[u], s.av[u + 1], s.av[u + 2], s.av[u + 3]});
 #pragma unroll
-      for (int j = 0; j < NB; ++j)
-        s.acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(s.av[u], bfix ? bf[u][j] : s.bv[u][j], s.acc[j], 0, 0, 0);
+        for (int j = 0; j < NB; ++j) {
+          const f32x4 b4 = bfix ? f32x4{bf[u][j], bf[u + 1][j], bf[u + 2][j], bf[u + 3][j]}
+                                : f32x4{s.bv[u][j], s.bv[u + 1][j], s.bv[u + 2][j], s.bv[u + 3][j]};
+          Io<BF16>::mma(s.acc[j], af, Io<BF16>::to_frag(b4));
+        }
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < KS; ++u)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          s.acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(s.av[u], bfix ? bf[u][j] : s.bv[u][j], s.acc[j], 0, 0, 0);
+    }
 #pragma unroll
     for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) C[coff + r * ldc + 16 * j] = s.acc[j][r];
     if (FZ) {
       const f32x4 xv = *reinterpret_cast<const f32x4*>(X + c * x_rs + 16 * tm + 4 * g);
+      if constexpr (BF) {
+        const auto xf = Io<BF16>::to_frag(xv);
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
+        for (int j = 0; j < NB; ++j) Io<BF16>::mma(zacc[j], xf, Io<BF16>::to_frag(s.acc[j]));
+      } else {
 #pragma unroll
-        for (int j = 0; j < NB; ++j) zacc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[r], s.acc[j][r], zacc[j], 0, 0, 0);
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int j = 0; j < NB; ++j) zacc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[r], s.acc[j][r], zacc[j], 0, 0, 0);
+      }
     }
   };
   int job = wave;
@@ -350,6 +428,13 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
   }
 }
 
+template <int MODE, int NW, int NB, int KS, bool FZ = false>
+__device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
+                                        int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
+                                        const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
+  mm_rank_t<false, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz);
+}
+
 // C[16 x 16*NT] (LDS, row stride ldc) op= A[16 x Kd] * B[Kd x 16*NT] with Kd = NW * 16 * KSTEPS split over the waves:
 // wave w takes k in [w*16*KSTEPS, (w+1)*16*KSTEPS) for ALL NT tile columns, leaves its partial product in
 // part[w] (LDS, NW tiles of 16 rows, stride ldc), and after a barrier the partials are summed in wave order
@@ -358,9 +443,9 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
 // element of A is fetched once instead of NT times, all NW waves work, and every operand of a wave is requested
 // before its first matrix instruction.  Contains a barrier: call from all threads; the caller's next barrier
 // publishes C.
-template <int MODE, int NW, int NT, int KSTEPS>
-__device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const float* A, int a_rs, const float* B,
-                                          int b_rs, int b_cs, int wave, int lane, int tid) {
+template <bool BF, int MODE, int NW, int NT, int KSTEPS>
+__device__ __forceinline__ void mm_splitk_t(float* C, int ldc, float* part, const float* A, int a_rs, const float* B,
+                                            int b_rs, int b_cs, int wave, int lane, int tid) {
   const int c = lane & 15, g = lane >> 4;
   const int kw = wave * 16 * KSTEPS, k0 = kw + 4 * g;
   const bool vecB = b_rs == 1 && (b_cs & 3) == 0;
@@ -392,12 +477,21 @@ __device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const 
   f32x4 acc[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if constexpr (BF) {
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s)
+    for (int s = 0; s < KSTEPS; ++s) {
+      const auto af = Io<BF16>::to_frag(av[s]);
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+      for (int j = 0; j < NT; ++j) Io<BF16>::mma(acc[j], af, Io<BF16>::to_frag(bv[s][j]));
+    }
+  } else {
 #pragma unroll
-      for (int j = 0; j < NT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s][r], bv[s][j][r], acc[j], 0, 0, 0);
+    for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s][r], bv[s][j][r], acc[j], 0, 0, 0);
+  }
   float* mine = part + wave * 16 * ldc;
 #pragma unroll
   for (int j = 0; j < NT; ++j)
@@ -412,6 +506,12 @@ __device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const 
     float* pc = C + row * ldc + col;
     *pc = MODE == 0 ? v : MODE == 1 ? *pc + v : *pc - v;
   }
+}
+
+template <int MODE, int NW, int NT, int KSTEPS>
+__device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const float* A, int a_rs, const float* B,
+                                          int b_rs, int b_cs, int wave, int lane, int tid) {
+  mm_splitk_t<false, MODE, NW, NT, KSTEPS>(C, ldc, part, A, a_rs, B, b_rs, b_cs, wave, lane, tid);
 }
 
 // Sum over r of p[r * stride] (+ q[r * stride]), r = 0..15, with all loads issued before the first add: written as

@@ -18,7 +18,8 @@
 // Data placement: [16 x d] tiles, the [16 x 16] causal matrices, biases and their gradients live
 // in LDS; the [16 x 4d] tiles, the rolling state and the gradient accumulators dW1, dW2 live in
 // global memory (caller's workspace / output buffers, an L2-resident working set) and are read
-// in place as MFMA operands.  All contractions are true-f32 MFMA for both I/O dtypes.
+// in place as MFMA operands.  Contractions are true-f32 MFMA, or (template flag BF) bf16-operand MFMA with f32
+// accumulation; the state, the gradient accumulators and every tile stay f32 in memory either way.
 #pragma once
 #include "ttt_engine_fwd.hip.h"
 
@@ -76,6 +77,29 @@ struct MlpBwdLds {
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
 
+// The tile engine's products with the operand type fixed for a whole kernel instantiation: BF = operands rounded to
+// bf16 (one v_mfma_f32_16x16x16_bf16 per 16-deep step), otherwise true f32.  Accumulation is f32 in both.
+template <bool BF>
+struct MlpBwdEng {
+  template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false>
+  static __device__ __forceinline__ void lds(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
+                                             int b_rs, int b_cs, int Mt, int Nt, int Kd, int wave, int lane,
+                                             int first = 0, int k0 = 0) {
+    mm_lds_t<BF, MODE, NW, NB, KU, BG>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, Kd, wave, lane, first, k0);
+  }
+  template <int MODE, int NW, int NB, int KS, bool FZ = false>
+  static __device__ __forceinline__ void rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
+                                              int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
+                                              const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
+    mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz);
+  }
+  template <int MODE, int NW, int NT, int KSTEPS>
+  static __device__ __forceinline__ void splitk(float* C, int ldc, float* part, const float* A, int a_rs,
+                                                const float* B, int b_rs, int b_cs, int wave, int lane, int tid) {
+    mm_splitk_t<BF, MODE, NW, NT, KSTEPS>(C, ldc, part, A, a_rs, B, b_rs, b_cs, wave, lane, tid);
+  }
+};
+
 // tanh-GELU with first and second derivative
 __device__ __forceinline__ void gelu_tanh_all(float x, float& y, float& dy, float& ddy) {
   const float c = 0.7978845608f, a = 0.044715f;
@@ -86,13 +110,17 @@ __device__ __forceinline__ void gelu_tanh_all(float x, float& y, float& dy, floa
   ddy = s * du + 0.5f * x * s * (ddu - 2.f * t * du * du);
 }
 
-template <class T, int D>
+// BF: every product takes its operands rounded to bf16 (bf16 I/O behind the register-resident forward sweep, whose
+// own products and state updates took bf16 operands: the states the scan walks back through are the ones that
+// sweep formed).  Otherwise all contractions are true-f32 MFMA.
+template <class T, int D, bool BF = false>
 // One workgroup per CU (the LDS use decides that), two waves per SIMD: said explicitly, because the scheduler
 // otherwise aims at a higher occupancy and, to save registers, issues independent loads one at a time.
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = MlpBwdLds<D>;
+  using E = MlpBwdEng<BF>;
   constexpr int M = L::M, LD = L::LD, LK = L::LK;
   constexpr int NW = 8, GW = 32, NJD = D / GW, NJM = M / GW, NTD = D / 16, NTM = M / 16;
   constexpr int NBM = NTM / NW;  // [16 x 4d] products: one job of NBM tile columns per wave
@@ -158,8 +186,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       const f32x4 xo = rows_to_operand(xa[s], lane), yo = rows_to_operand(ya[s], lane);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xo[r], yo[r], acc, 0, 0, 0);
+      mma16<BF>(acc, xo, yo);
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) lds[L::PART + wave * 256 + (4 * g + r) * 16 + c] = acc[r];
@@ -189,9 +216,9 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   auto prod_k = [&](auto mode, float* C, const float* A, const float* B, int b_rs, int b_cs) {
     constexpr int MODE = decltype(mode)::value;
     if constexpr (L::SPLITK)
-      mm_splitk<MODE, NW, NTD, M / (16 * NW)>(C, LD, lds + L::SKP, A, M, B, b_rs, b_cs, wave, lane, tid);
+      E::template splitk<MODE, NW, NTD, M / (16 * NW)>(C, LD, lds + L::SKP, A, M, B, b_rs, b_cs, wave, lane, tid);
     else
-      mm_lds<MODE, NW>(C, LD, A, M, 1, B, b_rs, b_cs, 1, NTD, M, wave, lane);
+      E::template lds<MODE, NW>(C, LD, A, M, 1, B, b_rs, b_cs, 1, NTD, M, wave, lane);
   };
   using M0 = std::integral_constant<int, 0>;
   using M1 = std::integral_constant<int, 1>;
@@ -223,7 +250,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     const float last = te_last * slr[t];
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
     // Z1 = XK W1 (step 3) rides along on the rolled-back tiles
-    mm_rank<1, NW, NBM, 4, true>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M);
+    E::template rank<1, NW, NBM, 4, true>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M);
     if (tid < M) sb1[tid] += col16_sum(G1l + tid, M);
     __syncthreads();
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
@@ -241,12 +268,12 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 4. roll W2, b2 back
-    mm_rank<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, wave, lane);
+    E::template rank<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, wave, lane);
     if (tid < D) sb2[tid] += col16_sum(G2l + tid, D);
     __syncthreads();
     // ---- 5. Z2 = X2 W2 ; A1 = XQ XK^T ; eta
     prod_k(M0{}, lds + L::XH, mX2, W2, D, 1);
-    mm_lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, NTD % NW);
+    E::template lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, NTD % NW);
     if (tid < 256) {
       const int tt = tid >> 4, s = tid & 15;
       lds[L::ETA + tt * LK + s] = (s <= tt) ? ste[tt] * slr[s] : 0.f;
@@ -279,8 +306,8 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 7. U = G2 W2^T ; Zbar1 = XQ W1
-    mm_lds<0, NW, NBM, 2, true>(mU, M, lds + L::G2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
-    mm_lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
+    E::template lds<0, NW, NBM, 2, true>(mU, M, lds + L::G2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    E::template lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 8. G1 = U gelu'(Z1)
     {
@@ -297,7 +324,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 9. Zbar1 -= M1 G1 ; then + b1, Xbar2 = gelu
-    mm_lds<2, NW, NBM, 4>(mZB1, M, lds + L::M1, LK, 1, mG1, M, 1, 1, NTM, 16, wave, lane);
+    E::template lds<2, NW, NBM, 4>(mZB1, M, lds + L::M1, LK, 1, mG1, M, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
     {
       float z[NJM], y[NJM];
@@ -321,7 +348,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       lds[L::M2 + tt * LK + s] = lds[L::ETA + tt * LK + s] * (1.f + part_sum(tt, s));
     }
     __syncthreads();
-    mm_lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M2, LK, 1, lds + L::G2, LD, 1, 1, NTD, 16, wave, lane);
+    E::template lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M2, LK, 1, lds + L::G2, LD, 1, 1, NTD, 16, wave, lane);
     __syncthreads();
     // ---- 11. output LayerNorm backward: dZbar2
     {
@@ -344,8 +371,8 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 12. P2 = dZbar2 G2^T ; dXbar2 = dZbar2 W2^T ; S2 = X2 dW2
-    mm_lds<0, NW>(lds + L::P, LK, lds + L::DZB2, LD, 1, lds + L::G2, 1, LD, 1, 1, D, wave, lane, NW - 1);
-    mm_lds<0, NW, NBM, 2, true>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    E::template lds<0, NW>(lds + L::P, LK, lds + L::DZB2, LD, 1, lds + L::G2, 1, LD, 1, 1, D, wave, lane, NW - 1);
+    E::template lds<0, NW, NBM, 2, true>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     prod_k(M0{}, lds + L::DG2, mX2, dW2, D, 1);
     __syncthreads();
     // ---- 13. dA2, d eta ; dG2 = -last (S2 + db2) ; d last
@@ -371,12 +398,12 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 14. dXbar2 += dA2 X2 ; dG2 -= M2^T dZbar2 ; dX2 = dA2^T Xbar2
-    mm_lds<1, NW, NBM, 4>(mDXB, M, lds + L::DA, LK, 1, mX2, M, 1, 1, NTM, 16, wave, lane);
-    mm_lds<2, NW, 1, 4>(lds + L::DG2, LD, lds + L::M2, 1, LK, lds + L::DZB2, LD, 1, 1, NTD, 16, wave, lane);
-    mm_lds<0, NW, NBM, 4>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
+    E::template lds<1, NW, NBM, 4>(mDXB, M, lds + L::DA, LK, 1, mX2, M, 1, 1, NTM, 16, wave, lane);
+    E::template lds<2, NW, 1, 4>(lds + L::DG2, LD, lds + L::M2, 1, LK, lds + L::DZB2, LD, 1, 1, NTD, 16, wave, lane);
+    E::template lds<0, NW, NBM, 4>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
     // ---- 15. dX2 -= (last G2) dW2^T ; dZbar1 = dXbar2 gelu'(Zbar1)
-    mm_lds<2, NW, NBM, 2, true>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
+    E::template lds<2, NW, NBM, 2, true>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
     {
       float z[NJM], v[NJM];
       ldm(mZB1, z);
@@ -393,7 +420,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     // ---- 16. P1 = dZbar1 G1^T (split-k) ; dQ = dZbar1 W1^T ; S1 = XK dW1
     splitk_xyT(mDXB, mG1);
     prod_k(M0{}, lds + L::DQ, mDXB, W1, 1, M);
-    mm_lds<0, NW, NBM>(mS1, M, lds + L::XK, LD, 1, dW1, M, 1, 1, NTM, D, wave, lane);
+    E::template lds<0, NW, NBM>(mS1, M, lds + L::XK, LD, 1, dW1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 17. dA1, d eta ; dG1 = -last (S1 + db1) ; d last
     if (tid < 256) {
@@ -418,9 +445,9 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 18. dG1 -= M1^T dZbar1 ; dQ += dA1 XK ; dK = dA1^T XQ
-    mm_lds<2, NW, NBM, 4>(mS1, M, lds + L::M1, 1, LK, mDXB, M, 1, 1, NTM, 16, wave, lane);
-    mm_lds<1, NW, 1, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NTD, 16, wave, lane);
-    mm_lds<0, NW, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NTD, 16, wave, lane, NTD % NW);
+    E::template lds<2, NW, NBM, 4>(mS1, M, lds + L::M1, 1, LK, mDXB, M, 1, 1, NTM, 16, wave, lane);
+    E::template lds<1, NW, 1, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NTD, 16, wave, lane);
+    E::template lds<0, NW, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NTD, 16, wave, lane, NTD % NW);
     __syncthreads();
     // ---- 19. dK -= (last G1) dW1^T ; dU = dG1 gelu'(Z1) (kept in mU's place after saving U * gelu'')
     prod_k(M2{}, lds + L::DK, G1l, dW1, 1, M);
@@ -484,7 +511,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 22. dX2 += dZ2 W2^T ; then dZ1 = dG1 U gelu''(Z1) + dX2 gelu'(Z1)
-    mm_lds<1, NW, NBM, 2, true>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    E::template lds<1, NW, NBM, 2, true>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     {
       float z[NJM], f1[NJM], dx[NJM];
@@ -502,9 +529,9 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 23. gradient accumulation; dK += dZ1 W1^T
     // dW2 += X2^T dZ2 + dU^T G2 + Xbar2^T dZbar2 as ONE rank-48 pass over dW2 (operands consecutive)
-    mm_rank<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, wave, lane);
+    E::template rank<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, wave, lane);
     // dW1 += XQ^T dZbar1 + XK^T dZ1 as one rank-32 pass
-    mm_rank<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, wave, lane);
+    E::template rank<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, wave, lane);
     prod_k(M1{}, lds + L::DK, mDX2, W1, 1, M);
     if (tid < M) sdb1[tid] += col16_sum2(mDXB + tid, mDX2 + tid, M);
     if (tid < D) {
