@@ -43,7 +43,9 @@ typedef struct ttt_desc {
   int32_t heads;               /* H */
   int32_t seq;                 /* tokens per sequence; must be a multiple of mini_batch */
   int32_t head_dim;            /* d */
-  int32_t mini_batch;          /* K (1..16) */
+  int32_t mini_batch;          /* K: 1..16; for ttt_linear_fwd / ttt_linear_bwd at head_dim 32 also 17..32 (the
+                                  reference's (mini_batch 32, head_dim 32) tile,
+                                  rust/fused/src/linear_fused_tile/mod.rs:31-38), with f32 row-major checkpoints */
   float eps;                   /* LayerNorm epsilon (reference default 1e-6) */
   int32_t checkpoint_interval; /* stages between W/b checkpoints, >= 1 */
   int32_t io_dtype;            /* ttt_dtype of xq, xk, xv, lr, out and their gradients */

@@ -47,7 +47,23 @@ def test_shape_validation(P):
     assert L.ttt_linear_supported(C.byref(desc(P, seq=33))) == P.TTT_ERR_SHAPE
     assert b"multiple" in L.ttt_last_error()
     assert L.ttt_linear_supported(C.byref(desc(P, head_dim=48))) == P.TTT_ERR_UNSUPPORTED
-    assert L.ttt_linear_supported(C.byref(desc(P, mini_batch=32, seq=64))) == P.TTT_ERR_UNSUPPORTED
+    # mini-batches beyond 16 tokens: up to 32 at head_dim 32, as the reference's tile table
+    # (rust/fused/src/linear_fused_tile/mod.rs:31-38: (8,32) (8,64) (16,32) (16,64) (32,32))
+    assert L.ttt_linear_supported(C.byref(desc(P, mini_batch=32, seq=64))) == P.TTT_ERR_UNSUPPORTED   # head_dim 64
+    assert b"head_dim 32" in L.ttt_last_error()
+    for K, d, want in ((8, 32, P.TTT_OK), (8, 64, P.TTT_OK), (16, 32, P.TTT_OK), (16, 64, P.TTT_OK),
+                       (32, 32, P.TTT_OK), (24, 32, P.TTT_OK), (33, 32, P.TTT_ERR_UNSUPPORTED),
+                       (32, 96, P.TTT_ERR_UNSUPPORTED)):
+        assert L.ttt_linear_supported(C.byref(desc(P, mini_batch=K, head_dim=d, seq=4 * K))) == want, (K, d)
+    big = lambda **kw: desc(P, mini_batch=32, head_dim=32, seq=128, **kw)
+    assert L.ttt_linear_bwd_supported(C.byref(big())) == P.TTT_OK
+    assert L.ttt_linear_bwd_supported(C.byref(big(checkpoint_interval=2, io_dtype=P.TTT_BF16))) == P.TTT_OK
+    assert L.ttt_linear_bwd_supported(C.byref(big(checkpoint_format=1))) == P.TTT_ERR_UNSUPPORTED
+    assert L.ttt_linear_bwd_supported(C.byref(big(checkpoint_format=2, io_dtype=P.TTT_BF16))) == P.TTT_ERR_UNSUPPORTED
+    assert L.ttt_linear_best_checkpoint_format(C.byref(big(io_dtype=P.TTT_BF16))) == 0
+    assert L.ttt_mlp_supported(C.byref(big())) == P.TTT_ERR_UNSUPPORTED
+    assert L.ttt_linear_adam_supported(C.byref(big())) == P.TTT_ERR_UNSUPPORTED
+    assert L.ttt_linear_fwd_fused_inputs_supported(C.byref(big(io_dtype=P.TTT_BF16)), 0, 0) == P.TTT_ERR_UNSUPPORTED
     assert L.ttt_linear_supported(C.byref(desc(P, checkpoint_interval=0))) == P.TTT_ERR_SHAPE
     assert L.ttt_linear_supported(C.byref(desc(P, io_dtype=7))) == P.TTT_ERR_UNSUPPORTED
     assert L.ttt_linear_supported(None) == P.TTT_ERR_NULL

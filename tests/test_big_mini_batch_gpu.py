@@ -1,0 +1,105 @@
+"""GPU parity for mini-batches of 17 .. 32 tokens at head_dim 32: the reference's tile table ends at
+(mini_batch 32, head_dim 32) (rust/fused/src/linear_fused_tile/mod.rs:31-38).  ttt_linear_fwd and ttt_linear_bwd
+through the C ABI against the float64 oracle, which is written for any mini-batch length."""
+import importlib
+
+import pytest
+import torch
+
+from helpers import TOL, assert_close, np_inputs, to_dev
+from oracle import ttt_oracle as orc
+from test_linear_bwd_gpu import compare, oracle_bwd, run_bwd
+from test_linear_fwd_gpu import oracle_case, run_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def P():
+    return importlib.import_module("ttt-rs_amd")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("style", ["ref", "baseline"])
+@pytest.mark.parametrize("B,H,K,N", [(2, 2, 32, 1), (1, 4, 32, 4), (2, 3, 24, 3), (1, 2, 17, 2), (1, 2, 32, 16)])
+def test_fwd_matches_oracle(P, B, H, K, N, style, dtype):
+    print(f"case big-K fwd {style} B{B} H{H} K{K} N{N} {dtype}", flush=True)
+    make = P.synthetic.reference_test_inputs if style == "ref" else P.synthetic.baseline_inputs
+    c = make(40 + B + K + N, B, H, N * K, 32, K, io_dtype=dtype)
+    out, W, b = run_case(P, c, K)
+    ro, rW, rb = oracle_case(c, K)
+    tol = TOL[dtype]
+    assert_close(out, ro, tol, "out")
+    assert_close(W, rW, tol, "W_out")
+    assert_close(b, rb, tol, "b_out")
+
+
+@pytest.mark.parametrize("ci", [1, 2, 3])
+def test_checkpoints_hold_state_entering_stage(P, ci):
+    print(f"case big-K checkpoints ci={ci}", flush=True)
+    B, H, d, K, N = 2, 2, 32, 32, 5
+    c = P.synthetic.reference_test_inputs(3, B, H, N * K, d, K)
+    out, W, b, Wc, bc = run_case(P, c, K, ci=ci, ckpt=True, per_batch=True)
+    ro, rW, rb, rWc, rbc = oracle_case(c, K, ci=ci)
+    assert_close(out, ro, 1e-4, "out")
+    assert_close(Wc, rWc, 1e-4, "W checkpoints")
+    assert_close(bc, rbc, 1e-4, "b checkpoints")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("B,H,K,N,ci", [(2, 2, 32, 1, 1), (1, 2, 32, 3, 1), (2, 2, 32, 4, 2), (1, 3, 24, 3, 1),
+                                        (1, 2, 17, 4, 4), (1, 1, 32, 8, 3)])
+def test_bwd_matches_oracle(P, B, H, K, N, ci, dtype):
+    print(f"case big-K bwd B{B} H{H} K{K} N{N} ci{ci} {dtype}", flush=True)
+    c = P.synthetic.reference_test_inputs(100 + B + K + N + ci, B, H, N * K, 32, K, io_dtype=dtype)
+    g = torch.Generator().manual_seed(5)
+    dO = torch.randn(B, H, N * K, 32, generator=g).to(dtype)
+    compare(run_bwd(P, c, dO, K, ci), oracle_bwd(c, dO, K), TOL[dtype])
+    # the reference's backward tests differentiate output.sum()
+    ones = torch.ones(B, H, N * K, 32).to(dtype)
+    compare(run_bwd(P, c, ones, K, ci), oracle_bwd(c, ones, K), TOL[dtype])
+
+
+def test_bwd_with_upstream_state_gradients(P):
+    print("case big-K bwd state grads", flush=True)
+    B, H, d, K, N = 2, 2, 32, 32, 3
+    c = P.synthetic.baseline_inputs(9, B, H, N * K, d, K)
+    g = torch.Generator().manual_seed(6)
+    dO = torch.randn(B, H, N * K, d, generator=g)
+    sg = (torch.randn(B, H, d, d, generator=g) * 0.1, torch.randn(B, H, d, generator=g) * 0.1)
+    compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), 1e-4)
+
+
+def test_inner_model_forward_with_remainder(P):
+    """Host class at mini_batch 32: the full mini-batches in one launch, then a remainder of 20 tokens as one short
+    mini-batch (rust/core/src/inner.rs:40-47), which is again one of more than 16 tokens."""
+    print("case big-K remainder", flush=True)
+    B, H, d, K, seq = 2, 2, 32, 32, 32 * 2 + 20
+    c = P.synthetic.reference_test_inputs(13, B, H, seq, d, K)
+    te_seq = c["token_eta"].repeat(seq // K + 1)[:seq]
+    dv = to_dev(c)
+    model = P.FusedTileMulti(P.ModelConfig(H, d, P.TTTConfig(mini_batch_size=K)), dv["W0"], dv["b0"],
+                             dv["gamma"], dv["beta"])
+    state = model.init_state(B)
+    inputs = P.TTTInputsInner(P.Qkv(dv["xq"], dv["xk"], dv["xv"]), te_seq.to("cuda:0"), dv["lr"])
+    out = model.forward(state, inputs)
+    torch.cuda.synchronize()
+    n = np_inputs(c)
+    ro, rW, rb = orc.linear_forward(n["W0"], n["b0"], n["xq"], n["xk"], n["xv"], te_seq.double().numpy(),
+                                    n["lr"], n["gamma"], n["beta"], K=K)
+    assert_close(out, ro, 1e-4, "out")
+    assert_close(state.weight, rW, 1e-4, "W")
+    assert_close(state.bias, rb, 1e-4, "b")
+
+
+def test_unsupported_combinations_are_refused(P):
+    print("case big-K refusals", flush=True)
+    c = to_dev(P.synthetic.reference_test_inputs(1, 1, 2, 64, 64, 32))
+    with pytest.raises(P.TttError):   # head_dim 64
+        P.ttt_linear_forward_raw(c["xq"], c["xk"], c["xv"], c["W0"], c["b0"], c["token_eta"], c["lr"], c["gamma"],
+                                 c["beta"], 32)
+    c = to_dev(P.synthetic.reference_test_inputs(1, 1, 2, 64, 32, 32, io_dtype=torch.bfloat16))
+    for fmt in (1, 2):                # packed states, update factors
+        with pytest.raises(P.TttError):
+            P.ttt_linear_forward_raw(c["xq"], c["xk"], c["xv"], c["W0"], c["b0"], c["token_eta"], c["lr"],
+                                     c["gamma"], c["beta"], 32, want_checkpoints=True, packed_checkpoints=fmt)

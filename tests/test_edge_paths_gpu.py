@@ -168,9 +168,10 @@ def test_mlp_bwd_token_eta_with_zeros(P, dtype, d, kind):
     n = np_inputs(c)
     ref = orc.mlp_backward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
                            n["gamma"], n["beta"], dO.double().numpy(), K=K)
+    # bf16 I/O up to head_dim 96: the scan's products take bf16 operands, so every gradient is held to the bf16 bar
     for k in MLP_GRADS:
-        io_out = k in ("d_xq", "d_xk", "d_xv", "d_lr")
-        assert_close(got[k], ref[k], TOL[dtype] if io_out else 1e-4, k)
+        io_out = k in ("d_xq", "d_xk", "d_xv", "d_lr") or dtype == torch.bfloat16
+        assert_close(got[k], ref[k], TOL[dtype] if io_out else 1e-4, k, min_frac=0.99 if dtype == torch.bfloat16 else 0.999)
 
 
 # ------------------------------------------------------------------ rows far from zero mean

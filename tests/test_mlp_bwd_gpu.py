@@ -20,7 +20,7 @@ def P():
     return importlib.import_module("ttt-rs_amd")
 
 
-def run_case(P, B, H, d, K, N, dtype, style, state_grads=False, seed=0):
+def run_case(P, B, H, d, K, N, dtype, style, state_grads=False, seed=0, kernel_hint=0):
     seq = N * K
     c = mlp_case(P, 300 + d + K + seed, B, H, seq, d, K, dtype, style)
     g = torch.Generator().manual_seed(77 + seed)
@@ -32,7 +32,8 @@ def run_case(P, B, H, d, K, N, dtype, style, state_grads=False, seed=0):
     dv = to_dev(c)
     got = P.ttt_mlp_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"],
                                  dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], d_out.to("cuda:0"), K,
-                                 d_state_out=None if dst is None else [x.to("cuda:0") for x in dst])
+                                 d_state_out=None if dst is None else [x.to("cuda:0") for x in dst],
+                                 kernel_hint=kernel_hint)
     torch.cuda.synchronize()
     n = np_inputs(c)
     ref = orc.mlp_backward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
@@ -48,15 +49,29 @@ def run_case(P, B, H, d, K, N, dtype, style, state_grads=False, seed=0):
 def test_mlp_bwd_matches_oracle(P, B, H, d, K, N, style, state_grads, dtype):
     print(f"case mlp bwd {style} B{B} H{H} d{d} K{K} N{N} {dtype} state_grads={state_grads}", flush=True)
     got, ref = run_case(P, B, H, d, K, N, dtype, style, state_grads)
-    # The reverse scan's arithmetic is f32 for both I/O dtypes; bf16 rounds the stored activation gradients.  With
-    # bf16 I/O up to head_dim 96 the update factors it rolls back and differentiates are those of the bf16-operand
-    # forward (rounded to bf16 as that forward applied them), so every gradient is held to the bf16 bar there;
-    # f32 I/O and head_dim 128 (f32 forward sweep) keep 1e-4 for the gradients stored in f32.
+    # bf16 rounds the stored activation gradients.  With bf16 I/O up to head_dim 96 the update factors the scan rolls
+    # back and differentiates are those of the bf16-operand forward (rounded to bf16 as that forward applied them)
+    # and the scan's own products take bf16 operands, so every gradient is held to the bf16 bar there;
+    # f32 I/O and head_dim 128 (f32 forward sweep, f32 products) keep 1e-4 for the gradients stored in f32.
     bf16_factors = dtype == torch.bfloat16 and d <= 96
     for k in GRADS:
         io_out = k in ("d_xq", "d_xk", "d_xv", "d_lr")
         assert_close(got[k], ref[k], TOL[dtype] if (io_out or bf16_factors) else 1e-4, k,
                      min_frac=0.99 if bf16_factors else 0.999)
+
+
+@pytest.mark.parametrize("d,N,style,sg", [(32, 3, "ref", False), (64, 4, "ref", True), (96, 3, "baseline", False)])
+def test_mlp_bwd_bf16_with_f32_products(P, d, N, style, sg):
+    """bf16 I/O up to head_dim 96: the scan with its products kept in f32 (TTT_HINT_F32_PRODUCTS) and the default scan
+    (bf16 operands) are two compilations of the same kernel; both are held to the oracle, and to each other."""
+    print(f"case mlp bwd bf16 f32-products d{d}", flush=True)
+    got32, ref = run_case(P, 1, 2, d, 16, N, torch.bfloat16, style, sg, kernel_hint=P.TTT_HINT_F32_PRODUCTS)
+    got16, _ = run_case(P, 1, 2, d, 16, N, torch.bfloat16, style, sg)
+    tol = TOL[torch.bfloat16]
+    for k in GRADS:
+        assert_close(got32[k], ref[k], tol, k + " (f32 products)", min_frac=0.99)
+        assert_close(got16[k], ref[k], tol, k + " (bf16 operands)", min_frac=0.99)
+        assert_close(got16[k], got32[k].double().cpu().numpy(), tol, k + " (bf16 operands vs f32 products)", min_frac=0.99)
 
 
 def test_mlp_bwd_is_linear_in_upstream_gradient(P):

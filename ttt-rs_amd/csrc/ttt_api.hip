@@ -262,14 +262,14 @@ int opt_in_lds(size_t bytes) {
   return rc;
 }
 
-template <class T, int D>
+template <class T, int D, int MT = 1>
 int launch_linear_fwd_lds(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s) {
   const ttt::LinearFwdArgs& a = probs[0];
-  constexpr auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D>;
-  constexpr size_t bytes = ttt::LinFwdLds<D>::BYTES;
+  constexpr auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D, MT>;
+  constexpr size_t bytes = ttt::LinFwdLds<D, MT>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H), ny), dim3(256), bytes, s, pack_of(probs, ny));
+  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H), ny), dim3(256 * MT), bytes, s, pack_of(probs, ny));
   return hip_status(hipGetLastError(), "ttt_linear_fwd (LDS kernel) launch");
 }
 
@@ -365,13 +365,13 @@ int uses_two_cu_mlp(const ttt_desc* d, int n_problems, bool* yes) {
   return TTT_OK;
 }
 
-template <class T, int D>
+template <class T, int D, int MT = 1>
 int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_linear_bwd_kernel<T, D>;
-  constexpr size_t bytes = ttt::BwdLds<D>::BYTES;
+  constexpr auto kern = ttt::ttt_linear_bwd_kernel<T, D, MT>;
+  constexpr size_t bytes = ttt::BwdLds<D, MT>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), bytes, s, a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * MT), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_bwd launch");
 }
 
@@ -438,6 +438,14 @@ int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
   }
   const bool packed = ckpt_format_of(d) == TTT_CKPT_PACKED;
   const bool factors = ckpt_format_of(d) == TTT_CKPT_FACTORS;
+  if (d->mini_batch > 16) {
+    // two tiles of token rows: the LDS-tile kernel, any checkpoint interval, f32 row-major checkpoints
+    if (packed || factors)
+      return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: mini_batch %d > 16 reads f32 row-major checkpoints only", d->mini_batch);
+    ch->kind = LinearBwdChoice::LDS;
+    ch->waves = 8;
+    return TTT_OK;
+  }
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && D <= 64;
   if (packed && (d->checkpoint_interval != 1 || want_lds))
     return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
@@ -629,8 +637,11 @@ const char* ttt_last_error(void) { return g_err; }
 int ttt_linear_supported(const ttt_desc* d) {
   int rc = check_common(d);
   if (rc != TTT_OK) return rc;
-  if (d->mini_batch > 16)
-    return fail(TTT_ERR_UNSUPPORTED, "mini_batch %d > 16 has no kernel", d->mini_batch);
+  // mini-batches of 17 .. 32 tokens: two tiles of token rows, at head_dim 32 only (the reference's own tile table,
+  // rust/fused/src/linear_fused_tile/mod.rs:31-38, ends at (32, 32))
+  if (d->mini_batch > 32 || (d->mini_batch > 16 && d->head_dim != 32))
+    return fail(TTT_ERR_UNSUPPORTED, "mini_batch %d has no kernel at head_dim %d (up to 16; up to 32 at head_dim 32)",
+                d->mini_batch, d->head_dim);
   if (d->head_dim != 32 && d->head_dim != 64 && d->head_dim != 96 && d->head_dim != 128)
     return fail(TTT_ERR_UNSUPPORTED, "TTT-Linear head_dim %d has no kernel (32, 64, 96, 128)", d->head_dim);
   return TTT_OK;
@@ -681,12 +692,16 @@ int prepare_linear_fwd(const ttt_desc* d, const void* xq, const void* xk, const 
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
   if (a.ckpt_packed == 1 && (d->checkpoint_interval != 1 || want_lds))
     return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
+  if (d->mini_batch > 16 && a.ckpt_packed != 0)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_fwd: mini_batch %d > 16 writes f32 row-major checkpoints only", d->mini_batch);
   return TTT_OK;
 }
 
 int dispatch_linear_fwd_pack(const ttt_desc* d, const ttt::LinearFwdArgs* a, unsigned ny, hipStream_t s) {
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
   const bool f32 = d->io_dtype == TTT_F32;
+  if (d->mini_batch > 16)  // head_dim 32 (ttt_linear_supported): the LDS-tile kernel on two tiles of token rows
+    return f32 ? launch_linear_fwd_lds<ttt::F32, 32, 2>(a, ny, s) : launch_linear_fwd_lds<ttt::BF16, 32, 2>(a, ny, s);
   switch (d->head_dim) {
     case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, d->kernel_hint, ny, s) : launch_linear_fwd<ttt::BF16, 32>(a, d->kernel_hint, ny, s);
     case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, d->kernel_hint, ny, s) : launch_linear_fwd<ttt::BF16, 64>(a, d->kernel_hint, ny, s);
@@ -788,6 +803,7 @@ int ttt_mlpn_fwd(const ttt_desc* d, int n_hidden, const void* xq, const void* xk
 int ttt_linear_adam_supported(const ttt_desc* d) {
   int rc = ttt_linear_supported(d);
   if (rc != TTT_OK) return rc;
+  if (d->mini_batch > 16) return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_adam_fwd: mini_batch up to 16 (got %d)", d->mini_batch);
   if (d->head_dim != 32 && d->head_dim != 64)
     return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_adam_fwd: head_dim 32 or 64 (got %d)", d->head_dim);
   if ((d->kernel_hint & TTT_HINT_LDS_TILES) != 0)
@@ -841,6 +857,8 @@ int ttt_linear_adam_fwd(const ttt_desc* d, const void* xq, const void* xk, const
 int ttt_linear_fwd_fused_inputs_supported(const ttt_desc* d, int pos_wrap, int has_rope) {
   int rc = ttt_linear_supported(d);
   if (rc != TTT_OK) return rc;
+  if (d->mini_batch > 16)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_fwd_fused_inputs: mini_batch up to 16 (got %d)", d->mini_batch);
   if (d->io_dtype != TTT_BF16 || (d->head_dim != 64 && d->head_dim != 32))
     return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_fwd_fused_inputs: bf16 I/O and head_dim 32 or 64 (got %s, %d)",
                 d->io_dtype == TTT_BF16 ? "bf16" : "f32", d->head_dim);
@@ -981,6 +999,8 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   const bool f32 = d->io_dtype == TTT_F32;
   const int waves = ch.waves;
   if (ch.kind == LinearBwdChoice::LDS) {
+    if (d->mini_batch > 16)
+      return f32 ? launch_linear_bwd<ttt::F32, 32, 2>(a, grid, s) : launch_linear_bwd<ttt::BF16, 32, 2>(a, grid, s);
     if (f32) return D == 64 ? launch_linear_bwd<ttt::F32, 64>(a, grid, s) : launch_linear_bwd<ttt::F32, 32>(a, grid, s);
     return D == 64 ? launch_linear_bwd<ttt::BF16, 64>(a, grid, s) : launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
   }
@@ -1190,6 +1210,7 @@ int plan_stack(const ttt_desc* d, int32_t n_layers, const ttt_stack_layer* layer
       return fail(TTT_ERR_UNSUPPORTED, "ttt_stack_fwd: layer %d has kind %d", l, layers[l].kind);
     rc = layers[l].kind == TTT_LAYER_LINEAR ? ttt_linear_supported(d) : ttt_mlp_supported(d);
     if (rc != TTT_OK) return rc;
+    if (d->mini_batch > 16) return fail(TTT_ERR_UNSUPPORTED, "ttt_stack_fwd: mini_batch up to 16 (got %d)", d->mini_batch);
   }
   // Windows of `chunk` tokens.  (Splitting the first window so that the upper layers start sooner was measured
   // and did not pay: the two-CU TTT-MLP kernel at the top of the benchmark stack bounds the call, and more

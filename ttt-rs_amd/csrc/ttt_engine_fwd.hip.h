@@ -66,24 +66,26 @@ __device__ __forceinline__ void ln_l2_grad(const float* zrow, const float* bias,
 }
 
 // ------------------------------------------------------------------------------------------
-// TTT-Linear forward, W resident in LDS.  256 threads, GW = 16.
+// TTT-Linear forward, W resident in LDS.  MT tiles of 16 token rows (mini_batch <= 16 MT), 256 MT threads, GW = 16.
+// MT = 2 is the kernel of the reference's (mini_batch 32, head_dim 32) tile
+// (rust/fused/src/linear_fused_tile/mod.rs:38).
 // ------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int MT = 1>
 struct LinFwdLds {
-  static constexpr int LD = D + 4, LK = 17, TILE = 16 * LD, KK = 16 * LK;
+  static constexpr int KT = 16 * MT, LD = D + 4, LK = KT + 1, TILE = KT * LD, KK = KT * LK;
   static constexpr int W = 0, XQ = W + D * LD, XK = XQ + TILE, TG = XK + TILE, G = TG + TILE,
                        ZB = G + TILE, A = ZB + TILE, M = A + KK, b = M + KK, gam = b + D,
-                       bet = gam + D, lr = bet + D, te = lr + 16, END = te + 16;
+                       bet = gam + D, lr = bet + D, te = lr + KT, END = te + KT;
   static constexpr size_t BYTES = sizeof(float) * END;
 };
 
-template <class T, int D>
-__global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(Problems<LinearFwdArgs> problems) {
+template <class T, int D, int MT = 1>
+__global__ void __launch_bounds__(256 * MT) ttt_linear_fwd_lds_kernel(Problems<LinearFwdArgs> problems) {
   const LinearFwdArgs& a = problems.p[blockIdx.y];
   using IO = Io<T>;
   using elem = typename IO::elem;
-  using L = LinFwdLds<D>;
-  constexpr int LD = L::LD, LK = L::LK, NJ = D / 16, NT = D / 16;
+  using L = LinFwdLds<D, MT>;
+  constexpr int LD = L::LD, LK = L::LK, KT = L::KT, NJ = D / 16, NT = D / 16, NTH = 256 * MT, NW = 4 * MT;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int t = tid >> 4, cg = tid & 15;
@@ -93,13 +95,13 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(Problems<Linear
         *slr = lds + L::lr, *ste = lds + L::te;
   const size_t sbase = a.state_per_batch ? bh : (size_t)h;
 
-  for (int i = tid; i < D * D; i += 256) sW[(i / D) * LD + (i % D)] = a.W0[sbase * D * D + i];
-  for (int i = tid; i < D; i += 256) {
+  for (int i = tid; i < D * D; i += NTH) sW[(i / D) * LD + (i % D)] = a.W0[sbase * D * D + i];
+  for (int i = tid; i < D; i += NTH) {
     sb[i] = a.b0[sbase * D + i];
     sgam[i] = a.gamma[h * D + i];
     sbet[i] = a.beta[h * D + i];
   }
-  if (tid < 16) ste[tid] = (tid < K) ? a.token_eta[tid] : 0.f;
+  if (tid < KT) ste[tid] = (tid < K) ? a.token_eta[tid] : 0.f;
   __syncthreads();
   const float te_last = ste[K - 1];
 
@@ -115,7 +117,7 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(Problems<Linear
       pk[j] = ok ? IO::load1(static_cast<const elem*>(a.xk) + r + o) : 0.f;
       pv[j] = ok ? IO::load1(static_cast<const elem*>(a.xv) + r + o) : 0.f;
     }
-    if (tid < 16)
+    if (tid < KT)
       plr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
   };
   fetch(0);
@@ -124,8 +126,8 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(Problems<Linear
     const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
     if (a.W_ckpt != nullptr && (st % a.ckpt_interval) == 0) {
       const size_t ci = bh * a.n_ckpt + st / a.ckpt_interval;
-      for (int i = tid; i < D * D; i += 256) a.W_ckpt[ci * D * D + i] = sW[(i / D) * LD + (i % D)];
-      for (int i = tid; i < D; i += 256) a.b_ckpt[ci * D + i] = sb[i];
+      for (int i = tid; i < D * D; i += NTH) a.W_ckpt[ci * D * D + i] = sW[(i / D) * LD + (i % D)];
+      for (int i = tid; i < D; i += NTH) a.b_ckpt[ci * D + i] = sb[i];
     }
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
@@ -134,24 +136,27 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(Problems<Linear
       lds[L::XK + t * LD + o] = pk[j];
       lds[L::TG + t * LD + o] = pv[j] - pk[j];
     }
-    if (tid < 16) slr[tid] = plr;
+    if (tid < KT) slr[tid] = plr;
     __syncthreads();
     if (st + 1 < a.n_stages) fetch(st + 1);
-    mm_lds<0>(lds + L::G, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NT, D, wave, lane);
-    mm_lds<0>(lds + L::ZB, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NT, D, wave, lane, NT & 3);
-    mm_lds<0>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, (2 * NT) & 3);
+    mm_lds<0, NW>(lds + L::G, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NT, D, wave, lane);
+    mm_lds<0, NW>(lds + L::ZB, LD, lds + L::XQ, LD, 1, sW, LD, 1, MT, NT, D, wave, lane, (MT * NT) % NW);
+    mm_lds<0, NW>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, MT, MT, D, wave, lane, (2 * MT * NT) % NW);
     __syncthreads();
     {
       float Gv[NJ];
       ln_l2_grad<D, 16>(lds + L::G + t * LD, sb, lds + L::TG + t * LD, sgam, sbet, cg, a.eps, Gv);
 #pragma unroll
       for (int j = 0; j < NJ; ++j) lds[L::G + t * LD + cg + 16 * j] = Gv[j];
-      const int s = cg;
-      const float at = lds[L::A + t * LK + s];
-      lds[L::M + t * LK + s] = (s <= t) ? ste[t] * slr[s] * (1.f + at) : 0.f;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int s = cg + 16 * i;
+        const float at = lds[L::A + t * LK + s];
+        lds[L::M + t * LK + s] = (s <= t) ? ste[t] * slr[s] * (1.f + at) : 0.f;
+      }
     }
     __syncthreads();
-    mm_lds<2, 4, 1, 4>(lds + L::ZB, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NT, 16, wave, lane);
+    mm_lds<2, NW, 1, 4>(lds + L::ZB, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, MT, NT, KT, wave, lane);
     __syncthreads();
     {
       float xh[NJ], rstd;
@@ -167,16 +172,16 @@ __global__ void __launch_bounds__(256) ttt_linear_fwd_lds_kernel(Problems<Linear
       }
     }
     __syncthreads();
-    mm_lds<2, 4, (NT % 4 == 0 ? 4 : 2), 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NT, NT, 16, wave, lane);
+    mm_lds<2, NW, (NT % 4 == 0 ? 4 : 2), 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NT, NT, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += lds[L::G + r * LD + tid];
+      for (int r = 0; r < KT; ++r) s += lds[L::G + r * LD + tid];
       sb[tid] -= s;
     }
     __syncthreads();
   }
-  for (int i = tid; i < D * D; i += 256) a.W_out[bh * D * D + i] = sW[(i / D) * LD + (i % D)];
-  for (int i = tid; i < D; i += 256) a.b_out[bh * D + i] = sb[i];
+  for (int i = tid; i < D * D; i += NTH) a.W_out[bh * D * D + i] = sW[(i / D) * LD + (i % D)];
+  for (int i = tid; i < D; i += NTH) a.b_out[bh * D + i] = sb[i];
 }
 
 // ------------------------------------------------------------------------------------------

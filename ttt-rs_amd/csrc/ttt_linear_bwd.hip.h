@@ -50,13 +50,16 @@ struct LinearBwdArgs {
   float eps;
 };
 
-template <int D>
+// MT tiles of 16 token rows: mini_batch <= KT = 16 MT.  MT = 2 serves the reference's (mini_batch 32, head_dim 32)
+// tile (rust/fused/src/linear_fused_tile/mod.rs:38).
+template <int D, int MT = 1>
 struct BwdLds {
+  static constexpr int KT = 16 * MT;
   static constexpr int LD = D + 4;     // padded row stride (floats) of every [*, D] array
-  static constexpr int LK = 17;        // row stride of the [16 x 16] matrices
-  static constexpr int TILE = 16 * LD;
+  static constexpr int LK = KT + 1;    // row stride of the [KT x KT] matrices
+  static constexpr int TILE = KT * LD;
   static constexpr int WSZ = D * LD;
-  static constexpr int KK = 16 * LK;
+  static constexpr int KK = KT * LK;
   // offsets in floats
   static constexpr int W = 0, dW = W + WSZ;
   static constexpr int XQ = dW + WSZ, XK = XQ + TILE, TG = XK + TILE, DO = TG + TILE, XH = DO + TILE,
@@ -66,16 +69,17 @@ struct BwdLds {
   static constexpr int A = DGM + TILE, ETA = A + KK, M = ETA + KK, P = M + KK, DA = P + KK,
                        DETA = DA + KK;
   static constexpr int b = DETA + KK, db = b + D, gam = db + D, bet = gam + D, lr = bet + D,
-                       te = lr + 16, rstd1 = te + 16, dlast = rstd1 + 16, END = dlast + 16;
+                       te = lr + KT, rstd1 = te + KT, dlast = rstd1 + KT, END = dlast + KT;
+  static_assert(sizeof(float) * END <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
   static constexpr size_t BYTES = sizeof(float) * END;
 };
 
-template <class T, int D>
-__global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
+template <class T, int D, int MT = 1>
+__global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using elem = typename IO::elem;
-  using L = BwdLds<D>;
-  constexpr int LD = L::LD, LK = L::LK, NJ = D / 16;
+  using L = BwdLds<D, MT>;
+  constexpr int LD = L::LD, LK = L::LK, KT = L::KT, NJ = D / 16, NTH = 256 * MT, NW = 4 * MT;
   constexpr int NB2 = NJ >= 2 ? 2 : 1;  // tile columns per job of a [16 x D] product
   constexpr float inv_d = 1.0f / D;
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -96,16 +100,16 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   float* ste = lds + L::te;
 
   // ---- one-time setup
-  for (int i = tid; i < D; i += 256) {
+  for (int i = tid; i < D; i += NTH) {
     sgam[i] = a.gamma[h * D + i];
     sbet[i] = a.beta[h * D + i];
     sdb[i] = a.d_b_out ? a.d_b_out[bh * D + i] : 0.f;
   }
-  for (int i = tid; i < D * D; i += 256) {
+  for (int i = tid; i < D * D; i += NTH) {
     const int r = i / D, cc = i - r * D;
     sdW[r * LD + cc] = a.d_W_out ? a.d_W_out[bh * D * D + i] : 0.f;
   }
-  if (tid < 16) ste[tid] = (tid < K) ? a.token_eta[tid] : 0.f;
+  if (tid < KT) ste[tid] = (tid < K) ? a.token_eta[tid] : 0.f;
   float dgam_acc[NJ], dbet_acc[NJ];
 #pragma unroll
   for (int j = 0; j < NJ; ++j) dgam_acc[j] = dbet_acc[j] = 0.f;
@@ -119,7 +123,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     for (int j = 0; j < NJ; ++j) dst[t * LD + cg + 16 * j] = (t < K) ? IO::load1(p + cg + 16 * j) : 0.f;
   };
   auto load_lr = [&](int stage) {
-    if (tid < 16)
+    if (tid < KT)
       slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
   };
 
@@ -159,8 +163,9 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   // activation tiles of the NEXT stage to be processed are fetched while the current one computes,
   // and only copied into LDS at the top of that stage.  Thread tid owns EP contiguous elements of
   // each [16 x D] tile and WP float4 pieces of the checkpoint.
-  constexpr int EP = D / 16;          // 16*D elements / 256 threads
-  constexpr int WP = D * D / 1024;    // D*D floats / (256 threads * 4)
+  constexpr int EP = D / 16;          // KT*D elements / NTH threads
+  constexpr int WP = (D * D + 4 * NTH - 1) / (4 * NTH);  // float4 pieces of the checkpoint per thread
+  constexpr bool WALL = D * D % (4 * NTH) == 0;          // every thread has all WP pieces
   const int pt = (tid * EP) / D, pc = (tid * EP) % D;  // token row / first feature of this thread's piece
   struct Prefetch {
     f32x4 w[WP];
@@ -176,7 +181,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     const int ckp = stage / a.ckpt_interval;
     const f32x4* Wg = reinterpret_cast<const f32x4*>(a.W_ckpt + (bh * a.n_ckpt + ckp) * D * D);
 #pragma unroll
-    for (int i = 0; i < WP; ++i) pre.w[i] = Wg[tid + 256 * i];
+    for (int i = 0; i < WP; ++i) pre.w[i] = Wg[(WALL || 4 * (tid + NTH * i) < D * D) ? tid + NTH * i : 0];
     pre.b = (tid < D) ? a.b_ckpt[(bh * a.n_ckpt + ckp) * D + tid] : 0.f;
     pre.lr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
     fetch_tile(pre.q, a.xq, stage);
@@ -187,8 +192,8 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   auto commit_state = [&]() {
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
-      const int idx = (tid + 256 * i) * 4;
-      *reinterpret_cast<f32x4*>(sW + (idx / D) * LD + (idx % D)) = pre.w[i];
+      const int idx = (tid + NTH * i) * 4;
+      if (WALL || idx < D * D) *reinterpret_cast<f32x4*>(sW + (idx / D) * LD + (idx % D)) = pre.w[i];
     }
     if (tid < D) sb[tid] = pre.b;
   };
@@ -200,7 +205,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       lds[L::TG + pt * LD + pc + e] = pre.v[e] - pre.k[e];
       lds[L::DO + pt * LD + pc + e] = pre.o[e];
     }
-    if (tid < 16) slr[tid] = pre.lr;
+    if (tid < KT) slr[tid] = pre.lr;
   };
   fetch_stage(a.n_stages - 1);
 
@@ -216,7 +221,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       lds_barrier();
 #pragma unroll
       for (int j = 0; j < NJ; ++j) lds[L::TG + t * LD + cg + 16 * j] -= lds[L::XK + t * LD + cg + 16 * j];
-      mm_lds<0>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane);
+      mm_lds<0, NW>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane);
       lds_barrier();
       {
         float xh[NJ], Gv[NJ], rstd;
@@ -227,10 +232,10 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       }
       lds_barrier();
       // W -= XK^T (last * G) ; b -= colsum(last * G)      (linear.rs:134-144)
-      mm_lds<2, 4, NJ, 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, 16, wave, lane);
+      mm_lds<2, NW, NJ, 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, KT, wave, lane);
       if (tid < D) {
         float s = 0.f;
-        for (int r = 0; r < 16; ++r) s += lds[L::G + r * LD + tid];
+        for (int r = 0; r < KT; ++r) s += lds[L::G + r * LD + tid];
         sb[tid] -= s;
       }
     }
@@ -243,9 +248,9 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     // Z1 = XK W ; Zq = XQ W ; A = XQ XK^T
     // every product is cut into jobs of NB2 tile columns: two or more accumulator chains per wave keep the
     // matrix pipe busy (a single chain waits out the full MFMA latency between dependent steps)
-    mm_lds<0, 4, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, 0);
-    mm_lds<0, 4, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, 1, NJ, D, wave, lane, 2);
-    mm_lds<0>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, 1);
+    mm_lds<0, NW, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane, 0);
+    mm_lds<0, NW, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane, 2);
+    mm_lds<0, NW>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, MT, MT, D, wave, lane, 1);
     lds_barrier();
 
     // ================= forward intermediates: x_hat, rstd, G; eta, A (tril), M = eta (1 + A)
@@ -256,8 +261,9 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
       lds[L::XH + t * LD + cg + 16 * j] = xh[j];
       lds[L::G + t * LD + cg + 16 * j] = Gv[j];
     }
-    {
-      const int s = cg;  // (t, s) entry of the [16 x 16] matrices
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int s = cg + 16 * i;  // (t, s) entry of the [KT x KT] matrices
       const bool low = s <= t;
       const float at = low ? lds[L::A + t * LK + s] : 0.f;
       const float et = low ? ste[t] * slr[s] : 0.f;
@@ -267,7 +273,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     }
     lds_barrier();
     // Zb = XQ W - M G  (+ b added when read)
-    mm_lds<2, 4, 1, 4>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, 1, NJ, 16, wave, lane);
+    mm_lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, MT, NJ, KT, wave, lane);
     lds_barrier();
 
     // ================= output LayerNorm and its backward (stage 4)
@@ -306,19 +312,22 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     lds_barrier();
 
     // ================= P = dZb G^T ; dQ = dZb W^T ; S = XK dW ; TMP = G dW^T
-    mm_lds<0, 4, NB2>(lds + L::DQ, LD, lds + L::DZB, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 0);
-    mm_lds<0, 4, NB2>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, LD, 1, NJ, D, wave, lane, 0);
-    mm_lds<0, 4, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, LD, 1, 1, NJ, D, wave, lane, 2);
-    mm_lds<0>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, 1, 1, D, wave, lane, 3);
+    mm_lds<0, NW, NB2>(lds + L::DQ, LD, lds + L::DZB, LD, 1, sW, 1, LD, MT, NJ, D, wave, lane, 0);
+    mm_lds<0, NW, NB2>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, LD, MT, NJ, D, wave, lane, 0);
+    mm_lds<0, NW, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, LD, 1, MT, NJ, D, wave, lane, 2);
+    mm_lds<0, NW>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, MT, MT, D, wave, lane, 3);
     lds_barrier();
 
     // ================= dA, d eta ; S += db ; dlast
     {
-      const int s = cg;
-      const bool low = s <= t;
-      const float p = lds[L::P + t * LK + s];
-      lds[L::DA + t * LK + s] = low ? -p * lds[L::ETA + t * LK + s] : 0.f;
-      lds[L::DETA + t * LK + s] = low ? -p * (1.f + lds[L::A + t * LK + s]) : 0.f;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int s = cg + 16 * i;
+        const bool low = s <= t;
+        const float p = lds[L::P + t * LK + s];
+        lds[L::DA + t * LK + s] = low ? -p * lds[L::ETA + t * LK + s] : 0.f;
+        lds[L::DETA + t * LK + s] = low ? -p * (1.f + lds[L::A + t * LK + s]) : 0.f;
+      }
       float dl = 0.f;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
@@ -332,27 +341,27 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     lds_barrier();
 
     // ================= dQ += dA XK ; dK = dA^T XQ ; DGM = M^T dZb ; dW += XQ^T dZb ; db += colsum(dZb)
-    mm_lds<1, 4, NJ, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NJ, 16, wave, lane, 0);
-    mm_lds<0, 4, NJ, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NJ, 16, wave, lane, 1);
-    mm_lds<0, 4, NJ, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, 1, NJ, 16, wave, lane, 2);
-    mm_lds<1, 4, NJ, 4>(sdW, LD, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, 16, wave, lane);
+    mm_lds<1, NW, NJ, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, MT, NJ, KT, wave, lane, 0);
+    mm_lds<0, NW, NJ, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, MT, NJ, KT, wave, lane, 1);
+    mm_lds<0, NW, NJ, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, MT, NJ, KT, wave, lane, 2);
+    mm_lds<1, NW, NJ, 4>(sdW, LD, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += lds[L::DZB + r * LD + tid];
+      for (int r = 0; r < KT; ++r) s += lds[L::DZB + r * LD + tid];
       sdb[tid] += s;
     }
-    // d lr and d token_eta (16 threads each)
-    if (tid < 16) {
+    // d lr and d token_eta (KT threads each, in different waves)
+    if (tid < KT) {
       float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += lds[L::DETA + r * LK + tid] * ste[r];
+      for (int r = 0; r < KT; ++r) s += lds[L::DETA + r * LK + tid] * ste[r];
       s += te_last * lds[L::dlast + tid];
       if (tid < K) IO::store1(static_cast<elem*>(a.d_lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid, s);
-    } else if (tid >= 64 && tid < 80) {
+    } else if (tid >= 64 && tid < 64 + KT) {
       const int tt = tid - 64;
       float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += lds[L::DETA + tt * LK + r] * slr[r];
+      for (int r = 0; r < KT; ++r) s += lds[L::DETA + tt * LK + r] * slr[r];
       if (tt == K - 1)
-        for (int r = 0; r < 16; ++r) s += lds[L::dlast + r] * slr[r];
+        for (int r = 0; r < KT; ++r) s += lds[L::dlast + r] * slr[r];
       if (tt < K) atomicAdd(a.d_token_eta + (size_t)st * K + tt, s);
     }
     lds_barrier();
@@ -402,11 +411,11 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
     lds_barrier();
 
     // ================= dK += dZ1 W^T ; dW += XK^T dZ1 ; db += colsum(dZ1)
-    mm_lds<1, 4, NB2>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, 1, NJ, D, wave, lane, 2);
-    mm_lds<1, 4, NJ, 4>(sdW, LD, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, 16, wave, lane);
+    mm_lds<1, NW, NB2>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, MT, NJ, D, wave, lane, 2);
+    mm_lds<1, NW, NJ, 4>(sdW, LD, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
-      for (int r = 0; r < 16; ++r) s += lds[L::DZ1 + r * LD + tid];
+      for (int r = 0; r < KT; ++r) s += lds[L::DZ1 + r * LD + tid];
       sdb[tid] += s;
     }
     lds_barrier();
@@ -426,7 +435,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   }
 
   // ---- results carried over the whole scan
-  for (int i = tid; i < D * D; i += 256) {
+  for (int i = tid; i < D * D; i += NTH) {
     const int r = i / D, cc = i - r * D;
     a.d_W0[bh * D * D + i] = sdW[r * LD + cc];
   }
@@ -439,7 +448,7 @@ __global__ void __launch_bounds__(256) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   __syncthreads();
   if (tid < D) {
     float sg = 0.f, sbt = 0.f;
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < KT; ++r) {
       sg += lds[L::XQ + r * LD + tid];
       sbt += lds[L::XK + r * LD + tid];
     }

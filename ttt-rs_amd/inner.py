@@ -356,7 +356,7 @@ def ttt_mlpn_forward_raw(xq, xk, xv, weights, biases, token_eta, ttt_lr_eta, ln_
 
 def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias, d_out,
                          mini_batch: int, eps: float = 1e-6, d_state_out=None, static_scratch: bool = False,
-                         into=None):
+                         into=None, kernel_hint: int = 0):
     """One call of ttt_mlp_bwd on the current stream: gradients of the TTT-MLP inner loop
     (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50; the reference gets them
     from Burn autodiff).  Arguments as ttt_mlp_forward_raw plus d_out [B,H,seq,d] and the optional
@@ -365,7 +365,8 @@ def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_w
     d_token_eta [seq], d_gamma, d_beta [H,d].
     static_scratch: call ttt_mlp_bwd_static (the library's built-in scratch buffer instead of a workspace
     allocated here); `into`: a dict returned by an earlier call of the same shape, whose tensors receive the
-    gradients (with both, the call allocates no device memory)."""
+    gradients (with both, the call allocates no device memory).  kernel_hint: TTT_HINT_F32_PRODUCTS keeps the
+    reverse scan's products in f32 where it would round their operands to bf16 (bf16 I/O, head_dim <= 96)."""
     B, H, seq, d = xq.shape
     m = w1.shape[-1]
     io = xq.dtype
@@ -388,6 +389,7 @@ def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_w
         raise _lib.TttError(_lib.TTT_ERR_SHAPE, "token_eta shorter than mini_batch")
     te = token_eta.to(torch.float32).contiguous()
     desc = TttDesc(B, H, seq, d, mini_batch, eps, 1, _io_dtype(xq), int(per_batch), 0)
+    desc.kernel_hint = int(kernel_hint)
     check(lib().ttt_mlp_supported(C.byref(desc)))
     dev = xq.device
     f32 = dict(dtype=torch.float32, device=dev)
