@@ -89,8 +89,11 @@ def test_best_checkpoint_format(P):
     # the hint is part of the question: the LDS-tile backward reads f32 matrices only
     assert best(io_dtype=P.TTT_BF16, kernel_hint=P.TTT_HINT_LDS_TILES) == 0
     assert best(io_dtype=P.TTT_F32, kernel_hint=P.TTT_HINT_LDS_TILES) == 0
-    # no backward kernel at all (f32 I/O at head_dim 128, an unsupported head_dim): the backward's status, no format
-    assert best(io_dtype=P.TTT_F32, head_dim=128) == P.TTT_ERR_UNSUPPORTED
+    # f32 I/O at head_dim 128: the LDS-tile backward that reads the row-major checkpoints in place
+    assert best(io_dtype=P.TTT_F32, head_dim=128) == 0
+    assert best(head_dim=96, checkpoint_interval=2) == 0
+    # no backward kernel at all: the backward's status, no format
+    assert best(head_dim=128, checkpoint_interval=2) == P.TTT_ERR_UNSUPPORTED
     assert best(head_dim=48) == P.TTT_ERR_UNSUPPORTED
     # what it names is accepted by the backward
     for kw in (dict(io_dtype=P.TTT_BF16), dict(io_dtype=P.TTT_F32), dict(io_dtype=P.TTT_BF16, head_dim=128),
@@ -112,9 +115,11 @@ def test_backward_support_query_and_kernel_hints(P):
     ok = lambda **kw: L.ttt_linear_bwd_supported(C.byref(desc(P, **kw)))
     assert ok() == P.TTT_OK
     assert ok(head_dim=128, io_dtype=P.TTT_BF16) == P.TTT_OK
-    assert ok(head_dim=128, io_dtype=P.TTT_F32) == P.TTT_ERR_UNSUPPORTED       # forward only
+    assert ok(head_dim=128, io_dtype=P.TTT_F32) == P.TTT_OK
+    assert ok(head_dim=128, io_dtype=P.TTT_F32, checkpoint_format=1) == P.TTT_ERR_UNSUPPORTED
     assert L.ttt_linear_supported(C.byref(desc(P, head_dim=128))) == P.TTT_OK
-    assert ok(head_dim=96, checkpoint_interval=2) == P.TTT_ERR_UNSUPPORTED
+    assert ok(head_dim=96, checkpoint_interval=2) == P.TTT_OK
+    assert ok(head_dim=128, checkpoint_interval=2) == P.TTT_ERR_UNSUPPORTED
     assert b"checkpoint_interval 1" in L.ttt_last_error()
     assert ok(head_dim=64, checkpoint_interval=2) == P.TTT_OK
     assert ok(checkpoint_format=1, checkpoint_interval=2) == P.TTT_ERR_UNSUPPORTED

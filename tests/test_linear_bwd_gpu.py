@@ -148,16 +148,13 @@ def test_bwd_multi_wave_kernel(P, B, H, d, K, N, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("B,H,d,K,N", [(1, 2, 96, 16, 3), (2, 1, 96, 7, 2), (1, 2, 128, 16, 3)])
 def test_bwd_wide_heads(P, B, H, d, K, N, dtype):
-    """head_dim 96 and 128 (feature-split kernel only; 128 needs bf16 I/O: the f32 staging does not fit LDS)."""
+    """head_dim 96 and 128: the feature-split kernel; f32 I/O at head_dim 128 (its f32 staging does not fit a CU) the
+    LDS-tile kernel with the state read in place from the checkpoints and the state gradient kept in d_W0."""
     print(f"case bwd wide B{B} H{H} d{d} K{K} N{N} {dtype}", flush=True)
     c = P.synthetic.reference_test_inputs(400 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
     g = torch.Generator().manual_seed(10)
     dO = torch.randn(B, H, N * K, d, generator=g).to(dtype)
     sg = (0.1 * torch.randn(B, H, d, d, generator=g), 0.1 * torch.randn(B, H, d, generator=g))
-    if d == 128 and dtype == torch.float32:
-        with pytest.raises(Exception, match="head_dim 128"):
-            run_bwd(P, c, dO, K, 1, sg)
-        return
     compare(run_bwd(P, c, dO, K, 1, sg), oracle_bwd(c, dO, K, sg), TOL[dtype])
     if K == 16:
         c = P.synthetic.baseline_inputs(4, B, H, N * K, d, K, io_dtype=dtype, with_dout=True)
@@ -165,10 +162,33 @@ def test_bwd_wide_heads(P, B, H, d, K, N, dtype):
         compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), TOL[dtype])
 
 
-def test_bwd_wide_heads_need_a_checkpoint_per_mini_batch(P):
-    c = P.synthetic.reference_test_inputs(1, 1, 1, 32, 96, 16)
+def test_bwd_head_dim_128_needs_a_checkpoint_per_mini_batch(P):
+    c = P.synthetic.reference_test_inputs(1, 1, 1, 32, 128, 16)
     with pytest.raises(Exception, match="checkpoint_interval 1"):
-        run_bwd(P, c, torch.ones(1, 1, 32, 96), 16, 2)
+        run_bwd(P, c, torch.ones(1, 1, 32, 128), 16, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("B,H,K,N,ci", [(1, 2, 16, 4, 2), (2, 1, 7, 5, 3), (1, 2, 16, 6, 6)])
+def test_bwd_head_dim_96_with_coarser_checkpoints(P, B, H, K, N, ci, dtype):
+    """head_dim 96 with a checkpoint every ci mini-batches: the LDS-tile kernel re-simulates the state in LDS and keeps
+    the state gradient in the d_W0 buffer."""
+    print(f"case bwd d96 ci{ci} B{B} H{H} K{K} N{N} {dtype}", flush=True)
+    c = P.synthetic.reference_test_inputs(430 + B + K + N + ci, B, H, N * K, 96, K, io_dtype=dtype)
+    g = torch.Generator().manual_seed(12)
+    dO = torch.randn(B, H, N * K, 96, generator=g).to(dtype)
+    sg = (0.1 * torch.randn(B, H, 96, 96, generator=g), 0.1 * torch.randn(B, H, 96, generator=g))
+    compare(run_bwd(P, c, dO, K, ci, sg), oracle_bwd(c, dO, K, sg), TOL[dtype])
+    compare(run_bwd(P, c, dO, K, ci), oracle_bwd(c, dO, K), TOL[dtype])
+
+
+def test_bwd_f32_head_dim_128_longer_sequence(P):
+    """f32 I/O at head_dim 128 over 24 mini-batches and two batch entries (per-batch checkpoints read in place)."""
+    print("case bwd f32 d128 long", flush=True)
+    B, H, d, K, N = 2, 2, 128, 16, 24
+    c = P.synthetic.baseline_inputs(6, B, H, N * K, d, K, with_dout=True)
+    dO = c.pop("d_out")
+    compare(run_bwd(P, c, dO, K, 1), oracle_bwd(c, dO, K), 1e-4)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -184,7 +204,7 @@ def test_bwd_packed_checkpoints_change_nothing(P, B, H, d, K, N, waves, dtype):
     if (d > 64 or dtype == torch.float32) and waves == "1":
         pytest.skip("wide heads and f32 I/O have the feature-split kernel only")
     if d == 128 and dtype == torch.float32:
-        pytest.skip("no f32 backward at head_dim 128")
+        pytest.skip("f32 I/O at head_dim 128 reads f32 row-major checkpoints only")
     print(f"case bwd packed ckpt B{B} H{H} d{d} K{K} N{N} waves {waves} {dtype}", flush=True)
     c = P.synthetic.reference_test_inputs(500 + B + d + K + N, B, H, N * K, d, K, io_dtype=dtype)
     dv = to_dev(c)

@@ -365,10 +365,10 @@ int uses_two_cu_mlp(const ttt_desc* d, int n_problems, bool* yes) {
   return TTT_OK;
 }
 
-template <class T, int D, int MT = 1>
+template <class T, int D, int MT = 1, bool WG = false, bool DG = false>
 int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_linear_bwd_kernel<T, D, MT>;
-  constexpr size_t bytes = ttt::BwdLds<D, MT>::BYTES;
+  constexpr auto kern = ttt::ttt_linear_bwd_kernel<T, D, MT, WG, DG>;
+  constexpr size_t bytes = ttt::BwdLds<D, MT, WG, DG>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * MT), bytes, s, a);
@@ -426,6 +426,8 @@ int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
 struct LinearBwdChoice {
   enum Kind { LDS, REG } kind;
   int waves;
+  // LDS-tile kernel only: the state gradient lives in the d_W0 buffer / the state is read in place from its checkpoint
+  bool dw_global = false, w_global = false;
 };
 int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
   int rc = ttt_linear_supported(d);
@@ -450,8 +452,15 @@ int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
   if (packed && (d->checkpoint_interval != 1 || want_lds))
     return fail(TTT_ERR_UNSUPPORTED, "packed checkpoints need checkpoint_interval 1 and the register-resident kernels");
   if (d->checkpoint_interval == 1 && !want_lds) {
-    if (f32 && D == 128)
-      return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O has no kernel (bf16 I/O has)");
+    if (f32 && D == 128) {
+      // the f32 staging of the register-resident kernel does not fit a CU at head_dim 128: the LDS-tile kernel with
+      // the state read in place from the (row-major) checkpoints and the state gradient kept in d_W0
+      if (packed) return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim 128 with f32 I/O reads f32 row-major checkpoints only");
+      ch->kind = LinearBwdChoice::LDS;
+      ch->waves = 4;
+      ch->w_global = ch->dw_global = true;
+      return TTT_OK;
+    }
     int waves = d->kernel_hint & TTT_HINT_WAVES_MASK;
     const long units = (long)d->batch * d->heads;
     // bf16 at head_dim 64 between 257 and 512 units, f32 row-major checkpoints: two waves per unit.  Four waves per
@@ -467,11 +476,14 @@ int choose_linear_bwd(const ttt_desc* d, LinearBwdChoice* ch) {
     ch->waves = waves;
     return TTT_OK;
   }
-  if (D > 64)
+  // coarser checkpoints: the state is re-simulated in LDS.  head_dim 96: with the state gradient in d_W0 the rest
+  // fits; head_dim 128: the state alone leaves too little LDS for the tiles of a stage
+  if (D > 96)
     return fail(TTT_ERR_UNSUPPORTED, "ttt_linear_bwd: head_dim %d needs checkpoint_interval 1 (got %d)", D,
                 d->checkpoint_interval);
   ch->kind = LinearBwdChoice::LDS;
   ch->waves = 4;
+  ch->dw_global = D == 96;
   return TTT_OK;
 }
 
@@ -986,6 +998,8 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
        !aligned16(d_xk) || !aligned16(d_xv) || !aligned16(W_ckpt) || !aligned16(b_ckpt) ||
        ((size_t)a.seq_stride * D) % 8 != 0))
     return fail(TTT_ERR_SHAPE, "ttt_linear_bwd: tensors must be 16-byte aligned");
+  if ((ch.w_global || ch.dw_global) && (!aligned16(W_ckpt) || !aligned16(d_W0)))
+    return fail(TTT_ERR_SHAPE, "ttt_linear_bwd: W_ckpt and d_W0 must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   // accumulated outputs start from zero; a fill kernel (not a memset node) so the sequence
   // can be captured into a graph
@@ -999,6 +1013,10 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   const bool f32 = d->io_dtype == TTT_F32;
   const int waves = ch.waves;
   if (ch.kind == LinearBwdChoice::LDS) {
+    if (ch.w_global) return launch_linear_bwd<ttt::F32, 128, 1, true, true>(a, grid, s);
+    if (ch.dw_global)
+      return f32 ? launch_linear_bwd<ttt::F32, 96, 1, false, true>(a, grid, s)
+                 : launch_linear_bwd<ttt::BF16, 96, 1, false, true>(a, grid, s);
     if (d->mini_batch > 16)
       return f32 ? launch_linear_bwd<ttt::F32, 32, 2>(a, grid, s) : launch_linear_bwd<ttt::BF16, 32, 2>(a, grid, s);
     if (f32) return D == 64 ? launch_linear_bwd<ttt::F32, 64>(a, grid, s) : launch_linear_bwd<ttt::F32, 32>(a, grid, s);

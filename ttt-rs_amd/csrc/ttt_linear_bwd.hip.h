@@ -52,7 +52,10 @@ struct LinearBwdArgs {
 
 // MT tiles of 16 token rows: mini_batch <= KT = 16 MT.  MT = 2 serves the reference's (mini_batch 32, head_dim 32)
 // tile (rust/fused/src/linear_fused_tile/mod.rs:38).
-template <int D, int MT = 1>
+// WG: the state W of a mini-batch is read in place from its checkpoint in global memory (one checkpoint per
+// mini-batch); DG: the state gradient dW lives in the d_W0 output buffer for the whole scan.  With both, head_dim 128
+// fits: LDS then holds only the tiles of a stage.
+template <int D, int MT = 1, bool WG = false, bool DG = false>
 struct BwdLds {
   static constexpr int KT = 16 * MT;
   static constexpr int LD = D + 4;     // padded row stride (floats) of every [*, D] array
@@ -61,8 +64,8 @@ struct BwdLds {
   static constexpr int WSZ = D * LD;
   static constexpr int KK = KT * LK;
   // offsets in floats
-  static constexpr int W = 0, dW = W + WSZ;
-  static constexpr int XQ = dW + WSZ, XK = XQ + TILE, TG = XK + TILE, DO = TG + TILE, XH = DO + TILE,
+  static constexpr int W = 0, dW = W + (WG ? 0 : WSZ);
+  static constexpr int XQ = dW + (DG ? 0 : WSZ), XK = XQ + TILE, TG = XK + TILE, DO = TG + TILE, XH = DO + TILE,
                        G = XH + TILE, XH2 = G + TILE, DZB = XH2 + TILE, S = DZB + TILE,
                        TMP = S + TILE, DK = TMP + TILE, DZ1 = DK + TILE, DQ = DZ1 + TILE,
                        DGM = DQ + TILE;
@@ -74,11 +77,11 @@ struct BwdLds {
   static constexpr size_t BYTES = sizeof(float) * END;
 };
 
-template <class T, int D, int MT = 1>
+template <class T, int D, int MT = 1, bool WG = false, bool DG = false>
 __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using elem = typename IO::elem;
-  using L = BwdLds<D, MT>;
+  using L = BwdLds<D, MT, WG, DG>;
   constexpr int LD = L::LD, LK = L::LK, KT = L::KT, NJ = D / 16, NTH = 256 * MT, NW = 4 * MT;
   constexpr int NB2 = NJ >= 2 ? 2 : 1;  // tile columns per job of a [16 x D] product
   constexpr float inv_d = 1.0f / D;
@@ -91,7 +94,19 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
   const int K = a.K;
 
   float* sW = lds + L::W;
-  float* sdW = lds + L::dW;
+  // W(k, n) = Wp[k * wld + n]: the LDS copy, or (WG) the checkpoint of the mini-batch itself, set per stage
+  const float* Wp = sW;
+  constexpr int wld = WG ? D : LD;
+  // dW likewise: LDS, or (DG) the caller's d_W0 buffer of this unit
+  float* sdW = DG ? a.d_W0 + bh * (size_t)D * D : lds + L::dW;
+  constexpr int dld = DG ? D : LD;
+  // stores to dW in global memory must have landed before another wave reads them: a full barrier then
+  auto bar = [&]() {
+    if constexpr (WG || DG)
+      __syncthreads();
+    else
+      lds_barrier();
+  };
   float* sb = lds + L::b;
   float* sdb = lds + L::db;
   float* sgam = lds + L::gam;
@@ -107,7 +122,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
   }
   for (int i = tid; i < D * D; i += NTH) {
     const int r = i / D, cc = i - r * D;
-    sdW[r * LD + cc] = a.d_W_out ? a.d_W_out[bh * D * D + i] : 0.f;
+    sdW[r * dld + cc] = a.d_W_out ? a.d_W_out[bh * D * D + i] : 0.f;
   }
   if (tid < KT) ste[tid] = (tid < K) ? a.token_eta[tid] : 0.f;
   float dgam_acc[NJ], dbet_acc[NJ];
@@ -164,7 +179,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
   // and only copied into LDS at the top of that stage.  Thread tid owns EP contiguous elements of
   // each [16 x D] tile and WP float4 pieces of the checkpoint.
   constexpr int EP = D / 16;          // KT*D elements / NTH threads
-  constexpr int WP = (D * D + 4 * NTH - 1) / (4 * NTH);  // float4 pieces of the checkpoint per thread
+  constexpr int WP = WG ? 1 : (D * D + 4 * NTH - 1) / (4 * NTH);  // float4 pieces of the checkpoint per thread
   constexpr bool WALL = D * D % (4 * NTH) == 0;          // every thread has all WP pieces
   const int pt = (tid * EP) / D, pc = (tid * EP) % D;  // token row / first feature of this thread's piece
   struct Prefetch {
@@ -180,8 +195,10 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
   auto fetch_stage = [&](int stage) {
     const int ckp = stage / a.ckpt_interval;
     const f32x4* Wg = reinterpret_cast<const f32x4*>(a.W_ckpt + (bh * a.n_ckpt + ckp) * D * D);
+    if constexpr (!WG) {
 #pragma unroll
-    for (int i = 0; i < WP; ++i) pre.w[i] = Wg[(WALL || 4 * (tid + NTH * i) < D * D) ? tid + NTH * i : 0];
+      for (int i = 0; i < WP; ++i) pre.w[i] = Wg[(WALL || 4 * (tid + NTH * i) < D * D) ? tid + NTH * i : 0];
+    }
     pre.b = (tid < D) ? a.b_ckpt[(bh * a.n_ckpt + ckp) * D + tid] : 0.f;
     pre.lr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
     fetch_tile(pre.q, a.xq, stage);
@@ -190,10 +207,12 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
     fetch_tile(pre.o, a.d_out, stage);
   };
   auto commit_state = [&]() {
+    if constexpr (!WG) {
 #pragma unroll
-    for (int i = 0; i < WP; ++i) {
-      const int idx = (tid + NTH * i) * 4;
-      if (WALL || idx < D * D) *reinterpret_cast<f32x4*>(sW + (idx / D) * LD + (idx % D)) = pre.w[i];
+      for (int i = 0; i < WP; ++i) {
+        const int idx = (tid + NTH * i) * 4;
+        if (WALL || idx < D * D) *reinterpret_cast<f32x4*>(sW + (idx / D) * LD + (idx % D)) = pre.w[i];
+      }
     }
     if (tid < D) sb[tid] = pre.b;
   };
@@ -212,17 +231,18 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
   for (int st = a.n_stages - 1; st >= 0; --st) {
     // ================= state entering stage st: checkpoint + re-simulated updates
     const int ck = st / a.ckpt_interval;
+    if constexpr (WG) Wp = a.W_ckpt + (bh * a.n_ckpt + st) * (size_t)D * D;  // checkpoint_interval is 1
     commit_state();
     for (int s2 = ck * a.ckpt_interval; s2 < st; ++s2) {
-      lds_barrier();
+      bar();
       load_tile(lds + L::XK, a.xk, s2);
       load_tile(lds + L::TG, a.xv, s2);
       load_lr(s2);
-      lds_barrier();
+      bar();
 #pragma unroll
       for (int j = 0; j < NJ; ++j) lds[L::TG + t * LD + cg + 16 * j] -= lds[L::XK + t * LD + cg + 16 * j];
       mm_lds<0, NW>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane);
-      lds_barrier();
+      bar();
       {
         float xh[NJ], Gv[NJ], rstd;
         ln1(lds + L::XH, lds + L::TG, xh, Gv, rstd);
@@ -230,7 +250,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
 #pragma unroll
         for (int j = 0; j < NJ; ++j) lds[L::G + t * LD + cg + 16 * j] = Gv[j] * last;
       }
-      lds_barrier();
+      bar();
       // W -= XK^T (last * G) ; b -= colsum(last * G)      (linear.rs:134-144)
       mm_lds<2, NW, NJ, 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, KT, wave, lane);
       if (tid < D) {
@@ -239,19 +259,19 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
         sb[tid] -= s;
       }
     }
-    if (ck * a.ckpt_interval < st) lds_barrier();  // the re-simulation used the XK / target tiles
+    if (ck * a.ckpt_interval < st) bar();  // the re-simulation used the XK / target tiles
 
     // ================= this stage's tiles (target = XV - XK formed on the way), then prefetch the next
     commit_tiles();
-    lds_barrier();
+    bar();
     if (st > 0) fetch_stage(st - 1);
     // Z1 = XK W ; Zq = XQ W ; A = XQ XK^T
     // every product is cut into jobs of NB2 tile columns: two or more accumulator chains per wave keep the
     // matrix pipe busy (a single chain waits out the full MFMA latency between dependent steps)
-    mm_lds<0, NW, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane, 0);
-    mm_lds<0, NW, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane, 2);
+    mm_lds<0, NW, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, Wp, wld, 1, MT, NJ, D, wave, lane, 0);
+    mm_lds<0, NW, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, Wp, wld, 1, MT, NJ, D, wave, lane, 2);
     mm_lds<0, NW>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, MT, MT, D, wave, lane, 1);
-    lds_barrier();
+    bar();
 
     // ================= forward intermediates: x_hat, rstd, G; eta, A (tril), M = eta (1 + A)
     float xh[NJ], Gv[NJ], rstd1;
@@ -271,10 +291,10 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
       lds[L::ETA + t * LK + s] = et;
       lds[L::M + t * LK + s] = et * (1.f + at);
     }
-    lds_barrier();
+    bar();
     // Zb = XQ W - M G  (+ b added when read)
     mm_lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, MT, NJ, KT, wave, lane);
-    lds_barrier();
+    bar();
 
     // ================= output LayerNorm and its backward (stage 4)
     {
@@ -309,14 +329,15 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
 #pragma unroll
       for (int j = 0; j < NJ; ++j) lds[L::DZB + t * LD + cg + 16 * j] = (gx2[j] - s1 - zv[j] * s2) * rstd2;
     }
-    lds_barrier();
+    bar();
 
     // ================= P = dZb G^T ; dQ = dZb W^T ; S = XK dW ; TMP = G dW^T
-    mm_lds<0, NW, NB2>(lds + L::DQ, LD, lds + L::DZB, LD, 1, sW, 1, LD, MT, NJ, D, wave, lane, 0);
-    mm_lds<0, NW, NB2>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, LD, MT, NJ, D, wave, lane, 0);
-    mm_lds<0, NW, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, LD, 1, MT, NJ, D, wave, lane, 2);
+    // a transposed matrix in global memory is contiguous along k: loaded four lanes to a row (BG)
+    mm_lds<0, NW, NB2, 4, WG>(lds + L::DQ, LD, lds + L::DZB, LD, 1, Wp, 1, wld, MT, NJ, D, wave, lane, 0);
+    mm_lds<0, NW, NB2, 4, DG>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, dld, MT, NJ, D, wave, lane, 0);
+    mm_lds<0, NW, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, dld, 1, MT, NJ, D, wave, lane, 2);
     mm_lds<0, NW>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, MT, MT, D, wave, lane, 3);
-    lds_barrier();
+    bar();
 
     // ================= dA, d eta ; S += db ; dlast
     {
@@ -338,13 +359,13 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
       dl = row16_sum(dl);
       if (cg == 0) lds[L::dlast + t] = -dl;
     }
-    lds_barrier();
+    bar();
 
     // ================= dQ += dA XK ; dK = dA^T XQ ; DGM = M^T dZb ; dW += XQ^T dZb ; db += colsum(dZb)
     mm_lds<1, NW, NJ, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, MT, NJ, KT, wave, lane, 0);
     mm_lds<0, NW, NJ, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, MT, NJ, KT, wave, lane, 1);
     mm_lds<0, NW, NJ, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, MT, NJ, KT, wave, lane, 2);
-    mm_lds<1, NW, NJ, 4>(sdW, LD, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, KT, wave, lane);
+    mm_lds<1, NW, NJ, 4>(sdW, dld, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < KT; ++r) s += lds[L::DZB + r * LD + tid];
@@ -364,7 +385,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
         for (int r = 0; r < KT; ++r) s += lds[L::dlast + r] * slr[r];
       if (tt < K) atomicAdd(a.d_token_eta + (size_t)st * K + tt, s);
     }
-    lds_barrier();
+    bar();
 
     // ================= through G: second-order LayerNorm (stage 2), token-local
     {
@@ -408,17 +429,17 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
         lds[L::DK + t * LD + o] += dy[j] - last * lds[L::TMP + t * LD + o];
       }
     }
-    lds_barrier();
+    bar();
 
     // ================= dK += dZ1 W^T ; dW += XK^T dZ1 ; db += colsum(dZ1)
-    mm_lds<1, NW, NB2>(lds + L::DK, LD, lds + L::DZ1, LD, 1, sW, 1, LD, MT, NJ, D, wave, lane, 2);
-    mm_lds<1, NW, NJ, 4>(sdW, LD, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, KT, wave, lane);
+    mm_lds<1, NW, NB2, 4, WG>(lds + L::DK, LD, lds + L::DZ1, LD, 1, Wp, 1, wld, MT, NJ, D, wave, lane, 2);
+    mm_lds<1, NW, NJ, 4>(sdW, dld, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < KT; ++r) s += lds[L::DZ1 + r * LD + tid];
       sdb[tid] += s;
     }
-    lds_barrier();
+    bar();
 
     // ================= store dXQ = dO + dQ, dXK
     if (t < K) {
@@ -431,13 +452,15 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
         IO::store1(pk + o, lds[L::DK + t * LD + o]);
       }
     }
-    lds_barrier();
+    bar();
   }
 
   // ---- results carried over the whole scan
-  for (int i = tid; i < D * D; i += NTH) {
-    const int r = i / D, cc = i - r * D;
-    a.d_W0[bh * D * D + i] = sdW[r * LD + cc];
+  if constexpr (!DG) {
+    for (int i = tid; i < D * D; i += NTH) {
+      const int r = i / D, cc = i - r * D;
+      a.d_W0[bh * D * D + i] = sdW[r * LD + cc];
+    }
   }
   if (tid < D) a.d_b0[bh * D + tid] = sdb[tid];
 #pragma unroll
