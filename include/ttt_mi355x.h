@@ -130,7 +130,8 @@ int ttt_linear_supported(const ttt_desc* desc);
  * (rust/fused/src/linear_fused_tile/forward/launch.rs:221-226). */
 int64_t ttt_linear_num_checkpoints(const ttt_desc* desc);
 /* TTT_OK if ttt_linear_bwd has a kernel for this desc (it supports fewer combinations than the forward:
- * checkpoint_interval > 1 only for head_dim <= 64, head_dim 128 only with bf16 I/O), else the status
+ * checkpoint_interval > 1 only for head_dim <= 96; f32 I/O at head_dim 128 and mini_batch > 16 with f32 row-major
+ * checkpoints only), else the status
  * ttt_linear_bwd would return.  A training caller asks this before the forward, as the reference asks
  * FusedTttConfig::is_supported (rust/fused/src/lib.rs:313-322) before it builds the layer. */
 int ttt_linear_bwd_supported(const ttt_desc* desc);
