@@ -404,20 +404,47 @@ __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int
   int job = wave;
   if (job >= njobs) return;
   const int last = job + ((njobs - 1 - job) / NW) * NW;  // this wave's last job
-  Set s0, s1;
-  request(job, s0);
+  if constexpr (BF) {
+    // With bf16 operands the matrix instructions of a job no longer cover a memory round trip: two jobs are kept in
+    // flight while a third is finished (three named sets; the ordering argument above holds unchanged: every request
+    // of a job not yet finished reads tiles that no store in flight touches, and what is re-requested past the end is
+    // never used).
+    Set s0, s1, s2;
+    auto at = [&](int j) { return j <= last ? j : last; };
+    request(job, s0);
+    request(at(job + NW), s1);
 #pragma nounroll
-  for (;;) {
-    const int j1 = job + NW, j2 = job + 2 * NW;
-    request(j1 <= last ? j1 : last, s1);
-    __builtin_amdgcn_sched_barrier(0);
-    finish(job, s0);
-    if (j1 > last) break;
-    request(j2 <= last ? j2 : last, s0);
-    __builtin_amdgcn_sched_barrier(0);
-    finish(j1, s1);
-    if (j2 > last) break;
-    job = j2;
+    for (;;) {
+      request(at(job + 2 * NW), s2);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(job, s0);
+      if (job + NW > last) break;
+      request(at(job + 3 * NW), s0);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(job + NW, s1);
+      if (job + 2 * NW > last) break;
+      request(at(job + 4 * NW), s1);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(job + 2 * NW, s2);
+      if (job + 3 * NW > last) break;
+      job += 3 * NW;
+    }
+  } else {
+    Set s0, s1;
+    request(job, s0);
+#pragma nounroll
+    for (;;) {
+      const int j1 = job + NW, j2 = job + 2 * NW;
+      request(j1 <= last ? j1 : last, s1);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(job, s0);
+      if (j1 > last) break;
+      request(j2 <= last ? j2 : last, s0);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(j1, s1);
+      if (j2 > last) break;
+      job = j2;
+    }
   }
   if (FZ) {
     const int zoff = 4 * g * ldz + 16 * (wave % nblk) * NB + c;

@@ -164,11 +164,28 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   __syncthreads();
   const float te_last = ste[K - 1];
 
-  auto load_tile = [&](float* dst, const void* src, int stage) {
-    const elem* p = static_cast<const elem*>(src) + (bh * (size_t)a.seq_stride + (size_t)stage * K + t) * D;
+  // the four activation tiles and the learning rates of the next mini-batch to be processed, in registers
+  struct {
+    float q[NJD], k[NJD], v[NJD], o[NJD], lr;
+  } pre;
+  auto fetch_inputs = [&](int stage) {
+    const size_t r = (bh * (size_t)a.seq_stride + (size_t)stage * K + (t < K ? t : 0)) * D;
+    const bool ok = t < K;
 #pragma unroll
-    for (int j = 0; j < NJD; ++j) dst[t * LD + cg + GW * j] = (t < K) ? IO::load1(p + cg + GW * j) : 0.f;
+    for (int j = 0; j < NJD; ++j) {
+      const float q = IO::load1(static_cast<const elem*>(a.xq) + r + cg + GW * j);
+      const float k = IO::load1(static_cast<const elem*>(a.xk) + r + cg + GW * j);
+      const float v = IO::load1(static_cast<const elem*>(a.xv) + r + cg + GW * j);
+      const float o = IO::load1(static_cast<const elem*>(a.d_out) + r + cg + GW * j);
+      pre.q[j] = ok ? q : 0.f, pre.k[j] = ok ? k : 0.f, pre.v[j] = ok ? v : 0.f, pre.o[j] = ok ? o : 0.f;
+    }
+    const int tl = (tid < K) ? tid : 0;
+    const float l = IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tl);
+    pre.lr = (tid < K) ? l : 0.f;
   };
+  // at head_dim 128 the kernel is at the register limit: there the tiles are fetched where they are needed
+  constexpr bool PFIN = D <= 96;
+  if constexpr (PFIN) fetch_inputs(N - 1);
   // C[16 x 16] (PART slices) = X Y^T over the 4d columns of two [16 x 4d] tiles, one k-slice per wave
   auto splitk_xyT = [&](const float* X, const float* Y) {
     const int c = lane & 15, g = lane >> 4;
@@ -237,16 +254,19 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     const float* G2l = a.G2s + ((bh * N + st) * (size_t)16) * D;
     const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
 
-    // ---- 1. inputs of this mini-batch
-    load_tile(lds + L::XQ, a.xq, st);
-    load_tile(lds + L::XK, a.xk, st);
-    load_tile(lds + L::TG, a.xv, st);
-    load_tile(lds + L::DO, a.d_out, st);
-    if (tid < 16)
-      slr[tid] = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)st * K + tid) : 0.f;
-    __syncthreads();
+    // ---- 1. inputs of this mini-batch (fetched while the previous one was computed); target = XV - XK
+    if constexpr (!PFIN) fetch_inputs(st);
 #pragma unroll
-    for (int j = 0; j < NJD; ++j) lds[L::TG + t * LD + cg + GW * j] -= lds[L::XK + t * LD + cg + GW * j];
+    for (int j = 0; j < NJD; ++j) {
+      const int o = t * LD + cg + GW * j;
+      lds[L::XQ + o] = pre.q[j];
+      lds[L::XK + o] = pre.k[j];
+      lds[L::TG + o] = pre.v[j] - pre.k[j];
+      lds[L::DO + o] = pre.o[j];
+    }
+    if (tid < 16) slr[tid] = pre.lr;
+    __syncthreads();
+    if constexpr (PFIN) fetch_inputs(st > 0 ? st - 1 : 0);  // always: a load under a branch weakens every later wait
     const float last = te_last * slr[t];
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
     // Z1 = XK W1 (step 3) rides along on the rolled-back tiles
