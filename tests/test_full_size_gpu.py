@@ -226,6 +226,46 @@ def test_config3_mlp_fwd_bf16_full(P):
             assert_close(gv[bs][:, hs], rv, TOL[torch.bfloat16], name)
 
 
+def test_config3_mlp_fwd_bwd_bf16_full(P):
+    """The TTT-MLP forward+backward as benchmarked (config-3 shape, bf16 I/O: register-resident sweep, bf16 operands in
+    the reverse scan), 128 chained mini-batches.  The gradients that belong to a unit are compared with the oracle on a
+    slice of units of the full call; the three that are sums over units (d_token_eta, d_gamma, d_beta) on a call of
+    that slice alone, which must also reproduce the per-unit gradients of the full call bit for bit (units are
+    independent)."""
+    B, H, d, seq, K = 8, 16, 96, 2048, 16
+    print("case config3 fwd+bwd full", flush=True)
+    c = P.synthetic.baseline_inputs(3, B, H, seq, d, K, io_dtype=torch.bfloat16, mlp=True, with_dout=True)
+    dv = dev(c)
+    run = lambda x: P.ttt_mlp_backward_raw(x["xq"], x["xk"], x["xv"], x["W1"], x["b1"], x["W2"], x["b2"], x["token_eta"],
+                                           x["lr"], x["gamma"], x["beta"], x["d_out"], K)
+    full = run(dv)
+    torch.cuda.synchronize()
+    for k, v in full.items():
+        assert torch.isfinite(v.float()).all(), k
+    bs, hs = [5], [0, 15]
+    per_bh, per_h = ("xq", "xk", "xv", "lr", "d_out"), ("W1", "b1", "W2", "b2", "gamma", "beta")
+    one = {k: dv[k][bs][:, hs].contiguous() for k in per_bh}
+    one.update({k: dv[k][hs].contiguous() for k in per_h})
+    one["token_eta"] = dv["token_eta"]
+    part = run(one)
+    torch.cuda.synchronize()
+    per_unit = ("d_xq", "d_xk", "d_xv", "d_W1", "d_b1", "d_W2", "d_b2", "d_lr")
+    for k in per_unit:
+        assert torch.equal(full[k][bs][:, hs], part[k]), f"{k}: a unit's gradient depends on the other units"
+    n = sub(c, bs, hs)
+    ref = orc.mlp_backward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                           n["gamma"], n["beta"], n["d_out"], K=K)
+    tol = TOL[torch.bfloat16]
+    for k in per_unit + ("d_token_eta", "d_gamma", "d_beta"):
+        g, r = to_np(part[k]), to_np(ref[k])
+        rel = np.abs(g - r).max() / np.abs(r).max()
+        print(f"  {k}: max-norm relative error {rel:.3e}", flush=True)
+        assert rel <= tol, f"{k}: max-norm relative error {rel:.3e} > {tol}"
+    # elementwise band where the tensors are not sums of thousands of bf16-rounded rows
+    for k in ("d_xq", "d_xk", "d_xv"):
+        assert_close(part[k], ref[k], tol, k, min_frac=0.99)
+
+
 def test_config4_layers_d128_seq8192(P):
     """One TTT-Linear and one TTT-MLP layer of the long-context stack at its real shape
     (512 chained mini-batches), checked on a slice of units."""
