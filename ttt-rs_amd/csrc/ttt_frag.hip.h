@@ -220,14 +220,16 @@ struct Io<BF16> {
     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
   }
   __device__ static __forceinline__ void load8(const elem* p, bool ok, frag& lo, frag& hi) {
-    u32x4 v = ok ? *reinterpret_cast<const u32x4*>(p) : u32x4{0u, 0u, 0u, 0u};
+    // activation tiles are read once per pass and written once: marked non-temporal (the `nt` bit), so that they do
+    // not displace the state and the checkpoints in L2
+    u32x4 v = ok ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)) : u32x4{0u, 0u, 0u, 0u};
     lo = __builtin_bit_cast(frag, u32x2{v[0], v[1]});
     hi = __builtin_bit_cast(frag, u32x2{v[2], v[3]});
   }
   __device__ static __forceinline__ void store8(elem* p, f32x4 lo, f32x4 hi) {
     u32x2 a = __builtin_bit_cast(u32x2, to_frag(lo));
     u32x2 b = __builtin_bit_cast(u32x2, to_frag(hi));
-    *reinterpret_cast<u32x4*>(p) = u32x4{a[0], a[1], b[0], b[1]};
+    __builtin_nontemporal_store(u32x4{a[0], a[1], b[0], b[1]}, reinterpret_cast<u32x4*>(p));
   }
   __device__ static __forceinline__ float load1(const elem* p) {
     return __builtin_bit_cast(float, static_cast<uint32_t>(*p) << 16);
