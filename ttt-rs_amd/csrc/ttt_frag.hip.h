@@ -220,8 +220,10 @@ struct Io<BF16> {
     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
   }
   __device__ static __forceinline__ void load8(const elem* p, bool ok, frag& lo, frag& hi) {
-    // activation tiles are read once per pass and written once: marked non-temporal (the `nt` bit), so that they do
-    // not displace the state and the checkpoints in L2
+    // activation tiles are read once per pass: loaded non-temporal (the `nt` bit), so that they do not displace the
+    // state and the checkpoints in L2.  (The stores stay plain: a token's row is written by several waves, 64 bytes
+    // each, and streaming stores are not always merged into one line on their way out: 20 % more bytes written for
+    // no measurable gain.)
     u32x4 v = ok ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)) : u32x4{0u, 0u, 0u, 0u};
     lo = __builtin_bit_cast(frag, u32x2{v[0], v[1]});
     hi = __builtin_bit_cast(frag, u32x2{v[2], v[3]});
@@ -229,7 +231,7 @@ struct Io<BF16> {
   __device__ static __forceinline__ void store8(elem* p, f32x4 lo, f32x4 hi) {
     u32x2 a = __builtin_bit_cast(u32x2, to_frag(lo));
     u32x2 b = __builtin_bit_cast(u32x2, to_frag(hi));
-    __builtin_nontemporal_store(u32x4{a[0], a[1], b[0], b[1]}, reinterpret_cast<u32x4*>(p));
+    *reinterpret_cast<u32x4*>(p) = u32x4{a[0], a[1], b[0], b[1]};
   }
   __device__ static __forceinline__ float load1(const elem* p) {
     return __builtin_bit_cast(float, static_cast<uint32_t>(*p) << 16);
