@@ -399,7 +399,8 @@ int ttt_linear_fwd_fused_inputs(const ttt_desc* desc, const void* xq, const void
  * [H,out_i] or [B,H,out_i] (state_per_batch selects; in_0 = out_last = d, every other side 4 d); W_out, b_out: the
  * same shapes per batch element, also the live state during the call (W_out[i] must not alias W0[i]).
  * Products are f32 for both I/O types.  head_dim 32 with 2 - 4 hidden layers, head_dim 64 with 2 (what fits the
- * LDS of a CU); ttt_mlpn_supported says so beforehand.  One hidden layer is ttt_mlp_fwd.
+ * LDS of a CU); ttt_mlpn_supported says so beforehand.  One hidden layer is ttt_mlp_fwd.  desc.seq_stride is
+ * honoured (a window of a longer sequence in place).
  */
 int ttt_mlpn_supported(const ttt_desc* desc, int n_hidden);
 int ttt_mlpn_fwd(const ttt_desc* desc, int n_hidden, const void* xq, const void* xk, const void* xv,

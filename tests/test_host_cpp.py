@@ -137,3 +137,57 @@ def test_cpp_host_state_buffers_across_a_forward_with_remainder(tmp_path):
     subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-I", ROOT, str(src), "-o", str(exe)], check=True)
     r = subprocess.run([str(exe)], capture_output=True, text=True)
     assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+
+
+def test_cpp_other_inner_models_compile_and_report_errors(tmp_path):
+    """host/fused_others.hpp (TTTLinearAdam, TTTMLP2/3/4): names as the reference's, incomplete states refused by the
+    classes, unsupported shapes and null tensors by the library, all before any launch."""
+    import importlib
+    P = importlib.import_module("ttt-rs_amd")
+    src = tmp_path / "o.cpp"
+    src.write_text(textwrap.dedent(r'''
+        #include <cstring>
+        #include "ttt-rs_amd/host/fused_others.hpp"
+        int main() {
+          ttt::ModelConfig cfg; cfg.num_heads = 2; cfg.head_dim = 64;
+          alignas(16) float dummy[4] = {0.f, 0.f, 0.f, 0.f};
+          alignas(16) char out[16];
+          ttt::TTTInputsInner in; in.batch = 2; in.seq_len = 32;
+          ttt::FusedLinearAdam adam(cfg, ttt::TTTLinearAdamConfig{}, dummy, dummy, dummy, dummy);
+          if (std::strcmp(adam.name(), "TTTLinearAdam")) return 1;
+          ttt::TTTLinearAdamState as;
+          try { adam.forward(as, in, out, nullptr); return 2; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 3; }
+          as.weight = as.bias = as.weight_m = as.bias_m = as.weight_v = as.bias_v = dummy;
+          as.next_weight = as.next_bias = as.next_weight_m = as.next_bias_m = as.next_weight_v = as.next_bias_v = dummy;
+          try { adam.forward_mini_batch(as, in, 0, 17, out, nullptr); return 4; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_SHAPE) return 5; }
+          try { adam.forward(as, in, out, nullptr); return 6; }          // null activations
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 7; }
+          if (as.initialised || as.step != 0) return 8;                    // a refused call leaves the state alone
+          const float* layers[5] = {dummy, dummy, dummy, dummy, dummy};
+          try { ttt::FusedMlpN bad(cfg, 5, layers, layers, dummy, dummy); return 9; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_UNSUPPORTED) return 10; }
+          ttt::FusedMlpN m3(cfg, 3, layers, layers, dummy, dummy);         // head_dim 64 has two hidden layers only
+          if (std::strcmp(m3.name(), "TTTMLP3")) return 11;
+          ttt::TTTMLPNState ms;
+          try { m3.forward(ms, in, out, nullptr); return 12; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 13; }
+          for (int i = 0; i < 4; ++i) ms.weight[i] = ms.bias[i] = ms.next_weight[i] = ms.next_bias[i] = dummy;
+          try { m3.forward(ms, in, out, nullptr); return 14; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_UNSUPPORTED) return 15; }
+          cfg.head_dim = 32;
+          ttt::FusedMlpN m4(cfg, 4, layers, layers, dummy, dummy);
+          if (std::strcmp(m4.name(), "TTTMLP4")) return 16;
+          for (int i = 0; i < 5; ++i) ms.weight[i] = ms.bias[i] = ms.next_weight[i] = ms.next_bias[i] = dummy;
+          try { m4.forward(ms, in, out, nullptr); return 17; }            // supported shape, null activations
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 18; }
+          return 0;
+        }
+    '''))
+    exe = tmp_path / "o"
+    libdir = os.path.dirname(P.LIB_PATH)
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-I", ROOT, str(src), "-o", str(exe),
+                    "-L", libdir, "-lttt_mi355x", f"-Wl,-rpath,{libdir}"], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)

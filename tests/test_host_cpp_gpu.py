@@ -196,3 +196,71 @@ def test_cpp_lost_workgroup_guard(P, drv):
     torch.cuda.synchronize()
     assert drv.ttt_host_lost_guard_verify_and_free(g) == P.TTT_ERR_HIP
     assert b"partner" in drv.ttt_host_last_error()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_cpp_linear_adam_forward_with_remainder_equals_python_mirror(P, drv, dtype):
+    """FusedLinearAdam of host/fused_others.hpp: full mini-batches in one launch, the remainder as one short mini-batch
+    that continues from the moments and the step count, both as in-place windows of the sequence."""
+    B, H, d, K, seq = 2, 2, 64, 16, 16 * 3 + 5
+    print(f"case host C++ linear-adam forward+remainder {dtype}", flush=True)
+    c = to_dev(P.synthetic.reference_test_inputs(23, B, H, seq, d, K, io_dtype=dtype))
+    te_seq = c["token_eta"].repeat(seq // K + 1)[:seq].contiguous()
+    hp = P.TTTLinearAdamConfig(beta1=0.8, beta2=0.95, epsilon=1e-7, lr=5e-3)
+    model = P.FusedLinearAdam(P.ModelConfig(H, d, P.TTTConfig(mini_batch_size=K)), hp, c["W0"], c["b0"], c["gamma"],
+                              c["beta"])
+    state = model.init_state(B)
+    ref = model.forward(state, P.TTTInputsInner(P.Qkv(c["xq"], c["xk"], c["xv"]), te_seq, c["lr"]))
+    nan = lambda *s: torch.full(s, float("nan"), device="cuda:0")
+    sets = [[nan(B, H, d, d), nan(B, H, d), nan(B, H, d, d), nan(B, H, d), nan(B, H, d, d), nan(B, H, d)] for _ in range(2)]
+    arr = lambda ts: (C.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    out = torch.full_like(c["xq"], float("nan"))
+    cur, step = C.c_int(-1), C.c_int(-1)
+    rc = drv.ttt_host_linear_adam_forward(B, H, d, K, seq, dt(P, c["xq"]), C.c_float(1e-6), C.c_float(hp.beta1),
+                                          C.c_float(hp.beta2), C.c_float(hp.epsilon), C.c_float(hp.lr), ptr(c["W0"]),
+                                          ptr(c["b0"]), ptr(c["gamma"]), ptr(c["beta"]), ptr(c["xq"]), ptr(c["xk"]),
+                                          ptr(c["xv"]), ptr(te_seq), ptr(c["lr"]), ptr(out), arr(sets[0]), arr(sets[1]),
+                                          C.byref(cur), C.byref(step),
+                                          C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert rc == P.TTT_OK, drv.ttt_host_last_error()
+    assert cur.value == 0 and step.value == state.step == 4   # two launches: back in the first set
+    assert torch.equal(out, ref)
+    got = sets[0]
+    for g, r, name in zip(got, (state.weight, state.bias, state.weight_m, state.bias_m, state.weight_v, state.bias_v),
+                          ("weight", "bias", "weight_m", "bias_m", "weight_v", "bias_v")):
+        assert torch.equal(g, r), name
+
+
+@pytest.mark.parametrize("n_hidden,d", [(2, 32), (4, 32), (2, 64)])
+def test_cpp_mlpn_forward_with_remainder_equals_python_mirror(P, drv, n_hidden, d):
+    """FusedMlpN of host/fused_others.hpp against the Python mirror, sequence with a remainder (the C++ class works on
+    windows of the sequence in place, the Python mirror on copies of the slices)."""
+    from test_mlpn_gpu import make_case
+    B, H, K, seq = 2, 2, 16, 16 * 2 + 7
+    print(f"case host C++ mlp{n_hidden} d{d} forward+remainder", flush=True)
+    c, Ws, bs = make_case(P, 31 + n_hidden, B, H, seq, d, K, n_hidden, torch.bfloat16)
+    c = to_dev(c)
+    Ws, bs = [w.to("cuda:0") for w in Ws], [b.to("cuda:0") for b in bs]
+    te_seq = c["token_eta"].repeat(seq // K + 1)[:seq].contiguous()
+    model = P.FusedMlpN(P.ModelConfig(H, d, P.TTTConfig(mini_batch_size=K)), Ws, bs, c["gamma"], c["beta"])
+    assert model.name() == f"TTTMLP{n_hidden}"
+    state = model.init_state(B)
+    ref = model.forward(state, P.TTTInputsInner(P.Qkv(c["xq"], c["xk"], c["xv"]), te_seq, c["lr"]))
+    nan = lambda *s: torch.full(s, float("nan"), device="cuda:0")
+    wa, wb = [nan(B, *w.shape) for w in Ws], [nan(B, *w.shape) for w in Ws]
+    ba, bb = [nan(B, *b.shape) for b in bs], [nan(B, *b.shape) for b in bs]
+    arr = lambda ts: (C.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    out = torch.full_like(c["xq"], float("nan"))
+    cur = C.c_int(-1)
+    rc = drv.ttt_host_mlpn_forward(B, H, d, K, seq, dt(P, c["xq"]), C.c_float(1e-6), n_hidden, arr(Ws), arr(bs),
+                                   ptr(c["gamma"]), ptr(c["beta"]), ptr(c["xq"]), ptr(c["xk"]), ptr(c["xv"]), ptr(te_seq),
+                                   ptr(c["lr"]), ptr(out), arr(wa), arr(ba), arr(wb), arr(bb), C.byref(cur),
+                                   C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert rc == P.TTT_OK, drv.ttt_host_last_error()
+    assert cur.value == 0
+    assert torch.equal(out, ref)
+    for i in range(n_hidden + 1):
+        assert torch.equal(wa[i], state.weights[i]), f"weight {i}"
+        assert torch.equal(ba[i], state.biases[i]), f"bias {i}"

@@ -768,8 +768,6 @@ int ttt_mlpn_supported(const ttt_desc* d, int n_hidden) {
   int rc = check_common(d);
   if (rc != TTT_OK) return rc;
   if (d->mini_batch > 16) return fail(TTT_ERR_UNSUPPORTED, "mini_batch %d > 16 has no kernel", d->mini_batch);
-  if (d->seq_stride != 0 && d->seq_stride != d->seq)
-    return fail(TTT_ERR_UNSUPPORTED, "ttt_mlpn_fwd: seq_stride must be 0");
   const bool ok = (d->head_dim == 32 && n_hidden >= 2 && n_hidden <= 4) || (d->head_dim == 64 && n_hidden == 2);
   if (!ok)
     return fail(TTT_ERR_UNSUPPORTED,
@@ -800,6 +798,7 @@ int ttt_mlpn_fwd(const ttt_desc* d, int n_hidden, const void* xq, const void* xk
   }
   a.xq = xq; a.xk = xk; a.xv = xv; a.token_eta = token_eta; a.lr = lr; a.gamma = gamma; a.beta = beta; a.out = out;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch; a.n_stages = d->seq / d->mini_batch;
+  a.seq_stride = d->seq_stride > 0 ? d->seq_stride : d->seq;
   a.state_per_batch = d->state_per_batch ? 1 : 0;
   a.eps = d->eps;
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -34,7 +34,7 @@ struct MlpNFwdArgs {
   const float* gamma;
   const float* beta;
   void* out;
-  int B, H, seq, K, n_stages, state_per_batch;
+  int B, H, seq, seq_stride, K, n_stages, state_per_batch;  // seq_stride: tokens between consecutive (b, h) units
   float eps;
 };
 
@@ -98,7 +98,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   // the next mini-batch's xq/xk/xv/lr are fetched into registers while this one computes
   float pq[NJD], pk[NJD], pv[NJD], plr = 0.f;
   auto fetch = [&](int stage) {
-    const size_t r = (bh * (size_t)a.seq + (size_t)stage * K + t) * D;
+    const size_t r = (bh * (size_t)a.seq_stride + (size_t)stage * K + t) * D;
     const bool ok = t < K;
 #pragma unroll
     for (int j = 0; j < NJD; ++j) {
@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       pv[j] = ok ? IO::load1(static_cast<const elem*>(a.xv) + r + o) : 0.f;
     }
     if (tid < 16)
-      plr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq + (size_t)stage * K + tid) : 0.f;
+      plr = (tid < K) ? IO::load1(static_cast<const elem*>(a.lr) + bh * (size_t)a.seq_stride + (size_t)stage * K + tid) : 0.f;
   };
   fetch(0);
 
@@ -117,7 +117,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     // recomputed here instead of being hoisted out of the scan into (spilled) registers
     asm volatile("" : "+v"(tid));
     lane = tid & 63, wave = tid >> 6, t = tid >> 5, cg = tid & 31;
-    const size_t row = bh * (size_t)a.seq + (size_t)st * K + t;
+    const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
 #pragma unroll
     for (int j = 0; j < NJD; ++j) {
       const int o = cg + GW * j;

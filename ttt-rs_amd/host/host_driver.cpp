@@ -1,4 +1,4 @@
-// Thin C entry points over the C++ host classes (fused_tile_multi.hpp, fused_mlp.hpp) so that a test
+// Thin C entry points over the C++ host classes (fused_tile_multi.hpp, fused_mlp.hpp, fused_others.hpp) so that a test
 // process can drive them with device buffers it already owns: each function builds the class the way a
 // C++ caller would and runs one forward (full mini-batches + remainder, as TTTInnerModel::forward,
 // rust/core/src/inner.rs:25-50) and, where the sequence allows it, one backward.  Built as
@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include "fused_mlp.hpp"
+#include "fused_others.hpp"
 #include "fused_tile_multi.hpp"
 
 namespace {
@@ -121,6 +122,77 @@ int ttt_host_mlp_forward_backward(int B, int H, int d, int K, int seq, int dtype
       g.grad_ln_bias = d_beta;
       model.backward(in, ttt::TTTMLPState{}, d_out, nullptr, nullptr, nullptr, nullptr, g, ws, stream);
     }
+    return TTT_OK;
+  } catch (const ttt::Error& e) {
+    return report(e);
+  }
+}
+
+// TTT-Linear with the Adam inner optimiser: forward over `seq` tokens (any length).  bufs_a / bufs_b: the two sets of
+// {weight, bias, weight_m, bias_m, weight_v, bias_v}; on return *cur says which set is current and *step holds the
+// step counter.
+int ttt_host_linear_adam_forward(int B, int H, int d, int K, int seq, int dtype, float eps, float beta1, float beta2,
+                                 float adam_eps, float adam_lr, const float* W0, const float* b0, const float* gamma,
+                                 const float* beta, const void* xq, const void* xk, const void* xv,
+                                 const float* token_eta, const void* lr, void* out, float* const* bufs_a,
+                                 float* const* bufs_b, int* cur, int* step, void* stream) {
+  try {
+    ttt::ModelConfig cfg;
+    cfg.num_heads = H;
+    cfg.head_dim = d;
+    cfg.ttt.mini_batch_size = K;
+    cfg.ttt.epsilon = eps;
+    ttt::TTTLinearAdamConfig ac;
+    ac.beta1 = beta1; ac.beta2 = beta2; ac.epsilon = adam_eps; ac.lr = adam_lr;
+    ttt::FusedLinearAdam model(cfg, ac, W0, b0, gamma, beta);
+    ttt::TTTInputsInner in;
+    in.qkv = ttt::Qkv{xq, xk, xv};
+    in.token_eta = token_eta;
+    in.ttt_lr_eta = lr;
+    in.batch = B;
+    in.seq_len = seq;
+    in.dtype = static_cast<ttt_dtype>(dtype);
+    ttt::TTTLinearAdamState st;
+    st.weight = bufs_a[0]; st.bias = bufs_a[1]; st.weight_m = bufs_a[2]; st.bias_m = bufs_a[3];
+    st.weight_v = bufs_a[4]; st.bias_v = bufs_a[5];
+    st.next_weight = bufs_b[0]; st.next_bias = bufs_b[1]; st.next_weight_m = bufs_b[2]; st.next_bias_m = bufs_b[3];
+    st.next_weight_v = bufs_b[4]; st.next_bias_v = bufs_b[5];
+    model.forward(st, in, out, stream);
+    *cur = st.weight == bufs_a[0] ? 0 : 1;
+    *step = st.step;
+    return TTT_OK;
+  } catch (const ttt::Error& e) {
+    return report(e);
+  }
+}
+
+// TTT-MLP with n_hidden hidden layers: forward over `seq` tokens (any length).  W0 / b0: the n_hidden + 1 parameter
+// layers; w_a / b_a and w_b / b_b: the two sets of state buffers; *cur says which set is current on return.
+int ttt_host_mlpn_forward(int B, int H, int d, int K, int seq, int dtype, float eps, int n_hidden,
+                          const float* const* W0, const float* const* b0, const float* gamma, const float* beta,
+                          const void* xq, const void* xk, const void* xv, const float* token_eta, const void* lr,
+                          void* out, float* const* w_a, float* const* b_a, float* const* w_b, float* const* b_b, int* cur,
+                          void* stream) {
+  try {
+    ttt::ModelConfig cfg;
+    cfg.num_heads = H;
+    cfg.head_dim = d;
+    cfg.ttt.mini_batch_size = K;
+    cfg.ttt.epsilon = eps;
+    ttt::FusedMlpN model(cfg, n_hidden, W0, b0, gamma, beta);
+    ttt::TTTInputsInner in;
+    in.qkv = ttt::Qkv{xq, xk, xv};
+    in.token_eta = token_eta;
+    in.ttt_lr_eta = lr;
+    in.batch = B;
+    in.seq_len = seq;
+    in.dtype = static_cast<ttt_dtype>(dtype);
+    ttt::TTTMLPNState st;
+    for (int i = 0; i <= n_hidden; ++i) {
+      st.weight[i] = w_a[i]; st.bias[i] = b_a[i]; st.next_weight[i] = w_b[i]; st.next_bias[i] = b_b[i];
+    }
+    model.forward(st, in, out, stream);
+    *cur = st.weight[0] == w_a[0] ? 0 : 1;
     return TTT_OK;
   } catch (const ttt::Error& e) {
     return report(e);

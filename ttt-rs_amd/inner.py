@@ -657,6 +657,68 @@ class FusedLinearAdam:
         return self._launch(state, inputs.slice_seq(r), len(r))
 
 
+@dataclass
+class TTTMLPNState:
+    """mlp2.rs:38-53, mlp3.rs:42-53, mlp4.rs:46-59: the n_hidden + 1 weight layers [B,H,in,out] and biases [B,H,out],
+    always f32."""
+    weights: list
+    biases: list
+
+
+class FusedMlpN:
+    """TTTMLP2 / TTTMLP3 / TTTMLP4 (rust/core/src/mlp2.rs, mlp3.rs, mlp4.rs) on the fused kernel: d -> 4d -> ... -> 4d
+    -> d with 2, 3 or 4 hidden layers, the TTTInnerModel interface of rust/core/src/inner.rs:13-58."""
+
+    def __init__(self, config: ModelConfig, weights_init, biases_init, ln_weight, ln_bias):
+        H, d = config.num_heads, config.head_dim
+        n = len(weights_init) - 1
+        if n < 2 or n > 4 or len(biases_init) != n + 1:
+            raise _lib.TttError(_lib.TTT_ERR_UNSUPPORTED, "FusedMlpN: 2, 3 or 4 hidden layers")
+        dims = [d] + [4 * d] * n + [d]
+        self.config, self.n_hidden = config, n
+        self.weights_init = [_need(w, (H, dims[i], dims[i + 1]), torch.float32, f"weights_init[{i}]")
+                             for i, w in enumerate(weights_init)]
+        self.biases_init = [_need(b, (H, dims[i + 1]), torch.float32, f"biases_init[{i}]")
+                            for i, b in enumerate(biases_init)]
+        self.ln_weight = _need(ln_weight, (H, d), torch.float32, "ln_weight")
+        self.ln_bias = _need(ln_bias, (H, d), torch.float32, "ln_bias")
+
+    def name(self) -> str:
+        return f"TTTMLP{self.n_hidden}"  # mlp2.rs:70-72, mlp3.rs:70-72, mlp4.rs:76-78
+
+    def get_config(self) -> ModelConfig:
+        return self.config
+
+    def init_state(self, batch_size: int) -> TTTMLPNState:
+        """mlp2.rs:129-145 and its siblings: the parameters repeated over the batch."""
+        rep = lambda t: t.unsqueeze(0).repeat(batch_size, *([1] * t.dim()))
+        return TTTMLPNState([rep(w) for w in self.weights_init], [rep(b) for b in self.biases_init])
+
+    def _launch(self, state: TTTMLPNState, inputs: TTTInputsInner, mini_batch: int):
+        out, ws, bs = ttt_mlpn_forward_raw(inputs.qkv.xq, inputs.qkv.xk, inputs.qkv.xv, state.weights, state.biases,
+                                           inputs.token_eta, inputs.ttt_lr_eta, self.ln_weight, self.ln_bias,
+                                           mini_batch, self.config.ttt.epsilon)
+        state.weights, state.biases = ws, bs
+        return out
+
+    def forward(self, state: TTTMLPNState, inputs: TTTInputsInner) -> torch.Tensor:
+        """inner.rs:25-50: all full mini-batches in one launch, a trailing remainder as one short mini-batch."""
+        K = self.config.ttt.mini_batch_size
+        seq = inputs.qkv.xq.shape[2]
+        full = (seq // K) * K
+        outs = []
+        if full > 0:
+            outs.append(self._launch(state, inputs.slice_seq(range(0, full)), K))
+        if full < seq:
+            outs.append(self._launch(state, inputs.slice_seq(range(full, seq)), seq - full))
+        return outs[0] if len(outs) == 1 else torch.cat(outs, 2)
+
+    def forward_mini_batch(self, state: TTTMLPNState, inputs: TTTInputsInner, r: range) -> torch.Tensor:
+        if len(r) > self.config.ttt.mini_batch_size or len(r) == 0:
+            raise _lib.TttError(_lib.TTT_ERR_SHAPE, "range longer than mini_batch_size")
+        return self._launch(state, inputs.slice_seq(r), len(r))
+
+
 def ttt_stack_workspace_bytes(B: int, H: int, seq: int, d: int, mini_batch: int, io: torch.dtype, mlp_flags,
                               chunk_tokens: int = 0) -> int:
     """ttt_stack_fwd_workspace_bytes for a stack whose layer l is TTT-MLP where mlp_flags[l] is true."""
