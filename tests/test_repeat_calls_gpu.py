@@ -65,7 +65,7 @@ def test_linear_fwd_repeat_calls(P, d, K, hint, fmt):
 # (d, K, mini-batches, waves hint): every NW / tiles-per-wave combination of the feature-split backward and the
 # single-wave kernel (bf16, head_dim <= 64)
 BWD_CASES = [(32, 16, 4, 0), (32, 7, 4, 0), (32, 7, 4, 1), (64, 16, 4, 0), (64, 7, 5, 0), (64, 3, 4, 2), (64, 7, 4, 1),
-             (96, 16, 3, 0), (96, 7, 4, 0), (128, 16, 3, 0), (128, 5, 4, 0)]
+             (96, 16, 3, 0), (96, 7, 4, 0), (128, 16, 3, 0), (128, 5, 4, 0), (32, 32, 3, 0), (32, 21, 4, 0)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -75,6 +75,8 @@ def test_linear_bwd_repeat_calls_and_short_mini_batches(P, d, K, N, hint, fmt, d
     f32 = dtype == torch.float32
     if fmt == 2 and (f32 or d > 96):
         pytest.skip("update factors: bf16 I/O up to head_dim 96")
+    if K > 16 and fmt != 0:
+        pytest.skip("mini-batches of more than 16 tokens: f32 row-major checkpoints only")
     if f32 and hint == 1:
         pytest.skip("f32 I/O: no single-wave kernel")
     if f32 and d == 128 and fmt != 0:
