@@ -262,10 +262,10 @@ int opt_in_lds(size_t bytes) {
   return rc;
 }
 
-template <class T, int D, int MT = 1>
+template <class T, int D, int MT = 1, bool BF = false>
 int launch_linear_fwd_lds(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s) {
   const ttt::LinearFwdArgs& a = probs[0];
-  constexpr auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D, MT>;
+  constexpr auto kern = ttt::ttt_linear_fwd_lds_kernel<T, D, MT, BF>;
   constexpr size_t bytes = ttt::LinFwdLds<D, MT>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
@@ -365,9 +365,9 @@ int uses_two_cu_mlp(const ttt_desc* d, int n_problems, bool* yes) {
   return TTT_OK;
 }
 
-template <class T, int D, int MT = 1, bool WG = false, bool DG = false>
+template <class T, int D, int MT = 1, bool WG = false, bool DG = false, bool BF = false>
 int launch_linear_bwd(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_linear_bwd_kernel<T, D, MT, WG, DG>;
+  constexpr auto kern = ttt::ttt_linear_bwd_kernel<T, D, MT, WG, DG, BF>;
   constexpr size_t bytes = ttt::BwdLds<D, MT, WG, DG>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
@@ -713,7 +713,9 @@ int dispatch_linear_fwd_pack(const ttt_desc* d, const ttt::LinearFwdArgs* a, uns
   const bool want_lds = (d->kernel_hint & TTT_HINT_LDS_TILES) != 0 && d->head_dim > 64;
   const bool f32 = d->io_dtype == TTT_F32;
   if (d->mini_batch > 16)  // head_dim 32 (ttt_linear_supported): the LDS-tile kernel on two tiles of token rows
-    return f32 ? launch_linear_fwd_lds<ttt::F32, 32, 2>(a, ny, s) : launch_linear_fwd_lds<ttt::BF16, 32, 2>(a, ny, s);
+    return f32 ? launch_linear_fwd_lds<ttt::F32, 32, 2>(a, ny, s)
+               : (d->kernel_hint & TTT_HINT_LDS_TILES) ? launch_linear_fwd_lds<ttt::BF16, 32, 2>(a, ny, s)
+                                                       : launch_linear_fwd_lds<ttt::BF16, 32, 2, true>(a, ny, s);
   switch (d->head_dim) {
     case 32: return f32 ? launch_linear_fwd<ttt::F32, 32>(a, d->kernel_hint, ny, s) : launch_linear_fwd<ttt::BF16, 32>(a, d->kernel_hint, ny, s);
     case 64: return f32 ? launch_linear_fwd<ttt::F32, 64>(a, d->kernel_hint, ny, s) : launch_linear_fwd<ttt::BF16, 64>(a, d->kernel_hint, ny, s);
@@ -1013,12 +1015,20 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   const int waves = ch.waves;
   if (ch.kind == LinearBwdChoice::LDS) {
     if (ch.w_global) return launch_linear_bwd<ttt::F32, 128, 1, true, true>(a, grid, s);
+    // bf16 I/O: operands rounded to bf16 like the register-resident kernels, unless f32 products were asked for
+    const bool bfops = !f32 && !(d->kernel_hint & TTT_HINT_LDS_TILES);
     if (ch.dw_global)
-      return f32 ? launch_linear_bwd<ttt::F32, 96, 1, false, true>(a, grid, s)
-                 : launch_linear_bwd<ttt::BF16, 96, 1, false, true>(a, grid, s);
+      return f32     ? launch_linear_bwd<ttt::F32, 96, 1, false, true>(a, grid, s)
+             : bfops ? launch_linear_bwd<ttt::BF16, 96, 1, false, true, true>(a, grid, s)
+                     : launch_linear_bwd<ttt::BF16, 96, 1, false, true>(a, grid, s);
     if (d->mini_batch > 16)
-      return f32 ? launch_linear_bwd<ttt::F32, 32, 2>(a, grid, s) : launch_linear_bwd<ttt::BF16, 32, 2>(a, grid, s);
+      return f32     ? launch_linear_bwd<ttt::F32, 32, 2>(a, grid, s)
+             : bfops ? launch_linear_bwd<ttt::BF16, 32, 2, false, false, true>(a, grid, s)
+                     : launch_linear_bwd<ttt::BF16, 32, 2>(a, grid, s);
     if (f32) return D == 64 ? launch_linear_bwd<ttt::F32, 64>(a, grid, s) : launch_linear_bwd<ttt::F32, 32>(a, grid, s);
+    if (bfops)
+      return D == 64 ? launch_linear_bwd<ttt::BF16, 64, 1, false, false, true>(a, grid, s)
+                     : launch_linear_bwd<ttt::BF16, 32, 1, false, false, true>(a, grid, s);
     return D == 64 ? launch_linear_bwd<ttt::BF16, 64>(a, grid, s) : launch_linear_bwd<ttt::BF16, 32>(a, grid, s);
   }
   if (a.ckpt_packed == ttt::kCkptFactors) {

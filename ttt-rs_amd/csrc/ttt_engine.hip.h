@@ -541,6 +541,29 @@ __device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const 
   mm_splitk_t<false, MODE, NW, NT, KSTEPS>(C, ldc, part, A, a_rs, B, b_rs, b_cs, wave, lane, tid);
 }
 
+// The tile engine's products with the operand type fixed for a whole kernel instantiation: BF = operands rounded to
+// bf16 (one v_mfma_f32_16x16x16_bf16 per 16-deep step), otherwise true f32.  Accumulation is f32 in both.
+template <bool BF>
+struct Eng {
+  template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false>
+  static __device__ __forceinline__ void lds(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
+                                             int b_rs, int b_cs, int Mt, int Nt, int Kd, int wave, int lane,
+                                             int first = 0, int k0 = 0) {
+    mm_lds_t<BF, MODE, NW, NB, KU, BG>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, Kd, wave, lane, first, k0);
+  }
+  template <int MODE, int NW, int NB, int KS, bool FZ = false>
+  static __device__ __forceinline__ void rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
+                                              int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
+                                              const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
+    mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz);
+  }
+  template <int MODE, int NW, int NT, int KSTEPS>
+  static __device__ __forceinline__ void splitk(float* C, int ldc, float* part, const float* A, int a_rs,
+                                                const float* B, int b_rs, int b_cs, int wave, int lane, int tid) {
+    mm_splitk_t<BF, MODE, NW, NT, KSTEPS>(C, ldc, part, A, a_rs, B, b_rs, b_cs, wave, lane, tid);
+  }
+};
+
 // Sum over r of p[r * stride] (+ q[r * stride]), r = 0..15, with all loads issued before the first add: written as
 // a plain loop the loads are issued one at a time, each waiting for the one before.
 __device__ __forceinline__ float col16_sum(const float* p, int stride) {

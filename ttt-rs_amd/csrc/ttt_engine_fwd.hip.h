@@ -79,9 +79,11 @@ struct LinFwdLds {
   static constexpr size_t BYTES = sizeof(float) * END;
 };
 
-template <class T, int D, int MT = 1>
+// BF: operands of the products rounded to bf16 (see ttt_linear_bwd_kernel)
+template <class T, int D, int MT = 1, bool BF = false>
 __global__ void __launch_bounds__(256 * MT) ttt_linear_fwd_lds_kernel(Problems<LinearFwdArgs> problems) {
   const LinearFwdArgs& a = problems.p[blockIdx.y];
+  using E = Eng<BF>;
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = LinFwdLds<D, MT>;
@@ -139,9 +141,9 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_fwd_lds_kernel(Problems<L
     if (tid < KT) slr[tid] = plr;
     __syncthreads();
     if (st + 1 < a.n_stages) fetch(st + 1);
-    mm_lds<0, NW>(lds + L::G, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NT, D, wave, lane);
-    mm_lds<0, NW>(lds + L::ZB, LD, lds + L::XQ, LD, 1, sW, LD, 1, MT, NT, D, wave, lane, (MT * NT) % NW);
-    mm_lds<0, NW>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, MT, MT, D, wave, lane, (2 * MT * NT) % NW);
+    E::template lds<0, NW>(lds + L::G, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NT, D, wave, lane);
+    E::template lds<0, NW>(lds + L::ZB, LD, lds + L::XQ, LD, 1, sW, LD, 1, MT, NT, D, wave, lane, (MT * NT) % NW);
+    E::template lds<0, NW>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, MT, MT, D, wave, lane, (2 * MT * NT) % NW);
     __syncthreads();
     {
       float Gv[NJ];
@@ -156,7 +158,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_fwd_lds_kernel(Problems<L
       }
     }
     __syncthreads();
-    mm_lds<2, NW, 1, 4>(lds + L::ZB, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, MT, NT, KT, wave, lane);
+    E::template lds<2, NW, 1, 4>(lds + L::ZB, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, MT, NT, KT, wave, lane);
     __syncthreads();
     {
       float xh[NJ], rstd;
@@ -172,7 +174,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_fwd_lds_kernel(Problems<L
       }
     }
     __syncthreads();
-    mm_lds<2, NW, (NT % 4 == 0 ? 4 : 2), 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NT, NT, KT, wave, lane);
+    E::template lds<2, NW, (NT % 4 == 0 ? 4 : 2), 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NT, NT, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < KT; ++r) s += lds[L::G + r * LD + tid];

@@ -77,11 +77,14 @@ struct BwdLds {
   static constexpr size_t BYTES = sizeof(float) * END;
 };
 
-template <class T, int D, int MT = 1, bool WG = false, bool DG = false>
+// BF: the operands of every product are rounded to bf16 (bf16 I/O when this kernel is the library's own choice, not
+// a request for f32 products): an eighth of the matrix-pipe time; tiles, state and accumulation stay f32.
+template <class T, int D, int MT = 1, bool WG = false, bool DG = false, bool BF = false>
 __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs a) {
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = BwdLds<D, MT, WG, DG>;
+  using E = Eng<BF>;
   constexpr int LD = L::LD, LK = L::LK, KT = L::KT, NJ = D / 16, NTH = 256 * MT, NW = 4 * MT;
   constexpr int NB2 = NJ >= 2 ? 2 : 1;  // tile columns per job of a [16 x D] product
   constexpr float inv_d = 1.0f / D;
@@ -241,7 +244,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
       bar();
 #pragma unroll
       for (int j = 0; j < NJ; ++j) lds[L::TG + t * LD + cg + 16 * j] -= lds[L::XK + t * LD + cg + 16 * j];
-      mm_lds<0, NW>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane);
+      E::template lds<0, NW>(lds + L::XH, LD, lds + L::XK, LD, 1, sW, LD, 1, MT, NJ, D, wave, lane);
       bar();
       {
         float xh[NJ], Gv[NJ], rstd;
@@ -252,7 +255,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
       }
       bar();
       // W -= XK^T (last * G) ; b -= colsum(last * G)      (linear.rs:134-144)
-      mm_lds<2, NW, NJ, 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, KT, wave, lane);
+      E::template lds<2, NW, NJ, 4>(sW, LD, lds + L::XK, 1, LD, lds + L::G, LD, 1, NJ, NJ, KT, wave, lane);
       if (tid < D) {
         float s = 0.f;
         for (int r = 0; r < KT; ++r) s += lds[L::G + r * LD + tid];
@@ -268,9 +271,9 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
     // Z1 = XK W ; Zq = XQ W ; A = XQ XK^T
     // every product is cut into jobs of NB2 tile columns: two or more accumulator chains per wave keep the
     // matrix pipe busy (a single chain waits out the full MFMA latency between dependent steps)
-    mm_lds<0, NW, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, Wp, wld, 1, MT, NJ, D, wave, lane, 0);
-    mm_lds<0, NW, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, Wp, wld, 1, MT, NJ, D, wave, lane, 2);
-    mm_lds<0, NW>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, MT, MT, D, wave, lane, 1);
+    E::template lds<0, NW, NB2>(lds + L::XH, LD, lds + L::XK, LD, 1, Wp, wld, 1, MT, NJ, D, wave, lane, 0);
+    E::template lds<0, NW, NB2>(lds + L::XH2, LD, lds + L::XQ, LD, 1, Wp, wld, 1, MT, NJ, D, wave, lane, 2);
+    E::template lds<0, NW>(lds + L::A, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, MT, MT, D, wave, lane, 1);
     bar();
 
     // ================= forward intermediates: x_hat, rstd, G; eta, A (tril), M = eta (1 + A)
@@ -293,7 +296,7 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
     }
     bar();
     // Zb = XQ W - M G  (+ b added when read)
-    mm_lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, MT, NJ, KT, wave, lane);
+    E::template lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M, LK, 1, lds + L::G, LD, 1, MT, NJ, KT, wave, lane);
     bar();
 
     // ================= output LayerNorm and its backward (stage 4)
@@ -333,10 +336,10 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
 
     // ================= P = dZb G^T ; dQ = dZb W^T ; S = XK dW ; TMP = G dW^T
     // a transposed matrix in global memory is contiguous along k: loaded four lanes to a row (BG)
-    mm_lds<0, NW, NB2, 4, WG>(lds + L::DQ, LD, lds + L::DZB, LD, 1, Wp, 1, wld, MT, NJ, D, wave, lane, 0);
-    mm_lds<0, NW, NB2, 4, DG>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, dld, MT, NJ, D, wave, lane, 0);
-    mm_lds<0, NW, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, dld, 1, MT, NJ, D, wave, lane, 2);
-    mm_lds<0, NW>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, MT, MT, D, wave, lane, 3);
+    E::template lds<0, NW, NB2, 4, WG>(lds + L::DQ, LD, lds + L::DZB, LD, 1, Wp, 1, wld, MT, NJ, D, wave, lane, 0);
+    E::template lds<0, NW, NB2, 4, DG>(lds + L::TMP, LD, lds + L::G, LD, 1, sdW, 1, dld, MT, NJ, D, wave, lane, 0);
+    E::template lds<0, NW, NB2>(lds + L::S, LD, lds + L::XK, LD, 1, sdW, dld, 1, MT, NJ, D, wave, lane, 2);
+    E::template lds<0, NW>(lds + L::P, LK, lds + L::DZB, LD, 1, lds + L::G, 1, LD, MT, MT, D, wave, lane, 3);
     bar();
 
     // ================= dA, d eta ; S += db ; dlast
@@ -362,10 +365,10 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
     bar();
 
     // ================= dQ += dA XK ; dK = dA^T XQ ; DGM = M^T dZb ; dW += XQ^T dZb ; db += colsum(dZb)
-    mm_lds<1, NW, NJ, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, MT, NJ, KT, wave, lane, 0);
-    mm_lds<0, NW, NJ, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, MT, NJ, KT, wave, lane, 1);
-    mm_lds<0, NW, NJ, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, MT, NJ, KT, wave, lane, 2);
-    mm_lds<1, NW, NJ, 4>(sdW, dld, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, KT, wave, lane);
+    E::template lds<1, NW, NJ, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, MT, NJ, KT, wave, lane, 0);
+    E::template lds<0, NW, NJ, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, MT, NJ, KT, wave, lane, 1);
+    E::template lds<0, NW, NJ, 4>(lds + L::DGM, LD, lds + L::M, 1, LK, lds + L::DZB, LD, 1, MT, NJ, KT, wave, lane, 2);
+    E::template lds<1, NW, NJ, 4>(sdW, dld, lds + L::XQ, 1, LD, lds + L::DZB, LD, 1, NJ, NJ, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < KT; ++r) s += lds[L::DZB + r * LD + tid];
@@ -432,8 +435,8 @@ __global__ void __launch_bounds__(256 * MT) ttt_linear_bwd_kernel(LinearBwdArgs 
     bar();
 
     // ================= dK += dZ1 W^T ; dW += XK^T dZ1 ; db += colsum(dZ1)
-    mm_lds<1, NW, NB2, 4, WG>(lds + L::DK, LD, lds + L::DZ1, LD, 1, Wp, 1, wld, MT, NJ, D, wave, lane, 2);
-    mm_lds<1, NW, NJ, 4>(sdW, dld, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, KT, wave, lane);
+    E::template lds<1, NW, NB2, 4, WG>(lds + L::DK, LD, lds + L::DZ1, LD, 1, Wp, 1, wld, MT, NJ, D, wave, lane, 2);
+    E::template lds<1, NW, NJ, 4>(sdW, dld, lds + L::XK, 1, LD, lds + L::DZ1, LD, 1, NJ, NJ, KT, wave, lane);
     if (tid < D) {
       float s = 0.f;
       for (int r = 0; r < KT; ++r) s += lds[L::DZ1 + r * LD + tid];

@@ -77,29 +77,6 @@ struct MlpBwdLds {
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
 };
 
-// The tile engine's products with the operand type fixed for a whole kernel instantiation: BF = operands rounded to
-// bf16 (one v_mfma_f32_16x16x16_bf16 per 16-deep step), otherwise true f32.  Accumulation is f32 in both.
-template <bool BF>
-struct MlpBwdEng {
-  template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false>
-  static __device__ __forceinline__ void lds(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
-                                             int b_rs, int b_cs, int Mt, int Nt, int Kd, int wave, int lane,
-                                             int first = 0, int k0 = 0) {
-    mm_lds_t<BF, MODE, NW, NB, KU, BG>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, Kd, wave, lane, first, k0);
-  }
-  template <int MODE, int NW, int NB, int KS, bool FZ = false>
-  static __device__ __forceinline__ void rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
-                                              int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
-                                              const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
-    mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz);
-  }
-  template <int MODE, int NW, int NT, int KSTEPS>
-  static __device__ __forceinline__ void splitk(float* C, int ldc, float* part, const float* A, int a_rs,
-                                                const float* B, int b_rs, int b_cs, int wave, int lane, int tid) {
-    mm_splitk_t<BF, MODE, NW, NT, KSTEPS>(C, ldc, part, A, a_rs, B, b_rs, b_cs, wave, lane, tid);
-  }
-};
-
 // tanh-GELU with first and second derivative
 __device__ __forceinline__ void gelu_tanh_all(float x, float& y, float& dy, float& ddy) {
   const float c = 0.7978845608f, a = 0.044715f;
@@ -120,7 +97,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   using IO = Io<T>;
   using elem = typename IO::elem;
   using L = MlpBwdLds<D>;
-  using E = MlpBwdEng<BF>;
+  using E = Eng<BF>;
   constexpr int M = L::M, LD = L::LD, LK = L::LK;
   constexpr int NW = 8, GW = 32, NJD = D / GW, NJM = M / GW, NTD = D / 16, NTM = M / 16;
   constexpr int NBM = NTM / NW;  // [16 x 4d] products: one job of NBM tile columns per wave
