@@ -368,12 +368,15 @@ def run_workload(name, a, pkg, torch):
                 return pkg.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
                                                dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
         else:
+            # the forward saves the update factors for the backward (ttt_mlp_fwd_saving + ttt_mlp_bwd_saved), as a
+            # training step does: the backward then runs no forward sweep of its own
             def step():
                 fw = pkg.ttt_mlp_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
-                                             dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K)
+                                             dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"], K,
+                                             save_for_backward=True)
                 g = pkg.ttt_mlp_backward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"],
                                              dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"], dv["beta"],
-                                             dv["d_out"], K)
+                                             dv["d_out"], K, saved=fw[5])
                 return (fw[0], g["d_xq"])
 
     # status word of the two-CU TTT-MLP kernel (head_dim 128): it must not move while this workload runs
@@ -502,8 +505,8 @@ def run_workload(name, a, pkg, torch):
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     elif kind == "mlp_fwd_bwd":
         # forward (56 d^2 + 20 K d) and the reverse scan's 14 state-sized and 7 rank-16 products:
-        # (56 + 14*8 + 7*8) d^2 flop per token-head, K-sized terms aside.  The backward's own forward sweep (the
-        # register-resident forward once more for bf16 I/O up to head_dim 96) is overhead, not algorithmic work.
+        # (56 + 14*8 + 7*8) d^2 flop per token-head, K-sized terms aside.  The forward saves the update factors, so the
+        # backward runs no forward sweep of its own.
         flops = th * (224 * d * d)
         # bf16 I/O up to head_dim 96: every product of the scan takes bf16 operands (f32 accumulation, f32 state and
         # gradient accumulators in memory); otherwise true-f32 products
@@ -513,7 +516,7 @@ def run_workload(name, a, pkg, torch):
         out["config"]["inner_model"] = "TTT-MLP"
         out["roofline"] = {"bound": "mfma", "achieved": flops / dev_s / 1e12, "peak": peak,
                            "unit": "TFLOP/s", "frac": flops / dev_s / 1e12 / peak, **counters,
-                           "kernel": "ttt_mlp_fwd_rr_kernel (forward, and again as the backward's sweep) + ttt_mlp_bwd_kernel (whole step)",
+                           "kernel": "ttt_mlp_fwd_rr_kernel (forward, saving the update factors) + ttt_mlp_bwd_kernel (whole step)",
                            "kernel_avg_us": dev_s * 1e6, "algorithmic_flops": flops}
     else:
         flops = th * (6 * (6 * d * d + 4 * K * d) + 2 * (56 * d * d + 20 * K * d))

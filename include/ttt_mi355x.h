@@ -259,6 +259,34 @@ int ttt_mlp_bwd(const ttt_desc* desc, const void* xq, const void* xk, const void
                 float* d_gamma, float* d_beta, void* workspace, void* stream);
 
 /*
+ * Forward that saves for the backward, and the backward that uses what was saved: ttt_mlp_fwd_saving +
+ * ttt_mlp_bwd_saved give the results of ttt_mlp_fwd + ttt_mlp_bwd (bit for bit) without the backward running the
+ * forward sweep a second time.  The reference differentiates TTTMLP::forward_mini_batch with Burn autodiff, which
+ * keeps the forward's activations for the backward (rust/core/src/mlp.rs:127-208); this pair is the fused counterpart
+ * of that: the forward leaves in `saved` (ttt_mlp_bwd_workspace_bytes(desc) bytes of device memory, 16-byte aligned,
+ * caller-owned) the two rank-16 factors of every mini-batch's state update and a copy of the final state, about
+ * 2 K (5 d) floats per mini-batch and unit instead of the activations.  ttt_mlp_bwd_saved takes the arguments of
+ * ttt_mlp_bwd with `saved` in place of the workspace, the same desc and the same inputs as the forward; it consumes
+ * `saved` (the state in it is walked back), so a second backward needs a second forward or ttt_mlp_bwd.
+ * Exists where the forward's kernel is also the backward's sweep: bf16 I/O up to head_dim 96 (one CU per unit) and
+ * f32 I/O; ttt_mlp_fwd_saving_supported says so beforehand (TTT_ERR_UNSUPPORTED for the forward on pairs of CUs:
+ * head_dim 128 with bf16 I/O, TTT_HINT_TWO_CU).
+ */
+int ttt_mlp_fwd_saving_supported(const ttt_desc* desc);
+int ttt_mlp_fwd_saving(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                       const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                       const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                       void* out, float* W1_out, float* b1_out, float* W2_out, float* b2_out, void* saved,
+                       void* stream);
+int ttt_mlp_bwd_saved(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                      const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                      const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                      const void* d_out, const float* d_W1_out, const float* d_b1_out,
+                      const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
+                      float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
+                      float* d_gamma, float* d_beta, void* saved, void* stream);
+
+/*
  * ttt_mlp_bwd without a workspace argument and without any allocation.  No counterpart in the
  * reference; it is for callers that cannot allocate device memory around the call (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same arguments, results

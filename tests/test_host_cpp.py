@@ -25,7 +25,7 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
           if (std::strcmp(m.name(), "FusedTileMultiTTTLinear")) return 1;
           if (m.num_checkpoints(2, 64) != 4) return 2;
           ttt::TTTInputsInner in; in.batch = 2; in.seq_len = 33;   // not a multiple of 16, > 16
-          ttt::TTTLinearState st; char out[4];
+          ttt::TTTLinearState st; alignas(16) char out[16];
           // a state without buffers is refused by the class itself
           in.seq_len = 32;
           try { m.forward(st, in, out, ttt::Checkpoints{}, nullptr); return 20; }
@@ -50,6 +50,16 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
           catch (const ttt::Error& e) { if (e.code != TTT_ERR_SHAPE) return 10; }
           try { mlp.backward(in, ms, out, nullptr, nullptr, nullptr, nullptr, ttt::TTTMLPGrads{}, out, nullptr); return 11; }
           catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 12; }
+          // the saving pair: null tensors are refused, and so is the forward that runs on pairs of CUs
+          in.dtype = TTT_BF16;
+          try { mlp.forward_saving(ms, in, out, out, nullptr); return 13; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 14; }
+          try { mlp.backward_saved(in, ms, out, nullptr, nullptr, nullptr, nullptr, ttt::TTTMLPGrads{}, out, nullptr); return 15; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_NULL) return 16; }
+          cfg.head_dim = 128;
+          ttt::FusedMlp wide(cfg, dummy, dummy, dummy, dummy, dummy, dummy);
+          try { wide.forward_saving(ms, in, out, out, nullptr); return 17; }
+          catch (const ttt::Error& e) { if (e.code != TTT_ERR_UNSUPPORTED) return 18; }
           return 0;
         }
     '''))

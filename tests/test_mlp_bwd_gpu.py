@@ -142,3 +142,46 @@ def test_mlp_bwd_d128_is_deterministic(P):
                 assert torch.equal(r[k], runs[0][k]), (k, dtype)
             for k in ("d_token_eta", "d_gamma", "d_beta"):
                 assert_close(r[k], runs[0][k].double().cpu().numpy(), 1e-5, k)
+
+
+@pytest.mark.parametrize("dtype,d,K,N", [(torch.bfloat16, 96, 16, 4), (torch.bfloat16, 64, 7, 3), (torch.bfloat16, 32, 16, 1),
+                                         (torch.float32, 64, 16, 3), (torch.float32, 128, 16, 2)],
+                         ids=["bf16-d96", "bf16-d64-K7", "bf16-d32-one", "f32-d64", "f32-d128"])
+def test_mlp_forward_saving_and_backward_from_saved(P, dtype, d, K, N):
+    """ttt_mlp_fwd_saving + ttt_mlp_bwd_saved against ttt_mlp_fwd + ttt_mlp_bwd: the same kernels without the backward's
+    own forward sweep, so outputs, final state and the eight per-unit gradients are the same bits (the three that
+    are accumulated with floating-point atomics to 1e-5); and against the oracle like the plain pair."""
+    print(f"case mlp saving fwd + saved bwd {dtype} d{d} K{K} N{N}", flush=True)
+    B, H = 2, 2
+    c = mlp_case(P, 700 + d + K, B, H, N * K, d, K, dtype, "ref")
+    g = torch.Generator().manual_seed(41)
+    dO = torch.randn(B, H, N * K, d, generator=g).to(dtype)
+    dv = to_dev(c)
+    args = (dv["xq"], dv["xk"], dv["xv"], dv["W1"], dv["b1"], dv["W2"], dv["b2"], dv["token_eta"], dv["lr"], dv["gamma"],
+            dv["beta"])
+    plain_f = P.ttt_mlp_forward_raw(*args, K)
+    plain_b = P.ttt_mlp_backward_raw(*args, dO.to("cuda:0"), K)
+    sv = P.ttt_mlp_forward_raw(*args, K, save_for_backward=True)
+    got = P.ttt_mlp_backward_raw(*args, dO.to("cuda:0"), K, saved=sv[5])
+    torch.cuda.synchronize()
+    for i, name in enumerate(("out", "W1", "b1", "W2", "b2")):
+        assert torch.equal(sv[i], plain_f[i]), name
+    for k in GRADS:
+        if k in ("d_token_eta", "d_gamma", "d_beta"):
+            assert_close(got[k], plain_b[k].double().cpu().numpy(), 1e-5, k)
+        else:
+            assert torch.equal(got[k], plain_b[k]), k
+    n = np_inputs(c)
+    ref = orc.mlp_backward(n["W1"], n["b1"], n["W2"], n["b2"], n["xq"], n["xk"], n["xv"], n["token_eta"], n["lr"],
+                           n["gamma"], n["beta"], dO.double().numpy(), K=K)
+    bf = dtype == torch.bfloat16
+    for k in GRADS:
+        io_out = k in ("d_xq", "d_xk", "d_xv", "d_lr")
+        assert_close(got[k], ref[k], TOL[dtype] if (io_out or bf) else 1e-4, k, min_frac=0.99 if bf else 0.999)
+
+
+def test_mlp_forward_saving_is_refused_on_pairs_of_cus(P):
+    c = to_dev(mlp_case(P, 5, 1, 2, 32, 128, 16, torch.bfloat16, "ref"))
+    with pytest.raises(P.TttError, match="pairs of CUs"):
+        P.ttt_mlp_forward_raw(c["xq"], c["xk"], c["xv"], c["W1"], c["b1"], c["W2"], c["b2"], c["token_eta"], c["lr"],
+                              c["gamma"], c["beta"], 16, save_for_backward=True)

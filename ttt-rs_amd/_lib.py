@@ -23,7 +23,7 @@ EXPORTS = (
     "ttt_linear_best_checkpoint_format",
     "ttt_linear_num_checkpoints",
     "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
-    "ttt_mlp_fwd_lost_workgroups", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue", "ttt_linear_fwd_fused_inputs_supported", "ttt_linear_fwd_fused_inputs", "ttt_linear_adam_supported", "ttt_linear_adam_fwd", "ttt_mlpn_supported", "ttt_mlpn_fwd", "ttt_selftest_mfma_mixed",
+    "ttt_mlp_fwd_lost_workgroups", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_mlp_fwd_saving_supported", "ttt_mlp_fwd_saving", "ttt_mlp_bwd_saved", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue", "ttt_linear_fwd_fused_inputs_supported", "ttt_linear_fwd_fused_inputs", "ttt_linear_adam_supported", "ttt_linear_adam_fwd", "ttt_mlpn_supported", "ttt_mlpn_fwd", "ttt_selftest_mfma_mixed",
 )
 
 
@@ -79,6 +79,9 @@ def lib() -> C.CDLL:
         L.ttt_mlp_bwd_workspace_bytes.restype = C.c_int64
         L.ttt_mlp_bwd.argtypes = [dp] + [vp] * 29
         L.ttt_mlp_bwd_static.argtypes = [dp] + [vp] * 28
+        L.ttt_mlp_fwd_saving_supported.argtypes = [dp]
+        L.ttt_mlp_fwd_saving.argtypes = [dp] + [vp] * 18
+        L.ttt_mlp_bwd_saved.argtypes = [dp] + [vp] * 29
         L.ttt_mlp_fwd_lost_workgroups.argtypes = [C.POINTER(C.c_int64)]
         L.ttt_stack_fwd_workspace_bytes.argtypes = [dp, C.c_int32, C.POINTER(TttStackLayer), C.c_int32]
         L.ttt_stack_fwd_workspace_bytes.restype = C.c_int64

@@ -547,13 +547,20 @@ int mlp_bwd_scratch(void** out) {
   return TTT_OK;
 }
 
+// Whether the forward sweep of a TTT-MLP backward is the register-resident forward (bf16 I/O up to head_dim 96, no
+// request for f32 products through TTT_HINT_LDS_TILES): the reverse scan then takes bf16 operands as well.
+bool mlp_rr_sweep(const ttt_desc* d) {
+  return d->io_dtype != TTT_F32 && d->head_dim <= 96 && !(d->kernel_hint & TTT_HINT_LDS_TILES);
+}
+
+// sweep = false: the workspace already holds what the sweep leaves there (ttt_mlp_fwd_saving wrote it)
 int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
                 const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
                 const float* token_eta, const void* lr, const float* gamma, const float* beta,
                 const void* d_out, const float* d_W1_out, const float* d_b1_out,
                 const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
                 float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
-                float* d_gamma, float* d_beta, void* workspace, void* stream) {
+                float* d_gamma, float* d_beta, void* workspace, void* stream, bool sweep = true) {
   int rc = ttt_mlp_supported(d);
   if (rc != TTT_OK) return rc;
   if (!xq || !xk || !xv || !W1_0 || !b1_0 || !W2_0 || !b2_0 || !token_eta || !lr || !gamma || !beta ||
@@ -574,7 +581,7 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   // head_dim 96: the register-resident forward itself (the factors are then the ones the forward of this step
   // applied, rounded to bf16 as its matrix instructions took them); its output goes to d_xq, which the reverse
   // scan overwrites afterwards.  Otherwise the LDS-tile kernel (f32 products, no output).
-  const bool rr_sweep = !f32 && d->head_dim <= 96 && !(d->kernel_hint & TTT_HINT_LDS_TILES);
+  const bool rr_sweep = mlp_rr_sweep(d);
   ttt::MlpFwdArgs fa;
   fa.xq = xq; fa.xk = xk; fa.xv = xv; fa.W1_0 = W1_0; fa.b1_0 = b1_0; fa.W2_0 = W2_0; fa.b2_0 = b2_0;
   fa.token_eta = token_eta; fa.lr = lr; fa.gamma = gamma; fa.beta = beta; fa.out = nullptr;
@@ -585,7 +592,9 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   fa.n_stages = d->seq / d->mini_batch;
   fa.state_per_batch = d->state_per_batch ? 1 : 0;
   fa.eps = d->eps;
-  if (rr_sweep) {
+  if (!sweep) {
+    rc = TTT_OK;
+  } else if (rr_sweep) {
     fa.out = d_xq;
     switch (d->head_dim) {
       case 32: rc = launch_mlp_fwd_rr<ttt::BF16, 32>(&fa, 1, s); break;
@@ -1181,6 +1190,61 @@ int ttt_mlp_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* x
   return mlp_bwd_impl(d, xq, xk, xv, W1_0, b1_0, W2_0, b2_0, token_eta, lr, gamma, beta, d_out, d_W1_out,
                       d_b1_out, d_W2_out, d_b2_out, d_xq, d_xk, d_xv, d_W1, d_b1, d_W2, d_b2, d_lr,
                       d_token_eta, d_gamma, d_beta, workspace, stream);
+}
+
+int ttt_mlp_fwd_saving_supported(const ttt_desc* d) {
+  int rc = ttt_mlp_supported(d);
+  if (rc != TTT_OK) return rc;
+  bool two_cu = false;
+  rc = uses_two_cu_mlp(d, 1, &two_cu);
+  if (rc != TTT_OK) return rc;
+  if (two_cu)
+    return fail(TTT_ERR_UNSUPPORTED, "ttt_mlp_fwd_saving: the forward on pairs of CUs saves nothing for the backward "
+                                     "(head_dim %d); call ttt_mlp_fwd and ttt_mlp_bwd", d->head_dim);
+  return TTT_OK;
+}
+
+int ttt_mlp_fwd_saving(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                       const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                       const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                       void* out, float* W1_out, float* b1_out, float* W2_out, float* b2_out, void* saved,
+                       void* stream) {
+  int rc = ttt_mlp_fwd_saving_supported(d);
+  if (rc != TTT_OK) return rc;
+  if (!saved) return fail(TTT_ERR_NULL, "ttt_mlp_fwd_saving: saved is NULL");
+  if (!aligned16(saved)) return fail(TTT_ERR_SHAPE, "ttt_mlp_fwd_saving: saved must be 16-byte aligned");
+  ttt::MlpFwdArgs a;
+  rc = prepare_mlp_fwd(d, xq, xk, xv, W1_0, b1_0, W2_0, b2_0, token_eta, lr, gamma, beta, out, W1_out, b1_out, W2_out,
+                       b2_out, &a);
+  if (rc != TTT_OK) return rc;
+  const MlpBwdWs w(d);
+  float* ws = static_cast<float*>(saved);
+  a.G1_save = ws + w.G1s;
+  a.G2_save = ws + w.G2s;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  rc = dispatch_mlp_fwd_pack(d, &a, 1, s);
+  if (rc != TTT_OK) return rc;
+  // the reverse scan walks the state back in place: it gets a copy of the final state of its own
+  const size_t U = (size_t)d->batch * d->heads, D = d->head_dim, M = 4 * D;
+  copy_or_zero(ws + w.W1, W1_out, U * D * M, s);
+  copy_or_zero(ws + w.b1, b1_out, U * M, s);
+  copy_or_zero(ws + w.W2, W2_out, U * M * D, s);
+  copy_or_zero(ws + w.b2, b2_out, U * D, s);
+  return hip_status(hipGetLastError(), "ttt_mlp_fwd_saving copies");
+}
+
+int ttt_mlp_bwd_saved(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                      const float* W1_0, const float* b1_0, const float* W2_0, const float* b2_0,
+                      const float* token_eta, const void* lr, const float* gamma, const float* beta,
+                      const void* d_out, const float* d_W1_out, const float* d_b1_out,
+                      const float* d_W2_out, const float* d_b2_out, void* d_xq, void* d_xk, void* d_xv,
+                      float* d_W1, float* d_b1, float* d_W2, float* d_b2, void* d_lr, float* d_token_eta,
+                      float* d_gamma, float* d_beta, void* saved, void* stream) {
+  int rc = ttt_mlp_fwd_saving_supported(d);
+  if (rc != TTT_OK) return rc;
+  return mlp_bwd_impl(d, xq, xk, xv, W1_0, b1_0, W2_0, b2_0, token_eta, lr, gamma, beta, d_out, d_W1_out,
+                      d_b1_out, d_W2_out, d_b2_out, d_xq, d_xk, d_xv, d_W1, d_b1, d_W2, d_b2, d_lr,
+                      d_token_eta, d_gamma, d_beta, saved, stream, /*sweep=*/false);
 }
 
 int ttt_mlp_bwd_static(const ttt_desc* d, const void* xq, const void* xk, const void* xv,

@@ -121,6 +121,40 @@ class FusedMlp {
                       g.grad_ln_bias, workspace, stream));
   }
 
+  /// forward over a sequence of whole mini-batches that also saves, in `saved` (backward_workspace_bytes of device
+  /// memory), what backward_saved needs: the training pair ttt_mlp_fwd_saving / ttt_mlp_bwd_saved, i.e. a backward
+  /// without a forward sweep of its own.  Throws TTT_ERR_UNSUPPORTED where the forward runs on pairs of CUs
+  /// (head_dim 128 with bf16 I/O): use forward + backward there.
+  void forward_saving(TTTMLPState& state, const TTTInputsInner& in, void* out, void* saved, void* stream) const {
+    if (in.seq_len % config_.ttt.mini_batch_size != 0)
+      throw Error(TTT_ERR_SHAPE, "forward_saving: the sequence must be whole mini-batches");
+    if (!state.next_w1 || !state.next_b1 || !state.next_w2 || !state.next_b2)
+      throw Error(TTT_ERR_NULL, "TTTMLPState: both sets of state buffers must be valid");
+    const bool per_batch = state.initialised;
+    ttt_desc d = desc(in.batch, in.seq_len, config_.ttt.mini_batch_size, in.dtype, per_batch);
+    check(ttt_mlp_fwd_saving(&d, in.qkv.xq, in.qkv.xk, in.qkv.xv, per_batch ? state.w1 : w1_,
+                             per_batch ? state.b1 : b1_, per_batch ? state.w2 : w2_, per_batch ? state.b2 : b2_,
+                             in.token_eta, in.ttt_lr_eta, ln_weight_, ln_bias_, out, state.next_w1, state.next_b1,
+                             state.next_w2, state.next_b2, saved, stream));
+    state.swap();
+    state.initialised = true;
+  }
+
+  /// backward with the arguments of backward(), `saved` (written by forward_saving on the same inputs and state0) in
+  /// place of the workspace; consumes `saved`.
+  void backward_saved(const TTTInputsInner& in, const TTTMLPState& state0, const void* grad_output,
+                      const float* grad_w1_out, const float* grad_b1_out, const float* grad_w2_out,
+                      const float* grad_b2_out, const TTTMLPGrads& g, void* saved, void* stream) const {
+    const bool per_batch = state0.initialised;
+    ttt_desc d = desc(in.batch, in.seq_len, config_.ttt.mini_batch_size, in.dtype, per_batch);
+    check(ttt_mlp_bwd_saved(&d, in.qkv.xq, in.qkv.xk, in.qkv.xv, per_batch ? state0.w1 : w1_,
+                            per_batch ? state0.b1 : b1_, per_batch ? state0.w2 : w2_, per_batch ? state0.b2 : b2_,
+                            in.token_eta, in.ttt_lr_eta, ln_weight_, ln_bias_, grad_output, grad_w1_out, grad_b1_out,
+                            grad_w2_out, grad_b2_out, g.grad_xq, g.grad_xk, g.grad_xv, g.grad_w1, g.grad_b1,
+                            g.grad_w2, g.grad_b2, g.grad_ttt_lr_eta, g.grad_token_eta, g.grad_ln_weight,
+                            g.grad_ln_bias, saved, stream));
+  }
+
  private:
   static const void* at(const void* p, std::size_t bytes) {
     return p ? static_cast<const char*>(p) + bytes : nullptr;

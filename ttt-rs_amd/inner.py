@@ -279,11 +279,13 @@ def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_
 
 
 def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias,
-                        mini_batch: int, eps: float = 1e-6, kernel_hint: int = 0):
+                        mini_batch: int, eps: float = 1e-6, kernel_hint: int = 0, save_for_backward: bool = False):
     """One call of ttt_mlp_fwd on the current stream: the fused counterpart of
     TTTMLP::forward (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50).
     w1 [B,H,d,4d] or [H,d,4d], b1 [..,4d], w2 [..,4d,d], b2 [..,d].
-    Returns (output, w1_out, b1_out, w2_out, b2_out), state per batch element."""
+    Returns (output, w1_out, b1_out, w2_out, b2_out), state per batch element.
+    save_for_backward: call ttt_mlp_fwd_saving instead and return a sixth element, the `saved` buffer that
+    ttt_mlp_backward_raw(saved=...) consumes (the backward then skips its own forward sweep)."""
     B, H, seq, d = xq.shape
     m = w1.shape[-1]
     io = xq.dtype
@@ -313,6 +315,13 @@ def ttt_mlp_forward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_we
          torch.empty((B, H, m, d), **f32), torch.empty((B, H, d), **f32)]
     stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     with torch.cuda.device(dev):
+        if save_for_backward:
+            check(lib().ttt_mlp_fwd_saving_supported(C.byref(desc)))
+            saved = torch.empty((lib().ttt_mlp_bwd_workspace_bytes(C.byref(desc)) + 3) // 4, **f32)
+            check(lib().ttt_mlp_fwd_saving(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(w1), _ptr(b1), _ptr(w2),
+                                           _ptr(b2), _ptr(te), _ptr(lr), _ptr(ln_weight), _ptr(ln_bias), _ptr(out),
+                                           *[_ptr(x) for x in o], _ptr(saved), stream))
+            return (out, *o, saved)
         check(lib().ttt_mlp_fwd(C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(w1), _ptr(b1), _ptr(w2),
                                 _ptr(b2), _ptr(te), _ptr(lr), _ptr(ln_weight), _ptr(ln_bias), _ptr(out),
                                 *[_ptr(x) for x in o], stream))
@@ -356,7 +365,7 @@ def ttt_mlpn_forward_raw(xq, xk, xv, weights, biases, token_eta, ttt_lr_eta, ln_
 
 def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_weight, ln_bias, d_out,
                          mini_batch: int, eps: float = 1e-6, d_state_out=None, static_scratch: bool = False,
-                         into=None, kernel_hint: int = 0):
+                         into=None, kernel_hint: int = 0, saved=None):
     """One call of ttt_mlp_bwd on the current stream: gradients of the TTT-MLP inner loop
     (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50; the reference gets them
     from Burn autodiff).  Arguments as ttt_mlp_forward_raw plus d_out [B,H,seq,d] and the optional
@@ -366,7 +375,9 @@ def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_w
     static_scratch: call ttt_mlp_bwd_static (the library's built-in scratch buffer instead of a workspace
     allocated here); `into`: a dict returned by an earlier call of the same shape, whose tensors receive the
     gradients (with both, the call allocates no device memory).  kernel_hint: TTT_HINT_F32_PRODUCTS keeps the
-    reverse scan's products in f32 where it would round their operands to bf16 (bf16 I/O, head_dim <= 96)."""
+    reverse scan's products in f32 where it would round their operands to bf16 (bf16 I/O, head_dim <= 96).
+    saved: the buffer a forward with save_for_backward=True returned (same inputs, same hint): ttt_mlp_bwd_saved, which
+    consumes it."""
     B, H, seq, d = xq.shape
     m = w1.shape[-1]
     io = xq.dtype
@@ -417,7 +428,9 @@ def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_w
             _ptr(ln_weight), _ptr(ln_bias), _ptr(d_out), *[null if g is None else _ptr(g) for g in up],
             *[_ptr(g) for g in g_act], *[_ptr(g) for g in g_st], _ptr(g_lr), _ptr(g_te), _ptr(g_gam), _ptr(g_bet)]
     with torch.cuda.device(dev):
-        if static_scratch:
+        if saved is not None:
+            check(lib().ttt_mlp_bwd_saved(*args, _ptr(saved), stream))
+        elif static_scratch:
             check(lib().ttt_mlp_bwd_static(*args, stream))
         else:
             nbytes = lib().ttt_mlp_bwd_workspace_bytes(C.byref(desc))
