@@ -173,3 +173,46 @@ def test_other_forwards_replay(P):
                 "mlp2 out": m[0], "mlp2 W2": m[1][1], "mlp2 b3": m[2][2]}
 
     replay_and_compare(calls, calls, refresh)
+
+
+def test_mlp_training_pair_and_long_mini_batches_replay(P):
+    """ttt_mlp_fwd_saving + ttt_mlp_bwd_saved (the forward's kernel, the copies of the final state into `saved`, the
+    fills and the reverse scan) and the TTT-Linear forward + backward at a mini-batch of 32 tokens (the LDS-tile kernels
+    on two tiles of token rows), recorded in one graph."""
+    print("case graph capture mlp saving pair + K32 linear", flush=True)
+    from test_mlp_fwd_gpu import mlp_case
+    B, H, d, N = 2, 2, 32, 3
+    dt = torch.bfloat16
+    gen = torch.Generator().manual_seed(33)
+    msets = [to_dev(mlp_case(P, 970 + i, B, H, N * 16, d, 16, dt, "ref")) for i in range(4)]
+    lsets = [to_dev(P.synthetic.reference_test_inputs(980 + i, B, H, N * 32, d, 32, io_dtype=dt)) for i in range(4)]
+    mdo = [torch.randn(B, H, N * 16, d, generator=gen).to(dt).to("cuda:0") for _ in range(4)]
+    ldo = [torch.randn(B, H, N * 32, d, generator=gen).to(dt).to("cuda:0") for _ in range(4)]
+    m = {k: v.clone() for k, v in msets[0].items()}
+    x = {k: v.clone() for k, v in lsets[0].items()}
+    dm, dl = mdo[0].clone(), ldo[0].clone()
+
+    def refresh(i):
+        for k in m:
+            m[k].copy_(msets[i][k])
+        for k in x:
+            x[k].copy_(lsets[i][k])
+        dm.copy_(mdo[i])
+        dl.copy_(ldo[i])
+
+    def calls():
+        margs = (m["xq"], m["xk"], m["xv"], m["W1"], m["b1"], m["W2"], m["b2"], m["token_eta"], m["lr"], m["gamma"],
+                 m["beta"])
+        f = P.ttt_mlp_forward_raw(*margs, 16, save_for_backward=True)
+        g = P.ttt_mlp_backward_raw(*margs, dm, 16, saved=f[5])
+        lf = P.ttt_linear_forward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"], x["gamma"],
+                                      x["beta"], 32, want_checkpoints=True)
+        lg = P.ttt_linear_backward_raw(x["xq"], x["xk"], x["xv"], x["W0"], x["b0"], x["token_eta"], x["lr"], x["gamma"],
+                                       x["beta"], lf[3], lf[4], dl, 32)
+        return {"mlp out": f[0], "mlp W2": f[3], "mlp d_xk": g["d_xk"], "mlp d_W1": g["d_W1"],
+                "mlp d_token_eta": g["d_token_eta"], "mlp d_gamma": g["d_gamma"], "lin out": lf[0], "lin W": lf[1],
+                "lin grad_xq": lg["grad_xq"], "lin grad_weight": lg["grad_weight"],
+                "lin grad_token_eta": lg["grad_token_eta"], "lin grad_ln_bias": lg["grad_ln_bias"]}
+
+    replay_and_compare(calls, calls, refresh,
+                       names_atomic=("mlp d_token_eta", "mlp d_gamma", "lin grad_token_eta", "lin grad_ln_bias"))
