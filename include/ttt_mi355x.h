@@ -110,6 +110,10 @@ typedef struct ttt_desc {
  * TTT_HINT_F32_PRODUCTS keeps every product of the scan in f32 (about twice the time).  Ignored elsewhere: f32 I/O and
  * head_dim 128 always compute in f32. */
 #define TTT_HINT_F32_PRODUCTS 0x4000
+/* ttt_mlp_bwd and its variants: with at most 128 (batch, head) units every unit is worked on by two workgroups on two
+ * CUs (see ttt_mlp_bwd); TTT_HINT_ONE_WORKGROUP keeps a unit on one.  Same results bit for bit (d_token_eta, which
+ * is summed over the units with atomic additions, aside); the workspace is smaller. */
+#define TTT_HINT_ONE_WORKGROUP 0x8000
 /* Testing only: the two workgroups that share a (batch, head) unit in ttt_mlp_fwd at head_dim 128 (bf16 I/O) give
  * up waiting for each other at once, as if the partner had never become resident.  Exercises the failure path
  * described at ttt_mlp_fwd: every output of the affected units is NaN.  All kernels still run to their end. */
@@ -213,7 +217,8 @@ int ttt_linear_bwd(const ttt_desc* desc, const void* xq, const void* xk, const v
  * A caller that shares the GPU checks one output element per unit, reads the status word below, or passes
  * TTT_HINT_LDS_TILES to use the single-workgroup kernel (slower, f32 products).
  *
- * ttt_mlp_fwd_lost_workgroups: the device's status word of that kernel, the number of workgroups whose wait for
+ * ttt_mlp_fwd_lost_workgroups: the device's status word of that kernel (and of ttt_mlp_bwd's kernel on two
+ * workgroups per unit, see there), the number of workgroups whose wait for
  * their partner ran out since the library was loaded on the current device (0 on a healthy run; it never
  * decreases, compare with the value before the call).  A blocking copy from the device: call it after the
  * stream's work has finished.  No counterpart in the reference.
@@ -248,6 +253,16 @@ int ttt_mlp_fwd(const ttt_desc* desc, const void* xq, const void* xk, const void
  * the caller and free to reuse after the call's work on `stream` has finished.  It holds the
  * rolling state, the per-mini-batch update factors of the forward sweep and scratch tiles.
  * seq must be a multiple of mini_batch.
+ *
+ * Two workgroups per unit.  With at most 128 (batch, head) units (and at least two CUs per unit on the device; no
+ * TTT_HINT_ONE_WORKGROUP) the reverse scan of a unit runs on two workgroups on two CUs: one walks the state back and
+ * recomputes the forward's intermediates a mini-batch ahead, the other carries the gradient; they hand their data
+ * over in the workspace (which is larger for such a desc) and follow each other through two counters there.  Same
+ * results as on one workgroup, bit for bit.  Both must be resident together, as in ttt_mlp_fwd at head_dim 128,
+ * and what is said there of a GPU shared with other work holds here: a workgroup that waits for its partner in
+ * vain (2^21 polls, seconds) gives up, both run to the end without waiting again, the unit's d_b1 is NaN in every
+ * element (the unit's other gradients are then meaningless) and ttt_mlp_fwd_lost_workgroups counts the two
+ * workgroups.  The workspace must be ordinary device memory (hipMalloc), not fine-grained or host memory.
  */
 int64_t ttt_mlp_bwd_workspace_bytes(const ttt_desc* desc);
 int ttt_mlp_bwd(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,

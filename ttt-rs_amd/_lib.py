@@ -17,6 +17,7 @@ TTT_HINT_OWN_LOADS = 0x1000
 TTT_HINT_ALL_LOADS = 0x2000
 TTT_HINT_TEST_OTHER_XCD = 0x800
 TTT_HINT_F32_PRODUCTS = 0x4000
+TTT_HINT_ONE_WORKGROUP = 0x8000
 
 EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_bwd_supported",

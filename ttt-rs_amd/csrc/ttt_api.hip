@@ -407,14 +407,22 @@ int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
   return hip_status(hipGetLastError(), "ttt_linear_bwd (multi-wave register-resident kernel) launch");
 }
 
-template <class T, int D, bool BF = false>
-int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
-  constexpr auto kern = ttt::ttt_mlp_bwd_kernel<T, D, BF>;
+template <class T, int D, bool BF, bool PIPE>
+int launch_mlp_bwd_as(const ttt::MlpBwdArgs& a, hipStream_t s) {
+  constexpr auto kern = ttt::ttt_mlp_bwd_kernel<T, D, BF, PIPE>;
   constexpr size_t bytes = ttt::MlpBwdLds<D>::BYTES;
   int rc = opt_in_lds<kern>(bytes);
   if (rc != TTT_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(a.B * a.H)), dim3(512), bytes, s, a);
+  // two workgroups per unit: workgroups b and b + 8 of every 16 share a unit
+  const unsigned units = (unsigned)(a.B * a.H), grid = PIPE ? (units + 7) / 8 * 16 : units;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_mlp_bwd launch");
+}
+template <class T, int D, bool BF = false>
+int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
+  static_assert(ttt::MlpBwdPipe<D>::FLOATS > 0, "");
+  if (a.pipe != nullptr) return launch_mlp_bwd_as<T, D, BF, true>(a, s);
+  return launch_mlp_bwd_as<T, D, BF, false>(a, s);
 }
 
 // Which TTT-Linear backward kernel serves a desc (and whether one does).
@@ -496,9 +504,17 @@ void copy_or_zero(float* dst, const float* src, size_t n, hipStream_t s) {
   hipLaunchKernelGGL(ttt_copy_or_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, dst, src, n);
 }
 
+// Whether the TTT-MLP reverse scan spreads every unit over two workgroups (producer and consumer, see
+// ttt_mlp_bwd_kernel): when every pair can have two CUs of its own.  A function of the desc alone, because the size of
+// the workspace follows from it; the launch checks the device's CU count on top.
+constexpr int kMlpBwdPipeMaxUnits = 128;
+bool mlp_bwd_pipe(const ttt_desc* d) {
+  return (int64_t)d->batch * d->heads <= kMlpBwdPipeMaxUnits && !(d->kernel_hint & TTT_HINT_ONE_WORKGROUP);
+}
+
 // float offsets of the pieces of the ttt_mlp_bwd workspace
 struct MlpBwdWs {
-  size_t W1, W2, b1, b2, G1s, G2s, mt, total;
+  size_t W1, W2, b1, b2, G1s, G2s, mt, pipe, flags, total;
   explicit MlpBwdWs(const ttt_desc* d) {
     const size_t U = (size_t)d->batch * d->heads, D = d->head_dim, M = 4 * D, N = d->seq / d->mini_batch;
     W1 = 0;
@@ -509,6 +525,14 @@ struct MlpBwdWs {
     G2s = G1s + U * N * 16 * M;
     mt = G2s + U * N * 16 * D;
     total = mt + U * ttt::kMlpBwdMTiles * 16 * M;
+    pipe = flags = total;
+    if (mlp_bwd_pipe(d)) {
+      // the same arithmetic as ttt::MlpBwdPipe<D>::FLOATS
+      const size_t xb = (48 * D + 4 * 256 + 16 + D + 3) / 4 * 4;
+      const size_t per_unit = 2 * D * M + ttt::kMlpBwdSharedTiles * 16 * M + 2 * xb;
+      flags = pipe + U * per_unit;
+      total = flags + U * ttt::kMlpBwdPipeFlagWords;
+    }
   }
 };
 
@@ -632,6 +656,22 @@ int mlp_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* 
   a.d_lr = d_lr; a.d_token_eta = d_token_eta; a.d_gamma = d_gamma; a.d_beta = d_beta;
   a.B = d->batch; a.H = d->heads; a.seq = d->seq; a.K = d->mini_batch;
   a.seq_stride = fa.seq_stride; a.n_stages = fa.n_stages; a.eps = d->eps;
+  a.pipe = nullptr; a.pipe_flags = nullptr; a.spin_limit = 1u << 21; a.agent_release = 0;
+  if (mlp_bwd_pipe(d)) {
+    // both workgroups of every unit must be resident together: as many CUs as workgroups
+    int cus = 0;
+    rc = device_cus(&cus);
+    if (rc != TTT_OK) return rc;
+    if ((int64_t)(U + 7) / 8 * 16 <= cus) {
+      a.pipe = ws + w.pipe;
+      a.pipe_flags = reinterpret_cast<unsigned*>(ws + w.flags);
+      if (d->kernel_hint & TTT_HINT_TEST_LOST_PARTNER) a.spin_limit = 0;
+      if (d->kernel_hint & TTT_HINT_TEST_OTHER_XCD) a.agent_release = 1;
+      copy_or_zero(ws + w.flags, nullptr, U * ttt::kMlpBwdPipeFlagWords, s);
+      rc = hip_status(hipGetLastError(), "ttt_mlp_bwd flag fill");
+      if (rc != TTT_OK) return rc;
+    }
+  }
   // behind the register-resident sweep the scan takes bf16 operands too (the states it walks back through were
   // formed from bf16 operands); TTT_HINT_F32_PRODUCTS keeps the scan's products in f32
   if (rr_sweep && !(d->kernel_hint & TTT_HINT_F32_PRODUCTS)) switch (d->head_dim) {

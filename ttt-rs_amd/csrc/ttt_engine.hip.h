@@ -11,6 +11,11 @@
 
 namespace ttt {
 
+// Status word of the kernels that spread a (batch, head) unit over two workgroups (TTT-MLP forward at head_dim 128,
+// TTT-MLP backward): workgroups whose wait for their partner ran out, counted since the library was loaded (one
+// copy per GPU).  Read by ttt_mlp_fwd_lost_workgroups.
+__device__ unsigned int g_mlp_fwd_lost_workgroups = 0u;
+
 // 16 rows x 64 bytes of a row-major matrix in GLOBAL memory, delivered in matrix-operand order: lane (c = lane % 16,
 // g = lane / 16) receives the 16 bytes at row c, byte offset 16 g.  Loaded directly in that order, each quarter
 // wave (16 lanes with the same g) touches 16 cache lines and the load runs at 16 B per cycle and CU; here lane l
@@ -318,8 +323,11 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
 template <bool BF, int MODE, int NW, int NB, int KS, bool FZ>
 __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                           int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
-                                          const float* X, int x_rs, float* Z, int ldz) {
+                                          const float* X, int x_rs, float* Z, int ldz, const float* Csrc = nullptr) {
   static_assert(MODE == 1 || MODE == 2, "read-modify-write modes only");
+  // Csrc: where the tiles of C are read from when the updated matrix goes to another buffer (same layout); the
+  // ordering argument below only gets easier, since no load ever meets a store
+  const float* Cin = Csrc != nullptr ? Csrc : C;
   static_assert(!BF || KS % 4 == 0, "bf16 operands: whole 16-deep steps");
   const int c = lane & 15, g = lane >> 4;
   const int nblk = Nt / NB, njobs = Mt * nblk;
@@ -347,7 +355,7 @@ __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int
 #pragma unroll
     for (int j = 0; j < NB; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) s.acc[j][r] = C[coff + r * ldc + 16 * j];
+      for (int r = 0; r < 4; ++r) s.acc[j][r] = Cin[coff + r * ldc + 16 * j];
     const int aoff = (16 * tm + c) * a_rs + g * a_cs, boff = g * b_rs + (16 * tn0 + c) * b_cs;
 #pragma unroll
     for (int u = 0; u < KS; ++u) {
@@ -554,8 +562,9 @@ struct Eng {
   template <int MODE, int NW, int NB, int KS, bool FZ = false>
   static __device__ __forceinline__ void rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                               int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
-                                              const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
-    mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz);
+                                              const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0,
+                                              const float* Csrc = nullptr) {
+    mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz, Csrc);
   }
   template <int MODE, int NW, int NT, int KSTEPS>
   static __device__ __forceinline__ void splitk(float* C, int ldc, float* part, const float* A, int a_rs,

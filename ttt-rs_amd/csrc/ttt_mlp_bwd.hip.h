@@ -54,9 +54,30 @@ struct MlpBwdArgs {
   float* d_beta;
   int B, H, seq, seq_stride, K, n_stages;
   float eps;
+  // two workgroups per unit (template flag PIPE of the kernel)
+  float* pipe;           // [B*H][MlpBwdPipe<d>::FLOATS]: second state buffer, second set of shared tiles, exchange blocks
+  unsigned* pipe_flags;  // [B*H][kMlpBwdPipeFlagWords] progress words, zero on entry
+  unsigned spin_limit;   // polls before a wait for the partner gives up; 0: give up at once (tests of that path)
+  int agent_release;     // 1: the producer always publishes with a device-scope release
 };
 
 constexpr int kMlpBwdMTiles = 9;  // [16 x 4d] scratch tiles per (batch, head)
+constexpr int kMlpBwdSharedTiles = 6;  // the first six are written by the recomputation and read by the gradient part
+constexpr int kMlpBwdPipeFlagWords = 32;  // per unit: [0] producer's count, [1] consumer's count, [2], [3] XCD ids
+constexpr unsigned kMlpBwdPipePoison = 0xffffffffu;
+
+// What the two workgroups of a unit share besides the kernel's ordinary workspace (float offsets within a.pipe's
+// slice of the unit): the second buffer of the rolling state, the second set of the shared [16 x 4d] tiles, and two
+// exchange blocks for what the one-workgroup kernel hands from its first half to its second in LDS.
+template <int D>
+struct MlpBwdPipe {
+  static constexpr int M = 4 * D;
+  // exchange block
+  static constexpr int XH = 0, G2 = XH + 16 * D, XH2 = G2 + 16 * D, A1 = XH2 + 16 * D, M1 = A1 + 256, M2 = M1 + 256,
+                       A2P = M2 + 256, RSTD = A2P + 256, B2 = RSTD + 16, XB = (B2 + D + 3) / 4 * 4;
+  static constexpr int W1X = 0, W2X = W1X + D * M, TILES = W2X + M * D, XBLK = TILES + kMlpBwdSharedTiles * 16 * M,
+                       FLOATS = XBLK + 2 * XB;
+};
 
 template <int D>
 struct MlpBwdLds {
@@ -69,7 +90,7 @@ struct MlpBwdLds {
                        DA = P + KK, DETA = DA + KK, PART = DETA + KK;
   static constexpr int b1 = PART + 8 * 256, b2 = b1 + M, db1 = b2 + D, db2 = db1 + M, gam = db2 + D,
                        bet = gam + D, lr = bet + D, te = lr + 16, rstd1 = te + 16, dlast = rstd1 + 16,
-                       SKP = dlast + 16;
+                       PIPEW = dlast + 16, SKP = PIPEW + 16;
   // partial products of the split-k [16 x d] products, one tile per wave: where LDS has the room (d <= 96)
   static constexpr bool SPLITK = D <= 96;
   static constexpr int END = SKP + (SPLITK ? 8 * TD : 0);
@@ -90,7 +111,18 @@ __device__ __forceinline__ void gelu_tanh_all(float x, float& y, float& dy, floa
 // BF: every product takes its operands rounded to bf16 (bf16 I/O behind the register-resident forward sweep, whose
 // own products and state updates took bf16 operands: the states the scan walks back through are the ones that
 // sweep formed).  Otherwise all contractions are true-f32 MFMA.
-template <class T, int D, bool BF = false>
+//
+// PIPE: two workgroups per unit on two CUs of one XCD.  A mini-batch's work falls into a part that needs only the
+// state walked back (steps 1 - 10: the roll-back and the recomputation of the forward's intermediates) and a part
+// that needs the gradient carried from the later mini-batches (steps 11 - 24).  The producer workgroup runs the
+// first part one mini-batch ahead of the consumer, which runs the second; what crosses (the rolled-back state,
+// six [16 x 4d] tiles, a block of LDS-sized tiles) lies in two sets of buffers used alternately, and two counters
+// in global memory say how far each side has come.  Workgroup b is the producer and b + 8 the consumer of one
+// unit: consecutive workgroup ids go to the XCDs in turn, so both run behind one L2; each reads its XCD id and the
+// producer publishes with a device-scope release (write-back of its L2) until it has seen that the ids agree.
+// Every wait is bounded: a side that waits in vain marks its counter, both run to the end without further waits, the
+// consumer makes the unit's d_b1 NaN and the status word g_mlp_fwd_lost_workgroups counts the event.
+template <class T, int D, bool BF = false, bool PIPE = false>
 // One workgroup per CU (the LDS use decides that), two waves per SIMD: said explicitly, because the scheduler
 // otherwise aims at a higher occupancy and, to save registers, issues independent loads one at a time.
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) ttt_mlp_bwd_kernel(MlpBwdArgs a) {
@@ -109,20 +141,68 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   // it would occupy several hundred registers and spill.
   int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int t = tid >> 5, cg = tid & 31;  // elementwise mapping: token t, columns cg + 32 j
-  const size_t bh = blockIdx.x;
+  using PX = MlpBwdPipe<D>;
+  size_t bh = blockIdx.x;
+  int role = 2;  // 0 producer, 1 consumer, 2 both
+  if constexpr (PIPE) {
+    bh = (size_t)(blockIdx.x >> 4) * 8 + (blockIdx.x & 7);
+    role = (blockIdx.x >> 3) & 1;
+    if (bh >= (size_t)a.B * a.H) return;
+  }
+  const bool do_p = !PIPE || role == 0, do_c = !PIPE || role == 1;
   const int h = (int)(bh % a.H), K = a.K, N = a.n_stages;
   float *sb1 = lds + L::b1, *sb2 = lds + L::b2, *sdb1 = lds + L::db1, *sdb2 = lds + L::db2,
         *sgam = lds + L::gam, *sbet = lds + L::bet, *slr = lds + L::lr, *ste = lds + L::te;
-  float* W1 = a.W1 + bh * (size_t)D * M;
-  float* W2 = a.W2 + bh * (size_t)M * D;
+  float* const W1h = a.W1 + bh * (size_t)D * M;
+  float* const W2h = a.W2 + bh * (size_t)M * D;
   float* dW1 = a.d_W1 + bh * (size_t)D * M;
   float* dW2 = a.d_W2 + bh * (size_t)M * D;
   // [16 x 4d] scratch tiles
   float* mt = a.mt + bh * (size_t)kMlpBwdMTiles * 16 * M;
-  // (X2, U, Xbar2) and (dZbar1, dZ1) are consecutive: each group is the k-side operand of one fused
-  // rank-48 / rank-32 accumulation into dW2 / dW1
-  float *mZ1 = mt, *mX2 = mt + 16 * M, *mU = mt + 2 * 16 * M, *mXB2 = mt + 3 * 16 * M, *mG1 = mt + 4 * 16 * M,
-        *mZB1 = mt + 5 * 16 * M, *mDXB = mt + 6 * 16 * M, *mDX2 = mt + 7 * 16 * M, *mS1 = mt + 8 * 16 * M;
+  float* const px = PIPE ? a.pipe + bh * (size_t)PX::FLOATS : nullptr;
+  unsigned* const fl = PIPE ? a.pipe_flags + bh * (size_t)kMlpBwdPipeFlagWords : nullptr;
+  int& lost = *reinterpret_cast<int*>(lds + L::PIPEW);  // written by thread 0 only
+  unsigned my_xcc = 0;
+  bool fast_release = false;  // producer: the consumer is known to sit behind the same L2
+  if constexpr (PIPE) {
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(my_xcc));
+    my_xcc &= 15u;
+    if (tid == 0) {
+      lost = a.spin_limit == 0 ? 1 : 0;
+      __hip_atomic_store(fl + 2 + role, 0x100u | my_xcc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  // Waits until the partner's counter has reached `want` (thread 0 polls), then every wave drops what its CU's
+  // vector cache holds, so that the loads that follow see what the partner stored before it raised the counter.
+  auto wait_for = [&](int which, int want) {
+    if (want > 0 && tid == 0 && lost == 0) {
+      bool got = false;
+      for (unsigned i = 0; i < a.spin_limit; ++i) {
+        const unsigned v = __hip_atomic_load(fl + which, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (v == kMlpBwdPipePoison) break;
+        if (v >= (unsigned)want) {
+          got = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      if (!got) lost = 1;
+    }
+    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  };
+  // Raises this side's counter once every store of every wave has reached the L2 (or, `wide`, device scope).  The
+  // barrier inside also closes the mini-batch for the reuse of LDS.
+  auto signal = [&](int which, int value, bool wide) {
+    if (wide)
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0)
+      __hip_atomic_store(fl + which, lost != 0 ? kMlpBwdPipePoison : (unsigned)value, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+  };
 
   for (int i = tid; i < M; i += 512) {
     sb1[i] = a.b1f[bh * M + i];
@@ -230,6 +310,38 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     const float* G1l = a.G1s + ((bh * N + st) * (size_t)16) * M;
     const float* G2l = a.G2s + ((bh * N + st) * (size_t)16) * D;
     const size_t row = bh * (size_t)a.seq_stride + (size_t)st * K + t;
+    // The state entering mini-batch st is formed in W1 / W2 from the state in W1r / W2r (the same buffers, walked
+    // back in place, unless two workgroups share the unit: then the buffer that held the final state on entry and
+    // the second one take turns, so that the consumer still reads one while the producer forms the next).
+    float *W1 = W1h, *W2 = W2h;
+    const float *W1r = nullptr, *W2r = nullptr;
+    // (X2, U, Xbar2) and (dZbar1, dZ1) are consecutive: each group is the k-side operand of one fused
+    // rank-48 / rank-32 accumulation into dW2 / dW1
+    float* sh = mt;
+    float* xb = nullptr;
+    if constexpr (PIPE) {
+      const bool home = ((st ^ N) & 1) == 0;
+      W1 = home ? W1h : px + PX::W1X;
+      W2 = home ? W2h : px + PX::W2X;
+      W1r = home ? px + PX::W1X : W1h;
+      W2r = home ? px + PX::W2X : W2h;
+      if (st & 1) sh = px + PX::TILES;
+      xb = px + PX::XBLK + (st & 1) * PX::XB;
+    }
+    float *mZ1 = sh, *mX2 = sh + 16 * M, *mU = sh + 2 * 16 * M, *mXB2 = sh + 3 * 16 * M, *mG1 = sh + 4 * 16 * M,
+          *mZB1 = sh + 5 * 16 * M, *mDXB = mt + 6 * 16 * M, *mDX2 = mt + 7 * 16 * M, *mS1 = mt + 8 * 16 * M;
+    if constexpr (PIPE) {
+      if (role == 0) {
+        // the buffers of this parity were last read by the consumer in mini-batch st + 2
+        wait_for(1, N - st - 2);
+        if (!fast_release && a.agent_release == 0 && N - st - 2 > 0) {
+          const unsigned other = __hip_atomic_load(fl + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          fast_release = other == (0x100u | my_xcc);
+        }
+      } else {
+        wait_for(0, N - st);
+      }
+    }
 
     // ---- 1. inputs of this mini-batch (fetched while the previous one was computed); target = XV - XK
     if constexpr (!PFIN) fetch_inputs(st);
@@ -242,12 +354,35 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       lds[L::DO + o] = pre.o[j];
     }
     if (tid < 16) slr[tid] = pre.lr;
+    if constexpr (PIPE) {
+      if (role == 1) {
+        // what the producer left for this mini-batch
+#pragma unroll
+        for (int j = 0; j < NJD; ++j) {
+          const int o = t * LD + cg + GW * j, x = t * D + cg + GW * j;
+          lds[L::XH + o] = xb[PX::XH + x];
+          lds[L::G2 + o] = xb[PX::G2 + x];
+          lds[L::XH2 + o] = xb[PX::XH2 + x];
+        }
+        if (tid < 256) {
+          const int o = (tid >> 4) * LK + (tid & 15);
+          lds[L::A1 + o] = xb[PX::A1 + tid];
+          lds[L::M1 + o] = xb[PX::M1 + tid];
+          lds[L::M2 + o] = xb[PX::M2 + tid];
+          lds[L::DETA + o] = xb[PX::A2P + tid];  // 1 + A2: read and replaced by the same thread in step 13
+        }
+        if (tid < 16) lds[L::rstd1 + tid] = xb[PX::RSTD + tid];
+        if (tid < D) sb2[tid] = xb[PX::B2 + tid];
+      }
+    }
     __syncthreads();
     if constexpr (PFIN) fetch_inputs(st > 0 ? st - 1 : 0);  // always: a load under a branch weakens every later wait
     const float last = te_last * slr[t];
+    float rstd1 = 0.f;
+    if (do_p) {
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
     // Z1 = XK W1 (step 3) rides along on the rolled-back tiles
-    E::template rank<1, NW, NBM, 4, true>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M);
+    E::template rank<1, NW, NBM, 4, true>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M, W1r);
     if (tid < M) sb1[tid] += col16_sum(G1l + tid, M);
     __syncthreads();
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
@@ -265,7 +400,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 4. roll W2, b2 back
-    E::template rank<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, wave, lane);
+    E::template rank<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, wave, lane, nullptr, 0, nullptr, 0, W2r);
     if (tid < D) sb2[tid] += col16_sum(G2l + tid, D);
     __syncthreads();
     // ---- 5. Z2 = X2 W2 ; A1 = XQ XK^T ; eta
@@ -277,7 +412,6 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 6. LayerNorm of Z2 + b2: x_hat, rstd, G2 ; M1 = eta (1 + A1)
-    float rstd1;
     {
       float xh[NJD], gx[NJD], s1 = 0.f, s2 = 0.f;
       ln_stats<D, GW>(lds + L::XH + t * LD, sb2, cg, a.eps, xh, rstd1);
@@ -342,11 +476,43 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     if (tid < 256) {
       const int tt = tid >> 4, s = tid & 15;
-      lds[L::M2 + tt * LK + s] = lds[L::ETA + tt * LK + s] * (1.f + part_sum(tt, s));
+      const float a2p = 1.f + part_sum(tt, s);
+      lds[L::M2 + tt * LK + s] = lds[L::ETA + tt * LK + s] * a2p;
+      if constexpr (PIPE) xb[PX::A2P + tid] = a2p;
     }
     __syncthreads();
     E::template lds<2, NW, 1, 4>(lds + L::XH2, LD, lds + L::M2, LK, 1, lds + L::G2, LD, 1, 1, NTD, 16, wave, lane);
-    __syncthreads();
+    if constexpr (PIPE) {
+      __syncthreads();
+      // hand the LDS-resident results to the consumer
+#pragma unroll
+      for (int j = 0; j < NJD; ++j) {
+        const int o = t * LD + cg + GW * j, x = t * D + cg + GW * j;
+        xb[PX::XH + x] = lds[L::XH + o];
+        xb[PX::G2 + x] = lds[L::G2 + o];
+        xb[PX::XH2 + x] = lds[L::XH2 + o];
+      }
+      if (tid < 256) {
+        const int o = (tid >> 4) * LK + (tid & 15);
+        xb[PX::A1 + tid] = lds[L::A1 + o];
+        xb[PX::M1 + tid] = lds[L::M1 + o];
+        xb[PX::M2 + tid] = lds[L::M2 + o];
+      }
+      if (cg == 0) xb[PX::RSTD + t] = rstd1;
+      if (tid < D) xb[PX::B2 + tid] = sb2[tid];
+      signal(0, N - st, !fast_release);
+    } else {
+      __syncthreads();
+    }
+    }  // do_p
+    if (do_c) {
+    if constexpr (PIPE) {
+      if (tid < 256) {
+        const int tt = tid >> 4, s = tid & 15;
+        lds[L::ETA + tt * LK + s] = (s <= tt) ? ste[tt] * slr[s] : 0.f;
+      }
+      rstd1 = lds[L::rstd1 + t];
+    }
     // ---- 11. output LayerNorm backward: dZbar2
     {
       float xh[NJD], rstd2, gx2[NJD], s1 = 0.f, s2 = 0.f;
@@ -378,8 +544,10 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       const float p = (s <= tt) ? lds[L::P + tt * LK + s] : 0.f;
       const float et = lds[L::ETA + tt * LK + s];
       lds[L::DA + tt * LK + s] = -p * et;
-      // 1 + A2 = M2 / eta is not safe for eta = 0: recompute from the split-k sums still in PART
-      lds[L::DETA + tt * LK + s] = -p * (1.f + part_sum(tt, s));
+      // 1 + A2 = M2 / eta is not safe for eta = 0: recompute from the split-k sums still in PART (two workgroups:
+      // the producer left it in this very element)
+      const float a2p = PIPE ? lds[L::DETA + tt * LK + s] : 1.f + part_sum(tt, s);
+      lds[L::DETA + tt * LK + s] = -p * a2p;
     }
     {
       float q = 0.f;
@@ -565,11 +733,20 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
         for (int r = 0; r < 16; ++r) s += lds[L::dlast + r] * slr[r];
       if (tt < K) atomicAdd(a.d_token_eta + (size_t)st * K + tt, s);
     }
-    __syncthreads();
+    if constexpr (PIPE)
+      signal(1, N - st, false);
+    else
+      __syncthreads();
+    }  // do_c
   }
+  if constexpr (PIPE) {
+    if (tid == 0 && lost != 0) atomicAdd(&g_mlp_fwd_lost_workgroups, 1u);
+    if (role == 0) return;
+  }
+  const bool poison = PIPE && lost != 0;
 
   // ---- results carried over the whole scan
-  for (int i = tid; i < M; i += 512) a.d_b1[bh * M + i] = sdb1[i];
+  for (int i = tid; i < M; i += 512) a.d_b1[bh * M + i] = poison ? __builtin_nanf("") : sdb1[i];
   for (int i = tid; i < D; i += 512) a.d_b2[bh * D + i] = sdb2[i];
 #pragma unroll
   for (int j = 0; j < NJD; ++j) {

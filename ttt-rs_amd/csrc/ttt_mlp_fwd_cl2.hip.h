@@ -126,10 +126,6 @@ __device__ __forceinline__ void recv_tagged(const unsigned long long* const (&sl
                    __uint_as_float((unsigned)wd[n][2]), __uint_as_float((unsigned)wd[n][3])};
 }
 
-// Status word of the two-CU kernel: workgroups whose wait for their partner ran out, counted since the library was
-// loaded (one copy per GPU).  Read by ttt_mlp_fwd_lost_workgroups.
-__device__ unsigned int g_mlp_fwd_lost_workgroups = 0u;
-
 #define RELANE() asm volatile("" : "+v"(lane))
 
 template <class T, int D>

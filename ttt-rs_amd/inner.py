@@ -429,6 +429,9 @@ def ttt_mlp_backward_raw(xq, xk, xv, w1, b1, w2, b2, token_eta, ttt_lr_eta, ln_w
             *[_ptr(g) for g in g_act], *[_ptr(g) for g in g_st], _ptr(g_lr), _ptr(g_te), _ptr(g_gam), _ptr(g_bet)]
     with torch.cuda.device(dev):
         if saved is not None:
+            if saved.numel() * saved.element_size() < lib().ttt_mlp_bwd_workspace_bytes(C.byref(desc)):
+                raise _lib.TttError(_lib.TTT_ERR_SHAPE, "saved is smaller than this desc's workspace (a forward with "
+                                                         "another kernel_hint?)")
             check(lib().ttt_mlp_bwd_saved(*args, _ptr(saved), stream))
         elif static_scratch:
             check(lib().ttt_mlp_bwd_static(*args, stream))
