@@ -320,10 +320,12 @@ __device__ __forceinline__ void mm_lds(float* C, int ldc, const float* A, int a_
 // in code generated for that form, which is why it is not used.  The head_dim-128 instance (256 VGPRs, a handful of
 // registers spilled outside the loops) is held by a test that runs it three times and asks for identical bits.
 // BF: bf16 operands, four k-steps per matrix instruction (mma16).
-template <bool BF, int MODE, int NW, int NB, int KS, bool FZ>
+// FZ == 2: a second product of the same kind, Z2 = X2 * C_new (same strides as X and Z), rides along as well.
+template <bool BF, int MODE, int NW, int NB, int KS, int FZ>
 __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                           int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
-                                          const float* X, int x_rs, float* Z, int ldz, const float* Csrc = nullptr) {
+                                          const float* X, int x_rs, float* Z, int ldz, const float* Csrc = nullptr,
+                                          const float* X2 = nullptr, float* Z2 = nullptr) {
   static_assert(MODE == 1 || MODE == 2, "read-modify-write modes only");
   // Csrc: where the tiles of C are read from when the updated matrix goes to another buffer (same layout); the
   // ordering argument below only gets easier, since no load ever meets a store
@@ -331,9 +333,11 @@ __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int
   static_assert(!BF || KS % 4 == 0, "bf16 operands: whole 16-deep steps");
   const int c = lane & 15, g = lane >> 4;
   const int nblk = Nt / NB, njobs = Mt * nblk;
-  f32x4 zacc[NB];
+  f32x4 zacc[NB], zacc2[FZ == 2 ? NB : 1];
 #pragma unroll
   for (int j = 0; j < NB; ++j) zacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < (FZ == 2 ? NB : 1); ++j) zacc2[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   // When the number of column blocks divides the number of waves, all jobs of a wave lie in one column block
   // and share their B operand: it is loaded once and kept in registers.
   const bool bfix = NW % nblk == 0;
@@ -407,6 +411,20 @@ __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int
 #pragma unroll
           for (int j = 0; j < NB; ++j) zacc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[r], s.acc[j][r], zacc[j], 0, 0, 0);
       }
+      if constexpr (FZ == 2) {
+        const f32x4 xw = *reinterpret_cast<const f32x4*>(X2 + c * x_rs + 16 * tm + 4 * g);
+        if constexpr (BF) {
+          const auto xf = Io<BF16>::to_frag(xw);
+#pragma unroll
+          for (int j = 0; j < NB; ++j) Io<BF16>::mma(zacc2[j], xf, Io<BF16>::to_frag(s.acc[j]));
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+              zacc2[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(xw[r], s.acc[j][r], zacc2[j], 0, 0, 0);
+        }
+      }
     }
   };
   int job = wave;
@@ -460,10 +478,16 @@ __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int
     for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) Z[zoff + r * ldz + 16 * j] = zacc[j][r];
+    if constexpr (FZ == 2) {
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Z2[zoff + r * ldz + 16 * j] = zacc2[j][r];
+    }
   }
 }
 
-template <int MODE, int NW, int NB, int KS, bool FZ = false>
+template <int MODE, int NW, int NB, int KS, int FZ = 0>
 __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                         int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
                                         const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0) {
@@ -559,12 +583,14 @@ struct Eng {
                                              int first = 0, int k0 = 0) {
     mm_lds_t<BF, MODE, NW, NB, KU, BG>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, Kd, wave, lane, first, k0);
   }
-  template <int MODE, int NW, int NB, int KS, bool FZ = false>
+  template <int MODE, int NW, int NB, int KS, int FZ = 0>
   static __device__ __forceinline__ void rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                               int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
                                               const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0,
-                                              const float* Csrc = nullptr) {
-    mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz, Csrc);
+                                              const float* Csrc = nullptr, const float* X2 = nullptr,
+                                              float* Z2 = nullptr) {
+    mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz, Csrc, X2,
+                                        Z2);
   }
   template <int MODE, int NW, int NT, int KSTEPS>
   static __device__ __forceinline__ void splitk(float* C, int ldc, float* part, const float* A, int a_rs,

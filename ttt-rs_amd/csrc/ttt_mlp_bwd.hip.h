@@ -1,4 +1,5 @@
-// TTT-MLP fused backward for gfx950: one workgroup (8 wavefronts) per (batch, head).
+// TTT-MLP fused backward for gfx950: one workgroup (8 wavefronts) per (batch, head), or two (template flag PIPE: a
+// producer that walks the state back and a consumer that carries the gradient, on two CUs).
 //
 // Arithmetic: the gradient of the TTT-MLP inner loop (reference rust/core/src/mlp.rs:127-208
 // looped as rust/core/src/inner.rs:25-50).  The reference has no fused MLP kernel and
@@ -135,6 +136,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   constexpr int NBM = NTM / NW;  // [16 x 4d] products: one job of NBM tile columns per wave
   constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
   constexpr float inv_d = 1.0f / D;
+  constexpr int RIDE = D <= 96 ? 2 : 1;  // products riding along on the W1 roll-back (head_dim 128 is at the register limit)
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // The thread indices are re-derived from an opaque copy at the top of every mini-batch (below): the
   // address arithmetic of the ~30 tile products is cheap, but hoisted out of the scan as loop invariants
@@ -381,8 +383,9 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     float rstd1 = 0.f;
     if (do_p) {
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
-    // Z1 = XK W1 (step 3) rides along on the rolled-back tiles
-    E::template rank<1, NW, NBM, 4, true>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M, W1r);
+    // Z1 = XK W1 (step 3) rides along on the rolled-back tiles, and where the registers allow so does XQ W1 (step 7)
+    E::template rank<1, NW, NBM, 4, RIDE>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M, W1r,
+                                          lds + L::XQ, mZB1);
     if (tid < M) sb1[tid] += col16_sum(G1l + tid, M);
     __syncthreads();
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
@@ -438,7 +441,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 7. U = G2 W2^T ; Zbar1 = XQ W1
     E::template lds<0, NW, NBM, 2, true>(mU, M, lds + L::G2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
-    E::template lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
+    if constexpr (RIDE != 2) E::template lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 8. G1 = U gelu'(Z1)
     {
@@ -537,6 +540,10 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     E::template lds<0, NW>(lds + L::P, LK, lds + L::DZB2, LD, 1, lds + L::G2, 1, LD, 1, 1, D, wave, lane, NW - 1);
     E::template lds<0, NW, NBM, 2, true>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     prod_k(M0{}, lds + L::DG2, mX2, dW2, D, 1);
+    // T2 = (last G2) dW2^T, the term step 15 used to subtract from dX2, right behind the other pass over dW2: a wave
+    // meets the same 4d/8 rows of dW2 in both, and the second pass finds them in the L2.  From here to step 22 the
+    // tile holds -dX2.
+    E::template lds<0, NW, NBM, 2, true>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 13. dA2, d eta ; dG2 = -last (S2 + db2) ; d last
     if (tid < 256) {
@@ -562,13 +569,12 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       if (cg == 0) lds[L::dlast + t] = -q;
     }
     __syncthreads();
-    // ---- 14. dXbar2 += dA2 X2 ; dG2 -= M2^T dZbar2 ; dX2 = dA2^T Xbar2
+    // ---- 14. dXbar2 += dA2 X2 ; dG2 -= M2^T dZbar2 ; -dX2 = T2 - dA2^T Xbar2
     E::template lds<1, NW, NBM, 4>(mDXB, M, lds + L::DA, LK, 1, mX2, M, 1, 1, NTM, 16, wave, lane);
     E::template lds<2, NW, 1, 4>(lds + L::DG2, LD, lds + L::M2, 1, LK, lds + L::DZB2, LD, 1, 1, NTD, 16, wave, lane);
-    E::template lds<0, NW, NBM, 4>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
+    E::template lds<2, NW, NBM, 4>(mDX2, M, lds + L::DA, 1, LK, mXB2, M, 1, 1, NTM, 16, wave, lane);
     __syncthreads();
-    // ---- 15. dX2 -= (last G2) dW2^T ; dZbar1 = dXbar2 gelu'(Zbar1)
-    E::template lds<2, NW, NBM, 2, true>(mDX2, M, G2l, D, 1, dW2, 1, D, 1, NTM, D, wave, lane);
+    // ---- 15. dZbar1 = dXbar2 gelu'(Zbar1)
     {
       float z[NJM], v[NJM];
       ldm(mZB1, z);
@@ -586,6 +592,11 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     splitk_xyT(mDXB, mG1);
     prod_k(M0{}, lds + L::DQ, mDXB, W1, 1, M);
     E::template lds<0, NW, NBM>(mS1, M, lds + L::XK, LD, 1, dW1, M, 1, 1, NTM, D, wave, lane);
+    // T1 = (last G1) dW1^T, the term step 19 used to subtract from dK, right behind the other pass over dW1 (a wave
+    // meets the same 4d/8 columns in both).  The barrier separates the two split-k products' partial sums.  From here
+    // on the DK tile holds -dK.
+    __syncthreads();
+    prod_k(M0{}, lds + L::DK, G1l, dW1, 1, M);
     __syncthreads();
     // ---- 17. dA1, d eta ; dG1 = -last (S1 + db1) ; d last
     if (tid < 256) {
@@ -609,13 +620,12 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       if (cg == 0) lds[L::dlast + t] -= q;
     }
     __syncthreads();
-    // ---- 18. dG1 -= M1^T dZbar1 ; dQ += dA1 XK ; dK = dA1^T XQ
+    // ---- 18. dG1 -= M1^T dZbar1 ; dQ += dA1 XK ; -dK = T1 - dA1^T XQ
     E::template lds<2, NW, NBM, 4>(mS1, M, lds + L::M1, 1, LK, mDXB, M, 1, 1, NTM, 16, wave, lane);
     E::template lds<1, NW, 1, 4>(lds + L::DQ, LD, lds + L::DA, LK, 1, lds + L::XK, LD, 1, 1, NTD, 16, wave, lane);
-    E::template lds<0, NW, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NTD, 16, wave, lane, NTD % NW);
+    E::template lds<2, NW, 1, 4>(lds + L::DK, LD, lds + L::DA, 1, LK, lds + L::XQ, LD, 1, 1, NTD, 16, wave, lane, NTD % NW);
     __syncthreads();
-    // ---- 19. dK -= (last G1) dW1^T ; dU = dG1 gelu'(Z1) (kept in mU's place after saving U * gelu'')
-    prod_k(M2{}, lds + L::DK, G1l, dW1, 1, M);
+    // ---- 19. dU = dG1 gelu'(Z1) (kept in mU's place after saving U * gelu'')
     {
       float z[NJM], dg1[NJM], u[NJM];
       ldm(mZ1, z);
@@ -675,8 +685,8 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       }
     }
     __syncthreads();
-    // ---- 22. dX2 += dZ2 W2^T ; then dZ1 = dG1 U gelu''(Z1) + dX2 gelu'(Z1)
-    E::template lds<1, NW, NBM, 2, true>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    // ---- 22. dX2 += dZ2 W2^T (the tile holds -dX2) ; then dZ1 = dG1 U gelu''(Z1) + dX2 gelu'(Z1)
+    E::template lds<2, NW, NBM, 2, true>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     {
       float z[NJM], f1[NJM], dx[NJM];
@@ -687,17 +697,17 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       for (int j = 0; j < NJM; ++j) {
         float y, dy;
         gelu_tanh_pair(z[j], y, dy);
-        dx[j] = f1[j] + dx[j] * dy;  // dZ1
+        dx[j] = f1[j] - dx[j] * dy;  // dZ1 (dx holds -dX2)
       }
       stm(mDX2, dx);
     }
     __syncthreads();
-    // ---- 23. gradient accumulation; dK += dZ1 W1^T
+    // ---- 23. gradient accumulation; dK += dZ1 W1^T (as -dK -= ...)
     // dW2 += X2^T dZ2 + dU^T G2 + Xbar2^T dZbar2 as ONE rank-48 pass over dW2 (operands consecutive)
     E::template rank<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, wave, lane);
     // dW1 += XQ^T dZbar1 + XK^T dZ1 as one rank-32 pass
     E::template rank<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, wave, lane);
-    prod_k(M1{}, lds + L::DK, mDX2, W1, 1, M);
+    prod_k(M2{}, lds + L::DK, mDX2, W1, 1, M);  // the tile holds -dK
     if (tid < M) sdb1[tid] += col16_sum2(mDXB + tid, mDX2 + tid, M);
     if (tid < D) {
       float s = 0.f;
@@ -715,7 +725,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
         const int o = cg + GW * j;
         const float dT = lds[L::DT + t * LD + o];
         IO::store1(pq + o, lds[L::DQ + t * LD + o] + lds[L::DO + t * LD + o]);
-        IO::store1(pk + o, lds[L::DK + t * LD + o] - dT);
+        IO::store1(pk + o, -lds[L::DK + t * LD + o] - dT);
         IO::store1(pv + o, dT);
       }
     }
