@@ -42,10 +42,11 @@ def test_cpp_host_class_compiles_links_and_reports_errors(tmp_path):
           ttt::FusedMlp mlp(cfg, dummy, dummy, dummy, dummy, dummy, dummy);
           if (std::strcmp(mlp.name(), "FusedTTTMLP")) return 7;
           // per (batch, head): 2 d M + M + d + N 16 (M + d) + 9 * 16 M floats, M = 4 d; up to 128 units (two
-          // workgroups per unit) a second state buffer, six more tiles, two exchange blocks and 32 counter words
+          // workgroups per unit) a second state buffer, six more tiles, two exchange blocks, bf16 copies of both state
+          // buffers and 32 counter words
           const long long xb = 48LL * 96 + 4 * 256 + 16 + 96;
           const long long per_unit = 2LL * 96 * 384 + 384 + 96 + 2LL * 16 * (384 + 96) + 9LL * 16 * 384
-                                     + 2LL * 96 * 384 + 6LL * 16 * 384 + 2 * xb + 32;
+                                     + 2LL * 96 * 384 + 6LL * 16 * 384 + 2 * xb + 2LL * 96 * 384 + 32;
           if (mlp.backward_workspace_bytes(2, 32, TTT_BF16) != 4 * 2 * 2 * per_unit) return 8;
           ttt::TTTMLPState ms;
           ms.w1 = ms.b1 = ms.w2 = ms.b2 = ms.next_w1 = ms.next_b1 = ms.next_w2 = ms.next_b2 = dummy;

@@ -420,7 +420,8 @@ int launch_mlp_bwd_as(const ttt::MlpBwdArgs& a, hipStream_t s) {
 }
 template <class T, int D, bool BF = false>
 int launch_mlp_bwd(const ttt::MlpBwdArgs& a, hipStream_t s) {
-  static_assert(ttt::MlpBwdPipe<D>::FLOATS > 0, "");
+  static_assert(ttt::MlpBwdPipe<D>::FLOATS == 4 * D * 4 * D + ttt::kMlpBwdSharedTiles * 16 * 4 * D + 2 * ((48 * D + 4 * 256 + 16 + D + 3) / 4 * 4),
+                "MlpBwdWs computes the same size");
   if (a.pipe != nullptr) return launch_mlp_bwd_as<T, D, BF, true>(a, s);
   return launch_mlp_bwd_as<T, D, BF, false>(a, s);
 }
@@ -529,7 +530,7 @@ struct MlpBwdWs {
     if (mlp_bwd_pipe(d)) {
       // the same arithmetic as ttt::MlpBwdPipe<D>::FLOATS
       const size_t xb = (48 * D + 4 * 256 + 16 + D + 3) / 4 * 4;
-      const size_t per_unit = 2 * D * M + ttt::kMlpBwdSharedTiles * 16 * M + 2 * xb;
+      const size_t per_unit = 2 * D * M + ttt::kMlpBwdSharedTiles * 16 * M + 2 * xb + 2 * D * M;
       flags = pipe + U * per_unit;
       total = flags + U * ttt::kMlpBwdPipeFlagWords;
     }

@@ -37,6 +37,20 @@ __device__ __forceinline__ f32x4 rows_to_operand(const f32x4& v, int lane) {
   return o;
 }
 
+// The same for a matrix kept as bf16 (a second copy of a state matrix, written for the operand reads): 16 rows x 32
+// bytes, lane l loads row l / 4, 8-byte chunk l % 4, and the exchange delivers a ready bf16 operand fragment.
+__device__ __forceinline__ u32x2 load_rows_raw_h(const uint16_t* block, int row_stride, int lane) {
+  return *reinterpret_cast<const u32x2*>(block + (lane >> 2) * row_stride + 4 * (lane & 3));
+}
+__device__ __forceinline__ u32x2 rows_to_operand(const u32x2& v, int lane) {
+  const int src = 4 * (4 * (lane & 15) + (lane >> 4));
+  const uint32_t x0 = v[0], x1 = v[1];
+  return u32x2{(uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)x0), (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)x1)};
+}
+// operand fragment of a 16-deep step from what was loaded: f32 values are rounded, bf16 bits are taken as they are
+__device__ __forceinline__ Io<BF16>::frag bf_frag(const f32x4& v) { return Io<BF16>::to_frag(v); }
+__device__ __forceinline__ Io<BF16>::frag bf_frag(const u32x2& v) { return __builtin_bit_cast(Io<BF16>::frag, v); }
+
 // One 16-deep step of a product: lane (c, g) holds four k slots of A (row c) and of B (column c).  BF: the operands
 // are rounded to bf16 and take one v_mfma_f32_16x16x16_bf16 (a quarter of the issue slots of the f32 form at an
 // eighth of the matrix-pipe time); otherwise four true-f32 v_mfma_f32_16x16x4_f32.  The accumulator is f32 either way.
@@ -60,11 +74,15 @@ __device__ __forceinline__ void mma16(f32x4& acc, const f32x4& a, const f32x4& b
 // BG: B is in global memory and contiguous along k (a transposed weight matrix): loaded four lanes to a row and
 // exchanged between lanes before use (load_rows_raw / rows_to_operand).
 // BF: bf16 operands (mma16); the k-steps outside the contiguous-A path are then taken four at a time.
-template <bool BF, int MODE, int NW, int NB, int KU0, bool BG>
+// BH (with BF and BG, A contiguous along k): B points at a bf16 copy of the matrix (uint16_t elements, same strides),
+// whose bits are the operands; half the bytes per pass, no conversion.
+template <bool BF, int MODE, int NW, int NB, int KU0, bool BG, bool BH = false>
 __device__ __forceinline__ void mm_lds_t(float* C, int ldc, const float* A, int a_rs, int a_cs,
                                          const float* B, int b_rs, int b_cs, int Mt, int Nt, int Kd,
                                          int wave, int lane, int first, int k0) {
   constexpr int KU = BF ? ((KU0 + 3) / 4) * 4 : KU0;
+  static_assert(!BH || (BF && BG), "a bf16 copy is read as a k-contiguous global operand of a bf16 product");
+  using bop = std::conditional_t<BH, u32x2, f32x4>;
   const int c = lane & 15, g = lane >> 4;
   const int nblk = (Nt + NB - 1) / NB;
   const int njobs = Mt * nblk;
@@ -139,24 +157,30 @@ __device__ __forceinline__ void mm_lds_t(float* C, int ldc, const float* A, int 
         // a tile column past the edge re-reads column tn0 and is zeroed afterwards (no load under a branch)
         const bool live = Nt % NB == 0 || tn0 + j < Nt;
         const float* pb = B + bo + kk * b_rs + (live ? j : 0) * bcol;
-        f32x4 v;
-        if (BG) {
-          v = load_rows_raw(B + (k0 + kk) * b_rs + 16 * (tn0 + (live ? j : 0)) * b_cs, b_cs, lane);
-        } else if (vecB) {
-          v = *reinterpret_cast<const f32x4*>(pb);
+        bop v;
+        if constexpr (BH) {
+          v = load_rows_raw_h(reinterpret_cast<const uint16_t*>(B) + (k0 + kk) * b_rs + 16 * (tn0 + (live ? j : 0)) * b_cs,
+                              b_cs, lane);
+          if (!live) v = u32x2{0u, 0u};
         } else {
+          if (BG) {
+            v = load_rows_raw(B + (k0 + kk) * b_rs + 16 * (tn0 + (live ? j : 0)) * b_cs, b_cs, lane);
+          } else if (vecB) {
+            v = *reinterpret_cast<const f32x4*>(pb);
+          } else {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = pb[r * b_rs];
+            for (int r = 0; r < 4; ++r) v[r] = pb[r * b_rs];
+          }
+          if (!live) v = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        if (!live) v = f32x4{0.f, 0.f, 0.f, 0.f};
         return v;
       };
-      auto step = [&](const f32x4& av, const f32x4 (&bv)[NB]) {
+      auto step = [&](const f32x4& av, const bop (&bv)[NB]) {
         if constexpr (BF) {
           const auto af = Io<BF16>::to_frag(av);
 #pragma unroll
-          for (int j = 0; j < NB; ++j) Io<BF16>::mma(acc[j], af, Io<BF16>::to_frag(bv[j]));
-        } else {
+          for (int j = 0; j < NB; ++j) Io<BF16>::mma(acc[j], af, bf_frag(bv[j]));
+        } else if constexpr (!BH) {
 #pragma unroll
           for (int r = 0; r < 4; ++r)
 #pragma unroll
@@ -169,7 +193,8 @@ __device__ __forceinline__ void mm_lds_t(float* C, int ldc, const float* A, int 
       // conditional; the scheduling barriers keep the refills where they are written.
       auto run = [&](auto pf_tag) {
         constexpr int PF = decltype(pf_tag)::value;
-        f32x4 av[PF], bv[PF][NB];
+        f32x4 av[PF];
+        bop bv[PF][NB];
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
           av[u] = loadA(16 * u);
@@ -325,7 +350,7 @@ template <bool BF, int MODE, int NW, int NB, int KS, int FZ>
 __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                           int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
                                           const float* X, int x_rs, float* Z, int ldz, const float* Csrc = nullptr,
-                                          const float* X2 = nullptr, float* Z2 = nullptr) {
+                                          const float* X2 = nullptr, float* Z2 = nullptr, uint16_t* Cb = nullptr) {
   static_assert(MODE == 1 || MODE == 2, "read-modify-write modes only");
   // Csrc: where the tiles of C are read from when the updated matrix goes to another buffer (same layout); the
   // ordering argument below only gets easier, since no load ever meets a store
@@ -399,6 +424,17 @@ __device__ __forceinline__ void mm_rank_t(float* C, int ldc, const float* A, int
     for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) C[coff + r * ldc + 16 * j] = s.acc[j][r];
+    // Cb: a bf16 copy of the updated matrix (same layout), rounded as an operand load of the f32 matrix would be
+    if (Cb != nullptr) {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const u32x2 h = __builtin_bit_cast(u32x2, Io<BF16>::to_frag(s.acc[j]));
+        Cb[coff + 16 * j] = (uint16_t)(h[0] & 0xffffu);
+        Cb[coff + ldc + 16 * j] = (uint16_t)(h[0] >> 16);
+        Cb[coff + 2 * ldc + 16 * j] = (uint16_t)(h[1] & 0xffffu);
+        Cb[coff + 3 * ldc + 16 * j] = (uint16_t)(h[1] >> 16);
+      }
+    }
     if (FZ) {
       const f32x4 xv = *reinterpret_cast<const f32x4*>(X + c * x_rs + 16 * tm + 4 * g);
       if constexpr (BF) {
@@ -502,24 +538,39 @@ __device__ __forceinline__ void mm_rank(float* C, int ldc, const float* A, int a
 // element of A is fetched once instead of NT times, all NW waves work, and every operand of a wave is requested
 // before its first matrix instruction.  Contains a barrier: call from all threads; the caller's next barrier
 // publishes C.
-template <bool BF, int MODE, int NW, int NT, int KSTEPS>
+// BH (with BF): B points at a bf16 copy of the matrix (uint16_t elements, same strides).
+template <bool BF, int MODE, int NW, int NT, int KSTEPS, bool BH = false>
 __device__ __forceinline__ void mm_splitk_t(float* C, int ldc, float* part, const float* A, int a_rs, const float* B,
                                             int b_rs, int b_cs, int wave, int lane, int tid) {
+  static_assert(!BH || BF, "a bf16 copy feeds a bf16 product");
+  using bop = std::conditional_t<BH, u32x2, f32x4>;
   const int c = lane & 15, g = lane >> 4;
   const int kw = wave * 16 * KSTEPS, k0 = kw + 4 * g;
   const bool vecB = b_rs == 1 && (b_cs & 3) == 0;
-  f32x4 av[KSTEPS], bv[KSTEPS][NT];
+  f32x4 av[KSTEPS];
+  bop bv[KSTEPS][NT];
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) {
     av[s] = load_rows_raw(A + kw + 16 * s, a_rs, lane);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      const float* pb = B + (k0 + 16 * s) * b_rs + (16 * j + c) * b_cs;
-      if (vecB) {
-        bv[s][j] = load_rows_raw(B + (kw + 16 * s) * b_rs + 16 * j * b_cs, b_cs, lane);
+      if constexpr (BH) {
+        const uint16_t* Bh = reinterpret_cast<const uint16_t*>(B);
+        if (vecB) {
+          bv[s][j] = load_rows_raw_h(Bh + (kw + 16 * s) * b_rs + 16 * j * b_cs, b_cs, lane);
+        } else {
+          const uint16_t* pb = Bh + (k0 + 16 * s) * b_rs + (16 * j + c) * b_cs;
+          const uint32_t h0 = pb[0], h1 = pb[b_rs], h2 = pb[2 * b_rs], h3 = pb[3 * b_rs];
+          bv[s][j] = u32x2{h0 | (h1 << 16), h2 | (h3 << 16)};
+        }
       } else {
+        const float* pb = B + (k0 + 16 * s) * b_rs + (16 * j + c) * b_cs;
+        if (vecB) {
+          bv[s][j] = load_rows_raw(B + (kw + 16 * s) * b_rs + 16 * j * b_cs, b_cs, lane);
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) bv[s][j][r] = pb[r * b_rs];
+          for (int r = 0; r < 4; ++r) bv[s][j][r] = pb[r * b_rs];
+        }
       }
     }
   }
@@ -541,9 +592,9 @@ __device__ __forceinline__ void mm_splitk_t(float* C, int ldc, float* part, cons
     for (int s = 0; s < KSTEPS; ++s) {
       const auto af = Io<BF16>::to_frag(av[s]);
 #pragma unroll
-      for (int j = 0; j < NT; ++j) Io<BF16>::mma(acc[j], af, Io<BF16>::to_frag(bv[s][j]));
+      for (int j = 0; j < NT; ++j) Io<BF16>::mma(acc[j], af, bf_frag(bv[s][j]));
     }
-  } else {
+  } else if constexpr (!BH) {
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s)
 #pragma unroll
@@ -577,25 +628,25 @@ __device__ __forceinline__ void mm_splitk(float* C, int ldc, float* part, const 
 // bf16 (one v_mfma_f32_16x16x16_bf16 per 16-deep step), otherwise true f32.  Accumulation is f32 in both.
 template <bool BF>
 struct Eng {
-  template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false>
+  template <int MODE, int NW = 4, int NB = 1, int KU = (NB >= 3 ? 2 : NB == 2 ? 4 : 8), bool BG = false, bool BH = false>
   static __device__ __forceinline__ void lds(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                              int b_rs, int b_cs, int Mt, int Nt, int Kd, int wave, int lane,
                                              int first = 0, int k0 = 0) {
-    mm_lds_t<BF, MODE, NW, NB, KU, BG>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, Kd, wave, lane, first, k0);
+    mm_lds_t<BF, MODE, NW, NB, KU, BG, BH>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, Kd, wave, lane, first, k0);
   }
   template <int MODE, int NW, int NB, int KS, int FZ = 0>
   static __device__ __forceinline__ void rank(float* C, int ldc, const float* A, int a_rs, int a_cs, const float* B,
                                               int b_rs, int b_cs, int Mt, int Nt, int wave, int lane,
                                               const float* X = nullptr, int x_rs = 0, float* Z = nullptr, int ldz = 0,
                                               const float* Csrc = nullptr, const float* X2 = nullptr,
-                                              float* Z2 = nullptr) {
+                                              float* Z2 = nullptr, uint16_t* Cb = nullptr) {
     mm_rank_t<BF, MODE, NW, NB, KS, FZ>(C, ldc, A, a_rs, a_cs, B, b_rs, b_cs, Mt, Nt, wave, lane, X, x_rs, Z, ldz, Csrc, X2,
-                                        Z2);
+                                        Z2, Cb);
   }
-  template <int MODE, int NW, int NT, int KSTEPS>
+  template <int MODE, int NW, int NT, int KSTEPS, bool BH = false>
   static __device__ __forceinline__ void splitk(float* C, int ldc, float* part, const float* A, int a_rs,
                                                 const float* B, int b_rs, int b_cs, int wave, int lane, int tid) {
-    mm_splitk_t<BF, MODE, NW, NT, KSTEPS>(C, ldc, part, A, a_rs, B, b_rs, b_cs, wave, lane, tid);
+    mm_splitk_t<BF, MODE, NW, NT, KSTEPS, BH>(C, ldc, part, A, a_rs, B, b_rs, b_cs, wave, lane, tid);
   }
 };
 

@@ -76,8 +76,10 @@ struct MlpBwdPipe {
   // exchange block
   static constexpr int XH = 0, G2 = XH + 16 * D, XH2 = G2 + 16 * D, A1 = XH2 + 16 * D, M1 = A1 + 256, M2 = M1 + 256,
                        A2P = M2 + 256, RSTD = A2P + 256, B2 = RSTD + 16, XB = (B2 + D + 3) / 4 * 4;
+  // SHB: bf16 copies of the two state buffers (W1 then W2, D * M uint16_t each, for the buffer that held the final
+  // state on entry and then for the second one), read as operands where the products take bf16 operands
   static constexpr int W1X = 0, W2X = W1X + D * M, TILES = W2X + M * D, XBLK = TILES + kMlpBwdSharedTiles * 16 * M,
-                       FLOATS = XBLK + 2 * XB;
+                       SHB = XBLK + 2 * XB, FLOATS = SHB + 2 * D * M;
 };
 
 template <int D>
@@ -136,6 +138,10 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
   constexpr int NBM = NTM / NW;  // [16 x 4d] products: one job of NBM tile columns per wave
   constexpr int NBD = NTD % 3 == 0 ? 3 : 2;
   constexpr float inv_d = 1.0f / D;
+  // Two workgroups with bf16 operands: the producer also writes every rolled-back state matrix as bf16, and the eight
+  // products that read W1 or W2 as an operand read that copy (half the bytes through the fabric; the same operand
+  // bits, since the copy is rounded as the operand load would round).
+  constexpr bool SHD = PIPE && BF;
   constexpr int RIDE = D <= 96 ? 2 : 1;  // products riding along on the W1 roll-back (head_dim 128 is at the register limit)
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // The thread indices are re-derived from an opaque copy at the top of every mini-batch (below): the
@@ -296,6 +302,15 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     else
       E::template lds<MODE, NW>(C, LD, A, M, 1, B, b_rs, b_cs, 1, NTD, M, wave, lane);
   };
+  // the same with W1 or W2 as B: from the bf16 copy where there is one
+  auto prod_w = [&](auto mode, float* C, const float* A, const float* B, int b_rs, int b_cs) {
+    constexpr int MODE = decltype(mode)::value;
+    if constexpr (L::SPLITK)
+      E::template splitk<MODE, NW, NTD, M / (16 * NW), SHD>(C, LD, lds + L::SKP, A, M, B, b_rs, b_cs, wave, lane, tid);
+    else
+      E::template lds<MODE, NW>(C, LD, A, M, 1, B, b_rs, b_cs, 1, NTD, M, wave, lane);
+  };
+  static_assert(!SHD || L::SPLITK, "bf16 operands exist up to head_dim 96");
   using M0 = std::integral_constant<int, 0>;
   using M1 = std::integral_constant<int, 1>;
   using M2 = std::integral_constant<int, 2>;
@@ -321,6 +336,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     // rank-48 / rank-32 accumulation into dW2 / dW1
     float* sh = mt;
     float* xb = nullptr;
+    uint16_t *W1b = nullptr, *W2b = nullptr;
     if constexpr (PIPE) {
       const bool home = ((st ^ N) & 1) == 0;
       W1 = home ? W1h : px + PX::W1X;
@@ -329,7 +345,14 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
       W2r = home ? px + PX::W2X : W2h;
       if (st & 1) sh = px + PX::TILES;
       xb = px + PX::XBLK + (st & 1) * PX::XB;
+      if constexpr (SHD) {
+        W1b = reinterpret_cast<uint16_t*>(px + PX::SHB + (home ? 0 : D * M));
+        W2b = W1b + D * M;
+      }
     }
+    // the state matrices as the products read them
+    const float* W1o = SHD ? reinterpret_cast<const float*>(W1b) : W1;
+    const float* W2o = SHD ? reinterpret_cast<const float*>(W2b) : W2;
     float *mZ1 = sh, *mX2 = sh + 16 * M, *mU = sh + 2 * 16 * M, *mXB2 = sh + 3 * 16 * M, *mG1 = sh + 4 * 16 * M,
           *mZB1 = sh + 5 * 16 * M, *mDXB = mt + 6 * 16 * M, *mDX2 = mt + 7 * 16 * M, *mS1 = mt + 8 * 16 * M;
     if constexpr (PIPE) {
@@ -385,7 +408,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     // ---- 2. roll W1, b1 back to the state entering this mini-batch
     // Z1 = XK W1 (step 3) rides along on the rolled-back tiles, and where the registers allow so does XQ W1 (step 7)
     E::template rank<1, NW, NBM, 4, RIDE>(W1, M, lds + L::XK, 1, LD, G1l, M, 1, NTD, NTM, wave, lane, lds + L::XK, LD, mZ1, M, W1r,
-                                          lds + L::XQ, mZB1);
+                                          lds + L::XQ, mZB1, W1b);
     if (tid < M) sb1[tid] += col16_sum(G1l + tid, M);
     __syncthreads();
     // ---- 3. Z1 = XK W1 + b1 ; X2 = gelu(Z1)
@@ -403,11 +426,12 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 4. roll W2, b2 back
-    E::template rank<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, wave, lane, nullptr, 0, nullptr, 0, W2r);
+    E::template rank<1, NW, NBD, 4>(W2, D, mX2, 1, M, G2l, D, 1, NTM, NTD, wave, lane, nullptr, 0, nullptr, 0, W2r, nullptr,
+                                    nullptr, W2b);
     if (tid < D) sb2[tid] += col16_sum(G2l + tid, D);
     __syncthreads();
     // ---- 5. Z2 = X2 W2 ; A1 = XQ XK^T ; eta
-    prod_k(M0{}, lds + L::XH, mX2, W2, D, 1);
+    prod_w(M0{}, lds + L::XH, mX2, W2o, D, 1);
     E::template lds<0, NW>(lds + L::A1, LK, lds + L::XQ, LD, 1, lds + L::XK, 1, LD, 1, 1, D, wave, lane, NTD % NW);
     if (tid < 256) {
       const int tt = tid >> 4, s = tid & 15;
@@ -440,7 +464,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 7. U = G2 W2^T ; Zbar1 = XQ W1
-    E::template lds<0, NW, NBM, 2, true>(mU, M, lds + L::G2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    E::template lds<0, NW, NBM, 2, true, SHD>(mU, M, lds + L::G2, LD, 1, W2o, 1, D, 1, NTM, D, wave, lane);
     if constexpr (RIDE != 2) E::template lds<0, NW, NBM>(mZB1, M, lds + L::XQ, LD, 1, W1, M, 1, 1, NTM, D, wave, lane);
     __syncthreads();
     // ---- 8. G1 = U gelu'(Z1)
@@ -475,7 +499,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 10. A2 = Xbar2 X2^T (split-k) ; Zbar2 = Xbar2 W2
     splitk_xyT(mXB2, mX2);
-    prod_k(M0{}, lds + L::XH2, mXB2, W2, D, 1);
+    prod_w(M0{}, lds + L::XH2, mXB2, W2o, D, 1);
     __syncthreads();
     if (tid < 256) {
       const int tt = tid >> 4, s = tid & 15;
@@ -538,7 +562,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 12. P2 = dZbar2 G2^T ; dXbar2 = dZbar2 W2^T ; S2 = X2 dW2
     E::template lds<0, NW>(lds + L::P, LK, lds + L::DZB2, LD, 1, lds + L::G2, 1, LD, 1, 1, D, wave, lane, NW - 1);
-    E::template lds<0, NW, NBM, 2, true>(mDXB, M, lds + L::DZB2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    E::template lds<0, NW, NBM, 2, true, SHD>(mDXB, M, lds + L::DZB2, LD, 1, W2o, 1, D, 1, NTM, D, wave, lane);
     prod_k(M0{}, lds + L::DG2, mX2, dW2, D, 1);
     // T2 = (last G2) dW2^T, the term step 15 used to subtract from dX2, right behind the other pass over dW2: a wave
     // meets the same 4d/8 rows of dW2 in both, and the second pass finds them in the L2.  From here to step 22 the
@@ -590,7 +614,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     // ---- 16. P1 = dZbar1 G1^T (split-k) ; dQ = dZbar1 W1^T ; S1 = XK dW1
     splitk_xyT(mDXB, mG1);
-    prod_k(M0{}, lds + L::DQ, mDXB, W1, 1, M);
+    prod_w(M0{}, lds + L::DQ, mDXB, W1o, 1, M);
     E::template lds<0, NW, NBM>(mS1, M, lds + L::XK, LD, 1, dW1, M, 1, 1, NTM, D, wave, lane);
     // T1 = (last G1) dW1^T, the term step 19 used to subtract from dK, right behind the other pass over dW1 (a wave
     // meets the same 4d/8 columns in both).  The barrier separates the two split-k products' partial sums.  From here
@@ -643,7 +667,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 20. dG2 += dU W2
-    prod_k(M1{}, lds + L::DG2, mU, W2, D, 1);
+    prod_w(M1{}, lds + L::DG2, mU, W2o, D, 1);
     __syncthreads();
     // ---- 21. second-order LayerNorm: dZ2, dT, d gamma, d beta
     {
@@ -686,7 +710,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     __syncthreads();
     // ---- 22. dX2 += dZ2 W2^T (the tile holds -dX2) ; then dZ1 = dG1 U gelu''(Z1) + dX2 gelu'(Z1)
-    E::template lds<2, NW, NBM, 2, true>(mDX2, M, lds + L::DZ2, LD, 1, W2, 1, D, 1, NTM, D, wave, lane);
+    E::template lds<2, NW, NBM, 2, true, SHD>(mDX2, M, lds + L::DZ2, LD, 1, W2o, 1, D, 1, NTM, D, wave, lane);
     __syncthreads();
     {
       float z[NJM], f1[NJM], dx[NJM];
@@ -707,7 +731,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
     E::template rank<1, NW, NBD, 12>(dW2, D, mX2, 1, M, lds + L::DZ2, LD, 1, NTM, NTD, wave, lane);
     // dW1 += XQ^T dZbar1 + XK^T dZ1 as one rank-32 pass
     E::template rank<1, NW, NBM, 8>(dW1, M, lds + L::XQ, 1, LD, mDXB, M, 1, NTD, NTM, wave, lane);
-    prod_k(M2{}, lds + L::DK, mDX2, W1, 1, M);  // the tile holds -dK
+    prod_w(M2{}, lds + L::DK, mDX2, W1o, 1, M);  // the tile holds -dK
     if (tid < M) sdb1[tid] += col16_sum2(mDXB + tid, mDX2 + tid, M);
     if (tid < D) {
       float s = 0.f;
