@@ -194,6 +194,13 @@ class LinearCalls:
                           lr=torch.empty_like(dv["lr"]), te=torch.empty(seq, **f32), gam=torch.empty((H, d), **f32),
                           bet=torch.empty((H, d), **f32))
         self.stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        # the backward takes a workspace where the library has a kernel that uses one (f32 I/O up to 128 units: two
+        # workgroups per unit); allocated once, outside the timed region
+        self.ws = None
+        if with_bwd:
+            nbytes = pkg.lib().ttt_linear_bwd_workspace_bytes(C.byref(self.desc))
+            if nbytes > 0:
+                self.ws = torch.empty((int(nbytes),), dtype=torch.uint8, device=dev)
 
     def _p(self, t):
         return None if t is None else self.C.c_void_p(t.data_ptr())
@@ -207,11 +214,11 @@ class LinearCalls:
 
     def bwd(self):
         d, p, g = self.dv, self._p, self.g
-        self.pkg._lib.check(self.pkg.lib().ttt_linear_bwd(
+        self.pkg._lib.check(self.pkg.lib().ttt_linear_bwd_ws(
             self.C.byref(self.desc), p(d["xq"]), p(d["xk"]), p(d["xv"]), p(d["W0"]), p(d["b0"]), p(d["token_eta"]),
             p(d["lr"]), p(d["gamma"]), p(d["beta"]), p(self.Wc), p(self.bc), p(d["d_out"]), None, None, p(g["xq"]),
             p(g["xk"]), p(g["xv"]), p(g["W"]), p(g["b"]), p(g["lr"]), p(g["te"]), p(g["gam"]), p(g["bet"]),
-            self.stream))
+            p(self.ws), self.stream))
 
 
 def measured_counters(workload):
@@ -474,7 +481,8 @@ def run_workload(name, a, pkg, torch):
         out["dtype"] = io
         out["config"].update(inner_model="TTT-Linear", checkpoint_interval=ci,
                              checkpoint_format=("f32 row-major", "packed", "update factors")[ckfmt])
-        kname = "ttt_linear_bwd_kernel" if lds else "ttt_linear_bwd_mw_kernel"
+        kname = ("ttt_linear_bwd_kernel" if lds else
+                 "ttt_linear_bwd_pair_kernel (two workgroups per unit)" if calls.ws is not None else "ttt_linear_bwd_mw_kernel")
         if io == "bf16" and not lds:
             alg = linear_bwd_bytes(B, H, seq, d, s)
             roof = {"bound": "hbm", "achieved": alg / bwd_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",

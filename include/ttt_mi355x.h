@@ -195,6 +195,33 @@ int ttt_linear_bwd(const ttt_desc* desc, const void* xq, const void* xk, const v
                    void* stream);
 
 /*
+ * ttt_linear_bwd with a caller-owned workspace: the same call (same interface of the reference replaced, same
+ * arguments, same results to rounding) for a caller that can hold ttt_linear_bwd_workspace_bytes(desc) bytes of
+ * device memory (16-byte aligned, ordinary hipMalloc memory, nothing in it has to be kept between calls).  The
+ * workspace argument itself has no counterpart in the reference.  Where that size is above zero -- f32 I/O,
+ * checkpoint_interval 1 (row-major or packed checkpoints), head_dim 32 or 64, at most 128 (batch, head) units, no
+ * TTT_HINT_ONE_WORKGROUP or wave hint -- and the device has two CUs per unit, the reverse scan of a unit runs on two
+ * workgroups on two CUs: one recomputes what depends only on the saved state (Z1, G, Zbar, dZbar, the attention
+ * block's gradients, d_xq), the other carries the state gradient (dZ1, d_xk, d_xv, d_lr, d_token_eta, dW, db); they
+ * hand their data over through a ring of three slots per unit in the workspace and follow each other through two
+ * counters there.  The f32 backward is bound by the matrix instructions of the CUs that hold a unit, and a batch of
+ * 8 x 12 heads leaves 160 of 256 CUs idle: BASELINE config 2 runs its backward in 0.45 instead of 0.72 ms.
+ * Both workgroups must be resident together, and what ttt_mlp_fwd says of a GPU shared with other work holds here: a
+ * workgroup that waits for its partner in vain (2^21 polls, seconds) gives up, both run to the end without waiting
+ * again, the unit's d_b0 is NaN in every element (its other gradients are then meaningless) and
+ * ttt_mlp_fwd_lost_workgroups counts the two workgroups.  With workspace == NULL, or where the size is zero, the call
+ * is ttt_linear_bwd.  ttt_linear_bwd_workspace_bytes returns a negative ttt_status for a desc without a backward.
+ */
+int64_t ttt_linear_bwd_workspace_bytes(const ttt_desc* desc);
+int ttt_linear_bwd_ws(const ttt_desc* desc, const void* xq, const void* xk, const void* xv,
+                      const float* W0, const float* b0, const float* token_eta, const void* lr,
+                      const float* gamma, const float* beta, const float* W_ckpt,
+                      const float* b_ckpt, const void* d_out, const float* d_W_out,
+                      const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
+                      float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
+                      void* workspace, void* stream);
+
+/*
  * TTT-MLP multi-stage forward (two-layer inner model d -> 4d -> d, tanh-GELU).  The reference
  * has no fused kernel for it; this is the fused counterpart of TTTMLP::forward
  * (rust/core/src/mlp.rs:127-208 looped as rust/core/src/inner.rs:25-50) behind the same

@@ -27,6 +27,27 @@ def flagged(lines):
     return list(isa_check.scan(["kern:"] + lines))
 
 
+def test_scanner_flags_a_scalar_select_on_a_vector_comparison():
+    """The second rule of the scan: s_cselect reads SCC; a comparison on the vector unit sets VCC.  The sequence the
+    compiler once produced for `lds_word != 0 ? a : b` (the word loaded from a wave-uniform LDS address) is reported,
+    the repaired form (v_readfirstlane + s_cmp) and the ordinary mask idiom (v_cmp, s_and_b64, s_cselect_b64) are not."""
+    wrong = ["kern:", "\ts_add_i32 s0, s23, 0", "\tv_mov_b32_e32 v0, s0", "\tds_read_b32 v0, v0", "\ts_waitcnt lgkmcnt(0)",
+             "\tv_cmp_eq_u32_e32 vcc, 0, v0", "\ts_cselect_b32 s0, s22, -1"]
+    bad = isa_check.scan_scc_select(wrong)
+    assert len(bad) == 1 and bad[0][0] == "kern" and bad[0][1] == 7
+    right = ["kern:", "\ts_add_i32 s0, s23, 0", "\tds_read_b32 v0, v0", "\ts_waitcnt lgkmcnt(0)", "\tv_readfirstlane_b32 s0, v0",
+             "\ts_cmp_eq_u32 s0, 0", "\tv_cmp_eq_u32_e32 vcc, 0, v0", "\ts_cselect_b32 s0, s22, -1"]
+    assert isa_check.scan_scc_select(right) == []
+    mask = ["kern:", "\ts_lshl_b32 s4, s5, 2", "\tv_cmp_gt_i32_e32 vcc, 4, v1", "\ts_and_b64 s[6:7], vcc, exec",
+            "\ts_cselect_b64 s[8:9], -1, 0"]
+    assert isa_check.scan_scc_select(mask) == []
+    # a label starts a new basic block: what set SCC in front of it is not known, nothing is reported
+    assert isa_check.scan_scc_select(["kern:", "\ts_add_i32 s0, s1, 4", ".LBB0_2:", "\tv_cmp_eq_u32_e32 vcc, 0, v0",
+                                      "\ts_cselect_b32 s0, s2, -1"]) == []
+    # the library's own self-test functions are skipped, as in the first rule
+    assert isa_check.scan_scc_select(["ttt_selftest_x:"] + wrong[1:]) == []
+
+
 def test_scanner_flags_a_close_mixed_pair_in_place():
     assert len(flagged([K32.format(c="0"), K16.format(d="v[0:3]", c="v[0:3]")])) == 1
     assert len(flagged([K16.format(d="v[0:3]", c="0"), K32.format(c="v[0:3]")])) == 1

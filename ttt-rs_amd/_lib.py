@@ -23,7 +23,7 @@ EXPORTS = (
     "ttt_version", "ttt_last_error", "ttt_linear_supported", "ttt_linear_bwd_supported",
     "ttt_linear_best_checkpoint_format",
     "ttt_linear_num_checkpoints",
-    "ttt_linear_fwd", "ttt_linear_bwd", "ttt_mlp_supported", "ttt_mlp_fwd",
+    "ttt_linear_fwd", "ttt_linear_bwd", "ttt_linear_bwd_workspace_bytes", "ttt_linear_bwd_ws", "ttt_mlp_supported", "ttt_mlp_fwd",
     "ttt_mlp_fwd_lost_workgroups", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_bwd", "ttt_mlp_bwd_static", "ttt_mlp_fwd_saving_supported", "ttt_mlp_fwd_saving", "ttt_mlp_bwd_saved", "ttt_stack_fwd_workspace_bytes", "ttt_stack_fwd", "ttt_inner_inputs", "ttt_layer_epilogue", "ttt_linear_fwd_fused_inputs_supported", "ttt_linear_fwd_fused_inputs", "ttt_linear_adam_supported", "ttt_linear_adam_fwd", "ttt_mlpn_supported", "ttt_mlpn_fwd", "ttt_selftest_mfma_mixed",
 )
 
@@ -74,6 +74,9 @@ def lib() -> C.CDLL:
         L.ttt_linear_num_checkpoints.restype = C.c_int64
         L.ttt_linear_fwd.argtypes = [dp] + [vp] * 15
         L.ttt_linear_bwd.argtypes = [dp] + [vp] * 24
+        L.ttt_linear_bwd_workspace_bytes.argtypes = [dp]
+        L.ttt_linear_bwd_workspace_bytes.restype = C.c_int64
+        L.ttt_linear_bwd_ws.argtypes = [dp] + [vp] * 25
         L.ttt_mlp_supported.argtypes = [dp]
         L.ttt_mlp_fwd.argtypes = [dp] + [vp] * 17
         L.ttt_mlp_bwd_workspace_bytes.argtypes = [dp]

@@ -54,6 +54,12 @@ def build_library(verbose: bool = False, extra_flags=()) -> str:
                 sys.stderr.write(f"{os.path.basename(path)}:{no}: in {func}: {ws} wait state(s) between\n    {a}\n    {b}\n")
             raise RuntimeError(f"{len(bad)} in-place accumulations onto a matrix instruction of another shape sit closer "
                                "than the hardware needs (see isa_check.py); library not installed")
+        sel = isa_check.check_scc_select_file(path)
+        if sel:
+            for func, no, a, b in sel[:20]:
+                sys.stderr.write(f"{os.path.basename(path)}:{no}: in {func}: scalar select on a vector comparison\n    {a}\n    {b}\n")
+            raise RuntimeError(f"{len(sel)} s_cselect instruction(s) read a condition code that the comparison in front "
+                               "of them does not set (see isa_check.py); library not installed")
     shutil.copyfile(out, LIB_PATH)
     shutil.copymode(out, LIB_PATH)
     shutil.rmtree(os.path.join(HERE, "build"), ignore_errors=True)

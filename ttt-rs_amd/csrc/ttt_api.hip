@@ -15,6 +15,7 @@
 #include "ttt_layer_io.hip.h"
 #include "ttt_linear_bwd.hip.h"
 #include "ttt_linear_bwd_mw.hip.h"
+#include "ttt_linear_bwd_pair.hip.h"
 #include "ttt_linear_bwd_rr.hip.h"
 #include "ttt_linear_fwd.hip.h"
 #include "ttt_linear_fwd_mw.hip.h"
@@ -405,6 +406,25 @@ int launch_linear_bwd_mw(const ttt::LinearBwdArgs& a, unsigned grid, hipStream_t
   if (rc != TTT_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), bytes, s, a);
   return hip_status(hipGetLastError(), "ttt_linear_bwd (multi-wave register-resident kernel) launch");
+}
+
+// f32 I/O, one checkpoint per mini-batch, two workgroups per (batch, head): workgroups b and b + 8 of every 16 share a unit
+template <int D, bool PK>
+int launch_linear_bwd_pair(const ttt::LinearBwdPairArgs& pa, hipStream_t s) {
+  constexpr size_t bytes = ttt::LinBwdPair<D, PK>::BYTES;
+  const unsigned units = (unsigned)(pa.a.B * pa.a.H), grid = (units + 7) / 8 * 16;
+  if (pa.a.K == 16) {
+    constexpr auto kern16 = ttt::ttt_linear_bwd_pair_kernel<D, PK, true>;
+    int rc = opt_in_lds<kern16>(bytes);
+    if (rc != TTT_OK) return rc;
+    hipLaunchKernelGGL(kern16, dim3(grid), dim3(64 * (D / 16 + 1)), bytes, s, pa);
+    return hip_status(hipGetLastError(), "ttt_linear_bwd_ws (two workgroups per unit) launch");
+  }
+  constexpr auto kern = ttt::ttt_linear_bwd_pair_kernel<D, PK, false>;
+  int rc = opt_in_lds<kern>(bytes);
+  if (rc != TTT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * (D / 16 + 1)), bytes, s, pa);
+  return hip_status(hipGetLastError(), "ttt_linear_bwd_ws (two workgroups per unit) launch");
 }
 
 template <class T, int D, bool BF, bool PIPE>
@@ -1011,17 +1031,55 @@ int ttt_linear_best_checkpoint_format(const ttt_desc* d) {
   return rc;  // no format has a backward kernel: the status ttt_linear_bwd would return for the f32 format
 }
 
-int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
-                   const float* W0, const float* b0, const float* token_eta, const void* lr,
-                   const float* gamma, const float* beta, const float* W_ckpt,
-                   const float* b_ckpt, const void* d_out, const float* d_W_out,
-                   const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
-                   float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
-                   void* stream) {
+}  // extern "C"
+
+namespace {
+// Whether a desc's TTT-Linear backward can spread every unit over two workgroups (producer and consumer,
+// ttt_linear_bwd_pair_kernel): f32 I/O, whose reverse scan is bound by the f32 matrix instructions of the SIMDs that
+// hold a unit, one checkpoint per mini-batch (row-major or packed), head_dim 32 or 64, at most 128 units.  A function
+// of the desc alone, because the size of the workspace follows from it; the launch checks the device's CU count on top.
+bool linear_bwd_pair_wanted(const ttt_desc* d) {
+  LinearBwdChoice ch;
+  if (choose_linear_bwd(d, &ch) != TTT_OK) return false;
+  if (ch.kind != LinearBwdChoice::REG || d->io_dtype != TTT_F32) return false;
+  if (d->head_dim != 32 && d->head_dim != 64) return false;
+  if ((d->kernel_hint & (TTT_HINT_ONE_WORKGROUP | TTT_HINT_WAVES_MASK)) != 0) return false;
+  if (d->seq / d->mini_batch < 2) return false;
+  return (int64_t)d->batch * d->heads <= 128;
+}
+struct LinBwdPairWs {
+  size_t hand, flags, total;
+};
+LinBwdPairWs linear_bwd_pair_ws(const ttt_desc* d) {
+  const size_t U = (size_t)d->batch * d->heads;
+  const size_t slot = d->head_dim == 64 ? ttt::LinBwdPair<64, true>::H_BYTES : ttt::LinBwdPair<32, true>::H_BYTES;
+  static_assert(ttt::LinBwdPair<64, true>::H_BYTES == ttt::LinBwdPair<64, false>::H_BYTES, "one slot size per head_dim");
+  LinBwdPairWs w;
+  w.hand = 0;
+  w.flags = U * ttt::kLinBwdPairSlots * slot;
+  w.total = w.flags + U * ttt::kLinBwdPairFlagWords * sizeof(unsigned);
+  return w;
+}
+
+int linear_bwd_impl(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                    const float* W0, const float* b0, const float* token_eta, const void* lr,
+                    const float* gamma, const float* beta, const float* W_ckpt,
+                    const float* b_ckpt, const void* d_out, const float* d_W_out,
+                    const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
+                    float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
+                    void* workspace, void* stream) {
   // the kernel is chosen (and a desc without one refused) before anything is enqueued
   LinearBwdChoice ch;
   int rc = choose_linear_bwd(d, &ch);
   if (rc != TTT_OK) return rc;
+  bool pair = workspace != nullptr && linear_bwd_pair_wanted(d);
+  if (pair) {
+    if (!aligned16(workspace)) return fail(TTT_ERR_SHAPE, "ttt_linear_bwd_ws: workspace must be 16-byte aligned");
+    int cus = 0;
+    rc = device_cus(&cus);
+    if (rc != TTT_OK) return rc;
+    pair = 2 * (int64_t)d->batch * d->heads <= cus;  // every workgroup a CU of its own, both sides resident together
+  }
   // W0/b0 are part of the saved state for interface parity; the state entering every stage is
   // rebuilt from the checkpoints (checkpoint 0 equals the initial state).
   (void)W0;
@@ -1063,6 +1121,19 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   const unsigned grid = (unsigned)(a.B * a.H);
   const bool f32 = d->io_dtype == TTT_F32;
   const int waves = ch.waves;
+  if (pair) {
+    const LinBwdPairWs w = linear_bwd_pair_ws(d);
+    ttt::LinearBwdPairArgs pa;
+    pa.a = a;
+    pa.hand = static_cast<unsigned char*>(workspace) + w.hand;
+    pa.flags = reinterpret_cast<unsigned*>(static_cast<unsigned char*>(workspace) + w.flags);
+    pa.spin_limit = (d->kernel_hint & TTT_HINT_TEST_LOST_PARTNER) ? 0u : (1u << 21);
+    pa.agent_release = (d->kernel_hint & TTT_HINT_TEST_OTHER_XCD) ? 1 : 0;
+    copy_or_zero(reinterpret_cast<float*>(pa.flags), nullptr, (size_t)grid * ttt::kLinBwdPairFlagWords, s);
+    if (a.ckpt_packed)
+      return D == 64 ? launch_linear_bwd_pair<64, true>(pa, s) : launch_linear_bwd_pair<32, true>(pa, s);
+    return D == 64 ? launch_linear_bwd_pair<64, false>(pa, s) : launch_linear_bwd_pair<32, false>(pa, s);
+  }
   if (ch.kind == LinearBwdChoice::LDS) {
     if (ch.w_global) return launch_linear_bwd<ttt::F32, 128, 1, true, true>(a, grid, s);
     // bf16 I/O: operands rounded to bf16 like the register-resident kernels, unless f32 products were asked for
@@ -1116,6 +1187,38 @@ int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void
   }
   if (D == 96) return launch_linear_bwd_mw<ttt::BF16, 96, 3>(a, grid, s);
   return launch_linear_bwd_mw<ttt::BF16, 128, 4>(a, grid, s);
+}
+}  // namespace
+
+extern "C" {
+
+int ttt_linear_bwd(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                   const float* W0, const float* b0, const float* token_eta, const void* lr,
+                   const float* gamma, const float* beta, const float* W_ckpt,
+                   const float* b_ckpt, const void* d_out, const float* d_W_out,
+                   const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
+                   float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
+                   void* stream) {
+  return linear_bwd_impl(d, xq, xk, xv, W0, b0, token_eta, lr, gamma, beta, W_ckpt, b_ckpt, d_out, d_W_out, d_b_out,
+                         d_xq, d_xk, d_xv, d_W0, d_b0, d_lr, d_token_eta, d_gamma, d_beta, nullptr, stream);
+}
+
+int64_t ttt_linear_bwd_workspace_bytes(const ttt_desc* d) {
+  LinearBwdChoice ch;
+  const int rc = choose_linear_bwd(d, &ch);
+  if (rc != TTT_OK) return rc;
+  return linear_bwd_pair_wanted(d) ? (int64_t)linear_bwd_pair_ws(d).total : 0;
+}
+
+int ttt_linear_bwd_ws(const ttt_desc* d, const void* xq, const void* xk, const void* xv,
+                      const float* W0, const float* b0, const float* token_eta, const void* lr,
+                      const float* gamma, const float* beta, const float* W_ckpt,
+                      const float* b_ckpt, const void* d_out, const float* d_W_out,
+                      const float* d_b_out, void* d_xq, void* d_xk, void* d_xv, float* d_W0,
+                      float* d_b0, void* d_lr, float* d_token_eta, float* d_gamma, float* d_beta,
+                      void* workspace, void* stream) {
+  return linear_bwd_impl(d, xq, xk, xv, W0, b0, token_eta, lr, gamma, beta, W_ckpt, b_ckpt, d_out, d_W_out, d_b_out,
+                         d_xq, d_xk, d_xv, d_W0, d_b0, d_lr, d_token_eta, d_gamma, d_beta, workspace, stream);
 }
 
 int ttt_mlp_supported(const ttt_desc* d) {

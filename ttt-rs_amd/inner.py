@@ -227,8 +227,10 @@ def ttt_linear_adam_forward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta,
 def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_weight, ln_bias,
                             weight_ckpt, bias_ckpt, grad_output, mini_batch: int, eps: float = 1e-6,
                             checkpoint_interval: int = 1, grad_weight_out=None, grad_bias_out=None, packed_checkpoints: bool = False,
-                            kernel_hint: int = 0):
-    """One call of ttt_linear_bwd on the current stream.
+                            kernel_hint: int = 0, workspace=None):
+    """One call of ttt_linear_bwd (or ttt_linear_bwd_ws, where the library has a kernel that uses a workspace: f32
+    I/O up to 128 units runs every unit on two workgroups) on the current stream.  workspace: a device tensor of
+    ttt_linear_bwd_workspace_bytes(desc) bytes, None to allocate one, False to call the entry point without.
 
     Counterpart of backward_multi (rust/fused/src/linear_fused_tile/backward/launch.rs:332-438).
     Returns a dict with the nine input gradients named as TttGradInputs
@@ -268,13 +270,24 @@ def ttt_linear_backward_raw(xq, xk, xv, weight, bias, token_eta, ttt_lr_eta, ln_
         grad_ln_bias=torch.empty((H, d), dtype=torch.float32, device=dev),
     )
     stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    with torch.cuda.device(dev):
-        check(lib().ttt_linear_bwd(
-            C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(weight), _ptr(bias), _ptr(te), _ptr(lr),
+    # a desc whose backward can use a workspace (two workgroups per unit) gets one: ttt_linear_bwd_ws
+    ws_bytes = lib().ttt_linear_bwd_workspace_bytes(C.byref(desc))
+    if ws_bytes < 0:
+        check(int(ws_bytes))
+    args = (C.byref(desc), _ptr(xq), _ptr(xk), _ptr(xv), _ptr(weight), _ptr(bias), _ptr(te), _ptr(lr),
             _ptr(ln_weight), _ptr(ln_bias), _ptr(w_ck), _ptr(b_ck), _ptr(go), _ptr(grad_weight_out),
             _ptr(grad_bias_out), _ptr(g["grad_xq"]), _ptr(g["grad_xk"]), _ptr(g["grad_xv"]),
             _ptr(g["grad_weight"]), _ptr(g["grad_bias"]), _ptr(g["grad_ttt_lr_eta"]),
-            _ptr(g["grad_token_eta"]), _ptr(g["grad_ln_weight"]), _ptr(g["grad_ln_bias"]), stream))
+            _ptr(g["grad_token_eta"]), _ptr(g["grad_ln_weight"]), _ptr(g["grad_ln_bias"]))
+    with torch.cuda.device(dev):
+        if ws_bytes > 0 and workspace is not False:
+            if workspace is None or workspace is True:
+                workspace = torch.empty((int(ws_bytes),), dtype=torch.uint8, device=dev)
+            if workspace.numel() * workspace.element_size() < ws_bytes:
+                raise _lib.TttError(_lib.TTT_ERR_SHAPE, f"workspace holds fewer than {ws_bytes} bytes")
+            check(lib().ttt_linear_bwd_ws(*args, _ptr(workspace), stream))
+        else:
+            check(lib().ttt_linear_bwd(*args, stream))
     return g
 
 

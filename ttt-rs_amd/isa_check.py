@@ -16,7 +16,10 @@ text order and, from every branch, on into the branch target while an earlier ma
 Functions whose name contains "selftest" are skipped: the library's own test of this fact places such pairs on
 purpose, in inline assembly.
 
-Usage: python isa_check.py file.s      (exit status 1 and a listing if a hazard is found)
+A second rule, described where it is implemented below (scan_scc_select), reports a scalar select that reads a
+condition code which the vector comparison in front of it does not set.
+
+Usage: python isa_check.py file.s      (exit status 1 and a listing if either rule finds something)
 """
 from __future__ import annotations
 
@@ -147,9 +150,71 @@ def check_file(path: str):
         return list(scan(fh))
 
 
+# ---- second rule: a scalar select on a vector comparison ---------------------------------------------------------
+# hipcc (ROCm 7.2) takes a value loaded from a wave-uniform LDS address for uniform.  Seen in this library's code: the
+# loaded word is compared on the vector unit (v_cmp ... vcc) and the result is then selected with s_cselect, which
+# reads the SCALAR condition code -- set by whatever scalar instruction came last (an address addition), not by that
+# comparison.  The kernel ran, and a status word read "given up" after a clean run.  Signature looked for, inside one
+# basic block: [scalar ARITHMETIC that writes SCC as a by-product: s_add, s_sub, a shift, s_and_saveexec ...] ...
+# v_cmp ... s_cselect, with nothing that writes SCC between the vector comparison and the select.  A scalar comparison
+# or a logical operation on a mask (s_cmp*, s_bitcmp*, s_and_b64 ... whose SCC is what a select is meant to read) in
+# that place is the ordinary, correct form and is not reported.  (The cure in source is to move the loaded word to a
+# scalar register by hand, __builtin_amdgcn_readfirstlane, before it is compared.)
+_SCC_ON_PURPOSE = ("s_cmp", "s_bitcmp", "s_and_b", "s_or_b", "s_xor_b", "s_andn2_b", "s_orn2_b", "s_not_b", "s_nand_b",
+                   "s_nor_b", "s_xnor_b")
+_NO_SCC = ("s_mov", "s_cmov", "s_load", "s_buffer_load", "s_waitcnt", "s_nop", "s_barrier", "s_branch", "s_cbranch",
+           "s_cselect", "s_getreg", "s_setreg", "s_mul_i32", "s_mul_hi", "s_bfm", "s_movk", "s_sext", "s_ff1", "s_ff0",
+           "s_flbit", "s_bitset", "s_getpc", "s_setpc", "s_swappc", "s_sleep", "s_sendmsg", "s_endpgm", "s_memtime",
+           "s_memrealtime", "s_dcache", "s_icache", "s_setprio", "s_sethalt", "s_trap", "s_setvskip", "s_set_gpr",
+           "s_brev", "s_bcnt0", "s_pack", "s_cmovk", "s_version", "s_code_end", "s_inst_prefetch", "s_clause",
+           "s_incperflevel", "s_decperflevel", "s_ttrace", "s_rfe", "s_wakeup")
+
+
+def scan_scc_select(lines):
+    """[(function, line number, vector comparison, select)] for every s_cselect whose nearest SCC-writing
+    predecessor in its basic block lies in front of a v_cmp that lies in front of the select."""
+    bad = []
+    func = "?"
+    scc_seen = False   # the last SCC writer of this block wrote SCC as a by-product of arithmetic
+    vcmp = None        # a vector comparison issued since that writer
+    for no, raw in enumerate(lines, 1):
+        line = raw.split(";")[0].strip()
+        m = _FUNC.match(line)
+        if m:
+            func = m.group(1)
+            scc_seen, vcmp = False, None
+            continue
+        if re.match(r"^\.L[\w.$]*:", line):  # a local label: a new basic block
+            scc_seen, vcmp = False, None
+            continue
+        if not line or line.startswith(".") or line.startswith("//"):
+            continue
+        op = line.split()[0]
+        if op.startswith("v_cmp"):
+            if scc_seen:
+                vcmp = (no, line)
+            continue
+        if op.startswith("s_cselect"):
+            if vcmp is not None and "selftest" not in func:
+                bad.append((func, no, vcmp[1], line))
+            continue
+        if op.startswith("s_") and not op.startswith(_NO_SCC):
+            scc_seen, vcmp = not op.startswith(_SCC_ON_PURPOSE), None
+    return bad
+
+
+def check_scc_select_file(path: str):
+    with open(path) as f:
+        return scan_scc_select(f.readlines())
+
+
 if __name__ == "__main__":
     bad = check_file(sys.argv[1])
     for func, no, a, b, ws in bad:
         print(f"{sys.argv[1]}:{no}: in {func}: {ws} wait state(s) between\n    {a}\n    {b}")
     print(f"{len(bad)} MFMA pair(s) of different shapes, the second accumulating from the first, closer than the first's passes + 1 wait states")
-    sys.exit(1 if bad else 0)
+    sel = check_scc_select_file(sys.argv[1])
+    for func, no, a, b in sel:
+        print(f"{sys.argv[1]}:{no}: in {func}: scalar select on a vector comparison\n    {a}\n    {b}")
+    print(f"{len(sel)} s_cselect instruction(s) behind a vector comparison with no scalar comparison between")
+    sys.exit(1 if bad or sel else 0)
