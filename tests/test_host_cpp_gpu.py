@@ -91,10 +91,13 @@ def test_cpp_linear_forward_backward_equals_python_mirror(P, drv, dtype, packed)
     rc = drv.ttt_host_linear_forward(*common, ptr(out), *[ptr(t) for t in st], ptr(Wc), ptr(bc), C.byref(cur), stream)
     assert rc == P.TTT_OK, drv.ttt_host_last_error()
     got = {k: torch.empty_like(v) for k, v in ref.items()}
+    # the class takes the same path as the mirror: a workspace where the library can use one (f32 I/O: two workgroups
+    # per unit), so the results can be held to each other bit for bit
+    ws = torch.empty((64 << 20,), dtype=torch.uint8, device="cuda:0")
     rc = drv.ttt_host_linear_backward(*common, ptr(Wc), ptr(bc), ptr(dO), ptr(got["grad_xq"]), ptr(got["grad_xk"]),
                                       ptr(got["grad_xv"]), ptr(got["grad_weight"]), ptr(got["grad_bias"]),
                                       ptr(got["grad_ttt_lr_eta"]), ptr(got["grad_token_eta"]), ptr(got["grad_ln_weight"]),
-                                      ptr(got["grad_ln_bias"]), stream)
+                                      ptr(got["grad_ln_bias"]), stream, ptr(ws), C.c_longlong(ws.numel()))
     torch.cuda.synchronize()
     assert rc == P.TTT_OK, drv.ttt_host_last_error()
     assert cur.value == 1  # one launch: the final state is in the second pair

@@ -1,25 +1,38 @@
 // TTT-Linear fused backward for gfx950 on TWO workgroups per (batch, head): f32 I/O, one checkpoint per mini-batch,
 // head_dim 32 / 64, one feature tile per wave (the feature-split scheme of ttt_linear_bwd_mw.hip.h).
 //
-// With f32 I/O the reverse scan is bound by the f32 matrix instructions of the four SIMDs that hold a unit, and a
-// batch of 8 x 12 heads leaves 160 of 256 CUs without work.  A mini-batch's work falls into two parts of about equal
-// matrix time (112 and 124 instructions per wave at head_dim 64):
+// With f32 I/O the reverse scan is bound by the f32 matrix instructions of the four SIMDs that hold a unit, and by the
+// chain of dependent steps of a mini-batch that one wave per SIMD cannot overlap; a batch of 8 x 12 heads leaves 160 of
+// 256 CUs without work.  A mini-batch's work falls into two parts of about equal matrix time (112 and 148
+// v_mfma_f32_16x16x4_f32 per wave at head_dim 64, packed checkpoints):
 //   producer  everything that needs only the saved state W_t and the inputs: Z1, its LayerNorm and G, the attention
 //             block, Zbar, the output-LayerNorm backward dZbar, P = dZbar G^T, dA, d eta, dXQ (final), dA^T XQ, M^T dZbar;
 //   consumer  everything that needs the state gradient carried from the later mini-batches: S = XK dW + db, G dW^T,
 //             the second-order LayerNorm backward dZ1, dXV, dXK, d lr, d token_eta, and the rank-32 update of dW, db.
 // Nothing of the consumer's flows back.  The producer workgroup runs ahead of the consumer; what crosses lies in a
 // ring of three slots per unit in global memory (the caller's workspace): the producer stores the consumer's operands
-// exactly as the consumer's lanes hold them (1 KiB per wave instruction), the consumer copies a slot global -> LDS
-// without passing registers, one mini-batch ahead, into one of two LDS buffers.  Two counters per unit say how far
-// each side has come: the producer raises its own when every store of a slot has been acknowledged, the consumer
-// waits for it, drops its CU's vector cache (device-scope acquire) and copies; the consumer raises its own when the
-// copies of a slot have landed, and the producer waits for slot t + 3 to have landed before it overwrites that slot.
+// exactly as the consumer's lanes hold them (1 KiB per wave instruction; 29 KiB per mini-batch at head_dim 64: dZbar^T
+// and G of every wave, xhat, gx, gO, M^T dZbar, dA^T XQ of the own features, eight scalars per token), the consumer
+// copies a slot global -> LDS without passing registers, one mini-batch ahead, into one of two LDS buffers, together
+// with what it takes from the inputs itself (the W tiles of the checkpoint, the rows of XK and XQ).
+//
+// Each workgroup has a CONTROL WAVE beside its NW compute waves.  It issues every global -> LDS copy, polls the
+// partner's counter and raises its own side's, and takes part in every barrier.  A copy costs the wave that issues it
+// about a hundred cycles of stalled issue (measured: the same copies dealt to the compute waves, between their matrix
+// instructions, made a mini-batch 1 000 - 1 600 cycles longer on either side), a poll is a round trip to the L2; with
+// the control wave neither sits in the instruction stream of a wave that feeds the matrix pipe.
+//
+// Two counters per unit say how far each side has come: the producer raises its own when every store of a slot has
+// been acknowledged (every compute wave waits for its stores in front of a barrier, the control wave raises behind it),
+// the consumer waits for it and copies -- with device-scope loads, which do not look in the CU's vector cache; the
+// consumer raises its own when the copies of a slot have landed, and the producer waits for slot t + 3 to have landed
+// before it overwrites that slot.
 // Workgroups b and b + 8 of every 16 share a unit: consecutive workgroup ids go to the XCDs in turn, so both run
-// behind one L2.  Each publishes its XCD number, and the producer publishes with a device-scope release (write-back
-// of its L2) until it has read the consumer's number and found it equal to its own.  Every wait is bounded; a side
-// that waits in vain marks its counter, both run to the end without waiting again, the consumer makes the unit's d_b0
-// NaN and the status word g_mlp_fwd_lost_workgroups counts both.
+// behind one L2.  Each publishes its XCD number; the producer publishes with a device-scope release (write-back
+// of its L2) until it has read the consumer's number and found it equal to its own, and the consumer puts a
+// device-scope acquire in front of its copies until it has found the producer's equal to its own.  Every wait is
+// bounded; a side that waits in vain marks its counter, both run to the end without waiting again, the consumer makes
+// the unit's d_b0 NaN and the status word g_mlp_fwd_lost_workgroups counts both.
 //
 // Arithmetic: that of ttt_linear_bwd_mw_kernel<F32, D, D/16, PK> term by term (reference
 // rust/fused/src/linear_fused_tile/backward/kernel.rs:253-429, backward/stage.rs:42-1006, layer_norm.rs:428-709).
@@ -34,6 +47,20 @@ __device__ __forceinline__ void lds_dma16_dev(const void* base, unsigned lane_of
   unsigned saved;
   asm volatile(
       "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 sc1\n\ts_nop 0\n\ts_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(lane_off), "s"(uniform_ptr(base)), "s"(lds_base)
+      : "memory");
+}
+
+// lds_dma16 with a non-temporal load: for rows that nothing reads again (the producer's xv and d_out, everything the
+// consumer takes from the inputs, which the producer has read before it).  Lines brought in this way do not push the
+// hand-over slots out of the L2, where they are meant to stay between their store and their one read: 170 MB per
+// step less between L2 and memory at 8 x 12 units of 2048 tokens.  (Non-temporal on every input copy lost as much as
+// it won: the consumer's read of the checkpoint then missed the L2.)
+__device__ __forceinline__ void lds_dma16_nt(const void* base, unsigned lane_off, unsigned lds_base) {
+  unsigned saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt\n\ts_nop 0\n\ts_mov_b32 m0, %0"
       : "=&s"(saved)
       : "v"(lane_off), "s"(uniform_ptr(base)), "s"(lds_base)
       : "memory");
@@ -54,22 +81,27 @@ constexpr unsigned kLinBwdPairPoison = 0xffffffffu;
 template <int D, bool PK>
 struct LinBwdPair {
   static constexpr int NT = D / 16, NW = NT;
-  // ---- a hand-over slot (bytes); every piece is a 1 KiB row: 16 bytes per lane of the wave that holds it
-  static constexpr int H_WN = 0;                          // NT*NT rows: row w*NT+J = W_t tile (own rows w, columns J), tokens along k
-  static constexpr int H_FRK = H_WN + NT * NT * 1024;     // 4 kinds x NT: XK^T, XQ^T, dZbar^T fragments, G fragments
-  static constexpr int H_OWN = H_FRK + 4 * NT * 1024;     // 5 kinds x NT: xhat, gx, gO, M^T dZbar, dA^T XQ of wave w's features
+  // ---- a hand-over slot (bytes); every piece is a 1 KiB row: 16 bytes per lane of the wave that holds it.  What the
+  // consumer can take from the inputs itself (the state W_t from the checkpoint, XK^T and XQ^T) is not handed over: a
+  // slot is written once and read once through the L2, and what does not fit there is written back to memory.
+  static constexpr int H_FRK = 0;                         // 2 kinds x NT: dZbar^T fragments, G fragments
+  static constexpr int H_OWN = H_FRK + 2 * NT * 1024;     // 5 kinds x NT: xhat, gx, gO, M^T dZbar, dA^T XQ of wave w's features
   static constexpr int H_SC = H_OWN + 5 * NT * 1024;      // 16 kinds x 16 tokens of f32 (8 used)
   static constexpr int H_BYTES = H_SC + 1024;
   static constexpr int H_ROWS = H_BYTES / 1024;
-  enum { KD = 0, QD, ZD, GF };
+  enum { ZD = 0, GF };
   enum { XH = 0, GX, GO, DGM, DKP };
   enum { S_RSTD = 0, S_AXH, S_AXH2, S_GX, S_GXXH, S_LR, S_E1, S_E2 };
-  // ---- consumer LDS: two buffers of (slot image, XK rows), then its own exchange areas
+  // ---- consumer LDS: two buffers of (slot image, XK rows, XQ rows, the W tiles of the checkpoint), then its own
+  // exchange areas
   static constexpr int C_XK = H_BYTES;                    // NT rows
-  static constexpr int C_BUF = C_XK + NT * 1024;
+  static constexpr int C_XQ = C_XK + NT * 1024;           // NT rows
+  static constexpr int C_W = C_XQ + NT * 1024;            // NT*NT rows, as the producer stages them
+  static constexpr int C_BUF = C_W + NT * NT * 1024;
   static constexpr int C_SUM = 2 * C_BUF;                 // [8 sums][16 tokens][NW]
-  static constexpr int C_FR = C_SUM + 8 * 16 * NW * 4;    // dZ1 fragments in both forms: 2 kinds x NT rows
-  static constexpr int C_CTL = C_FR + 2 * NT * 1024;      // control words
+  static constexpr int C_FR = C_SUM + 8 * 16 * NW * 4;    // 4 kinds x NT rows: dZ1 fragments in both forms, XK^T, XQ^T
+  static constexpr int C_M0 = C_FR + 4 * NT * 1024;       // D row means of the initial W, then mean(b)
+  static constexpr int C_CTL = C_M0 + (D + 4) * 4;        // control words
   static constexpr int C_BYTES = C_CTL + 16;
   // ---- producer LDS: the staging of ttt_linear_bwd_mw_kernel in two buffers used alternately, its exchange areas
   static constexpr int P_W = 0;
@@ -88,7 +120,7 @@ struct LinBwdPair {
   static constexpr int BYTES_RAW = C_BYTES > P_BYTES ? C_BYTES : P_BYTES;
   static constexpr int BYTES = BYTES_RAW > 81 * 1024 ? BYTES_RAW : 81 * 1024;
   static_assert(BYTES <= 160 * 1024, "exceeds the 160 KiB of LDS of a gfx950 CU");
-  static_assert(P_M0 % 16 == 0 && C_FR % 16 == 0, "16-byte aligned areas");
+  static_assert(P_M0 % 16 == 0 && C_FR % 16 == 0 && C_M0 % 16 == 0, "16-byte aligned areas");
 };
 
 template <int D, bool PK, bool FULL>
@@ -207,6 +239,31 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
     *reinterpret_cast<f32x4*>(static_cast<float*>(base) + tokoff + fo) = x;
   };
 
+  // the scan works on the centred state, as the one-workgroup kernel does: row means of the initial W (a packed
+  // checkpoint holds the centred matrix already) and the mean of the initial bias
+  float* const M0p = reinterpret_cast<float*>(smem + (role == 0 ? L::P_M0 : L::C_M0));
+  {
+    const size_t c0 = bh * (size_t)a.n_ckpt;
+    if (!PK) {
+      for (int i = threadIdx.x; i < D; i += 64 * (NW + 1)) {
+        const f32x4* row = reinterpret_cast<const f32x4*>(a.W_ckpt + c0 * D * D + (size_t)i * D);
+        float sum = 0.f;
+        for (int j = 0; j < D / 4; ++j) {
+          const f32x4 v = row[j];
+          sum += (v[0] + v[1]) + (v[2] + v[3]);
+        }
+        M0p[i] = sum * inv_d;
+      }
+    }
+    if (threadIdx.x == 0) {
+      float sum = 0.f;
+      for (int f = 0; f < D; ++f) sum += a.b_ckpt[c0 * D + f];
+      M0p[D] = sum * inv_d;
+    }
+    __syncthreads();
+  }
+  const float mrowo = PK ? 0.f : M0p[feat(w, c)];  // mean of row feat(w, c): the wave's own row tile
+
   if (role == 0) {
     // =============================================================================================== producer
     float* const SUMp = reinterpret_cast<float*>(smem + L::P_SUM);
@@ -224,32 +281,9 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
 #pragma unroll
     for (int r = 0; r < 4; ++r) te_s[r] = (4 * g + r < K) ? a.token_eta[4 * g + r] : 0.f;
 
-    // the scan works on the centred state, as the one-workgroup kernel does
-    float* const M0p = reinterpret_cast<float*>(smem + L::P_M0);
-    {
-      const size_t c0 = bh * (size_t)a.n_ckpt;
-      if (!PK) {
-        for (int i = threadIdx.x; i < D; i += 64 * (NW + 1)) {
-          const f32x4* row = reinterpret_cast<const f32x4*>(a.W_ckpt + c0 * D * D + (size_t)i * D);
-          float sum = 0.f;
-          for (int j = 0; j < D / 4; ++j) {
-            const f32x4 v = row[j];
-            sum += (v[0] + v[1]) + (v[2] + v[3]);
-          }
-          M0p[i] = sum * inv_d;
-        }
-      }
-      if (threadIdx.x == 0) {
-        float sum = 0.f;
-        for (int f = 0; f < D; ++f) sum += a.b_ckpt[c0 * D + f];
-        M0p[D] = sum * inv_d;
-      }
-      __syncthreads();
-    }
     float mrow[NT];
 #pragma unroll
     for (int I = 0; I < NT; ++I) mrow[I] = PK ? 0.f : M0p[feat(I, c)];
-    const float mrowo = PK ? 0.f : M0p[feat(w, c)];
     const float bbar = M0p[D];
 
     // copies of one mini-batch into staging buffer (stage & 1): the control wave's
@@ -273,8 +307,8 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
         if (FULL || c < K) {
           lds_dma16(static_cast<const float*>(a.xq) + tok0, ((unsigned)(c * D) + foJ) * 4u, dst + L::P_X + (0 * NT + J) * 1024);
           lds_dma16(static_cast<const float*>(a.xk) + tok0, ((unsigned)(c * D) + foJ) * 4u, dst + L::P_X + (1 * NT + J) * 1024);
-          lds_dma16(static_cast<const float*>(a.xv) + tok0, ((unsigned)(c * D) + foJ) * 4u, dst + L::P_X + (2 * NT + J) * 1024);
-          lds_dma16(static_cast<const float*>(a.d_out) + tok0, ((unsigned)(c * D) + foJ) * 4u, dst + L::P_X + (3 * NT + J) * 1024);
+          lds_dma16_nt(static_cast<const float*>(a.xv) + tok0, ((unsigned)(c * D) + foJ) * 4u, dst + L::P_X + (2 * NT + J) * 1024);
+          lds_dma16_nt(static_cast<const float*>(a.d_out) + tok0, ((unsigned)(c * D) + foJ) * 4u, dst + L::P_X + (3 * NT + J) * 1024);
         }
       }
       if (lane < 16) {
@@ -309,9 +343,9 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
 
     // The counted wait of the compute waves.  Memory operations of a wave retire in the order they were issued, stores
     // included, so "s_waitcnt vmcnt(n)" with n = the number of operations a wave is KNOWN to have issued behind the
-    // ones it waits for leaves those younger operations in flight.  In front of X1 every compute wave has stored, in
-    // this mini-batch, its NT state tiles and XK^T, XQ^T: NT + 2 stores behind the last store of the mini-batch before.
-    constexpr int kStoresBeforeX1 = NT + 2;
+    // ones it waits for leaves those younger operations in flight.  In front of X1 a compute wave stores nothing of
+    // this mini-batch (the first store, xhat, follows the exchange), so everything it has in flight is waited for.
+    constexpr int kStoresBeforeX1 = 0;
     auto open_slot = [&](int) { lds_barrier(); };
     // in front of the X1 barrier of mini-batch st: every store of the slot of mini-batch st + 1 has been acknowledged
     // (the stores of this mini-batch so far may stay in flight), or, while the partner is not known to share the L2,
@@ -355,11 +389,8 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
           Wn[J] = tokens_k(*reinterpret_cast<const frag*>(sl + L::P_W + (w * NT + J) * 1024));
         else
           Wn[J] = *reinterpret_cast<const f32x4*>(sl + L::P_W + (w * NT + J) * 1024) - mrowo;
-        put(L::H_WN + (w * NT + J) * 1024, Wn[J]);
       }
       const frag kdo = tokens_k(ko), qdo = tokens_k(qo);
-      put(L::H_FRK + (L::KD * NT + w) * 1024, kdo);
-      put(L::H_FRK + (L::QD * NT + w) * 1024, qdo);
 
       // ---- forward intermediates of the own features: Z1 = XK W + b, Zq = XQ W + b; partial attention blocks
       f32x4 z1 = bT, zb = bT;
@@ -549,19 +580,34 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
   // slot is read with device-scope loads: the producer's stores were acknowledged by the L2 both sit behind.
   // In three portions, one per stretch between the barriers of a mini-batch and sized like the stretches: the compute
   // waves must not find the control wave still issuing copies when they reach a barrier.
-  constexpr int kRowsA = L::H_ROWS * 3 / 8, kRowsB = L::H_ROWS / 2;
+  constexpr int kRowsA = L::H_ROWS / 4, kRowsB = L::H_ROWS / 2;
   auto copy_in = [&](int stage, int part) {
     const unsigned char* hs = hand + (size_t)(stage % R) * L::H_BYTES;
     const unsigned dst = stg + (unsigned)(stage & 1) * L::C_BUF;
     const int n0 = part == 0 ? 0 : part == 1 ? kRowsA : kRowsB, n1 = part == 0 ? kRowsA : part == 1 ? kRowsB : L::H_ROWS;
 #pragma unroll 4
     for (int n = n0; n < n1; ++n) lds_dma16_dev(hs, (unsigned)(n * 1024 + lane * 16), dst + n * 1024);
+    if (part == 0) {
+      // the W tiles of the checkpoint, as the producer stages them
+      const float* Wg = a.W_ckpt + (bh * (size_t)a.n_ckpt + stage) * D * D;
+#pragma unroll 4
+      for (int n = 0; n < NT * NT; ++n) {
+        const int I = n / NT, J = n - I * NT;
+        if (PK)
+          lds_dma16_nt(Wg, (unsigned)(n * 1024 + lane * 16), dst + L::C_W + n * 1024);
+        else
+          lds_dma16_nt(Wg, (unsigned)(feat(I, c) * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, dst + L::C_W + n * 1024);
+      }
+    }
     if (part == 2) {
-      const float* src = static_cast<const float*>(a.xk) + (bh * (size_t)a.seq_stride + (size_t)stage * K) * D;
+      const size_t tok0 = (bh * (size_t)a.seq_stride + (size_t)stage * K) * D;
       if (FULL || c < K) {
 #pragma unroll
-        for (int J = 0; J < NT; ++J)
-          lds_dma16(src, (unsigned)(c * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u, dst + L::C_XK + J * 1024);
+        for (int J = 0; J < NT; ++J) {
+          const unsigned off = (unsigned)(c * D + 32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u;
+          lds_dma16_nt(static_cast<const float*>(a.xk) + tok0, off, dst + L::C_XK + J * 1024);
+          lds_dma16_nt(static_cast<const float*>(a.xq) + tok0, off, dst + L::C_XQ + J * 1024);
+        }
       }
     }
   };
@@ -612,6 +658,12 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
     const float rstd1 = sc[L::S_RSTD * 16], sa_xh = sc[L::S_AXH * 16], sa_xh2 = sc[L::S_AXH2 * 16];
     const float s_gx = sc[L::S_GX * 16], s_gxxh = sc[L::S_GXXH * 16], lr_c = sc[L::S_LR * 16];
     const float mgx = s_gx * inv_d, sgx = s_gxxh * inv_d;
+    // ---- XK^T, XQ^T of the own features (tokens along k) for the state gradient: published for the other waves, read
+    // behind the X4 barrier
+    const frag kdo = tokens_k(*reinterpret_cast<const frag*>(sl + L::C_XK + w * 1024));
+    const frag qdo = tokens_k(*reinterpret_cast<const frag*>(sl + L::C_XQ + w * 1024));
+    fr2(2, w) = kdo;
+    fr2(3, w) = qdo;
     // ---- S = XK dW + db, TMP = G dW^T (own features)
     f32x4 S = dbT, TMP = zero4;
     {
@@ -674,7 +726,10 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
 #pragma unroll
       for (int J = 0; J < NT; ++J) {
         Z1fa[J] = fr2(0, J);
-        Wn[J] = *reinterpret_cast<const frag*>(sl + L::H_WN + (w * NT + J) * 1024);
+        if constexpr (PK)  // stored as (m = j, k = i): transposed on the matrix pipe
+          Wn[J] = tokens_k(*reinterpret_cast<const frag*>(sl + L::C_W + (w * NT + J) * 1024));
+        else
+          Wn[J] = *reinterpret_cast<const f32x4*>(sl + L::C_W + (w * NT + J) * 1024) - mrowo;
       }
       mma_all(dK, Wn, Z1fa);
       if (tok_ok) store_own(a.d_xk, tokoff, dK);
@@ -692,10 +747,10 @@ __global__ void __launch_bounds__(64 * (D / 16 + 1)) ttt_linear_bwd_pair_kernel(
     }
     // ---- state gradient: dW += XQ^T dZb + XK^T dZ1 (column slice and transposed row slice), db
     {
-      const frag Zd = frk(L::ZD, w), qdo = frk(L::QD, w), kdo = frk(L::KD, w);
+      const frag Zd = frk(L::ZD, w);
 #pragma unroll
       for (int I = 0; I < NT; ++I) {
-        const frag qa = frk(L::QD, I), ka = frk(L::KD, I), za = frk(L::ZD, I), z1a = fr2(1, I);
+        const frag qa = fr2(3, I), ka = fr2(2, I), za = frk(L::ZD, I), z1a = fr2(1, I);
         IO::mma2(dWc[I], qa, ka, Zd, Z1d);
         IO::mma2(DT[I], za, z1a, qdo, kdo);
       }

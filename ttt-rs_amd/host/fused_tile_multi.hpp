@@ -169,16 +169,26 @@ class FusedTileMulti {
   /// backward_multi (backward/launch.rs:332-438): consumes the saved inputs, the checkpoints
   /// written by forward and grad_output [B,H,seq,d]; upstream gradients of the final state are
   /// optional (null = zero, as the reference assumes, launch.rs:188-194).
+  /// `workspace`: null, or backward_workspace_bytes() bytes of device memory (16-byte aligned): where that size is
+  /// above zero the backward then runs every (batch, head) unit on two workgroups (ttt_linear_bwd_ws).
   void backward(const TTTInputsInner& in, const float* weight0, const float* bias0,
                 bool state_per_batch, const Checkpoints& ck, const void* grad_output,
                 const float* grad_weight_out, const float* grad_bias_out, const TTTLinearGrads& g,
-                void* stream) const {
+                void* stream, void* workspace = nullptr) const {
     ttt_desc d = desc(in.batch, in.seq_len, config_.ttt.mini_batch_size, in.dtype, state_per_batch);
-    check(ttt_linear_bwd(&d, in.qkv.xq, in.qkv.xk, in.qkv.xv, weight0, bias0, in.token_eta,
-                         in.ttt_lr_eta, ln_weight_, ln_bias_, ck.weight, ck.bias, grad_output,
-                         grad_weight_out, grad_bias_out, g.grad_xq, g.grad_xk, g.grad_xv,
-                         g.grad_weight, g.grad_bias, g.grad_ttt_lr_eta, g.grad_token_eta,
-                         g.grad_ln_weight, g.grad_ln_bias, stream));
+    check(ttt_linear_bwd_ws(&d, in.qkv.xq, in.qkv.xk, in.qkv.xv, weight0, bias0, in.token_eta,
+                            in.ttt_lr_eta, ln_weight_, ln_bias_, ck.weight, ck.bias, grad_output,
+                            grad_weight_out, grad_bias_out, g.grad_xq, g.grad_xk, g.grad_xv,
+                            g.grad_weight, g.grad_bias, g.grad_ttt_lr_eta, g.grad_token_eta,
+                            g.grad_ln_weight, g.grad_ln_bias, workspace, stream));
+  }
+
+  /// Bytes of device workspace backward() can use for this batch and sequence length (0: it needs none).
+  std::int64_t backward_workspace_bytes(int batch, int seq, ttt_dtype dtype, bool state_per_batch) const {
+    ttt_desc d = desc(batch, seq, config_.ttt.mini_batch_size, dtype, state_per_batch);
+    const std::int64_t n = ttt_linear_bwd_workspace_bytes(&d);
+    if (n < 0) check((int)n);
+    return n;
   }
 
  private:

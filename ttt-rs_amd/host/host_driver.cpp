@@ -59,7 +59,8 @@ int ttt_host_linear_backward(int B, int H, int d, int K, int seq, int dtype, flo
                              const float* beta, const void* xq, const void* xk, const void* xv,
                              const float* token_eta, const void* lr, const float* ck_w, const float* ck_b,
                              const void* d_out, void* d_xq, void* d_xk, void* d_xv, float* d_W, float* d_b,
-                             void* d_lr, float* d_te, float* d_gamma, float* d_beta, void* stream) {
+                             void* d_lr, float* d_te, float* d_gamma, float* d_beta, void* stream,
+                             void* workspace, long long workspace_bytes) {
   try {
     ttt::ModelConfig cfg;
     cfg.num_heads = H;
@@ -69,6 +70,10 @@ int ttt_host_linear_backward(int B, int H, int d, int K, int seq, int dtype, flo
     cfg.ttt.checkpoint_interval = ckpt_interval;
     cfg.ttt.checkpoint_format = ckpt_format;
     ttt::FusedTileMulti model(cfg, W0, b0, gamma, beta);
+    // the caller's workspace is used when it is large enough for what the class asks for
+    if (workspace != nullptr &&
+        model.backward_workspace_bytes(B, seq, static_cast<ttt_dtype>(dtype), false) > workspace_bytes)
+      throw ttt::Error(TTT_ERR_SHAPE, "workspace smaller than FusedTileMulti::backward_workspace_bytes");
     ttt::TTTInputsInner in;
     in.qkv = ttt::Qkv{xq, xk, xv};
     in.token_eta = token_eta;
@@ -80,7 +85,7 @@ int ttt_host_linear_backward(int B, int H, int d, int K, int seq, int dtype, flo
     g.grad_xq = d_xq; g.grad_xk = d_xk; g.grad_xv = d_xv; g.grad_weight = d_W; g.grad_bias = d_b;
     g.grad_ttt_lr_eta = d_lr; g.grad_token_eta = d_te; g.grad_ln_weight = d_gamma; g.grad_ln_bias = d_beta;
     model.backward(in, W0, b0, false, ttt::Checkpoints{const_cast<float*>(ck_w), const_cast<float*>(ck_b)}, d_out,
-                   nullptr, nullptr, g, stream);
+                   nullptr, nullptr, g, stream, workspace);
     return TTT_OK;
   } catch (const ttt::Error& e) {
     return report(e);
