@@ -221,6 +221,12 @@ class LinearCalls:
             p(self.ws), self.stream))
 
 
+def fwd_kernel_name(io, units):
+    """The TTT-Linear forward kernel the library picks at head_dim 64 and mini_batch 16: with f32 I/O and a CU per
+    (batch, head) unit the variant with a control wave that copies the operands global -> LDS."""
+    return "ttt_linear_fwd_dma_kernel" if io == "f32" and units <= 256 else "ttt_linear_fwd_sk_kernel"
+
+
 def measured_counters(workload):
     """HBM bytes per launch and matrix-pipe utilisation of a workload's dominant kernel, as measured with rocprofv3
     counters and kept in profiles/traffic.json (not quantities of this run: counters cannot be read from inside it)."""
@@ -439,7 +445,7 @@ def run_workload(name, a, pkg, torch):
         out["config"]["inner_model"] = "TTT-Linear"
         out["roofline"] = {"bound": "hbm", "achieved": alg / k_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": alg / k_s / 1e9 / HBM_PEAK_GBS, **counters,
-                           "kernel": "ttt_linear_fwd_sk_kernel", "kernel_avg_us": k_s * 1e6,
+                           "kernel": fwd_kernel_name(io, B * H), "kernel_avg_us": k_s * 1e6,
                            "kernel_avg_source": "HIP events around the timed region / steps (launches back to back)",
                            "single_call_event_us": part_s["ttt_linear_fwd"] * 1e6,
                            "step_avg_us": dev_s * 1e6, "algorithmic_bytes": alg}
@@ -494,7 +500,7 @@ def run_workload(name, a, pkg, torch):
                     "algorithmic_bytes": linear_bwd_bytes(B, H, seq, d, s)}
         out["roofline"] = {**roof, **counters, "kernel": kname, "kernel_avg_us": bwd_s * 1e6,
                            "step_avg_us": dev_s * 1e6, "checkpoint_bytes_each_way": ck_bytes,
-                           "other_kernels": [{"kernel": "ttt_linear_fwd_sk_kernel (writes checkpoints)",
+                           "other_kernels": [{"kernel": fwd_kernel_name(io, B * H) + " (writes checkpoints)",
                                               "kernel_avg_us": fwd_s * 1e6,
                                               "algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s)}],
                            "step_algorithmic_bytes": linear_fwd_bytes(B, H, seq, d, s) + linear_bwd_bytes(B, H, seq, d, s),

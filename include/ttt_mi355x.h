@@ -102,7 +102,11 @@ typedef struct ttt_desc {
 /* ttt_linear_fwd, bf16 I/O at head_dim 64 with two waves per unit: TTT_HINT_OWN_LOADS = every wave loads only the
  * features it owns of xq, xk, xv and the full rows reach the waves through LDS (half the vector loads; the library's
  * choice above 256 units, where two workgroups share a CU); TTT_HINT_ALL_LOADS = every wave loads every row (the
- * library's choice up to 256 units).  Same results bit for bit.  Ignored where only one of the two exists. */
+ * library's choice up to 256 units).  Same results bit for bit.  Ignored where only one of the two exists.
+ * ttt_linear_fwd, f32 I/O with one wave per feature tile (head_dim 32 / 64), whole mini-batches of 16 tokens and at
+ * most one (batch, head) unit per CU: the library's choice is a kernel with a fifth wave that copies the operands
+ * global -> LDS, so that the four compute waves issue no loads; TTT_HINT_ALL_LOADS keeps the loads in the compute
+ * waves.  Same results bit for bit. */
 #define TTT_HINT_OWN_LOADS 0x1000
 #define TTT_HINT_ALL_LOADS 0x2000
 /* ttt_mlp_bwd / ttt_mlp_bwd_static, bf16 I/O up to head_dim 96: the reverse scan normally rounds the operands of its

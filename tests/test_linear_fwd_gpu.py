@@ -168,3 +168,32 @@ def test_sequence_windows_in_place(P, d):
     assert o1.data_ptr() == win(out_full).data_ptr()
     assert torch.equal(o1, o2) and torch.equal(W1, W2) and torch.equal(b1, b2)
     assert torch.isnan(out_full[:, :, :lo]).all() and torch.isnan(out_full[:, :, hi:]).all()
+
+
+@pytest.mark.parametrize("fmt", [0, 1], ids=["rowmajor", "packed"])
+@pytest.mark.parametrize("B,H,d,N", [(1, 4, 64, 16), (3, 2, 64, 5), (2, 3, 32, 3), (1, 1, 64, 1), (2, 2, 32, 2), (1, 2, 64, 9)])
+def test_f32_forward_with_control_wave_equals_forward_with_own_loads(P, B, H, d, N, fmt):
+    """f32 I/O, whole mini-batches of 16 tokens, a CU per workgroup: the library's choice is the kernel with a control
+    wave that copies the operands global -> LDS (the compute waves issue no loads); TTT_HINT_ALL_LOADS keeps the loads in
+    the compute waves.  Same arithmetic in the same order: the same bits, output, final state and checkpoints; and the
+    oracle holds the library's choice at the f32 bar."""
+    print(f"case f32 fwd control wave B{B} H{H} d{d} N{N} fmt{fmt}", flush=True)
+    K = 16
+    c = P.synthetic.reference_test_inputs(61 + B + H + d + N, B, H, N * K, d, K)
+    dv = to_dev(c)
+
+    def run(hint):
+        r = P.ttt_linear_forward_raw(dv["xq"], dv["xk"], dv["xv"], dv["W0"], dv["b0"], dv["token_eta"], dv["lr"],
+                                     dv["gamma"], dv["beta"], K, 1e-6, 1, want_checkpoints=True,
+                                     packed_checkpoints=fmt, kernel_hint=hint)
+        torch.cuda.synchronize()
+        return r
+
+    ctl, own, again = run(0), run(P.TTT_HINT_ALL_LOADS), run(0)
+    for name, x, y, z in zip(("out", "W", "b", "W_ckpt", "b_ckpt"), ctl, own, again):
+        assert torch.equal(x, y), f"{name}: control wave against own loads"
+        assert torch.equal(x, z), f"{name}: second call"
+    ro, rW, rb = oracle_case(c, K)
+    assert_close(ctl[0], ro, TOL[torch.float32], "out")
+    assert_close(ctl[1], rW, TOL[torch.float32], "W")
+    assert_close(ctl[2], rb, TOL[torch.float32], "b")

@@ -107,11 +107,23 @@ bool any_input_sums(const ttt::LinearFwdArgs* probs, unsigned ny) {
 // bound until there are more units than SIMDs.  Few units: split each unit over several waves
 // (skewed workgroup kernel).  Many units: one wave per unit (no exchange at all).
 // desc.kernel_hint (low byte) = 1 | 2 | 4 overrides the number of waves per unit (tuning / tests).
+int device_cus(int* cus);
+
+// ctl_wave: f32 I/O, one feature tile per wave, whole mini-batches, a CU per workgroup: the variant with a control
+// wave that copies the operands global -> LDS, so that the compute waves issue no loads (same bits; config-2 forward
+// 246 -> 216 us, with packed checkpoints 278 -> 250 us)
 template <class T, int D, int NW>
-int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s, bool own_loads = false) {
+int launch_linear_fwd_nw(const ttt::LinearFwdArgs* probs, unsigned ny, hipStream_t s, bool own_loads = false,
+                         bool ctl_wave = false) {
   const ttt::LinearFwdArgs& a = probs[0];
   const bool sums = any_input_sums(probs, ny);
   const auto P = pack_of(probs, ny);
+  if constexpr (sizeof(typename ttt::Io<T>::elem) == 4 && NW == D / 16 && NW > 1) {
+    if (ctl_wave && a.K == 16 && !sums) {
+      hipLaunchKernelGGL((ttt::ttt_linear_fwd_dma_kernel<T, D, NW, 2>), dim3((unsigned)(a.B * a.H), ny), dim3(64 * (NW + 1)), 0, s, P);
+      return hip_status(hipGetLastError(), "ttt_linear_fwd launch");
+    }
+  }
   // mini-batches prefetched ahead, in registers (f32 fragments are twice as large: the one-wave f32 kernel, which
   // holds the whole state and all rows in one wave, has registers for one mini-batch ahead only)
   constexpr int PF = (NW == 1 && sizeof(typename ttt::Io<T>::elem) == 4) ? 1 : 2;
@@ -200,12 +212,18 @@ int launch_linear_fwd(const ttt::LinearFwdArgs* probs, int hint, unsigned ny, hi
   if constexpr (!f32 && D == 64) {
     if (any_input_sums(probs, ny)) nw = 2;  // the kernel that forms x + projections is the two-wave one
   }
+  // f32 I/O with a CU per workgroup: the control-wave variant (TTT_HINT_ALL_LOADS keeps the loads in the compute waves)
+  bool ctl_wave = false;
+  if constexpr (f32) {
+    int cus = 0;
+    if ((hint & TTT_HINT_ALL_LOADS) == 0 && device_cus(&cus) == TTT_OK) ctl_wave = units <= cus;
+  }
   if constexpr (max_nw >= 4) {
-    if (nw >= 4) return launch_linear_fwd_nw<T, D, 4>(probs, ny, s);
+    if (nw >= 4) return launch_linear_fwd_nw<T, D, 4>(probs, ny, s, false, ctl_wave);
   }
   // a launch that puts two workgroups on a CU, or a caller that asks for it
   const bool own_loads = units > 256 ? (hint & TTT_HINT_ALL_LOADS) == 0 : (hint & TTT_HINT_OWN_LOADS) != 0;
-  if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(probs, ny, s, own_loads);
+  if (nw >= 2) return launch_linear_fwd_nw<T, D, 2>(probs, ny, s, own_loads, ctl_wave && max_nw == 2);
   return launch_linear_fwd_nw<T, D, 1>(probs, ny, s);
 }
 

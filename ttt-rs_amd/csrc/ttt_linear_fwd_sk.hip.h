@@ -36,6 +36,14 @@ namespace ttt {
 // input is the output of the layer below plus its own projections); x may be the memory `out` is written to: a wave
 // reads a row's own features three mini-batches before it writes that row's own features, and no other wave
 // touches them.
+// RAW = 5: the operands are given, and a CONTROL WAVE beside the NW compute waves brings them in: it copies the rows of
+// xq, xk, xv and lr of a mini-batch global -> LDS without passing registers (one 1 KiB row per feature tile and
+// tensor, 16 bytes per lane: exactly the fragment that lane holds of the tile), four mini-batches ahead into a ring of
+// four slots, and takes part in every barrier.  The compute waves issue no global load at all: behind the barrier of a
+// mini-batch they read the next one's fragments from LDS.  (A load costs the wave that issues it up to a hundred
+// cycles of stalled issue, nine of them per wave and mini-batch with f32 I/O.)  For f32 I/O with one feature tile per
+// wave, where a unit has a CU to itself (the control wave shares a SIMD with a compute wave: the kernel must stay
+// within 256 registers) and whole mini-batches of 16 tokens.
 // ADAM: the state update W -= XK^T (eta_last G) is replaced by one Adam step on that gradient per mini-batch
 // (reference rust/core/src/linear_adam.rs:76-128): the gradient tile is formed by the same matrix instructions into a
 // zero accumulator, the moments live in registers beside the state (three times the state's registers), bias
@@ -61,7 +69,11 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   __shared__ f32x4 kdx[SHARE ? 2 : 1][SHARE ? NT : 1][64];
   __shared__ f32x4 atx[SHARE ? 2 : 1][SHARE ? NW : 1][64];
 
+  constexpr bool DMA = RAW == 5;
   const int lane = threadIdx.x & 63, w = (threadIdx.x >> 6) % NW;
+  // RAW = 5: the wave behind the compute waves is the control wave; up to the point where it branches off it does what
+  // wave 0 does (w == 0: valid loads, LDS writes of the same values) and it stores nothing
+  const bool ctlw = DMA && __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) == NW;
   const int c = lane & 15, g = lane >> 4;
   const size_t bh = blockIdx.x;
   const int h = (int)(bh % a.H);
@@ -268,7 +280,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   f32x2 cs_fix[TPW], sn_fix[TPW];  // RAW = 1: cosines and sines of the lane's token position and own feature pairs
   u32x4* xrot = nullptr;           // rotated rows in LDS: [2 buffers][xq, xk][feature pair][lane]
   float lr_bias_h = 0.f;
-  if constexpr (RAW != 0) {
+  if constexpr (RAW != 0 && !DMA) {
     static_assert(BF && PF == 2, "rows shared through LDS: bf16 I/O");
     static_assert(!FORM || NT <= 4, "operands formed from the projections: head_dim <= 64");
     __shared__ u32x4 xrot_s[2][2][NT / 2][64];
@@ -298,7 +310,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   const size_t bidx = bh / a.H;
   const unsigned raw_row = (unsigned)a.H * (unsigned)(D * sizeof(elem));  // bytes from one token to the next
   auto load_raw = [&](RawIn& r, int stage) {
-    if constexpr (RAW != 0) {
+    if constexpr (RAW != 0 && !DMA) {
       if (FULL) stage = min(stage, n_stages_ - 1);
       const bool ok = FULL || ((c < K) && (stage < n_stages_));
       const unsigned t = (unsigned)stage * (unsigned)K + (unsigned)c;
@@ -350,7 +362,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   };
   // own features of a mini-batch: rotate, keep (own-feature operands of dst), share through LDS buffer `pb`, store
   auto rotate_share = [&](const RawIn& r, StageInMw<T, NT, TPW>& dst, int stage, int pb) {
-    if constexpr (RAW != 0) {
+    if constexpr (RAW != 0 && !DMA) {
       const bool tok = FULL || c < K;
 #pragma unroll
       for (int jj = 0; jj < TPW; ++jj) {
@@ -417,7 +429,7 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
   };
   // the full rotated rows of a mini-batch, from LDS buffer `pb` (behind a barrier that follows rotate_share)
   auto gather_rows = [&](StageInMw<T, NT, TPW>& dst, int pb) {
-    if constexpr (RAW != 0) {
+    if constexpr (RAW != 0 && !DMA) {
       const u32x4* xb = xrot + (size_t)pb * 2 * (NT / 2) * 64;
 #pragma unroll
       for (int q = 0; q < NT / 2; ++q) {
@@ -429,7 +441,65 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
       }
     }
   };
-  if constexpr (RAW != 0) {
+  // ---- RAW = 5: the ring the control wave fills, and the control wave itself
+  constexpr int RS = 4;                                  // slots = mini-batches in flight
+  constexpr int kCopies = 3 * NT + 1;                    // copies per mini-batch: the tile rows of xq, xk, xv, and lr
+  __shared__ f32x4 ring_s[DMA ? RS : 1][3][DMA ? NT : 1][64];  // [slot][xq, xk, xv][feature tile][lane]
+  __shared__ float ringlr_s[DMA ? RS : 1][64];           // lr of the lane's token c
+  auto gather_dma = [&](StageInMw<T, NT, TPW>& dst, int stage) {
+    if constexpr (DMA) {
+      static_assert(!BF && TPW == 1 && FULL && !FAC, "control-wave loads: f32 I/O, one feature tile per wave, whole mini-batches");
+      const int sl = stage & (RS - 1);
+#pragma unroll
+      for (int J = 0; J < NT; ++J) {
+        dst.q[J] = ring_s[sl][0][J][lane];
+        dst.k[J] = ring_s[sl][1][J][lane];
+      }
+      dst.qo[0] = ring_s[sl][0][w][lane];
+      dst.ko[0] = ring_s[sl][1][w][lane];
+      dst.vo[0] = ring_s[sl][2][w][lane];
+      dst.lr = ringlr_s[sl][c];
+    }
+  };
+  if constexpr (DMA) {
+    if (ctlw) {
+      const unsigned ring0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)&ring_s[0][0][0][0];
+      const unsigned lr0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)&ringlr_s[0][0];
+      // the copies of one mini-batch (past the end: the last one again, into a slot nobody reads)
+      auto copy_in = [&](int stage) {
+        const unsigned dst = ring0 + (unsigned)(stage & (RS - 1)) * (3 * NT * 1024);
+        const int st_ld = min(stage, n_stages_ - 1);
+        const unsigned off = UnitBase<T, D>::row_off(st_ld, K, c);
+#pragma unroll
+        for (int J = 0; J < NT; ++J) {
+          const unsigned fo = (unsigned)(32 * (J >> 1) + 8 * g + 4 * (J & 1)) * 4u;  // the lane's four features of tile J
+          lds_dma16(ub.xq, off + fo, dst + (0 * NT + J) * 1024);
+          lds_dma16(ub.xk, off + fo, dst + (1 * NT + J) * 1024);
+          lds_dma16(ub.xv, off + fo, dst + (2 * NT + J) * 1024);
+        }
+        // every lane issues (the count of copies in flight must not depend on the lane): lanes 16.. repeat token c's
+        lds_dma4(ub.lr, ((unsigned)st_ld * (unsigned)K + (unsigned)c) * 4u, lr0 + (unsigned)(stage & (RS - 1)) * 256u);
+      };
+#pragma unroll
+      for (int u = 0; u < RS; ++u) copy_in(u);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RS - 1) * kCopies) : "memory");  // mini-batch 0 has landed
+      asm volatile("s_barrier" ::: "memory");
+      for (int st = 0; st < n_stages_; ++st) {
+        // mini-batch st + 1 has landed (st + 2 .. st + RS - 1 may be in flight); behind the barrier the compute waves
+        // read it, and the slot of mini-batch st, read behind the barrier before, is free
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((RS - 2) * kCopies) : "memory");
+        asm volatile("s_barrier" ::: "memory");
+        copy_in(st + RS);
+      }
+      asm volatile("s_barrier" ::: "memory");  // the exchange that flushes the last output
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      return;
+    }
+  }
+  if constexpr (DMA) {
+    lds_barrier();
+    gather_dma(buf[0], 0);
+  } else if constexpr (RAW != 0) {
     // mini-batch 0 complete, mini-batch 1 rotated and on its way through LDS (read behind the first barrier of the
     // loop), the raw rows of mini-batch 2 in flight
 #pragma unroll
@@ -543,7 +613,8 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
       if (!CHECKED || st > 1) emit_output(so0, so1, st - 2, zbo, qoo);
       exchange8_collect(S, st & 1);
       // RAW: the rows of the next mini-batch, rotated by their owners before this barrier
-      if constexpr (RAW != 0) gather_rows(buf[(u + 1) % R], (st + 1) & 1);
+      if constexpr (DMA) gather_dma(buf[(u + 1) % R], st + 1);
+      else if constexpr (RAW != 0) gather_rows(buf[(u + 1) % R], (st + 1) & 1);
       so0 = S[6];
       so1 = S[7];
 #pragma unroll
@@ -813,6 +884,12 @@ __device__ __forceinline__ void linear_fwd_sk_body(const LinearFwdArgs& a, const
 template <class T, int D, int NW, int PF, bool FULL, bool FAC = false, int OWN = 0>
 __global__ void __launch_bounds__(64 * NW) ttt_linear_fwd_sk_kernel(Problems<LinearFwdArgs> problems) {
   linear_fwd_sk_body<T, D, NW, PF, FULL, FAC, OWN == 0 ? 0 : OWN + 2>(problems.p[blockIdx.y], nullptr);
+}
+
+// The forward with a control wave that brings the operands in: see RAW = 5 above.
+template <class T, int D, int NW, int PF>
+__global__ void __launch_bounds__(64 * (NW + 1)) ttt_linear_fwd_dma_kernel(Problems<LinearFwdArgs> problems) {
+  linear_fwd_sk_body<T, D, NW, PF, true, false, 5>(problems.p[blockIdx.y], nullptr);
 }
 
 // TTT-Linear with the Adam inner optimiser: see ADAM above.
