@@ -249,8 +249,8 @@ int ttt_linear_bwd_ws(const ttt_desc* desc, const void* xq, const void* xk, cons
  * A caller that shares the GPU checks one output element per unit, reads the status word below, or passes
  * TTT_HINT_LDS_TILES to use the single-workgroup kernel (slower, f32 products).
  *
- * ttt_mlp_fwd_lost_workgroups: the device's status word of that kernel (and of ttt_mlp_bwd's kernel on two
- * workgroups per unit, see there), the number of workgroups whose wait for
+ * ttt_mlp_fwd_lost_workgroups: the device's status word of that kernel (and of the kernels of ttt_mlp_bwd and
+ * ttt_linear_bwd_ws on two workgroups per unit, see there), the number of workgroups whose wait for
  * their partner ran out since the library was loaded on the current device (0 on a healthy run; it never
  * decreases, compare with the value before the call).  A blocking copy from the device: call it after the
  * stream's work has finished.  No counterpart in the reference.
@@ -388,6 +388,10 @@ int ttt_mlp_bwd_static(const ttt_desc* desc, const void* xq, const void* xk, con
  * copy of every layer's state).  `out` doubles as the hand-over tensor between layers:
  * it holds intermediate layers' outputs while the call runs.
  * checkpoint fields of desc are ignored (forward only); seq_stride must be 0.
+ * A stack that holds a TTT-MLP layer at head_dim 128 with bf16 I/O runs the two-CU kernel of ttt_mlp_fwd, and what is
+ * said there of a GPU shared with other work holds: the call returns when the work is enqueued, so a caller compares
+ * ttt_mlp_fwd_lost_workgroups before the call and after the stream's work has finished (an affected unit's outputs
+ * are NaN from that layer on).
  */
 #define TTT_LAYER_LINEAR 0
 #define TTT_LAYER_MLP 1
